@@ -1,0 +1,190 @@
+/*
+ * lightop_mi355 - C ABI of the block-INT8 fused-MoE path for AMD Instinct MI355X (gfx950).
+ *
+ * Every entry point takes raw device pointers, extents and a HIP stream, launches
+ * on that stream, never synchronises, never reads device results on the host and
+ * never allocates.  Return value: 0 on success, a negative LO_E* code otherwise;
+ * lo_last_error() returns a thread-local description of the last failure.
+ *
+ * Each function names the reference interface it replaces (paths relative to the
+ * HYGON-AI/lightop tree).
+ */
+#ifndef LIGHTOP_MI355_H
+#define LIGHTOP_MI355_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *lo_stream_t; /* hipStream_t */
+
+enum {
+  LO_OK = 0,
+  LO_EINVAL = -1,   /* bad shape, alignment, dtype or null pointer */
+  LO_ENOSPC = -2,   /* caller buffer / workspace too small */
+  LO_ELAUNCH = -3,  /* hipGetLastError() after a launch */
+  LO_ENOTSUP = -4   /* valid request that this build has no kernel for */
+};
+
+/* activation element types */
+enum { LO_BF16 = 0, LO_F16 = 1 };
+/* index element types of topk_ids */
+enum { LO_I32 = 0, LO_I64 = 1 };
+
+/* flags of lo_moe_gemm_block_int8 / lo_fused_experts_block_int8 */
+enum {
+  LO_GEMM_DEFAULT = 0,
+  /* accumulate acc += f32(d) * (a_s * b_s) with one fused multiply-add per
+   * 128-K block instead of the canonical (f32(d) * a_s) * b_s then add.  The
+   * int32 partial sums are identical; the fp32 rounding differs in the last ulp. */
+  LO_GEMM_FUSED_SCALE = 1
+};
+
+int lo_version(void);
+const char *lo_last_error(void);
+
+/*
+ * Routing alignment.
+ * Replaces op.moe_align_block_size (csrc/pybind/export.cpp:1593-1605,
+ * csrc/kernels/moe_align_sum_kernels.cu:1210-1314) together with the
+ * expert_map post-mapping of python/lightop/_lmslim_native/vllm_compat/
+ * moe_align_block_size.py:117-118.
+ *
+ *   topk_ids      [numel] int32 or int64 (ids_dtype = LO_I32 / LO_I64), values in [0, num_experts)
+ *   expert_map    [num_experts] int32 or NULL
+ *   ignore_invalid 0: count on the given ids, expert_ids[b] = expert_map[e] (or e)
+ *                  1: drop ids whose expert_map entry is -1, count on mapped ids
+ *   sorted_ids    [sorted_cap] int32  - slot ids grouped by expert, ascending inside an
+ *                                       expert, every other entry = numel
+ *   expert_ids    [expert_ids_cap] int32 - expert of each block, -1 past the last block
+ *   num_tokens_post_pad [1] int32
+ * sorted_cap must be >= numel + num_experts*(block_size-1) or numel*block_size,
+ * whichever is smaller; expert_ids_cap >= ceil(sorted_cap / block_size).
+ */
+int lo_moe_align_block_size(const void *topk_ids, int ids_dtype, int64_t numel,
+                            int32_t num_experts, int32_t block_size,
+                            const int32_t *expert_map, int ignore_invalid,
+                            int32_t *sorted_ids, int64_t sorted_cap,
+                            int32_t *expert_ids, int64_t expert_ids_cap,
+                            int32_t *num_tokens_post_pad, lo_stream_t stream);
+
+/*
+ * 1x128 group quantisation of activations to int8 with fp32 scales.
+ * Replaces per_token_group_quant_int8 (python/lightop/_lmslim_native/layers/gemm/
+ * int8_utils.py:125-195, Triton kernel :74-122).
+ *   x [rows, cols] contiguous, cols % 128 == 0;  q [rows, cols] int8;  s [rows, cols/128] f32
+ *   amax = max(max|x|, eps); s = amax / 127; q = trunc(clamp(x / s, -128, 127))
+ */
+int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t rows, int64_t cols,
+                                  float eps, int8_t *q, float *s, lo_stream_t stream);
+
+/*
+ * One grouped GEMM stage over the aligned routing.
+ * Replaces invoke_fused_moe_kernel_int8 / Triton fused_moe_kernel
+ * (python/lightop/_lmslim_native/layers/fused_moe/int8.py:543-626, :320-541) for
+ * use_int8_w8a8=True, block_shape=[128,128].
+ *
+ *   A  [a_rows, K] int8;  As [a_rows, K/128] f32;  the row of slot f is f / top_k
+ *   W  [E, N, K] int8 (K contiguous);  Ws [E, ceil(N/128), K/128] f32
+ *   C  [num_valid, N] c_dtype, row f;  rows of blocks whose expert id is -1 are zeroed
+ *   topk_w [num_valid] f32, used when mul_routed != 0
+ *   sorted_ids / expert_ids / num_tokens_post_pad as produced by lo_moe_align_block_size
+ *   with block_size == block_size_m; sorted_cap is the extent of sorted_ids.
+ * K % 128 == 0, N % 16 == 0.
+ */
+int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W, const float *Ws,
+                           void *C, int c_dtype, const float *topk_w, const int32_t *sorted_ids,
+                           const int32_t *expert_ids, const int32_t *num_tokens_post_pad,
+                           int64_t sorted_cap, int64_t num_valid, int64_t a_rows, int32_t E,
+                           int64_t N, int64_t K, int32_t top_k, int32_t block_size_m,
+                           int mul_routed, int flags, lo_stream_t stream);
+
+/*
+ * First grouped GEMM with the activation fused into its epilogue:
+ * GEMM1 -> bf16 round -> SiLU(gate) * up -> 1x128 group quant, i.e. the sequence
+ * int8.py:784-823 without materialising intermediate_cache1 / intermediate_cache2.
+ *   W [E, 2I, K] (gate rows first, then up rows), Ws [E, 2I/128, K/128]
+ *   A2q [num_valid, I] int8, A2s [num_valid, I/128] f32 (rows of -1 blocks untouched)
+ * I % 128 == 0, K % 128 == 0.
+ */
+int lo_moe_gemm1_silu_quant_block_int8(const int8_t *A, const float *As, const int8_t *W,
+                                       const float *Ws, int8_t *A2q, float *A2s, int c_dtype,
+                                       const float *topk_w, const int32_t *sorted_ids,
+                                       const int32_t *expert_ids,
+                                       const int32_t *num_tokens_post_pad, int64_t sorted_cap,
+                                       int64_t num_valid, int64_t a_rows, int32_t E, int64_t I,
+                                       int64_t K, int32_t top_k, int32_t block_size_m,
+                                       int mul_routed, int flags, lo_stream_t stream);
+
+/*
+ * SiLU-and-mul: act[f, i] = T( T(silu(c1[f, i])) * c1[f, I + i] ).
+ * Replaces torch.ops._C.silu_and_mul at int8.py:811 (in-repo twin:
+ * csrc/kernels/gated_activation/fuse_silu_mul_quant.cu:893-905).
+ */
+int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *act,
+                    lo_stream_t stream);
+
+/*
+ * Top-k reduction back to token order: out[t, :] = factor * sum_j in[t, j, :] (+ bias[t, :]).
+ * Replaces op.moe_sum (csrc/pybind/export.cpp:1584-1592,
+ * csrc/kernels/moe_align_sum_kernels.cu:1315-2092).  fp32 accumulation in slot
+ * order; without bias one rounding (:619-633), with bias the three roundings of :886-909.
+ */
+int lo_moe_sum(const void *in, void *out, const void *bias, int dtype, int64_t M, int32_t topk,
+               int64_t H, float factor, lo_stream_t stream);
+
+/*
+ * Tile table: block_size_m (the alignment block and GEMM token tile) chosen for a
+ * problem.  Replaces get_w8a8moe_json / W8a8GetCacheJSON (int8.py:220-256,
+ * vllm_compat/w8a8_get_cache_json.py:12-174) and the per-device JSON files
+ * configs/w8a8/MOE_BLOCKINT8[128,128]_*.json.
+ */
+typedef struct lo_moe_tile {
+  int32_t block_size_m; /* 16, 32, 64 or 128 */
+  int32_t kernel;       /* implementation id, for reporting */
+  int32_t waves;        /* wavefronts per workgroup */
+  int32_t block_n;      /* weight rows per workgroup */
+} lo_moe_tile;
+
+int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k, int64_t H,
+                      int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2);
+
+/*
+ * Whole path for one chunk of tokens: quant -> align -> GEMM1(+SiLU*mul+quant) -> GEMM2
+ * -> weighted top-k reduce.  Replaces the body of fused_experts_impl_int8
+ * (int8.py:703-888); the reduce is always performed.
+ *
+ *   x [M, H] bf16;  w1 [E, 2I, H], w2 [E, H, I] int8;  w1s [E, 2I/128, H/128], w2s [E, H/128, I/128]
+ *   topk_w [M, top_k] f32;  topk_ids [M, top_k] int32/int64;  expert_map [num_experts] or NULL
+ *   cache3 [M*top_k, H] act dtype: the caller's cache13 workspace (second GEMM's output)
+ *   shared_output [M, H] or NULL;  out [M, H]
+ *   workspace: lo_fused_experts_workspace_bytes(...) bytes of device memory, 256-byte aligned
+ *   block_size_m: 0 = take it from the tile table
+ */
+int64_t lo_fused_experts_workspace_bytes(int64_t M, int32_t top_k, int64_t H, int64_t I,
+                                         int32_t num_experts, int32_t block_size_m);
+
+int lo_fused_experts_block_int8(const void *x, int dtype, int64_t M, int64_t H, int64_t I,
+                                int32_t E, int32_t num_experts, int32_t top_k, const int8_t *w1,
+                                const float *w1s, const int8_t *w2, const float *w2s,
+                                const float *topk_w, const void *topk_ids, int ids_dtype,
+                                const int32_t *expert_map, int apply_router_weight_on_input,
+                                float routed_scaling_factor, const void *shared_output,
+                                void *cache3, void *out, void *workspace, int64_t workspace_bytes,
+                                int32_t block_size_m, int flags, lo_stream_t stream);
+
+/*
+ * Views into the workspace of the last layout computed for the same arguments, so
+ * that tests can read every intermediate of lo_fused_experts_block_int8:
+ * which = 0 a1q, 1 a1s, 2 sorted_ids, 3 expert_ids, 4 num_tokens_post_pad, 5 a2q, 6 a2s.
+ * Returns the byte offset inside the workspace or a negative error.
+ */
+int64_t lo_fused_experts_workspace_offset(int which, int64_t M, int32_t top_k, int64_t H, int64_t I,
+                                          int32_t num_experts, int32_t block_size_m);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LIGHTOP_MI355_H */

@@ -1,0 +1,81 @@
+"""ctypes binding of the C ABI declared in include/lightop_mi355.h."""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(_CSRC, "liblightop_mi355.so")
+
+LO_BF16, LO_F16 = 0, 1
+LO_I32, LO_I64 = 0, 1
+LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE = 0, 1
+
+
+class LoMoeTile(ctypes.Structure):
+    _fields_ = [("block_size_m", c_int32), ("kernel", c_int32), ("waves", c_int32), ("block_n", c_int32)]
+
+
+# name -> (restype, argtypes); must list every symbol of include/lightop_mi355.h
+SIGNATURES = {
+    "lo_version": (c_int, []),
+    "lo_last_error": (c_char_p, []),
+    "lo_moe_align_block_size": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,
+                                        c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
+    "lo_per_token_group_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_float, c_void_p,
+                                              c_void_p, c_void_p]),
+    "lo_moe_gemm_block_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                       c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32,
+                                       c_int64, c_int64, c_int32, c_int32, c_int, c_int, c_void_p]),
+    "lo_moe_gemm1_silu_quant_block_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                   c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                   c_int64, c_int64, c_int64, c_int32, c_int64, c_int64,
+                                                   c_int32, c_int32, c_int, c_int, c_void_p]),
+    "lo_silu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
+    "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float, c_void_p]),
+    "lo_moe_tile_query": (c_int, [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
+                                  ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
+    "lo_fused_experts_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
+    "lo_fused_experts_workspace_offset": (c_int64, [c_int, c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
+    "lo_fused_experts_block_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int32, c_int32,
+                                            c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_int64, c_int32, c_int, c_void_p]),
+}
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded HIP library.  A missing library is an error: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m lightop_amd.build` "
+                "(lightop_amd has no CPU or PyTorch fallback)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc: int) -> None:
+    """Map a negative return code to RuntimeError, as TORCH_CHECK does in the reference."""
+    if rc < 0:
+        msg = lib().lo_last_error()
+        raise RuntimeError(f"lightop_amd: {msg.decode() if msg else 'error'} (code {rc})")
+
+
+def ptr(t) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def stream_of(t) -> c_void_p:
+    import torch
+
+    return c_void_p(torch.cuda.current_stream(t.device).cuda_stream)

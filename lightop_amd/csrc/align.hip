@@ -1,0 +1,184 @@
+// moe_align_block_size for gfx950: expert histogram, padded prefix sum and a stable
+// (ascending slot id) counting sort, in one workgroup, with wavefront ballots and
+// LDS counters and no atomics on the ranking path, so the result is deterministic.
+//
+// Semantics follow python/lightop/_lmslim_native/vllm_compat/moe_align_block_size.py:17-120
+// and csrc/kernels/moe_align_sum_kernels.cu:1034-1115 of the reference; the order
+// inside an expert is the ascending one of test/test_moe_align_block_size.py:81-88.
+#include "common.h"
+
+namespace lo {
+
+// Lanes of the wave that hold the same key as this lane (key < 2^bits), as a mask.
+__device__ __forceinline__ uint64_t match_any(int key, int bits, bool active) {
+  uint64_t peers = __ballot(active);
+  for (int b = 0; b < bits; ++b) {
+    uint64_t set = __ballot(active && ((key >> b) & 1));
+    peers &= ((key >> b) & 1) ? set : ~set;
+  }
+  return peers;
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(1024) void moe_align_kernel(
+    const IdT *__restrict__ ids, int64_t numel, int num_experts, int bs,
+    const int32_t *__restrict__ expert_map, int ignore_invalid, int32_t *__restrict__ sorted,
+    int64_t sorted_cap, int32_t *__restrict__ expert_ids, int64_t expert_ids_cap,
+    int32_t *__restrict__ ntpp, int key_bits) {
+  extern __shared__ int32_t lds[];
+  const int nw = blockDim.x / kWave;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int E = num_experts;
+  int32_t *offs = lds;               // [E + 1] padded exclusive prefix
+  int32_t *total = lds + (E + 1);    // [E] tokens per expert
+  int32_t *wcnt = total + E;         // [nw][E] per-wave counts, later running bases
+
+  for (int i = tid; i < nw * E; i += blockDim.x) wcnt[i] = 0;
+  __syncthreads();
+
+  // Each wave owns a contiguous range of slot ids, rounded to whole 64-id tiles.
+  const int64_t tiles = (numel + kWave - 1) / kWave;
+  const int64_t tiles_per_wave = (tiles + nw - 1) / nw;
+  const int64_t t0 = wave * tiles_per_wave;
+  const int64_t t1 = (t0 + tiles_per_wave < tiles) ? t0 + tiles_per_wave : tiles;
+
+  auto key_of = [&](int64_t f, bool &ok) -> int {
+    ok = f < numel;
+    int e = 0;
+    if (ok) {
+      int64_t raw = static_cast<int64_t>(ids[f]);
+      ok = raw >= 0 && raw < E;
+      e = ok ? static_cast<int>(raw) : 0;
+      if (ok && ignore_invalid && expert_map) {
+        e = expert_map[e];
+        ok = e >= 0 && e < E;
+        if (!ok) e = 0;
+      }
+    }
+    return e;
+  };
+
+  // pass 1: per-wave histogram
+  for (int64_t t = t0; t < t1; ++t) {
+    bool ok;
+    int e = key_of(t * kWave + lane, ok);
+    uint64_t peers = match_any(e, key_bits, ok);
+    if (ok) {
+      int leader = __ffsll(static_cast<unsigned long long>(peers)) - 1;
+      if (lane == leader) wcnt[wave * E + e] += __popcll(peers);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  __syncthreads();
+
+  // pass 2: totals, padded sizes, exclusive scan over experts (one thread per
+  // expert; wave-level inclusive scan, then a scan over wave sums)
+  __shared__ int32_t wave_sum[16];
+  for (int base = 0; base < E; base += blockDim.x) {
+    int e = base + tid;
+    int c = 0;
+    if (e < E) {
+      for (int w = 0; w < nw; ++w) {
+        int v = wcnt[w * E + e];
+        wcnt[w * E + e] = c; // tokens of expert e held by earlier waves
+        c += v;
+      }
+      total[e] = c;
+    }
+    int padded = (e < E) ? (c + bs - 1) / bs * bs : 0;
+    int incl = padded;
+    for (int d = 1; d < kWave; d <<= 1) {
+      int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) wave_sum[wave] = incl;
+    __syncthreads();
+    int carry = (base == 0) ? 0 : offs[base];
+    for (int w = 0; w < wave; ++w) carry += wave_sum[w];
+    if (e < E) offs[e + 1] = carry + incl;
+    if (base == 0 && tid == 0) offs[0] = 0;
+    __syncthreads();
+  }
+  const int P = offs[E];
+  if (tid == 0) ntpp[0] = P;
+
+  // expert id of every block; -1 past the last block
+  for (int e = tid; e < E; e += blockDim.x) {
+    int v = (expert_map && !ignore_invalid) ? expert_map[e] : e;
+    for (int b = offs[e] / bs; b < offs[e + 1] / bs; ++b) expert_ids[b] = v;
+  }
+  for (int64_t b = P / bs + tid; b < expert_ids_cap; b += blockDim.x) expert_ids[b] = -1;
+
+  // padding entries: the tail of every expert's range and everything past P
+  for (int e = wave; e < E; e += nw)
+    for (int i = offs[e] + total[e] + lane; i < offs[e + 1]; i += kWave)
+      sorted[i] = static_cast<int32_t>(numel);
+  for (int64_t i = P + tid; i < sorted_cap; i += blockDim.x) sorted[i] = static_cast<int32_t>(numel);
+
+  // pass 3: stable scatter.  wcnt[wave][e] is the running number of slots of expert
+  // e that precede the current tile.
+  for (int64_t t = t0; t < t1; ++t) {
+    bool ok;
+    int64_t f = t * kWave + lane;
+    int e = key_of(f, ok);
+    uint64_t peers = match_any(e, key_bits, ok);
+    if (ok) {
+      int before = __popcll(peers & ((1ull << lane) - 1ull));
+      int leader = __ffsll(static_cast<unsigned long long>(peers)) - 1;
+      int base = wcnt[wave * E + e];
+      sorted[offs[e] + base + before] = static_cast<int32_t>(f);
+      __builtin_amdgcn_wave_barrier();
+      if (lane == leader) wcnt[wave * E + e] = base + __popcll(peers);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+} // namespace lo
+
+extern "C" int lo_moe_align_block_size(const void *topk_ids, int ids_dtype, int64_t numel,
+                                       int32_t num_experts, int32_t block_size,
+                                       const int32_t *expert_map, int ignore_invalid,
+                                       int32_t *sorted_ids, int64_t sorted_cap,
+                                       int32_t *expert_ids, int64_t expert_ids_cap,
+                                       int32_t *num_tokens_post_pad, lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(topk_ids && sorted_ids && expert_ids && num_tokens_post_pad, LO_EINVAL,
+             "moe_align_block_size: null pointer");
+  LO_REQUIRE(ids_dtype == LO_I32 || ids_dtype == LO_I64, LO_EINVAL,
+             "moe_align_block_size: topk_ids must be int32 or int64");
+  LO_REQUIRE(numel >= 0 && numel < (1ll << 31) - 1, LO_EINVAL, "moe_align_block_size: bad numel %lld",
+             (long long)numel);
+  LO_REQUIRE(num_experts >= 1 && num_experts <= 2048, LO_EINVAL,
+             "moe_align_block_size: num_experts %d outside [1, 2048]", num_experts);
+  LO_REQUIRE(block_size >= 1, LO_EINVAL, "moe_align_block_size: block_size %d", block_size);
+  int64_t need = numel + static_cast<int64_t>(num_experts) * (block_size - 1);
+  if (numel < num_experts && numel * block_size < need) need = numel * block_size;
+  LO_REQUIRE(sorted_cap >= need, LO_ENOSPC, "moe_align_block_size: sorted_ids holds %lld, needs %lld",
+             (long long)sorted_cap, (long long)need);
+  LO_REQUIRE(expert_ids_cap >= (need + block_size - 1) / block_size, LO_ENOSPC,
+             "moe_align_block_size: expert_ids holds %lld, needs %lld", (long long)expert_ids_cap,
+             (long long)((need + block_size - 1) / block_size));
+
+  // waves per workgroup: as many as the per-wave LDS counters allow (<= 60 KB)
+  int nw = 16;
+  while (nw > 1 && (static_cast<int64_t>(nw) + 2) * num_experts + 1 > 15360) nw >>= 1;
+  if (numel <= 64 * 4) nw = nw < 4 ? nw : 4;
+  size_t lds_bytes = (static_cast<size_t>(nw + 2) * num_experts + 1) * sizeof(int32_t);
+  int key_bits = 1;
+  while ((1 << key_bits) < num_experts) ++key_bits;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (ids_dtype == LO_I32)
+    hipLaunchKernelGGL(moe_align_kernel<int32_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
+                       static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,
+                       expert_map, ignore_invalid, sorted_ids, sorted_cap, expert_ids,
+                       expert_ids_cap, num_tokens_post_pad, key_bits);
+  else
+    hipLaunchKernelGGL(moe_align_kernel<int64_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
+                       static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size,
+                       expert_map, ignore_invalid, sorted_ids, sorted_cap, expert_ids,
+                       expert_ids_cap, num_tokens_post_pad, key_bits);
+  return check_launch("moe_align_block_size");
+}

@@ -1,0 +1,162 @@
+// Host side of the C ABI: error reporting, the gfx950 tile table and the whole-path
+// entry point that chains the stage kernels on one stream.
+#include <cstdarg>
+#include <cstdio>
+
+#include "common.h"
+
+namespace lo {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return LO_ELAUNCH;
+  }
+  return LO_OK;
+}
+
+static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+// Extents of the alignment buffers (moe_align_block_size.py:80-93 of the reference).
+static void align_caps(int64_t numel, int32_t num_experts, int32_t bs, int64_t *sorted_cap,
+                       int64_t *blocks_cap) {
+  int64_t cap = numel + static_cast<int64_t>(num_experts) * (bs - 1);
+  if (numel < num_experts && numel * bs < cap) cap = numel * bs;
+  *sorted_cap = cap;
+  *blocks_cap = (cap + bs - 1) / bs;
+}
+
+struct WsLayout {
+  int64_t off[7];
+  int64_t total;
+  int64_t sorted_cap, blocks_cap;
+};
+
+static WsLayout ws_layout(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_t num_experts,
+                          int32_t bs) {
+  WsLayout L{};
+  const int64_t S = M * top_k;
+  align_caps(S, num_experts, bs, &L.sorted_cap, &L.blocks_cap);
+  const int64_t sizes[7] = {M * H,                 // a1q
+                            M * (H / kGroup) * 4,  // a1s
+                            L.sorted_cap * 4,      // sorted_ids
+                            L.blocks_cap * 4,      // expert_ids
+                            4,                     // num_tokens_post_pad
+                            S * I,                 // a2q
+                            S * (I / kGroup) * 4}; // a2s
+  int64_t o = 0;
+  for (int i = 0; i < 7; ++i) {
+    L.off[i] = o;
+    o += align_up(sizes[i] > 0 ? sizes[i] : 1, 256);
+  }
+  L.total = o;
+  return L;
+}
+
+// gfx950 tile table.  The token tile (= alignment block) follows the expected number
+// of slots per expert: small tiles waste no MFMA columns on padding while the layer
+// is weight-streaming bound, larger ones amortise each pass over an expert's weights.
+static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k) {
+  const double per_expert = static_cast<double>(M) * top_k / (num_experts > 0 ? num_experts : 1);
+  if (per_expert <= 12.0) return 16;
+  if (per_expert <= 24.0) return 32;
+  if (per_expert <= 96.0) return 64;
+  return 128;
+}
+
+} // namespace lo
+
+extern "C" int lo_version(void) { return 100; }
+
+extern "C" const char *lo_last_error(void) { return lo::g_err; }
+
+extern "C" int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
+                                 int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
+  using namespace lo;
+  (void)E_local;
+  LO_REQUIRE(M >= 0 && num_experts >= 1 && top_k >= 1 && H > 0 && I > 0, LO_EINVAL,
+             "moe_tile_query: bad problem size");
+  const int32_t bm = pick_block_m(M, num_experts, top_k);
+  if (gemm1) *gemm1 = lo_moe_tile{bm, 1, 8, 256};
+  if (gemm2) *gemm2 = lo_moe_tile{bm, 0, 4, 64};
+  return LO_OK;
+}
+
+extern "C" int64_t lo_fused_experts_workspace_bytes(int64_t M, int32_t top_k, int64_t H, int64_t I,
+                                                    int32_t num_experts, int32_t block_size_m) {
+  using namespace lo;
+  if (M < 0 || top_k < 1 || H < kGroup || I < kGroup || num_experts < 1) return LO_EINVAL;
+  if (block_size_m == 0) block_size_m = 128; // the largest tile bounds every choice of the table
+  return ws_layout(M, top_k, H, I, num_experts, block_size_m).total + 256;
+}
+
+extern "C" int64_t lo_fused_experts_workspace_offset(int which, int64_t M, int32_t top_k, int64_t H,
+                                                     int64_t I, int32_t num_experts,
+                                                     int32_t block_size_m) {
+  using namespace lo;
+  if (which < 0 || which > 6 || block_size_m <= 0) return LO_EINVAL;
+  return ws_layout(M, top_k, H, I, num_experts, block_size_m).off[which];
+}
+
+extern "C" int lo_fused_experts_block_int8(
+    const void *x, int dtype, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts,
+    int32_t top_k, const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s,
+    const float *topk_w, const void *topk_ids, int ids_dtype, const int32_t *expert_map,
+    int apply_router_weight_on_input, float routed_scaling_factor, const void *shared_output,
+    void *cache3, void *out, void *workspace, int64_t workspace_bytes, int32_t block_size_m,
+    int flags, lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(x && w1 && w1s && w2 && w2s && topk_w && topk_ids && cache3 && out && workspace,
+             LO_EINVAL, "fused_experts: null pointer");
+  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "fused_experts: only bf16 activations are built");
+  LO_REQUIRE(M >= 0 && H >= kGroup && H % kGroup == 0 && I >= kGroup && I % kGroup == 0, LO_EINVAL,
+             "fused_experts: hidden (%lld) and intermediate (%lld) sizes must be multiples of 128",
+             (long long)H, (long long)I);
+  LO_REQUIRE(E >= 1 && num_experts >= E && top_k >= 1, LO_EINVAL, "fused_experts: bad expert counts");
+  LO_REQUIRE(num_experts == E || expert_map, LO_EINVAL,
+             "fused_experts: global_num_experts (%d) != local experts (%d) needs an expert_map",
+             num_experts, E);
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, LO_EINVAL,
+             "fused_experts: workspace must be 256-byte aligned");
+  if (M == 0) return LO_OK;
+  if (block_size_m == 0) block_size_m = pick_block_m(M, num_experts, top_k);
+  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
+             LO_EINVAL, "fused_experts: block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
+  const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
+  LO_REQUIRE(workspace_bytes >= L.total, LO_ENOSPC, "fused_experts: workspace holds %lld bytes, needs %lld",
+             (long long)workspace_bytes, (long long)L.total);
+  char *ws = static_cast<char *>(workspace);
+  int8_t *a1q = reinterpret_cast<int8_t *>(ws + L.off[0]);
+  float *a1s = reinterpret_cast<float *>(ws + L.off[1]);
+  int32_t *sorted = reinterpret_cast<int32_t *>(ws + L.off[2]);
+  int32_t *eids = reinterpret_cast<int32_t *>(ws + L.off[3]);
+  int32_t *ntpp = reinterpret_cast<int32_t *>(ws + L.off[4]);
+  int8_t *a2q = reinterpret_cast<int8_t *>(ws + L.off[5]);
+  float *a2s = reinterpret_cast<float *>(ws + L.off[6]);
+  const int64_t S = M * top_k;
+
+  int rc = lo_per_token_group_quant_int8(x, dtype, M, H, 1e-10f, a1q, a1s, stream);
+  if (rc) return rc;
+  rc = lo_moe_align_block_size(topk_ids, ids_dtype, S, num_experts, block_size_m, expert_map, 0,
+                               sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, stream);
+  if (rc) return rc;
+  rc = lo_moe_gemm1_silu_quant_block_int8(a1q, a1s, w1, w1s, a2q, a2s, dtype, topk_w, sorted, eids,
+                                          ntpp, L.sorted_cap, S, M, E, I, H, top_k, block_size_m,
+                                          apply_router_weight_on_input, flags, stream);
+  if (rc) return rc;
+  rc = lo_moe_gemm_block_int8(a2q, a2s, w2, w2s, cache3, dtype, topk_w, sorted, eids, ntpp,
+                              L.sorted_cap, S, S, E, H, I, 1, block_size_m,
+                              !apply_router_weight_on_input, flags, stream);
+  if (rc) return rc;
+  return lo_moe_sum(cache3, out, shared_output, dtype, M, top_k, H, routed_scaling_factor, stream);
+}

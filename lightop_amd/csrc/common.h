@@ -1,0 +1,106 @@
+// Shared device/host helpers of the gfx950 block-INT8 fused-MoE kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/lightop_mi355.h"
+
+namespace lo {
+
+constexpr int kWave = 64;   // CDNA wavefront
+constexpr int kGroup = 128; // quantisation group along K and weight block edge
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned short v4u16 __attribute__((ext_vector_type(4)));
+typedef unsigned short v8u16 __attribute__((ext_vector_type(8)));
+
+// ---- error reporting (host) -------------------------------------------------
+void set_error(const char *fmt, ...);
+int check_launch(const char *what);
+
+#define LO_REQUIRE(cond, code, ...)  \
+  do {                               \
+    if (!(cond)) {                   \
+      ::lo::set_error(__VA_ARGS__);  \
+      return (code);                 \
+    }                                \
+  } while (0)
+
+// ---- 16-bit float helpers (device) ------------------------------------------
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+  return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+
+// Round-to-nearest-even; NaN stays a quiet NaN.
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+__device__ __forceinline__ float f16_to_f32(uint16_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, h));
+}
+__device__ __forceinline__ uint16_t f32_to_f16(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+
+template <int DT> __device__ __forceinline__ float to_f32(uint16_t h) {
+  if constexpr (DT == LO_BF16) return bf16_to_f32(h);
+  else return f16_to_f32(h);
+}
+template <int DT> __device__ __forceinline__ uint16_t from_f32(float f) {
+  if constexpr (DT == LO_BF16) return f32_to_bf16(f);
+  else return f32_to_f16(f);
+}
+
+// exp(x) as a fixed sequence of IEEE single operations (Cody-Waite reduction,
+// degree-7 polynomial, exact power-of-two scaling), so that the result does not
+// depend on a math library.  Used for SiLU: g / (1 + exp(-g)).
+__device__ __forceinline__ float det_expf(float x) {
+  if (x > 88.72283f) return __uint_as_float(0x7f800000u);
+  if (x < -87.0f) return 0.0f;
+  float n = __builtin_rintf(x * 1.44269504088896341f);
+  float r = __builtin_fmaf(n, -0.693145751953125f, x);
+  r = __builtin_fmaf(n, -1.42860682030941723212e-6f, r);
+  float p = 1.9841270114e-4f;
+  p = __builtin_fmaf(p, r, 1.3888889225e-3f);
+  p = __builtin_fmaf(p, r, 8.3333337680e-3f);
+  p = __builtin_fmaf(p, r, 4.1666667908e-2f);
+  p = __builtin_fmaf(p, r, 1.6666667163e-1f);
+  p = __builtin_fmaf(p, r, 5.0000000000e-1f);
+  p = __builtin_fmaf(p, r, 1.0f);
+  p = __builtin_fmaf(p, r, 1.0f);
+  int ni = static_cast<int>(n);
+  int h = ni / 2;
+  float a = __uint_as_float(static_cast<uint32_t>(h + 127) << 23);
+  float b = __uint_as_float(static_cast<uint32_t>(ni - h + 127) << 23);
+  return (p * a) * b;
+}
+
+// act = T( T(silu(g)) * u ), everything in fp32 between the roundings.
+template <int DT> __device__ __forceinline__ uint16_t silu_mul(uint16_t g16, uint16_t u16) {
+  float g = to_f32<DT>(g16);
+  float e = det_expf(-g);
+  float sg = to_f32<DT>(from_f32<DT>(g / (1.0f + e)));
+  return from_f32<DT>(sg * to_f32<DT>(u16));
+}
+
+// q = (int8) trunc(clamp(v / s, -128, 127))
+__device__ __forceinline__ int quant_one(float v, float s) {
+  float t = v / s;
+  t = fmaxf(t, -128.0f);
+  t = fminf(t, 127.0f);
+  return static_cast<int>(t);
+}
+
+__device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
+  return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
+         ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+}
+
+} // namespace lo

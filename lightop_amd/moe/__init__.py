@@ -1,0 +1,38 @@
+"""Mixture-of-Experts APIs of the block-INT8 path (reference: python/lightop/moe/__init__.py)."""
+from importlib import import_module
+
+from .cache import get_moe_cache
+from .routing import moe_align_block_size, moe_align_block_size_out, moe_sum
+
+# resolved on first access, like the reference's lazily imported "LMSlim native" entry points
+# (moe/__init__.py:57-78)
+_NATIVE_APIS = {
+    "fused_experts_impl_int8",
+    "get_w8a8moe_json",
+    "invoke_fused_moe_kernel_int8",
+    "invoke_fused_moe_gemm1_silu_quant",
+    "silu_and_mul",
+    "fused_experts_workspace_bytes",
+}
+
+
+def __getattr__(name):
+    if name not in _NATIVE_APIS:
+        raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+    value = getattr(import_module(f"{__name__}.native"), name)
+    globals()[name] = value
+    return value
+
+
+__all__ = [
+    "fused_experts_impl_int8",
+    "fused_experts_workspace_bytes",
+    "get_moe_cache",
+    "get_w8a8moe_json",
+    "invoke_fused_moe_gemm1_silu_quant",
+    "invoke_fused_moe_kernel_int8",
+    "moe_align_block_size",
+    "moe_align_block_size_out",
+    "moe_sum",
+    "silu_and_mul",
+]

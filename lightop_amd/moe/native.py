@@ -1,0 +1,251 @@
+"""Block-INT8 fused experts (reference:
+python/lightop/_lmslim_native/layers/fused_moe/int8.py:543-908)."""
+from __future__ import annotations
+
+from typing import Any, Dict, List, Optional, Tuple
+
+import torch
+
+from .. import _lib, envs
+from ..op import _act_dtype, _ids_dtype, _on_device, _require_cuda
+
+
+def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bool,
+                     block_shape: Optional[List[int]], topk: int,
+                     global_num_experts: int = -1) -> Tuple[Dict[str, Any], Dict[str, Any]]:
+    """Tile configuration of both GEMMs for ``m`` tokens (reference: get_w8a8moe_json,
+    int8.py:220-256, backed there by per-device JSON files).  Here the table is compiled
+    into the library; the dictionaries keep the reference's keys.  ``n1`` = 2*I, ``n2`` = H,
+    ``k`` = I."""
+    del use_int8_w8a8, block_shape
+    t1, t2 = _lib.LoMoeTile(), _lib.LoMoeTile()
+    Eg = E if global_num_experts in (-1, None) else global_num_experts
+    _lib.check(_lib.lib().lo_moe_tile_query(m, E, Eg, topk, n2, k, t1, t2))
+
+    def as_dict(t):
+        return {"BLOCK_SIZE_M": t.block_size_m, "BLOCK_SIZE_N": t.block_n, "BLOCK_SIZE_K": 128,
+                "GROUP_SIZE_M": 1, "num_warps": t.waves, "num_stages": 0, "kernel": t.kernel}
+
+    return as_dict(t1), as_dict(t2)
+
+
+def _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded):
+    _require_cuda(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)
+    assert A.dtype == torch.int8 and B.dtype == torch.int8, "A and B must be int8"
+    assert A.is_contiguous() and A_scale.is_contiguous() and A_scale.dtype == torch.float32
+    assert B.is_contiguous(), "weights must be contiguous [E, N, K]"
+    assert B_scale.is_contiguous() and B_scale.dtype == torch.float32
+    assert sorted_token_ids.stride(0) == 1 and sorted_token_ids.dtype == torch.int32
+    assert expert_ids.dtype == torch.int32 and num_tokens_post_padded.dtype == torch.int32
+    E, N, K = B.shape
+    assert A.shape[1] == K and A_scale.shape == (A.shape[0], K // 128)
+    assert B_scale.shape == (E, (N + 127) // 128, K // 128), "weight scales must be [E, N/128, K/128]"
+
+
+def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
+                                 A_scale: torch.Tensor, B_scale: torch.Tensor,
+                                 topk_weights: Optional[torch.Tensor],
+                                 sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
+                                 num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
+                                 top_k: int, config: Dict[str, Any], fused_scale: bool = False) -> None:
+    """One grouped block-INT8 GEMM stage: C[f] = bf16(sum_kb dot(A[f // top_k], B[e])_kb *
+    A_scale * B_scale) (* topk_weights[f]) for every routed slot f (reference:
+    invoke_fused_moe_kernel_int8, int8.py:543-626).  ``C`` is [M, topk, N] or [S, N]."""
+    assert topk_weights is not None or not mul_routed_weight
+    _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)
+    E, N, K = B.shape
+    assert C.is_contiguous() and C.shape[-1] == N
+    num_valid = C.numel() // N
+    tw = None
+    if topk_weights is not None:
+        tw = topk_weights
+        if tw.dtype != torch.float32 or not tw.is_contiguous():
+            tw = tw.to(torch.float32).contiguous()
+    with _on_device(A):
+        _lib.check(_lib.lib().lo_moe_gemm_block_int8(
+            _lib.ptr(A), _lib.ptr(A_scale), _lib.ptr(B), _lib.ptr(B_scale), _lib.ptr(C), _act_dtype(C),
+            _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(expert_ids),
+            _lib.ptr(num_tokens_post_padded), sorted_token_ids.numel(), num_valid, A.shape[0], E, N, K,
+            int(top_k), int(config["BLOCK_SIZE_M"]), 1 if mul_routed_weight else 0,
+            _lib.LO_GEMM_FUSED_SCALE if fused_scale else 0, _lib.stream_of(A)))
+
+
+def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale: torch.Tensor,
+                                      B_scale: torch.Tensor, topk_weights: Optional[torch.Tensor],
+                                      sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
+                                      num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
+                                      top_k: int, num_valid: int, config: Dict[str, Any],
+                                      fused_scale: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """First GEMM with SiLU-and-mul and the 1x128 re-quantisation in its epilogue: the
+    sequence int8.py:784-823 in one kernel.  Returns (A2q [num_valid, I] int8,
+    A2s [num_valid, I/128] f32); rows of slots routed to non-local experts are not written."""
+    assert topk_weights is not None or not mul_routed_weight
+    _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)
+    E, N, K = B.shape
+    I = N // 2
+    a2q = torch.empty(num_valid, I, dtype=torch.int8, device=A.device)
+    a2s = torch.empty(num_valid, I // 128, dtype=torch.float32, device=A.device)
+    tw = None
+    if topk_weights is not None:
+        tw = topk_weights
+        if tw.dtype != torch.float32 or not tw.is_contiguous():
+            tw = tw.to(torch.float32).contiguous()
+    with _on_device(A):
+        _lib.check(_lib.lib().lo_moe_gemm1_silu_quant_block_int8(
+            _lib.ptr(A), _lib.ptr(A_scale), _lib.ptr(B), _lib.ptr(B_scale), _lib.ptr(a2q), _lib.ptr(a2s),
+            _lib.LO_BF16, _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(expert_ids),
+            _lib.ptr(num_tokens_post_padded), sorted_token_ids.numel(), num_valid, A.shape[0], E, I, K,
+            int(top_k), int(config["BLOCK_SIZE_M"]), 1 if mul_routed_weight else 0,
+            _lib.LO_GEMM_FUSED_SCALE if fused_scale else 0, _lib.stream_of(A)))
+    return a2q, a2s
+
+
+def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
+    """out[:, i] = T(T(silu(x[:, i])) * x[:, d + i])  (the op called at int8.py:811)."""
+    _require_cuda(out, x)
+    assert x.is_contiguous() and out.is_contiguous() and x.shape[-1] == 2 * out.shape[-1]
+    I = out.shape[-1]
+    rows = out.numel() // I
+    with _on_device(x):
+        _lib.check(_lib.lib().lo_silu_and_mul(_lib.ptr(x), _act_dtype(x), rows, I, _lib.ptr(out),
+                                              _lib.stream_of(x)))
+
+
+def fused_experts_workspace_bytes(M: int, top_k: int, H: int, I: int, num_experts: int,
+                                  block_size_m: int = 0) -> int:
+    n = _lib.lib().lo_fused_experts_workspace_bytes(M, top_k, H, I, num_experts, block_size_m)
+    _lib.check(n)
+    return int(n)
+
+
+def fused_experts_impl_int8(hidden_states: torch.Tensor,
+                            w1: torch.Tensor,
+                            w2: torch.Tensor,
+                            topk_weights: torch.Tensor,
+                            topk_ids: torch.Tensor,
+                            cache13: torch.Tensor,
+                            inplace: bool = False,
+                            activation: str = "silu",
+                            apply_router_weight_on_input: bool = False,
+                            use_fp8_w8a8: bool = False,
+                            use_int8_w8a8: bool = False,
+                            use_int8_w8a16: bool = False,
+                            use_int4_w4a16: bool = False,
+                            per_channel_quant: bool = False,
+                            global_num_experts: int = -1,
+                            expert_map: Optional[torch.Tensor] = None,
+                            w1_scale: Optional[torch.Tensor] = None,
+                            w2_scale: Optional[torch.Tensor] = None,
+                            w1_zp: Optional[torch.Tensor] = None,
+                            w2_zp: Optional[torch.Tensor] = None,
+                            a1_scale: Optional[torch.Tensor] = None,
+                            a2_scale: Optional[torch.Tensor] = None,
+                            block_shape: Optional[List[int]] = None,
+                            use_nn_moe: Optional[bool] = False,
+                            routed_scaling_factor: Optional[float] = 1.0,
+                            shared_output: Optional[torch.Tensor] = None,
+                            i_q: Optional[torch.Tensor] = None,
+                            i_s: Optional[torch.Tensor] = None, **_):
+    """Fused MoE experts with block-quantised INT8 weights (128x128 blocks, fp32 scales) and
+    activations quantised per 1x128 group on the fly.
+
+    Same signature as the reference (int8.py:628-656).  This build implements the branch
+    ``use_int8_w8a8=True, block_shape=[128, 128], activation="silu"``; every other
+    combination raises.  ``cache13`` is the caller's workspace (dtype of ``hidden_states``,
+    at least ``min(M, CHUNK) * topk * max(2I, H)`` elements); its first ``M*topk*H``
+    elements receive the second GEMM's per-slot output.  The top-k reduction is always
+    performed: ``out = routed_scaling_factor * sum_k(...) (+ shared_output)``.
+    Unknown keyword arguments are ignored, as in the reference.
+    """
+    extra = _  # private tuning knobs: lightop_amd_flags, lightop_amd_block_size_m
+    # Check constraints (int8.py:658-667).
+    assert use_int8_w8a8 or use_fp8_w8a8
+    assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
+    assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.stride(-1) == 1, "Stride of last dimension must be 1"
+    assert w2.stride(-1) == 1, "Stride of last dimension must be 1"
+    assert hidden_states.dtype in [torch.float32, torch.float16, torch.bfloat16]
+    if not use_int8_w8a8 or use_fp8_w8a8 or use_int8_w8a16 or use_int4_w4a16 or per_channel_quant:
+        raise NotImplementedError("lightop_amd: only use_int8_w8a8=True with block_shape=[128, 128] is built")
+    if block_shape is None or list(block_shape) != [128, 128]:
+        raise NotImplementedError("lightop_amd: block_shape must be [128, 128]")
+    if activation != "silu":
+        if activation == "gelu":
+            raise NotImplementedError("lightop_amd: the gelu activation is not built")
+        raise ValueError(f"Unsupported FusedMoe activation: {activation}")
+    if hidden_states.dtype != torch.bfloat16:
+        raise NotImplementedError("lightop_amd: hidden_states must be bfloat16")
+    assert w1_scale is not None and w2_scale is not None
+    del w1_zp, w2_zp, a1_scale, a2_scale, use_nn_moe, i_q, i_s
+    _require_cuda(hidden_states, w1, w2, topk_weights, topk_ids, cache13, w1_scale, w2_scale,
+                  expert_map, shared_output)
+
+    num_tokens, H = hidden_states.shape
+    E, N = w1.shape[0], w1.shape[1]
+    I = N // 2
+    assert w2.shape == (E, H, I), "w2 must be [E, H, I]"
+    assert w1.is_contiguous() and w2.is_contiguous(), "expert weights must be contiguous"
+    assert w1.dtype == torch.int8 and w2.dtype == torch.int8
+    assert w1_scale.shape == (E, N // 128, H // 128) and w2_scale.shape == (E, H // 128, I // 128)
+    if global_num_experts == -1:
+        global_num_experts = E
+    top_k_num = topk_ids.shape[1]
+    CHUNK_SIZE = envs.LMSLIM_FUSED_MOE_CHUNK_SIZE
+    M = min(num_tokens, CHUNK_SIZE)
+    assert cache13.dtype == hidden_states.dtype and cache13.is_contiguous()
+    assert cache13.numel() >= M * top_k_num * max(N, H), "cache13 is too small"
+
+    out_hidden_states = hidden_states if inplace else torch.empty_like(hidden_states)
+    if num_tokens == 0:
+        return out_hidden_states
+
+    w1_scale = w1_scale if w1_scale.dtype == torch.float32 and w1_scale.is_contiguous() \
+        else w1_scale.to(torch.float32).contiguous()
+    w2_scale = w2_scale if w2_scale.dtype == torch.float32 and w2_scale.is_contiguous() \
+        else w2_scale.to(torch.float32).contiguous()
+    if topk_weights.dtype != torch.float32 or not topk_weights.is_contiguous():
+        topk_weights = topk_weights.to(torch.float32).contiguous()
+    if not topk_ids.is_contiguous():
+        topk_ids = topk_ids.contiguous()
+    if expert_map is not None and (expert_map.dtype != torch.int32 or not expert_map.is_contiguous()):
+        expert_map = expert_map.to(torch.int32).contiguous()
+    if shared_output is not None:
+        assert shared_output.shape == hidden_states.shape and shared_output.dtype == hidden_states.dtype
+        shared_output = shared_output.contiguous()
+
+    lib = _lib.lib()
+    ws_bytes = fused_experts_workspace_bytes(M, top_k_num, H, I, global_num_experts, 0)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=hidden_states.device)
+    ws_ptr = (workspace.data_ptr() + 255) // 256 * 256
+    ws_avail = ws_bytes - (ws_ptr - workspace.data_ptr())
+    flags = int(extra.get("lightop_amd_flags", 0))
+    block_size_m = int(extra.get("lightop_amd_block_size_m", 0))
+
+    with _on_device(hidden_states):
+        stream = _lib.stream_of(hidden_states)
+        for chunk in range((num_tokens // CHUNK_SIZE) + 1):
+            begin, end = chunk * CHUNK_SIZE, min((chunk + 1) * CHUNK_SIZE, num_tokens)
+            m = end - begin
+            if m <= 0:
+                break
+            x = hidden_states[begin:end]
+            _lib.check(lib.lo_fused_experts_block_int8(
+                _lib.ptr(x), _act_dtype(x), m, H, I, E, global_num_experts, top_k_num,
+                _lib.ptr(w1), _lib.ptr(w1_scale), _lib.ptr(w2), _lib.ptr(w2_scale),
+                _lib.ptr(topk_weights[begin:end]), _lib.ptr(topk_ids[begin:end]), _ids_dtype(topk_ids),
+                _lib.ptr(expert_map), 1 if apply_router_weight_on_input else 0,
+                float(routed_scaling_factor), _lib.ptr(None if shared_output is None else shared_output[begin:end]),
+                _lib.ptr(cache13), _lib.ptr(out_hidden_states[begin:end]),
+                ctypes_void(ws_ptr), ws_avail, block_size_m, flags, stream))
+    return out_hidden_states
+
+
+def ctypes_void(addr: int):
+    import ctypes
+
+    return ctypes.c_void_p(addr)
+
+
+__all__ = ["fused_experts_impl_int8", "get_w8a8moe_json", "invoke_fused_moe_kernel_int8",
+           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes"]

@@ -1,0 +1,108 @@
+"""Flat native-op namespace (reference: the pybind module ``lightop.op``,
+csrc/pybind/export.cpp:1584-1605).  Only the two operators of the block-INT8 fused-MoE
+path exist here; both write into caller-allocated tensors and return None.
+"""
+from __future__ import annotations
+
+import contextlib
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("lightop_amd: tensors must live on the GPU (there is no CPU path)")
+
+
+@contextlib.contextmanager
+def _on_device(t: torch.Tensor):
+    if torch.cuda.current_device() == t.device.index:
+        yield
+    else:
+        with torch.cuda.device(t.device):
+            yield
+
+
+def _ids_dtype(t: torch.Tensor) -> int:
+    if t.dtype == torch.int32:
+        return _lib.LO_I32
+    if t.dtype == torch.int64:
+        return _lib.LO_I64
+    raise RuntimeError(f"lightop_amd: topk_ids must be int32 or int64, got {t.dtype}")
+
+
+def _act_dtype(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.LO_BF16
+    if t.dtype == torch.float16:
+        return _lib.LO_F16
+    raise RuntimeError(f"lightop_amd: unsupported activation dtype {t.dtype}")
+
+
+def _align(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad,
+           expert_map, ignore_invalid):
+    _require_cuda(topk_ids, sorted_token_ids, experts_ids, num_tokens_post_pad, expert_map)
+    if not topk_ids.is_contiguous():
+        topk_ids = topk_ids.contiguous()
+    for t, name in ((sorted_token_ids, "sorted_token_ids"), (experts_ids, "experts_ids"),
+                    (num_tokens_post_pad, "num_tokens_post_pad")):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError(f"lightop_amd: {name} must be a contiguous int32 tensor")
+    if expert_map is not None and (expert_map.dtype != torch.int32 or not expert_map.is_contiguous()):
+        expert_map = expert_map.to(torch.int32).contiguous()
+    with _on_device(topk_ids):
+        _lib.check(_lib.lib().lo_moe_align_block_size(
+            _lib.ptr(topk_ids), _ids_dtype(topk_ids), topk_ids.numel(), int(num_experts), int(block_size),
+            _lib.ptr(expert_map), 1 if ignore_invalid else 0, _lib.ptr(sorted_token_ids),
+            sorted_token_ids.numel(), _lib.ptr(experts_ids), experts_ids.numel(),
+            _lib.ptr(num_tokens_post_pad), _lib.stream_of(topk_ids)))
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: int,
+                         sorted_token_ids: torch.Tensor, experts_ids: torch.Tensor,
+                         num_tokens_post_pad: torch.Tensor,
+                         expert_map: Optional[torch.Tensor] = None,
+                         expert_mask: Optional[torch.Tensor] = None,
+                         num_local_tokens: Optional[torch.Tensor] = None,
+                         Is_EP: bool = False, Is_fuse_fill: bool = True) -> None:
+    """``op.moe_align_block_size`` (export.cpp:1593-1605).  An ``expert_map`` given here is
+    applied to the ids before counting and ids mapped to -1 are dropped
+    (csrc/kernels/moe_align_sum_kernels.cu:62-90); the DeepEP-only arguments
+    ``expert_mask``, ``num_local_tokens`` and ``Is_EP`` are not part of this path."""
+    if expert_mask is not None or num_local_tokens is not None or Is_EP:
+        raise NotImplementedError(
+            "lightop_amd.op.moe_align_block_size: expert_mask / num_local_tokens / Is_EP belong to the "
+            "DeepEP layout, which this build does not cover")
+    del Is_fuse_fill  # the pad value is always written
+    _align(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad,
+           expert_map, ignore_invalid=True)
+
+
+def moe_sum(input: torch.Tensor, output: torch.Tensor, bias: Optional[torch.Tensor] = None,
+            expert_mask: Optional[torch.Tensor] = None, num_local_tokens: Optional[torch.Tensor] = None,
+            factor: float = 1.0, expect_m: int = -1) -> None:
+    """``op.moe_sum`` (export.cpp:1584-1592): output[t] = factor * sum_k input[t, k] (+ bias[t])."""
+    if expert_mask is not None or num_local_tokens is not None:
+        raise NotImplementedError(
+            "lightop_amd.op.moe_sum: expert_mask / num_local_tokens belong to the DeepEP layout, "
+            "which this build does not cover")
+    del expect_m
+    _require_cuda(input, output, bias)
+    if input.dim() != 3:
+        raise RuntimeError("lightop_amd.op.moe_sum: input must be [num_tokens, topk, hidden]")
+    if not input.is_contiguous():
+        input = input.contiguous()
+    M, k, H = input.shape
+    if not output.is_contiguous() or output.numel() != M * H or output.dtype != input.dtype:
+        raise RuntimeError("lightop_amd.op.moe_sum: output must be a contiguous [num_tokens, hidden] "
+                           "tensor of the input dtype")
+    if bias is not None and (not bias.is_contiguous() or bias.numel() != M * H or bias.dtype != input.dtype):
+        raise RuntimeError("lightop_amd.op.moe_sum: bias must match output")
+    with _on_device(input):
+        _lib.check(_lib.lib().lo_moe_sum(_lib.ptr(input), _lib.ptr(output), _lib.ptr(bias),
+                                         _act_dtype(input), M, k, H, float(factor),
+                                         _lib.stream_of(input)))

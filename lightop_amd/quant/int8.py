@@ -1,0 +1,40 @@
+"""1x128 group INT8 quantisation (reference:
+python/lightop/_lmslim_native/layers/gemm/int8_utils.py:125-195)."""
+from __future__ import annotations
+
+from typing import Tuple
+
+import torch
+
+from .. import _lib
+from ..op import _act_dtype, _on_device, _require_cuda
+
+
+def per_token_group_quant_int8(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float = 1e-10,
+    dtype: torch.dtype = torch.int8,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Quantise every ``group_size`` contiguous values of the last dimension to int8:
+    ``amax = max(|x|.max(), eps); s = amax / 127; q = trunc(clamp(x / s, -128, 127))``.
+    Returns ``(x_q, x_s)`` with ``x_s`` of shape ``x.shape[:-1] + (x.shape[-1] // group_size,)``
+    in fp32.  The kernel is built for ``group_size == 128`` (int8_utils.py:112).
+    """
+    assert x.shape[-1] % group_size == 0, "the last dimension of `x` cannot be divisible by `group_size`"
+    if dtype != torch.int8:
+        raise RuntimeError("per_token_group_quant_int8: only torch.int8 output is supported")
+    if group_size != 128:
+        raise RuntimeError("per_token_group_quant_int8: group_size must be 128")
+    _require_cuda(x)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    x_q = torch.empty_like(x, dtype=torch.int8)
+    x_s = torch.empty(x.shape[:-1] + (x.shape[-1] // group_size,), device=x.device, dtype=torch.float32)
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    with _on_device(x):
+        _lib.check(_lib.lib().lo_per_token_group_quant_int8(
+            _lib.ptr(x), _act_dtype(x), rows, cols, float(eps), _lib.ptr(x_q), _lib.ptr(x_s),
+            _lib.stream_of(x)))
+    return x_q, x_s

@@ -1,0 +1,128 @@
+"""Synthetic block-INT8 MoE workloads: layer shapes, weights, activations and routing.
+
+Weights: int8 uniform in [-127, 127] with one fp32 scale per 128x128 block drawn
+lognormal(mu = ln 1e-3, sigma = 0.3).  Activations: bf16 ~ N(0, 1).  Routing: softmax
+top-k (renormalised), DeepSeek-V3 grouped sigmoid top-k (8 groups, top-4 groups, group
+score = sum of the group's two best experts, renormalised, x2.5; reference form:
+test/ci_tests/test_fused_moe_gate.py:9-61), optionally Zipf-skewed.  Everything is
+drawn from a seeded torch.Generator on the CPU (or, for layers too large to copy, on
+the device) so that a CPU checker and the GPU see the same bits.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class MoeLayer:
+    name: str
+    E: int              # experts resident on this GPU
+    E_global: int       # experts the router chooses from
+    top_k: int
+    H: int
+    I: int
+    routing: str        # "softmax" | "grouped_sigmoid" | "grouped_sigmoid_zipf"
+    n_group: int = 1
+    topk_group: int = 1
+    routed_scaling: float = 1.0
+
+    @property
+    def weight_bytes(self) -> int:
+        return self.E * 3 * self.I * self.H
+
+
+TINY = MoeLayer("tiny-e8", E=8, E_global=8, top_k=2, H=1024, I=512, routing="softmax")
+QWEN3_30B = MoeLayer("qwen3-30b-a3b", E=128, E_global=128, top_k=8, H=2048, I=768, routing="softmax")
+DSV3_EP = MoeLayer("deepseek-v3-ep8-share", E=32, E_global=256, top_k=8, H=7168, I=2048,
+                   routing="grouped_sigmoid", n_group=8, topk_group=4, routed_scaling=2.5)
+DSV3_FULL = MoeLayer("deepseek-v3-full", E=256, E_global=256, top_k=8, H=7168, I=2048,
+                     routing="grouped_sigmoid_zipf", n_group=8, topk_group=4, routed_scaling=2.5)
+
+LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL)}
+
+
+def make_weights(layer: MoeLayer, seed: int = 0, device="cpu", gen_device: Optional[str] = None):
+    """(w1 [E,2I,H] int8, w2 [E,H,I] int8, w1_scale [E,2I/128,H/128], w2_scale [E,H/128,I/128])."""
+    gen_device = gen_device or "cpu"
+    g = torch.Generator(device=gen_device).manual_seed(seed)
+    E, H, I = layer.E, layer.H, layer.I
+
+    def w(shape):
+        return torch.randint(-127, 128, shape, generator=g, dtype=torch.int8, device=gen_device)
+
+    def s(shape):
+        return torch.exp(torch.randn(shape, generator=g, dtype=torch.float32, device=gen_device) * 0.3
+                         + math.log(1e-3))
+
+    w1 = w((E, 2 * I, H))
+    w2 = w((E, H, I))
+    w1s = s((E, 2 * I // 128, H // 128))
+    w2s = s((E, H // 128, I // 128))
+    return tuple(t.to(device) for t in (w1, w2, w1s, w2s))
+
+
+def expert_map_for(layer: MoeLayer, device="cpu") -> Optional[torch.Tensor]:
+    """Global id -> local id for the first ``E`` experts, -1 elsewhere; None if all are local."""
+    if layer.E == layer.E_global:
+        return None
+    m = torch.full((layer.E_global,), -1, dtype=torch.int32)
+    m[: layer.E] = torch.arange(layer.E, dtype=torch.int32)
+    return m.to(device)
+
+
+def route(layer: MoeLayer, logits: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(topk_weights [M,k] f32, topk_ids [M,k] int32) from router logits [M, E_global]."""
+    k = layer.top_k
+    if layer.routing == "softmax":
+        p = torch.softmax(logits.float(), dim=-1)
+        w, ids = torch.topk(p, k, dim=-1)
+        w = w / w.sum(dim=-1, keepdim=True)
+        return w.contiguous(), ids.to(torch.int32).contiguous()
+    scores = torch.sigmoid(logits.float())
+    M, Eg = scores.shape
+    per = Eg // layer.n_group
+    group_scores = scores.view(M, layer.n_group, per).topk(2, dim=-1)[0].sum(dim=-1)
+    gidx = torch.topk(group_scores, layer.topk_group, dim=-1, sorted=False)[1]
+    gmask = torch.zeros_like(group_scores)
+    gmask.scatter_(1, gidx, 1.0)
+    mask = gmask.unsqueeze(-1).expand(M, layer.n_group, per).reshape(M, Eg)
+    masked = scores.masked_fill(mask == 0, float("-inf"))
+    ids = torch.topk(masked, k, dim=-1, sorted=False)[1]
+    w = scores.gather(1, ids)
+    w = w / w.sum(dim=-1, keepdim=True) * layer.routed_scaling
+    return w.contiguous(), ids.to(torch.int32).contiguous()
+
+
+def make_inputs(layer: MoeLayer, M: int, seed: int = 0, device="cpu"):
+    """(x [M,H] bf16, topk_weights [M,k] f32, topk_ids [M,k] int32) for one step."""
+    g = torch.Generator(device="cpu").manual_seed(seed * 7919 + M)
+    x = torch.randn((M, layer.H), generator=g, dtype=torch.float32).to(torch.bfloat16)
+    logits = torch.randn((M, layer.E_global), generator=g, dtype=torch.float32)
+    if layer.routing.endswith("zipf"):
+        perm = torch.randperm(layer.E_global, generator=g)
+        zipf = 1.0 / torch.arange(1, layer.E_global + 1, dtype=torch.float32) ** 1.2
+        bias = torch.empty(layer.E_global)
+        bias[perm] = torch.log(zipf / zipf.sum())
+        logits = logits + bias
+    w, ids = route(layer, logits)
+    return x.to(device), w.to(device), ids.to(device)
+
+
+def algorithmic_work(layer: MoeLayer, topk_ids: torch.Tensor, expert_map: Optional[torch.Tensor]):
+    """(int8 ops, bytes, local slots, active local experts) of one call: ops = 6*S_loc*I*H;
+    bytes = every active expert's weights and block scales once + bf16 activations in and
+    out + routing tensors.  Intermediates are not counted."""
+    ids = topk_ids.reshape(-1).long().cpu()
+    local = ids if expert_map is None else expert_map.cpu().long()[ids]
+    local = local[local >= 0]
+    S_loc = int(local.numel())
+    E_act = int(torch.unique(local).numel())
+    H, I = layer.H, layer.I
+    M = topk_ids.shape[0]
+    per_expert = 3 * I * H + 4 * ((2 * I // 128) * (H // 128) + (H // 128) * (I // 128))
+    nbytes = E_act * per_expert + 2 * M * H * 2 + M * layer.top_k * 8
+    return 6 * S_loc * I * H, nbytes, S_loc, E_act

@@ -1,0 +1,173 @@
+"""ctypes front end of the C oracle (oracle/moe_oracle.c).  TEST INFRASTRUCTURE ONLY.
+
+Nothing in ``lightop_amd`` may import this module: it is the checker used by
+``tests/``, ``__graft_entry__.smoke()`` and the cpu-baseline leg of ``bench.py``.
+All functions take and return torch CPU tensors; bf16 tensors are handed to C
+as their raw 16-bit patterns.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "_build", "libmoe_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (a few seconds).  Returns the .so path."""
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(
+        os.path.join(_HERE, "moe_oracle.c")
+    ):
+        subprocess.run(["make", "-C", _HERE, "-B"], check=True, capture_output=True)
+    return _SO
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        _lib = ctypes.CDLL(_SO)
+        _lib.orc_expf.restype = ctypes.c_float
+        _lib.orc_expf.argtypes = [ctypes.c_float]
+        _lib.orc_bf16_to_f32.restype = ctypes.c_float
+        _lib.orc_bf16_to_f32.argtypes = [ctypes.c_uint16]
+        _lib.orc_f32_to_bf16.restype = ctypes.c_uint16
+        _lib.orc_f32_to_bf16.argtypes = [ctypes.c_float]
+        _lib.orc_silu_bf16.restype = ctypes.c_uint16
+        _lib.orc_silu_bf16.argtypes = [ctypes.c_uint16]
+        _lib.orc_silu_bf16_libm.restype = ctypes.c_uint16
+        _lib.orc_silu_bf16_libm.argtypes = [ctypes.c_uint16]
+    return _lib
+
+
+def _p(t: Optional[torch.Tensor]):
+    if t is None:
+        return ctypes.c_void_p(0)
+    assert t.device.type == "cpu" and t.is_contiguous(), "oracle wants contiguous CPU tensors"
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _i32(v):
+    return ctypes.c_int32(int(v))
+
+
+def align_buffer_sizes(numel: int, num_experts: int, block_size: int, pad_sorted_ids: bool = False):
+    """Buffer extents of moe_align_block_size.py:80-93."""
+    max_pad = numel + num_experts * (block_size - 1)
+    if pad_sorted_ids:
+        max_pad = (max_pad + block_size - 1) // block_size * block_size
+    if numel < num_experts:
+        max_pad = min(numel * block_size, max_pad)
+    return max_pad, (max_pad + block_size - 1) // block_size
+
+
+def moe_align_block_size(topk_ids, block_size, num_experts, expert_map=None,
+                         pad_sorted_ids=False, ignore_invalid_experts=False):
+    ids = topk_ids.reshape(-1).to(torch.int32).contiguous()
+    S = ids.numel()
+    max_pad, max_blocks = align_buffer_sizes(S, num_experts, block_size, pad_sorted_ids)
+    sorted_ids = torch.empty(max_pad, dtype=torch.int32)
+    expert_ids = torch.empty(max_blocks, dtype=torch.int32)
+    ntpp = torch.zeros(1, dtype=torch.int32)
+    emap = None if expert_map is None else expert_map.to(torch.int32).contiguous()
+    rc = lib().orc_moe_align_block_size(
+        _p(ids), _i64(S), _i32(num_experts), _i32(block_size), _p(emap),
+        ctypes.c_int(1 if ignore_invalid_experts else 0), _p(sorted_ids), _i64(max_pad),
+        _p(expert_ids), _i64(max_blocks), _p(ntpp))
+    if rc != 0:
+        raise RuntimeError("oracle moe_align_block_size: id out of range or buffer too small")
+    return sorted_ids, expert_ids, ntpp
+
+
+def per_token_group_quant_int8(x, group_size=128, eps=1e-10):
+    assert group_size == 128 and x.dtype == torch.bfloat16
+    x = x.contiguous()
+    C = x.shape[-1]
+    R = x.numel() // C
+    q = torch.empty(x.shape, dtype=torch.int8)
+    s = torch.empty(x.shape[:-1] + (C // 128,), dtype=torch.float32)
+    lib().orc_group_quant_int8(_p(x), _i64(R), _i64(C), ctypes.c_float(eps), _p(q), _p(s))
+    return q, s
+
+
+def moe_gemm_block_int8(A, As, W, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_routed,
+                        top_k, num_valid, block_size, dump_acc=False, out=None):
+    """One grouped-GEMM stage.  Returns C[num_valid, N] bf16 (and the int32
+    per-128-block dot products when dump_acc)."""
+    E, N, K = W.shape
+    C = torch.zeros(num_valid, N, dtype=torch.bfloat16) if out is None else out
+    acc = torch.zeros(num_valid, N, K // 128, dtype=torch.int32) if dump_acc else None
+    tw = None if topk_w is None else topk_w.reshape(-1).to(torch.float32).contiguous()
+    lib().orc_moe_gemm_block_int8(
+        _p(A.contiguous()), _p(As.contiguous()), _p(W.contiguous()), _p(Ws.contiguous()),
+        _p(sorted_ids), _p(expert_ids), _p(ntpp), _p(tw), ctypes.c_int(1 if mul_routed else 0),
+        _i32(top_k), _i64(num_valid), _i64(N), _i64(K), _i32(block_size), _p(C), _p(acc))
+    return (C, acc) if dump_acc else C
+
+
+def silu_and_mul(c1):
+    S, N = c1.shape
+    act = torch.empty(S, N // 2, dtype=torch.bfloat16)
+    lib().orc_silu_and_mul(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(act))
+    return act
+
+
+def moe_sum(inp, bias=None, factor=1.0):
+    M, k, H = inp.shape
+    out = torch.empty(M, H, dtype=torch.bfloat16)
+    lib().orc_moe_sum(_p(inp.contiguous()), _i64(M), _i32(k), _i64(H),
+                      _p(None if bias is None else bias.contiguous()), ctypes.c_float(factor), _p(out))
+    return out
+
+
+def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids, block_size_m,
+                             global_num_experts=-1, expert_map=None,
+                             apply_router_weight_on_input=False, routed_scaling_factor=1.0,
+                             shared_output=None, return_intermediates=False):
+    """Whole path; with return_intermediates a dict of every stage's output."""
+    M, H = x.shape
+    E, N1, _ = w1.shape
+    I = N1 // 2
+    k = topk_ids.shape[1]
+    S = M * k
+    Eg = E if global_num_experts == -1 else global_num_experts
+    max_pad, max_blocks = align_buffer_sizes(S, Eg, block_size_m)
+    out = torch.empty(M, H, dtype=torch.bfloat16)
+    sorted_ids = torch.empty(max_pad, dtype=torch.int32)
+    expert_ids = torch.empty(max_blocks, dtype=torch.int32)
+    ntpp = torch.zeros(1, dtype=torch.int32)
+    inter = {}
+    if return_intermediates:
+        inter = dict(
+            a1q=torch.empty(M, H, dtype=torch.int8), a1s=torch.empty(M, H // 128, dtype=torch.float32),
+            c1=torch.zeros(S, 2 * I, dtype=torch.bfloat16), act=torch.empty(S, I, dtype=torch.bfloat16),
+            a2q=torch.empty(S, I, dtype=torch.int8), a2s=torch.empty(S, I // 128, dtype=torch.float32),
+            c3=torch.zeros(S, H, dtype=torch.bfloat16))
+    ids = topk_ids.to(torch.int32).contiguous()
+    tw = topk_weights.to(torch.float32).contiguous()
+    emap = None if expert_map is None else expert_map.to(torch.int32).contiguous()
+    rc = lib().orc_fused_experts_block_int8(
+        _p(x.contiguous()), _i64(M), _i64(H), _i64(I), _i32(E), _i32(Eg), _i32(k),
+        _p(w1.contiguous()), _p(w1_scale.contiguous()), _p(w2.contiguous()), _p(w2_scale.contiguous()),
+        _p(tw), _p(ids), _p(emap), _i32(block_size_m),
+        ctypes.c_int(1 if apply_router_weight_on_input else 0), ctypes.c_float(routed_scaling_factor),
+        _p(None if shared_output is None else shared_output.contiguous()), _p(out),
+        _p(sorted_ids), _i64(max_pad), _p(expert_ids), _i64(max_blocks), _p(ntpp),
+        _p(inter.get("a1q")), _p(inter.get("a1s")), _p(inter.get("c1")), _p(inter.get("act")),
+        _p(inter.get("a2q")), _p(inter.get("a2s")), _p(inter.get("c3")))
+    if rc != 0:
+        raise RuntimeError("oracle fused_experts: alignment failed")
+    if return_intermediates:
+        inter.update(sorted_ids=sorted_ids, expert_ids=expert_ids, num_tokens_post_pad=ntpp, out=out)
+        return inter
+    return out

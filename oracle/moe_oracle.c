@@ -1,0 +1,360 @@
+/*
+ * CPU oracle for the block-INT8 fused-MoE path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain C, the arithmetic of the reference's
+ * `fused_experts_impl_int8(use_int8_w8a8=True, block_shape=[128,128])` path.
+ * It is the checker that the HIP kernels are compared with; nothing in the
+ * shipped library links, imports or calls it.  Only the tests, the smoke
+ * check and the benchmark's cpu-baseline leg may load it.
+ *
+ * Reference (all paths relative to the reference tree):
+ *   routing alignment   python/lightop/_lmslim_native/vllm_compat/moe_align_block_size.py:17-120
+ *                       csrc/kernels/moe_align_sum_kernels.cu:1034-1115, :1210-1314
+ *                       test/test_moe_align_block_size.py:26-101 (stable ascending order)
+ *   1x128 group quant   python/lightop/_lmslim_native/layers/gemm/int8_utils.py:74-195
+ *   grouped GEMM        python/lightop/_lmslim_native/layers/fused_moe/int8.py:320-541
+ *   SiLU-and-mul        call site int8.py:811; in-repo twin
+ *                       csrc/kernels/gated_activation/fuse_silu_mul_quant.cu:893-905
+ *   top-k reduce        csrc/kernels/moe_align_sum_kernels.cu:551-637, :860-909
+ *   orchestration       int8.py:628-908
+ *
+ * Arithmetic rules: every fp32 operation is a single IEEE-754 RN operation
+ * (compile with -ffp-contract=off, never -ffast-math); bf16 conversion is
+ * round-to-nearest-even; float->int8 is truncation toward zero after the
+ * clamp; int8 dot products are exact in int32.
+ *
+ * Pinning status (which independent check fixes each function) is listed in
+ * tests/test_oracle.py; a function without one is marked "parity unpinned"
+ * there.  Known unpinned points: the intra-expert order of sorted_token_ids
+ * (the reference kernels rank with atomics; the stable ascending order of the
+ * reference's own Python test is taken as canonical) and the last-ulp
+ * behaviour of the third-party expf inside vLLM's silu_and_mul (orc_expf below
+ * is checked against libm's expf over every bf16 input instead).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_GROUP 128
+
+/* ---------------------------------------------------------------- bf16 -- */
+
+static inline float bf16_to_f32(uint16_t h) {
+  union { uint32_t u; float f; } v;
+  v.u = (uint32_t)h << 16;
+  return v.f;
+}
+
+/* Round-to-nearest-even, the rule of moe_sum_from_float
+ * (moe_align_sum_kernels.cu:577-589) and of torch's BFloat16 conversion;
+ * NaN is kept quiet. */
+static inline uint16_t f32_to_bf16(float f) {
+  union { uint32_t u; float f; } v;
+  v.f = f;
+  if ((v.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((v.u >> 16) | 0x0040u);
+  v.u += 0x7fffu + ((v.u >> 16) & 1u);
+  return (uint16_t)(v.u >> 16);
+}
+
+uint16_t orc_f32_to_bf16(float f) { return f32_to_bf16(f); }
+float orc_bf16_to_f32(uint16_t h) { return bf16_to_f32(h); }
+
+/* ----------------------------------------------------------- alignment -- */
+
+/*
+ * moe_align_block_size.  ids[S] are expert ids in [0, num_experts).
+ *
+ *   ignore_invalid == 0 (the reference default): count on the given ids;
+ *     expert_ids[b] is map[e] when a map is given (moe_align_block_size.py:117-118),
+ *     else e.
+ *   ignore_invalid != 0: ids with map[id] == -1 are dropped, counting and
+ *     expert_ids use the mapped id (moe_align_sum_kernels.cu:83-90).
+ *
+ * sorted[0:sorted_cap] is filled with S (the pad value) first; within an
+ * expert the flat slot ids are ascending.  expert_ids beyond P/bs are set to -1.
+ * Returns 0, or -1 if an id is out of range or a buffer is too small.
+ */
+int orc_moe_align_block_size(const int32_t *ids, int64_t S, int32_t num_experts,
+                             int32_t bs, const int32_t *map, int ignore_invalid,
+                             int32_t *sorted, int64_t sorted_cap,
+                             int32_t *expert_ids, int64_t expert_ids_cap,
+                             int32_t *num_tokens_post_pad) {
+  int64_t *cnt = (int64_t *)calloc((size_t)num_experts + 1, sizeof(int64_t));
+  int64_t *off = (int64_t *)calloc((size_t)num_experts + 1, sizeof(int64_t));
+  int rc = 0;
+  for (int64_t f = 0; f < S; ++f) {
+    int32_t e = ids[f];
+    if (e < 0 || e >= num_experts) { rc = -1; goto done; }
+    if (ignore_invalid && map) {
+      e = map[e];
+      if (e < 0) continue;
+      if (e >= num_experts) { rc = -1; goto done; }
+    }
+    cnt[e]++;
+  }
+  for (int32_t e = 0; e < num_experts; ++e)
+    off[e + 1] = off[e] + (cnt[e] + bs - 1) / bs * bs;
+  {
+    int64_t P = off[num_experts];
+    if (P > sorted_cap || P / bs > expert_ids_cap) { rc = -1; goto done; }
+    for (int64_t i = 0; i < sorted_cap; ++i) sorted[i] = (int32_t)S;
+    for (int64_t b = 0; b < expert_ids_cap; ++b) expert_ids[b] = -1;
+    for (int32_t e = 0; e < num_experts; ++e)
+      for (int64_t b = off[e] / bs; b < off[e + 1] / bs; ++b)
+        expert_ids[b] = (map && !ignore_invalid) ? map[e] : e;
+    memset(cnt, 0, ((size_t)num_experts + 1) * sizeof(int64_t));
+    for (int64_t f = 0; f < S; ++f) {
+      int32_t e = ids[f];
+      if (ignore_invalid && map) {
+        e = map[e];
+        if (e < 0) continue;
+      }
+      sorted[off[e] + cnt[e]++] = (int32_t)f;
+    }
+    *num_tokens_post_pad = (int32_t)P;
+  }
+done:
+  free(cnt);
+  free(off);
+  return rc;
+}
+
+/* --------------------------------------------------------- group quant -- */
+
+/*
+ * per_token_group_quant_int8 for contiguous bf16 x[R, C], groups of 128 along
+ * the last dimension (int8_utils.py:110-116):
+ *   amax = max(max|x|, eps);  s = amax / 127;  q = (int8) trunc(clamp(x / s, -128, 127))
+ */
+void orc_group_quant_int8(const uint16_t *x, int64_t R, int64_t C, float eps,
+                          int8_t *q, float *s) {
+  int64_t G = C / ORC_GROUP;
+#pragma omp parallel for schedule(static)
+  for (int64_t g = 0; g < R * G; ++g) {
+    const uint16_t *xg = x + g * ORC_GROUP;
+    float amax = 0.0f;
+    for (int i = 0; i < ORC_GROUP; ++i) {
+      float a = fabsf(bf16_to_f32(xg[i]));
+      if (a > amax) amax = a;
+    }
+    if (!(amax > eps)) amax = eps;
+    float sc = amax / 127.0f;
+    s[g] = sc;
+    for (int i = 0; i < ORC_GROUP; ++i) {
+      float v = bf16_to_f32(xg[i]) / sc;
+      if (v < -128.0f) v = -128.0f;
+      if (v > 127.0f) v = 127.0f;
+      q[g * ORC_GROUP + i] = (int8_t)(int32_t)v; /* C cast truncates toward zero */
+    }
+  }
+}
+
+/* ------------------------------------------------------- grouped GEMM -- */
+
+/*
+ * One stage of the fused-MoE grouped GEMM (Triton fused_moe_kernel,
+ * int8.py:320-541) in the block-quantised int8 form.
+ *
+ *   A   [*, K] int8, row of slot f is f / top_k;   As [*, K/128] f32
+ *   W   [E, N, K] int8 (K contiguous);             Ws [E, ceil(N/128), K/128] f32
+ *   C   [num_valid, N] bf16, row f
+ *
+ * For every block b < P/bs with e = expert_ids[b] and every row
+ * f = sorted[b*bs + i] < num_valid:
+ *   acc = 0;  for kb: d = sum_k A*W (int32, exact);
+ *             acc = acc + (f32(d) * As[row, kb]) * Ws[e, n/128, kb]   (int8.py:499-508)
+ *   if mul_routed: acc = acc * topk_w[f]                              (int8.py:521-525)
+ *   C[f, n] = bf16(acc);  e == -1 -> C[f, :] = 0                      (int8.py:441-449)
+ *
+ * acc_dump (optional, [num_valid, N, K/128] int32) receives the exact
+ * per-128-block integer dot products, so that the integer part can be checked
+ * on its own.
+ */
+void orc_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W,
+                             const float *Ws, const int32_t *sorted,
+                             const int32_t *expert_ids,
+                             const int32_t *num_tokens_post_pad,
+                             const float *topk_w, int mul_routed, int32_t top_k,
+                             int64_t num_valid, int64_t N, int64_t K, int32_t bs,
+                             uint16_t *C, int32_t *acc_dump) {
+  int64_t KB = K / ORC_GROUP;
+  int64_t NB = (N + ORC_GROUP - 1) / ORC_GROUP;
+  int64_t P = num_tokens_post_pad[0];
+  int64_t nblk = P / bs;
+#pragma omp parallel for schedule(dynamic, 1) collapse(2)
+  for (int64_t b = 0; b < nblk; ++b) {
+    for (int32_t i = 0; i < bs; ++i) {
+      int64_t f = sorted[b * bs + i];
+      if (f >= num_valid) continue;
+      int32_t e = expert_ids[b];
+      uint16_t *c = C + f * N;
+      if (e < 0) {
+        for (int64_t n = 0; n < N; ++n) c[n] = 0;
+        continue;
+      }
+      int64_t row = f / top_k;
+      const int8_t *a = A + row * K;
+      const float *as = As + row * KB;
+      const int8_t *w = W + (int64_t)e * N * K;
+      const float *ws = Ws + (int64_t)e * NB * KB;
+      for (int64_t n = 0; n < N; ++n) {
+        const int8_t *wn = w + n * K;
+        float acc = 0.0f;
+        for (int64_t kb = 0; kb < KB; ++kb) {
+          int32_t d = 0;
+          for (int k = 0; k < ORC_GROUP; ++k)
+            d += (int32_t)a[kb * ORC_GROUP + k] * (int32_t)wn[kb * ORC_GROUP + k];
+          if (acc_dump) acc_dump[(f * N + n) * KB + kb] = d;
+          float t = (float)d * as[kb];
+          t = t * ws[(n / ORC_GROUP) * KB + kb];
+          acc = acc + t;
+        }
+        if (mul_routed) acc = acc * topk_w[f];
+        c[n] = f32_to_bf16(acc);
+      }
+    }
+  }
+}
+
+/* ------------------------------------------------------------ SiLU*mul -- */
+
+/*
+ * expf restated with explicit single operations so that the same sequence can
+ * be issued on any IEEE machine: n = rint(x*log2e), Cody-Waite reduction with
+ * fmaf, degree-7 polynomial, exact scaling by 2^n.  tests/test_oracle.py checks
+ * it against libm's expf (<= 1 ulp on the working range) and, exhaustively over
+ * all 65536 bf16 inputs, that bf16(silu(x)) built on it equals the one built
+ * on libm's expf.
+ */
+float orc_expf(float x) {
+  if (x > 88.72283f) return INFINITY;
+  if (x < -87.0f) return 0.0f; /* 1 + e == 1 for every e this small */
+  float n = rintf(x * 1.44269504088896341f);
+  float r = fmaf(n, -0.693145751953125f, x);
+  r = fmaf(n, -1.42860682030941723212e-6f, r);
+  float p = 1.9841270114e-4f;
+  p = fmaf(p, r, 1.3888889225e-3f);
+  p = fmaf(p, r, 8.3333337680e-3f);
+  p = fmaf(p, r, 4.1666667908e-2f);
+  p = fmaf(p, r, 1.6666667163e-1f);
+  p = fmaf(p, r, 5.0000000000e-1f);
+  p = fmaf(p, r, 1.0f);
+  p = fmaf(p, r, 1.0f);
+  /* scale by 2^n in two exact steps so that neither factor leaves the normal range */
+  int32_t ni = (int32_t)n;
+  int32_t h = ni / 2;
+  union { uint32_t u; float f; } a, b;
+  a.u = (uint32_t)(h + 127) << 23;
+  b.u = (uint32_t)(ni - h + 127) << 23;
+  return (p * a.f) * b.f;
+}
+
+/*
+ * silu_and_mul on bf16 c1[S, 2I] -> act[S, I]:
+ *   sg = bf16( g / (1 + expf(-g)) );  act = bf16( f32(sg) * u )
+ * gate = first half, up = second half (fuse_silu_mul_quant.cu:893-905).
+ */
+static inline uint16_t silu_mul_one(uint16_t g16, uint16_t u16) {
+  float g = bf16_to_f32(g16);
+  float e = orc_expf(-g);
+  float sg = bf16_to_f32(f32_to_bf16(g / (1.0f + e)));
+  return f32_to_bf16(sg * bf16_to_f32(u16));
+}
+
+uint16_t orc_silu_bf16(uint16_t g16) {
+  float g = bf16_to_f32(g16);
+  return f32_to_bf16(g / (1.0f + orc_expf(-g)));
+}
+
+uint16_t orc_silu_bf16_libm(uint16_t g16) {
+  float g = bf16_to_f32(g16);
+  return f32_to_bf16(g / (1.0f + expf(-g)));
+}
+
+void orc_silu_and_mul(const uint16_t *c1, int64_t S, int64_t I, uint16_t *act) {
+#pragma omp parallel for schedule(static)
+  for (int64_t f = 0; f < S; ++f)
+    for (int64_t i = 0; i < I; ++i)
+      act[f * I + i] = silu_mul_one(c1[f * 2 * I + i], c1[f * 2 * I + I + i]);
+}
+
+/* ------------------------------------------------------------ moe_sum -- */
+
+/*
+ * out[t, h] from in[M, k, H] bf16.
+ *   bias == NULL: bf16( (sum_j f32(in[t,j,h])) * factor ), sequential j in fp32,
+ *                 one rounding (moe_align_sum_kernels.cu:619-633).
+ *   bias != NULL: x = bf16(sum); x = bf16(f32(x) * factor); x = bf16(f32(x) + f32(bias))
+ *                 (moe_align_sum_kernels.cu:886-909).
+ */
+void orc_moe_sum(const uint16_t *in, int64_t M, int32_t k, int64_t H,
+                 const uint16_t *bias, float factor, uint16_t *out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t t = 0; t < M; ++t)
+    for (int64_t h = 0; h < H; ++h) {
+      float acc = 0.0f;
+      for (int32_t j = 0; j < k; ++j) acc = acc + bf16_to_f32(in[(t * k + j) * H + h]);
+      if (!bias) {
+        out[t * H + h] = f32_to_bf16(acc * factor);
+      } else {
+        uint16_t x = f32_to_bf16(acc);
+        x = f32_to_bf16(bf16_to_f32(x) * factor);
+        x = f32_to_bf16(bf16_to_f32(x) + bf16_to_f32(bias[t * H + h]));
+        out[t * H + h] = x;
+      }
+    }
+}
+
+/* ------------------------------------------------------- whole path ---- */
+
+/*
+ * fused_experts_impl_int8 for one chunk (int8.py:703-888, with the final
+ * reduce always performed).  Intermediates are returned when the pointers are
+ * non-NULL so that each stage of the HIP path can be compared on its own:
+ *   a1q[M,H] a1s[M,H/128]  c1[S,2I]  act[S,I]  a2q[S,I] a2s[S,I/128]  c3[S,H]
+ * sorted/expert_ids/ntpp are outputs too (capacities as in
+ * moe_align_block_size.py:80-93).  Returns 0 or -1.
+ */
+int orc_fused_experts_block_int8(
+    const uint16_t *x, int64_t M, int64_t H, int64_t I, int32_t E_local,
+    int32_t num_experts_global, int32_t top_k, const int8_t *w1, const float *w1s,
+    const int8_t *w2, const float *w2s, const float *topk_w, const int32_t *topk_ids,
+    const int32_t *expert_map, int32_t bs, int apply_router_weight_on_input,
+    float routed_scaling_factor, const uint16_t *shared_output, uint16_t *out,
+    int32_t *sorted, int64_t sorted_cap, int32_t *expert_ids, int64_t expert_ids_cap,
+    int32_t *ntpp, int8_t *a1q, float *a1s, uint16_t *c1, uint16_t *act, int8_t *a2q,
+    float *a2s, uint16_t *c3) {
+  (void)E_local;
+  int64_t S = M * top_k;
+  int own_a1q = !a1q, own_a1s = !a1s, own_c1 = !c1, own_act = !act, own_a2q = !a2q,
+      own_a2s = !a2s, own_c3 = !c3;
+  if (own_a1q) a1q = (int8_t *)malloc((size_t)(M * H));
+  if (own_a1s) a1s = (float *)malloc(sizeof(float) * (size_t)(M * (H / ORC_GROUP)));
+  if (own_c1) c1 = (uint16_t *)calloc((size_t)(S * 2 * I), 2);
+  if (own_act) act = (uint16_t *)malloc(2 * (size_t)(S * I));
+  if (own_a2q) a2q = (int8_t *)malloc((size_t)(S * I));
+  if (own_a2s) a2s = (float *)malloc(sizeof(float) * (size_t)(S * (I / ORC_GROUP)));
+  if (own_c3) c3 = (uint16_t *)calloc((size_t)(S * H), 2);
+
+  orc_group_quant_int8(x, M, H, 1e-10f, a1q, a1s);
+  int rc = orc_moe_align_block_size(topk_ids, S, num_experts_global, bs, expert_map, 0,
+                                    sorted, sorted_cap, expert_ids, expert_ids_cap, ntpp);
+  if (rc == 0) {
+    orc_moe_gemm_block_int8(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
+                            apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL);
+    orc_silu_and_mul(c1, S, I, act);
+    orc_group_quant_int8(act, S, I, 1e-10f, a2q, a2s);
+    orc_moe_gemm_block_int8(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
+                            !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL);
+    orc_moe_sum(c3, M, top_k, H, shared_output, routed_scaling_factor, out);
+  }
+  if (own_a1q) free(a1q);
+  if (own_a1s) free(a1s);
+  if (own_c1) free(c1);
+  if (own_act) free(act);
+  if (own_a2q) free(a2q);
+  if (own_a2s) free(a2s);
+  if (own_c3) free(c3);
+  return rc;
+}

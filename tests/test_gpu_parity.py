@@ -1,0 +1,348 @@
+"""GPU parity: every stage of the HIP path against the CPU oracle, through the C ABI
+(ctypes) exactly as a caller would reach it.  Integer, int8 and index outputs must be
+bit-exact; bf16 outputs of the canonical-order kernels are bit-exact as well, and the
+fused-scale variants must stay within max-abs <= 1e-2 * max|ref| and mean-rel <= 2e-3."""
+import math
+import sys
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+BS_ALL = (16, 32, 64, 128)
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from lightop_amd import _lib
+
+    _lib.lib()  # a missing HIP library must fail the run, not skip it
+    return torch.device("cuda:0")
+
+
+def within_tolerance(out, ref):
+    o, r = out.float().cpu(), ref.float().cpu()
+    err = (o - r).abs()
+    return err.max().item() <= 1e-2 * r.abs().max().item() and \
+        (err.sum() / r.abs().sum().clamp(min=1e-30)).item() <= 2e-3
+
+
+# ------------------------------------------------------------------ alignment --
+
+@pytest.mark.parametrize("S,E,bs", [(1, 8, 16), (2, 64, 16), (7, 4, 16), (128, 8, 16), (512, 256, 16),
+                                    (1000, 33, 32), (4096, 128, 64), (8191, 5, 128), (32768, 256, 64),
+                                    (65536, 256, 128), (131072, 256, 16), (3000, 1000, 16)])
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+def test_align_bit_exact(dev, oracle, S, E, bs, idt):
+    from lightop_amd.moe import moe_align_block_size
+
+    say(f"align S={S} E={E} bs={bs} {idt}")
+    g = torch.Generator().manual_seed(S + E)
+    ids = torch.randint(0, E, (S,), generator=g, dtype=torch.int32)
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, E)
+    s, e, p = moe_align_block_size(ids.to(idt).to(dev).view(-1, 1), bs, E)
+    torch.cuda.synchronize()
+    assert torch.equal(p.cpu(), rp)
+    assert torch.equal(s.cpu(), rs), "sorted_token_ids differ"
+    assert torch.equal(e.cpu(), re), "expert_ids differ"
+
+
+@pytest.mark.parametrize("ignore", [False, True])
+def test_align_expert_map(dev, oracle, ignore):
+    from lightop_amd.moe import moe_align_block_size
+
+    say(f"align expert_map ignore={ignore}")
+    g = torch.Generator().manual_seed(11)
+    E = 256
+    ids = torch.randint(0, E, (333, 8), generator=g, dtype=torch.int32)
+    emap = torch.full((E,), -1, dtype=torch.int32)
+    emap[64:96] = torch.arange(32, dtype=torch.int32)
+    rs, re, rp = oracle.moe_align_block_size(ids, 16, E, expert_map=emap, ignore_invalid_experts=ignore)
+    s, e, p = moe_align_block_size(ids.to(dev), 16, E, expert_map=emap.to(dev), ignore_invalid_experts=ignore)
+    torch.cuda.synchronize()
+    assert torch.equal(p.cpu(), rp) and torch.equal(s.cpu(), rs) and torch.equal(e.cpu(), re)
+
+
+def test_align_skewed_and_docstring(dev, oracle):
+    from lightop_amd.moe import moe_align_block_size
+
+    say("align docstring + all-one-expert")
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]], dtype=torch.int32)
+    s, e, p = moe_align_block_size(ids.to(dev), 4, 5)
+    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert p.item() == 16 and e[:4].tolist() == [1, 2, 3, 4]
+    ids = torch.full((5000,), 3, dtype=torch.int32)
+    rs, re, rp = oracle.moe_align_block_size(ids, 64, 8)
+    s, e, p = moe_align_block_size(ids.to(dev).view(-1, 1), 64, 8)
+    assert torch.equal(s.cpu(), rs) and torch.equal(e.cpu(), re) and torch.equal(p.cpu(), rp)
+
+
+def test_align_out_variant_and_errors(dev, oracle):
+    from lightop_amd.moe import moe_align_block_size_out
+
+    say("align out variant")
+    ids = torch.randint(0, 16, (64, 2), dtype=torch.int32)
+    cap, nb = oracle.align_buffer_sizes(128, 16, 16)
+    s = torch.empty(cap, dtype=torch.int32, device=dev)
+    e = torch.empty(nb, dtype=torch.int32, device=dev)
+    p = torch.empty(1, dtype=torch.int32, device=dev)
+    moe_align_block_size_out(ids.to(dev), 16, 16, s, e, p)
+    rs, re, rp = oracle.moe_align_block_size(ids, 16, 16)
+    assert torch.equal(s.cpu(), rs) and torch.equal(e.cpu(), re) and torch.equal(p.cpu(), rp)
+    with pytest.raises(RuntimeError):
+        moe_align_block_size_out(ids.to(dev), 16, 16, s[:10], e, p)
+
+
+# ---------------------------------------------------------------- group quant --
+
+@pytest.mark.parametrize("rows,cols", [(1, 128), (1, 7168), (3, 2048), (64, 1024), (257, 768), (4096, 2048)])
+def test_group_quant_bit_exact(dev, oracle, rows, cols):
+    from lightop_amd.quant import per_token_group_quant_int8
+
+    say(f"quant {rows}x{cols}")
+    g = torch.Generator().manual_seed(rows * 13 + cols)
+    x = (torch.randn(rows, cols, generator=g) * torch.rand(rows, 1, generator=g) * 8).to(torch.bfloat16)
+    x[0, :128] = 0  # an all-zero group
+    if rows > 1:
+        x[1, 5] = 300.0
+    rq, rs = oracle.per_token_group_quant_int8(x)
+    q, s = per_token_group_quant_int8(x.to(dev), 128)
+    torch.cuda.synchronize()
+    assert q.dtype == torch.int8 and s.dtype == torch.float32 and s.shape == (rows, cols // 128)
+    assert torch.equal(s.cpu(), rs), "scales differ"
+    assert torch.equal(q.cpu(), rq), "int8 values differ"
+
+
+def test_group_quant_truncation_cases(dev):
+    from lightop_amd.quant import per_token_group_quant_int8
+
+    say("quant truncation cases")
+    row = [127.0, 1.5, -1.5, 2.5, -2.5, 0.75, -0.75, 126.5] + [0.0] * 120
+    q, s = per_token_group_quant_int8(torch.tensor([row]).to(torch.bfloat16).to(dev), 128)
+    assert s.item() == 1.0 and q[0, :8].tolist() == [127, 1, -1, 2, -2, 0, 0, 126]
+    with pytest.raises(AssertionError):
+        per_token_group_quant_int8(torch.zeros(2, 100, dtype=torch.bfloat16, device=dev), 128)
+
+
+# --------------------------------------------------------------- SiLU * mul ----
+
+def test_silu_and_mul_every_bf16(dev, oracle):
+    from lightop_amd.moe import silu_and_mul
+
+    say("silu_and_mul over all bf16 gates")
+    gate = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).view(512, 128)
+    finite = torch.isfinite(gate.float())
+    gate = torch.where(finite, gate, torch.zeros_like(gate))
+    g = torch.Generator().manual_seed(4)
+    up = torch.randn(512, 128, generator=g).to(torch.bfloat16)
+    c1 = torch.cat([gate, up], dim=1).contiguous()
+    ref = oracle.silu_and_mul(c1)
+    out = torch.empty(512, 128, dtype=torch.bfloat16, device=dev)
+    silu_and_mul(out, c1.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+# ------------------------------------------------------------------ moe_sum ----
+
+@pytest.mark.parametrize("M,k,H", [(1, 8, 7168), (5, 2, 1024), (64, 8, 2048), (33, 1, 256), (300, 6, 4096)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_moe_sum_bit_exact(dev, oracle, M, k, H, with_bias):
+    from lightop_amd.moe import moe_sum
+
+    say(f"moe_sum M={M} k={k} H={H} bias={with_bias}")
+    g = torch.Generator().manual_seed(M + k + H)
+    x = torch.randn(M, k, H, generator=g).to(torch.bfloat16)
+    b = torch.randn(M, H, generator=g).to(torch.bfloat16) if with_bias else None
+    ref = oracle.moe_sum(x, bias=b, factor=2.5)
+    out = torch.empty(M, H, dtype=torch.bfloat16, device=dev)
+    moe_sum(x.to(dev), out, bias=None if b is None else b.to(dev), factor=2.5)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+# --------------------------------------------------------------------- GEMM ----
+
+def gemm_case(seed, M, k, E, Eg, N, K, small_values=False):
+    g = torch.Generator().manual_seed(seed)
+    lo, hi = (-7, 8) if small_values else (-127, 128)
+    Aq = torch.randint(lo, hi, (M, K), generator=g, dtype=torch.int8)
+    W = torch.randint(lo, hi, (E, N, K), generator=g, dtype=torch.int8)
+    if small_values:
+        As = torch.ones(M, K // 128)
+        Ws = torch.ones(E, (N + 127) // 128, K // 128)
+    else:
+        As = torch.rand(M, K // 128, generator=g) * 0.05 + 0.005
+        Ws = torch.exp(torch.randn(E, (N + 127) // 128, K // 128, generator=g) * 0.3 + math.log(1e-3))
+    ids = torch.stack([torch.randperm(Eg, generator=g)[:k] for _ in range(M)]).to(torch.int32)
+    tw = torch.rand(M, k, generator=g) + 0.1
+    emap = None
+    if Eg != E:
+        emap = torch.full((Eg,), -1, dtype=torch.int32)
+        emap[:E] = torch.arange(E, dtype=torch.int32)
+    return Aq, As, W, Ws, ids, tw, emap
+
+
+@pytest.mark.parametrize("M,k,E,Eg,N,K", [(1, 2, 4, 4, 64, 128), (5, 2, 4, 4, 256, 512), (40, 4, 8, 8, 320, 1024),
+                                          (64, 2, 8, 8, 1024, 1024), (100, 8, 4, 16, 512, 768),
+                                          (300, 2, 3, 3, 128, 2048)])
+@pytest.mark.parametrize("bs", BS_ALL)
+def test_gemm_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
+    from lightop_amd.moe import invoke_fused_moe_kernel_int8, moe_align_block_size
+
+    say(f"gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs}")
+    Aq, As, W, Ws, ids, tw, emap = gemm_case(M + N + bs, M, k, E, Eg, N, K)
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
+    S = M * k
+    for mul in (False, True):
+        ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, k, S, bs)
+        C = torch.full((M, k, N), 7.0, dtype=torch.bfloat16, device=dev)
+        s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
+        invoke_fused_moe_kernel_int8(Aq.to(dev), W.to(dev), C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
+                                     mul, k, {"BLOCK_SIZE_M": bs})
+        torch.cuda.synchronize()
+        assert torch.equal(C.view(S, N).cpu().view(torch.int16), ref.view(torch.int16)), f"mul_routed={mul}"
+    # fused-scale variant: same integers, fp32 rounding differs in the last place only
+    C2 = torch.empty((M, k, N), dtype=torch.bfloat16, device=dev)
+    invoke_fused_moe_kernel_int8(Aq.to(dev), W.to(dev), C2, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
+                                 True, k, {"BLOCK_SIZE_M": bs}, fused_scale=True)
+    torch.cuda.synchronize()
+    assert within_tolerance(C2.view(S, N), ref)
+    differs = (C2.view(S, N).cpu().view(torch.int16) != ref.view(torch.int16)).float().mean().item()
+    assert differs < 0.02, differs
+
+
+@pytest.mark.parametrize("bs", BS_ALL)
+def test_gemm_int32_accumulators_exact(dev, oracle, bs):
+    """Unit scales and small integers: the bf16 output is then the exactly rounded integer
+    dot product, in any summation order, for both scale modes."""
+    from lightop_amd.moe import invoke_fused_moe_kernel_int8, moe_align_block_size
+
+    say(f"gemm integer exactness bs={bs}")
+    M, k, E, N, K = 70, 2, 4, 256, 7168
+    Aq, As, W, Ws, ids, tw, emap = gemm_case(99 + bs, M, k, E, E, N, K, small_values=True)
+    exact = torch.einsum("mk,enk->men", Aq.double(), W.double())  # [M, E, N], exact in float64
+    s, e, p = moe_align_block_size(ids.to(dev), bs, E)
+    for fused in (False, True):
+        C = torch.empty((M, k, N), dtype=torch.bfloat16, device=dev)
+        invoke_fused_moe_kernel_int8(Aq.to(dev), W.to(dev), C, As.to(dev), Ws.to(dev), None, s, e, p,
+                                     False, k, {"BLOCK_SIZE_M": bs}, fused_scale=fused)
+        torch.cuda.synchronize()
+        want = torch.stack([exact[m, ids[m].long()] for m in range(M)])  # [M, k, N]
+        assert torch.equal(C.cpu(), want.float().to(torch.bfloat16)), f"fused_scale={fused}"
+
+
+@pytest.mark.parametrize("M,k,E,Eg,I,K", [(1, 2, 4, 4, 128, 256), (9, 2, 4, 4, 256, 512), (64, 2, 8, 8, 512, 1024),
+                                          (50, 8, 4, 16, 256, 768), (200, 4, 6, 6, 384, 1024)])
+@pytest.mark.parametrize("bs", BS_ALL)
+def test_gemm1_silu_quant_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
+    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size
+
+    say(f"gemm1+silu+quant M={M} k={k} E={E}/{Eg} I={I} K={K} bs={bs}")
+    Aq, As, W, Ws, ids, tw, emap = gemm_case(M + I + bs + 1, M, k, E, Eg, 2 * I, K)
+    Ws = Ws * 30  # bring the gate into the range where SiLU is neither 0 nor identity
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
+    S = M * k
+    s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
+    for mul in (False, True):
+        c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, k, S, bs)
+        rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+        q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), W.to(dev), As.to(dev), Ws.to(dev), tw.to(dev),
+                                                  s, e, p, mul, k, S, {"BLOCK_SIZE_M": bs})
+        torch.cuda.synchronize()
+        local = torch.ones(S, dtype=torch.bool) if emap is None else emap.long()[ids.reshape(-1).long()] >= 0
+        assert torch.equal(sc.cpu()[local], rsc[local]), f"scales differ (mul_routed={mul})"
+        assert torch.equal(q.cpu()[local], rq[local]), f"int8 activations differ (mul_routed={mul})"
+
+
+# ---------------------------------------------------------------- whole path ---
+
+def run_fused(dev, layer, M, seed, bs=0, flags=0, shared=False, on_input=False, inplace=False):
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import fused_experts_impl_int8
+
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=seed)
+    x, tw, ids = wl.make_inputs(layer, M, seed=seed)
+    emap = wl.expert_map_for(layer)
+    g = torch.Generator().manual_seed(seed + 5)
+    sh = torch.randn(M, layer.H, generator=g).to(torch.bfloat16) if shared else None
+    cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
+    xd = x.to(dev)
+    out = fused_experts_impl_int8(
+        xd, w1.to(dev), w2.to(dev), tw.to(dev), ids.to(dev), cache13, inplace=inplace,
+        apply_router_weight_on_input=on_input, use_int8_w8a8=True, global_num_experts=layer.E_global,
+        expert_map=None if emap is None else emap.to(dev), w1_scale=w1s.to(dev), w2_scale=w2s.to(dev),
+        block_shape=[128, 128], routed_scaling_factor=1.0 if not shared else 2.5,
+        shared_output=None if sh is None else sh.to(dev), lightop_amd_block_size_m=bs, lightop_amd_flags=flags)
+    torch.cuda.synchronize()
+    if inplace:
+        assert out.data_ptr() == xd.data_ptr()
+    return (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out.cpu()
+
+
+@pytest.mark.parametrize("bs", BS_ALL)
+def test_fused_experts_tiny_config_bit_exact(dev, oracle, bs):
+    """BASELINE config 1: E=8, top-2, H=1024, I=512, M=64, seed 0."""
+    from lightop_amd import workloads as wl
+
+    say(f"fused tiny bs={bs}")
+    (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, wl.TINY, 64, 0, bs=bs)
+    ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, bs)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 77])
+@pytest.mark.parametrize("variant", ["plain", "shared", "on_input", "inplace"])
+def test_fused_experts_ep_share_bit_exact(dev, oracle, M, variant):
+    from lightop_amd import workloads as wl
+
+    say(f"fused ep-share M={M} {variant}")
+    layer = wl.MoeLayer("ep", E=4, E_global=32, top_k=8, H=512, I=256, routing="grouped_sigmoid",
+                        n_group=8, topk_group=4, routed_scaling=2.5)
+    kw = dict(shared=variant == "shared", on_input=variant == "on_input", inplace=variant == "inplace")
+    (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, layer, M, 3, bs=16, **kw)
+    ref = oracle.fused_experts_block_int8(
+        x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=32, expert_map=emap,
+        apply_router_weight_on_input=kw["on_input"], routed_scaling_factor=2.5 if kw["shared"] else 1.0,
+        shared_output=sh)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+def test_fused_experts_default_tile_and_fused_scale(dev, oracle):
+    from lightop_amd import _lib, workloads as wl
+
+    say("fused default tile + fused-scale tolerance")
+    layer = wl.MoeLayer("q", E=16, E_global=16, top_k=4, H=512, I=256, routing="softmax")
+    (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, layer, 200, 1, flags=_lib.LO_GEMM_FUSED_SCALE)
+    ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 64)
+    assert within_tolerance(out, ref)
+
+
+def test_fused_experts_rejects_unsupported(dev):
+    from lightop_amd.moe import fused_experts_impl_int8
+
+    x = torch.zeros(2, 256, dtype=torch.bfloat16, device=dev)
+    w1 = torch.zeros(2, 256, 256, dtype=torch.int8, device=dev)
+    w2 = torch.zeros(2, 256, 128, dtype=torch.int8, device=dev)
+    tw = torch.ones(2, 1, device=dev)
+    ids = torch.zeros(2, 1, dtype=torch.int32, device=dev)
+    c = torch.empty(2 * 256, dtype=torch.bfloat16, device=dev)
+    s1 = torch.ones(2, 2, 2, device=dev)
+    s2 = torch.ones(2, 2, 1, device=dev)
+    with pytest.raises(NotImplementedError):
+        fused_experts_impl_int8(x, w1, w2, tw, ids, c, use_int8_w8a8=True, per_channel_quant=True,
+                                w1_scale=s1, w2_scale=s2)
+    with pytest.raises(ValueError):
+        fused_experts_impl_int8(x, w1, w2, tw, ids, c, use_int8_w8a8=True, block_shape=[128, 128],
+                                activation="relu", w1_scale=s1, w2_scale=s2)
+    with pytest.raises(AssertionError):
+        fused_experts_impl_int8(x[:, :128], w1, w2, tw, ids, c, use_int8_w8a8=True, block_shape=[128, 128],
+                                w1_scale=s1, w2_scale=s2)

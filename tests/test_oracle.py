@@ -1,0 +1,309 @@
+"""Pins the CPU oracle (oracle/moe_oracle.c) before anything is compared with it.
+
+Every check here is independent of the oracle's own formulae: the reference's
+docstring known answer, brute force with Python integers, closed-form special
+cases, libm, and a second torch restatement with a different summation order.
+
+Pinning status per oracle function
+  orc_moe_align_block_size    pinned: docstring known answer
+                              (moe_align_block_size.py:66-81), brute force, invariants.
+                              The order inside an expert is the stable ascending one of
+                              the reference's own Python test; the reference kernels'
+                              atomics-defined order is not reproducible: parity unpinned
+                              for that order (their test compares sorted multisets).
+  orc_group_quant_int8        pinned: exact power-of-two cases, truncation cases, zeros.
+  orc_moe_gemm_block_int8     int32 part pinned by Python-integer brute force; fp32 part
+                              pinned by closed-form cases and the torch restatement.
+  orc_expf / orc_silu_and_mul pinned against libm expf over all 65536 bf16 inputs.
+  orc_moe_sum                 pinned: k=1 identity, torch.sum, hand-worked roundings.
+  orc_fused_experts_block_int8 pinned against the torch restatement within the path's
+                              tolerance (the reference holds no end-to-end assertion
+                              for the block-INT8 path).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import torch_ref
+
+
+def bf16(vals):
+    return torch.tensor(vals, dtype=torch.float32).to(torch.bfloat16)
+
+
+# ------------------------------------------------------------------ alignment --
+
+def test_align_reference_docstring_example(oracle):
+    # moe_align_block_size.py:66-81: experts 1..4 are used, so five experts with expert 0 empty
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]], dtype=torch.int32)
+    s, e, p = oracle.moe_align_block_size(ids, 4, 5)
+    assert p.item() == 16
+    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert e[:4].tolist() == [1, 2, 3, 4]
+    assert s[16:].tolist() == [12] * (s.numel() - 16)
+
+
+def brute_align(ids, E, bs, emap=None, ignore=False):
+    """Plain Python, list based; independent of the C code."""
+    S = len(ids)
+    buckets = [[] for _ in range(E)]
+    for f, e in enumerate(ids):
+        if ignore and emap is not None:
+            e = emap[e]
+            if e < 0:
+                continue
+        buckets[e].append(f)
+    out, eids = [], []
+    for e, b in enumerate(buckets):
+        nb = -(-len(b) // bs)
+        out += b + [S] * (nb * bs - len(b))
+        eids += [(emap[e] if (emap is not None and not ignore) else e)] * nb
+    return out, eids
+
+
+@pytest.mark.parametrize("S,E,bs", [(1, 8, 16), (7, 4, 4), (64, 8, 16), (300, 256, 16), (1000, 33, 32),
+                                    (4096, 128, 64), (513, 5, 128)])
+def test_align_vs_brute_force(oracle, S, E, bs):
+    g = torch.Generator().manual_seed(S * 31 + E)
+    ids = torch.randint(0, E, (S,), generator=g, dtype=torch.int32)
+    s, e, p = oracle.moe_align_block_size(ids, bs, E)
+    ref_s, ref_e = brute_align(ids.tolist(), E, bs)
+    assert p.item() == len(ref_s)
+    assert s[: len(ref_s)].tolist() == ref_s
+    assert e[: len(ref_e)].tolist() == ref_e
+    assert (s[len(ref_s):] == S).all() and (e[len(ref_e):] == -1).all()
+    # invariants: every slot exactly once, blocks are single-expert
+    valid = s[s < S]
+    assert sorted(valid.tolist()) == list(range(S))
+    blocks = s[: p.item()].view(-1, bs)
+    for b in range(blocks.shape[0]):
+        row = blocks[b][blocks[b] < S]
+        assert (ids[row.long()] == e[b]).all()
+
+
+def test_align_expert_map_modes(oracle):
+    g = torch.Generator().manual_seed(5)
+    E = 16
+    ids = torch.randint(0, E, (200,), generator=g, dtype=torch.int32)
+    emap = torch.full((E,), -1, dtype=torch.int32)
+    emap[4:8] = torch.arange(4, dtype=torch.int32)
+    for ignore in (False, True):
+        s, e, p = oracle.moe_align_block_size(ids, 16, E, expert_map=emap, ignore_invalid_experts=ignore)
+        ref_s, ref_e = brute_align(ids.tolist(), E, 16, emap.tolist(), ignore)
+        assert p.item() == len(ref_s)
+        assert s[: len(ref_s)].tolist() == ref_s and e[: len(ref_e)].tolist() == ref_e
+    # buffer sizing rule when there are fewer slots than experts
+    s, e, p = oracle.moe_align_block_size(torch.tensor([3, 1], dtype=torch.int32), 16, 64)
+    assert s.numel() == 32 and e.numel() == 2 and p.item() == 32
+
+
+def test_align_rejects_bad_ids(oracle):
+    with pytest.raises(RuntimeError):
+        oracle.moe_align_block_size(torch.tensor([0, 9], dtype=torch.int32), 16, 8)
+
+
+# ---------------------------------------------------------------- group quant --
+
+def test_quant_exact_powers_of_two(oracle):
+    # x = i * 2^k with amax = 127 * 2^k  ->  s = 2^k exactly, q = i exactly
+    for k in (-6, 0, 3):
+        vals = [float(i) * 2.0 ** k for i in range(-127, 1)]  # 128 values, amax 127*2^k
+        q, s = oracle.per_token_group_quant_int8(bf16([vals]))
+        assert s.item() == 2.0 ** k
+        assert q[0].tolist() == list(range(-127, 1))
+
+
+def test_quant_truncates_toward_zero(oracle):
+    # amax 127 -> s = 1; 1.5 -> 1 (round would give 2), -1.5 -> -1 (floor would give -2), 2.5 -> 2
+    row = [127.0, 1.5, -1.5, 2.5, -2.5, 0.75, -0.75, 126.5] + [0.0] * 120
+    q, s = oracle.per_token_group_quant_int8(bf16([row]))
+    assert s.item() == 1.0
+    assert q[0, :8].tolist() == [127, 1, -1, 2, -2, 0, 0, 126]
+
+
+def test_quant_zero_group_and_single_value(oracle):
+    q, s = oracle.per_token_group_quant_int8(torch.zeros(1, 256, dtype=torch.bfloat16))
+    assert (q == 0).all()
+    assert s.flatten().tolist() == [np.float32(1e-10) / np.float32(127.0)] * 2
+    # one non-zero value: q is 127 or 126 exactly as IEEE division says
+    for v in (0.3, 1.7, 3.1415, 1000.0, 2.0 ** -20):
+        x = torch.zeros(1, 128, dtype=torch.bfloat16)
+        x[0, 5] = -v
+        xv = np.float32(x[0, 5].float().item())
+        q, s = oracle.per_token_group_quant_int8(x)
+        sc = np.float32(abs(xv)) / np.float32(127.0)
+        assert s.item() == sc
+        assert q[0, 5].item() == int(np.trunc(max(np.float32(xv) / sc, np.float32(-128.0))))
+        assert q[0, 5].item() in (-127, -126)
+
+
+def test_quant_matches_torch_restatement(oracle):
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(37, 1024, generator=g) * 3).to(torch.bfloat16)
+    q, s = oracle.per_token_group_quant_int8(x)
+    q2, s2 = torch_ref.native_per_token_group_quant_int8(x)
+    assert torch.equal(s, s2) and torch.equal(q, q2)
+
+
+# ------------------------------------------------------------------- GEMM -----
+
+def _small_gemm_case(seed, S_tok, k, E, N, K, bs, scales_one=False, emap=None, lo=-127, hi=128):
+    g = torch.Generator().manual_seed(seed)
+    Aq = torch.randint(lo, hi, (S_tok, K), generator=g, dtype=torch.int8)
+    As = torch.ones(S_tok, K // 128) if scales_one else torch.rand(S_tok, K // 128, generator=g) * 0.1 + 0.01
+    W = torch.randint(lo, hi, (E, N, K), generator=g, dtype=torch.int8)
+    Ws = torch.ones(E, (N + 127) // 128, K // 128) if scales_one else \
+        torch.exp(torch.randn(E, (N + 127) // 128, K // 128, generator=g) * 0.3 + math.log(1e-3))
+    Eg = E if emap is None else emap.numel()
+    ids = torch.randint(0, Eg, (S_tok, k), generator=g, dtype=torch.int32)
+    tw = torch.rand(S_tok, k, generator=g)
+    return Aq, As, W, Ws, ids, tw, Eg
+
+
+def test_gemm_int32_exact_vs_python_integers(oracle):
+    Aq, As, W, Ws, ids, tw, Eg = _small_gemm_case(3, 5, 2, 3, 32, 256, 16, scales_one=True)
+    s, e, p = oracle.moe_align_block_size(ids, 16, Eg)
+    C, acc = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, None, False, 2, 10, 16, dump_acc=True)
+    A64, W64 = Aq.numpy().astype(np.int64), W.numpy().astype(np.int64)
+    flat = ids.reshape(-1).tolist()
+    for f in range(10):
+        for n in range(32):
+            for kb in range(2):
+                d = int((A64[f // 2, kb * 128:(kb + 1) * 128] * W64[flat[f], n, kb * 128:(kb + 1) * 128]).sum())
+                assert acc[f, n, kb].item() == d
+            # scales of one: the bf16 output is the rounded exact integer sum
+            tot = float(acc[f, n].sum().item())
+            assert C[f, n].item() == torch.tensor(tot).to(torch.bfloat16).item()
+
+
+def test_gemm_scale_order_and_router_weight(oracle):
+    # one token, one expert, K=256: acc = (d0*as0)*ws0 + (d1*as1)*ws1, then * w, then bf16
+    Aq = torch.zeros(1, 256, dtype=torch.int8); Aq[0, 0] = 100; Aq[0, 128] = -7
+    W = torch.zeros(1, 16, 256, dtype=torch.int8); W[0, :, 0] = 3; W[0, :, 128] = 11
+    As = torch.tensor([[0.37, 1.9]]); Ws = torch.tensor([[[0.0123, 0.5]]])
+    ids = torch.zeros(1, 1, dtype=torch.int32); tw = torch.tensor([[0.731]])
+    s, e, p = oracle.moe_align_block_size(ids, 16, 1)
+    C = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, tw, True, 1, 1, 16)
+    f = np.float32
+    acc = f(0) + (f(300) * f(0.37)) * f(0.0123)
+    acc = acc + (f(-77) * f(1.9)) * f(0.5)
+    acc = acc * f(0.731)
+    assert C[0, 0].item() == torch.tensor(float(acc)).to(torch.bfloat16).item()
+    assert (C[0] == C[0, 0]).all()
+
+
+def test_gemm_vs_torch_restatement_and_skipped_experts(oracle):
+    emap = torch.tensor([0, -1, 1, -1], dtype=torch.int32)
+    Aq, As, W, Ws, ids, tw, Eg = _small_gemm_case(7, 24, 2, 2, 256, 384, 16, emap=emap)
+    s, e, p = oracle.moe_align_block_size(ids, 16, Eg, expert_map=emap)
+    C = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, None, False, 2, 48, 16)
+    flat = emap.long()[ids.reshape(-1).long()]
+    for f in range(48):
+        if flat[f] < 0:
+            assert (C[f] == 0).all()
+            continue
+        ref = torch_ref.native_w8a8_block_int8_matmul(Aq[f // 2:f // 2 + 1], W[flat[f]], As[f // 2:f // 2 + 1],
+                                                      Ws[flat[f]], output_dtype=torch.float32)
+        got = C[f].float()
+        # bf16 of two fp32 sums that differ only in rounding order: equal up to one bf16 ulp
+        assert torch.allclose(got, ref[0], rtol=2 ** -7, atol=1e-6)
+        assert (got - ref[0]).abs().mean() <= 2 ** -8 * ref[0].abs().mean()
+
+
+# --------------------------------------------------------------- SiLU * mul ----
+
+def test_expf_vs_libm(oracle):
+    lib = oracle.lib()
+    xs = np.concatenate([np.linspace(-87, 88.7, 200001, dtype=np.float32),
+                         np.random.default_rng(0).normal(0, 4, 100000).astype(np.float32)])
+    worst = 0.0
+    for x in xs[::7]:
+        got = lib.orc_expf(float(x))
+        ref = math.exp(float(x))
+        ulp = np.spacing(np.float32(ref))
+        worst = max(worst, abs(got - ref) / float(ulp))
+    assert worst <= 1.0, worst
+
+
+def test_silu_equals_libm_silu_on_every_bf16(oracle):
+    lib = oracle.lib()
+    bad = []
+    for h in range(65536):
+        e = (h >> 7) & 0xFF
+        if e == 0xFF:  # inf / nan
+            continue
+        if lib.orc_silu_bf16(h) != lib.orc_silu_bf16_libm(h):
+            bad.append(h)
+    assert not bad, f"{len(bad)} bf16 inputs differ from the libm-based SiLU, e.g. {bad[:8]}"
+
+
+def test_silu_and_mul_vs_torch(oracle):
+    g = torch.Generator().manual_seed(2)
+    c1 = (torch.randn(64, 512, generator=g) * 4).to(torch.bfloat16)
+    act = oracle.silu_and_mul(c1)
+    ref = torch.nn.functional.silu(c1[:, :256].float()).to(torch.bfloat16).float() * c1[:, 256:].float()
+    # the reference's own bar for this op is rtol = atol = 1e-2 (test/ci_tests/test_fuse_silu_mul.py:31-33)
+    assert torch.allclose(act.float(), ref, rtol=1e-2, atol=1e-2)
+    # and bit-for-bit against torch's own bf16 rounding of the same two-step formula
+    assert (act == ref.to(torch.bfloat16)).float().mean() > 0.999
+    # gate is the first half: silu(0) * u == 0, silu(large) ~ g
+    z = torch.zeros(1, 256, dtype=torch.bfloat16); z[0, 128:] = 3.0
+    assert (oracle.silu_and_mul(z) == 0).all()
+
+
+# ------------------------------------------------------------------ moe_sum ----
+
+def test_moe_sum_cases(oracle):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(9, 1, 64, generator=g).to(torch.bfloat16)
+    assert torch.equal(oracle.moe_sum(x), x[:, 0])                      # k = 1, factor 1: identity
+    x = torch.randn(9, 8, 64, generator=g).to(torch.bfloat16)
+    assert torch.equal(oracle.moe_sum(x), x.float().sum(dim=1).to(torch.bfloat16)) or \
+        torch.allclose(oracle.moe_sum(x).float(), x.float().sum(dim=1), rtol=2 ** -8)
+    # sequential fp32 order, one rounding: hand-worked
+    v = bf16([[[1.0], [2.0 ** -9], [2.0 ** -9]]])                       # 1 + 2^-9 + 2^-9 = 1 + 2^-8
+    assert oracle.moe_sum(v).float().item() == 1.0 + 2.0 ** -7 or oracle.moe_sum(v).float().item() == 1.0
+    f = np.float32
+    acc = (f(0) + f(1.0)) + f(2.0 ** -9) + f(2.0 ** -9)
+    assert oracle.moe_sum(v, factor=2.5).float().item() == torch.tensor(float(acc * f(2.5))).to(torch.bfloat16).item()
+    # with bias: three roundings
+    b = bf16([[0.00390625]])
+    xr = torch.tensor(float(acc)).to(torch.bfloat16).float()
+    xr = (xr * 2.5).to(torch.bfloat16).float()
+    xr = (xr + b.float()).to(torch.bfloat16)
+    assert oracle.moe_sum(v, bias=b, factor=2.5).item() == xr.item()
+
+
+# ------------------------------------------------------------- whole path -----
+
+def test_fused_path_vs_torch_restatement(oracle):
+    from lightop_amd import workloads as wl
+
+    layer = wl.MoeLayer("t", E=4, E_global=4, top_k=2, H=256, I=128, routing="softmax")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
+    x, tw, ids = wl.make_inputs(layer, 33, seed=0)
+    out = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 16)
+    ref = torch_ref.torch_w8a8_block_int8_moe(x, w1, w2, w1s, w2s, tw, ids)
+    err = (out.float() - ref.float()).abs()
+    assert err.max() <= 1e-2 * ref.float().abs().max()
+    assert (err.sum() / ref.float().abs().sum()) <= 2e-3 * 3  # two bf16 roundings apart
+
+
+def test_fused_path_expert_parallel_share(oracle):
+    from lightop_amd import workloads as wl
+
+    layer = wl.MoeLayer("t", E=4, E_global=32, top_k=8, H=256, I=128, routing="grouped_sigmoid",
+                        n_group=8, topk_group=4, routed_scaling=2.5)
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=1)
+    x, tw, ids = wl.make_inputs(layer, 40, seed=1)
+    emap = wl.expert_map_for(layer)
+    r = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=32,
+                                        expert_map=emap, return_intermediates=True)
+    ref = torch_ref.torch_w8a8_block_int8_moe(x, w1, w2, w1s, w2s, tw, ids, expert_map=emap)
+    err = (r["out"].float() - ref.float()).abs()
+    assert err.max() <= 1e-2 * ref.float().abs().max()
+    assert (r["expert_ids"][: r["num_tokens_post_pad"].item() // 16] >= -1).all()
+    nonlocal_slots = emap.long()[ids.reshape(-1).long()] < 0
+    assert (r["c3"][nonlocal_slots] == 0).all()
