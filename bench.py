@@ -1,0 +1,265 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-INT8 fused-MoE path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--tokens M]
+                    [--sweep {default,none,full}] [--no-cpu-baseline]
+
+A step is one call of ``fused_experts_impl_int8`` on one batch of synthetic tokens with
+every input already resident in HBM.  Between steps a 512 MiB buffer is overwritten so
+that weights are streamed from HBM and not served from the 256 MB Infinity Cache; the
+step time is taken with HIP events on the launching stream and excludes that flush.
+The last line printed is one JSON object (see README / DESIGN for the fields).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0        # MI355X dense INT8 MFMA, published (5.0 POP/s)
+
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc
+# (FETCH_SIZE and WRITE_SIZE runs, scaled by a copy kernel of known size); keyed by
+# (workload, tokens).  None until measured for that point.
+MEASURED_TRAFFIC = {}
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--workload", default="qwen3-30b-a3b")
+    p.add_argument("--tokens", type=int, default=8192)
+    p.add_argument("--sweep", default="default", choices=["default", "none", "full"])
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--block-size-m", type=int, default=0)
+    p.add_argument("--fused-scale", type=int, default=-1, help="-1: library default per tile, 0/1: force")
+    return p.parse_args()
+
+
+class Flusher:
+    """Evicts the Infinity Cache between steps by overwriting 512 MiB."""
+
+    def __init__(self, dev):
+        self.buf = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.int32, device=dev)
+        self.i = 0
+
+    def __call__(self):
+        self.i += 1
+        self.buf.fill_(self.i)
+
+
+def time_steps(fn, steps, warmup, flush):
+    """Mean / median / min of `steps` event-timed calls (ms), each after a cache flush."""
+    for _ in range(warmup):
+        flush()
+        fn()
+    torch.cuda.synchronize()
+    evs = []
+    for _ in range(steps):
+        flush()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    ts = [a.elapsed_time(b) for a, b in evs]
+    return sum(ts) / len(ts), statistics.median(ts), min(ts)
+
+
+class Point:
+    """One (layer, M) measurement: whole path plus the two GEMM kernels on their own."""
+
+    def __init__(self, layer, weights, M, dev, seed=0):
+        from lightop_amd import workloads as wl
+
+        self.layer, self.M, self.dev = layer, M, dev
+        self.w1, self.w2, self.w1s, self.w2s = weights
+        self.emap = wl.expert_map_for(layer, dev)
+        # a pool of different batches so that consecutive steps hit different experts
+        pool = 8 if M <= 64 else 2
+        self.batches = [tuple(t.to(dev) for t in wl.make_inputs(layer, M, seed=seed + i)) for i in range(pool)]
+        self.cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
+        self.i = 0
+        ops = byts = sloc = eact = 0
+        for (_, _, ids) in self.batches:
+            o, b, s, e = wl.algorithmic_work(layer, ids, self.emap)
+            ops, byts, sloc, eact = ops + o, byts + b, sloc + s, eact + e
+        n = len(self.batches)
+        self.ops, self.bytes, self.S_loc, self.E_act = ops / n, byts / n, sloc / n, eact / n
+
+    def step(self, bs=0, flags=0):
+        from lightop_amd.moe import fused_experts_impl_int8
+
+        x, tw, ids = self.batches[self.i % len(self.batches)]
+        self.i += 1
+        L = self.layer
+        return fused_experts_impl_int8(
+            x, self.w1, self.w2, tw, ids, self.cache13, use_int8_w8a8=True, global_num_experts=L.E_global,
+            expert_map=self.emap, w1_scale=self.w1s, w2_scale=self.w2s, block_shape=[128, 128],
+            lightop_amd_block_size_m=bs, lightop_amd_flags=flags)
+
+    def stage_times(self, steps, warmup, flush, bs=0, fused_scale=False):
+        """Event-timed duration of each stage kernel launched on its own (ms, mean)."""
+        from lightop_amd import moe
+        from lightop_amd.quant import per_token_group_quant_int8
+
+        L = self.layer
+        if bs == 0:
+            bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, [128, 128], L.top_k, L.E_global)[0]["BLOCK_SIZE_M"]
+        cfg = {"BLOCK_SIZE_M": bs}
+        S = self.M * L.top_k
+        c3 = self.cache13[: S * L.H].view(self.M, L.top_k, L.H)
+        out = torch.empty(self.M, L.H, dtype=torch.bfloat16, device=self.dev)
+        names = ["quant", "align", "gemm1_silu_quant", "gemm2", "moe_sum"]
+        acc = {n: [] for n in names}
+        for it in range(warmup + steps):
+            x, tw, ids = self.batches[it % len(self.batches)]
+            flush()
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+            ev[0].record()
+            a1q, a1s = per_token_group_quant_int8(x, 128)
+            ev[1].record()
+            s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
+            ev[2].record()
+            a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
+                                                             L.top_k, S, cfg, fused_scale=fused_scale)
+            ev[3].record()
+            moe.invoke_fused_moe_kernel_int8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, True, 1, cfg,
+                                             fused_scale=fused_scale)
+            ev[4].record()
+            moe.moe_sum(c3, out)
+            ev[5].record()
+            if it >= warmup:
+                torch.cuda.synchronize()
+                for i, n in enumerate(names):
+                    acc[n].append(ev[i].elapsed_time(ev[i + 1]))
+        return {n: sum(v) / len(v) for n, v in acc.items()}, bs
+
+
+def measure_point(pt, steps, warmup, flush, bs, flags):
+    mean_ms, med_ms, min_ms = time_steps(lambda: pt.step(bs, flags), steps, warmup, flush)
+    t = mean_ms * 1e-3
+    L = pt.layer
+    hbm = pt.bytes / t / 1e9
+    tops = pt.ops / t / 1e12
+    t_hbm, t_mfma = pt.bytes / (HBM_PEAK_GBS * 1e9), pt.ops / (INT8_PEAK_TOPS * 1e12)
+    bound = "mfma" if t_mfma > t_hbm else "hbm"
+    return {
+        "workload": L.name, "tokens": pt.M, "ms_per_step": round(mean_ms, 4), "ms_median": round(med_ms, 4),
+        "ms_min": round(min_ms, 4), "tokens_per_s": round(pt.M / t, 1), "int8_tops": round(tops, 2),
+        "hbm_gbs": round(hbm, 1), "S_loc": pt.S_loc, "E_act": pt.E_act, "bound": bound,
+        "roofline_frac": round((tops / INT8_PEAK_TOPS) if bound == "mfma" else (hbm / HBM_PEAK_GBS), 4),
+        "frac_hbm": round(hbm / HBM_PEAK_GBS, 4), "frac_mfma": round(tops / INT8_PEAK_TOPS, 4),
+    }
+
+
+def cpu_baseline(layer, weights, M_sample, seed=0):
+    """The torch-CPU restatement of the reference path on the host cores, on the first
+    M_sample tokens of the benchmark's batch."""
+    from lightop_amd import workloads as wl
+    from oracle import torch_ref
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    w1, w2, w1s, w2s = (t.cpu() for t in weights)
+    x, tw, ids = wl.make_inputs(layer, M_sample, seed=seed)
+    emap = wl.expert_map_for(layer)
+    t0 = time.perf_counter()
+    torch_ref.torch_w8a8_block_int8_moe(x, w1, w2, w1s, w2s, tw, ids, expert_map=emap)
+    dt = time.perf_counter() - t0
+    return {"value": round(M_sample / dt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{layer.name}, first {M_sample} tokens of the same synthetic batch, one timed run of "
+                      f"oracle/torch_ref.py ({dt:.1f} s), torch {torch.__version__} CPU"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (one process, one MI355X, no collectives); "
+              f"--gpus {args.gpus} is not supported. Expert-parallel sharding is described in DESIGN.md.",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from lightop_amd import _lib, workloads as wl
+
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    flush = Flusher(dev)
+    flags_default = 0 if args.fused_scale <= 0 else _lib.LO_GEMM_FUSED_SCALE
+
+    layer = wl.LAYERS[args.workload]
+    weights = wl.make_weights(layer, seed=0, device=dev, gen_device="cuda")
+    pt = Point(layer, weights, args.tokens, dev)
+    head = measure_point(pt, args.steps, args.warmup, flush, args.block_size_m, flags_default)
+    stages, bs_used = pt.stage_times(args.steps, args.warmup, flush, args.block_size_m,
+                                     fused_scale=bool(flags_default))
+
+    # dominant kernel: the first grouped GEMM with its fused SiLU*mul + re-quantisation
+    L = layer
+    g1_ops = 4.0 * pt.S_loc * L.I * L.H
+    # weights and block scales of the active experts once, int8 activations and their
+    # group scales in (M rows) and out (S_loc rows)
+    g1_bytes = pt.E_act * (2 * L.I * L.H + 4 * (2 * L.I // 128) * (L.H // 128)) \
+        + args.tokens * (L.H + 4 * L.H // 128) + pt.S_loc * (L.I + 4 * L.I // 128)
+    g1_t = stages["gemm1_silu_quant"] * 1e-3
+    if head["bound"] == "mfma":
+        ach, peak, unit = g1_ops / g1_t / 1e12, INT8_PEAK_TOPS, "TFLOP/s"
+    else:
+        ach, peak, unit = g1_bytes / g1_t / 1e9, HBM_PEAK_GBS, "GB/s"
+    roofline = {"bound": head["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
+                "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
+                "kernel": "moe_gemm_ws_kernel (GEMM1 + SiLU*mul + 1x128 re-quant)",
+                "kernel_ms": round(stages["gemm1_silu_quant"], 4),
+                "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately)"}
+
+    sweep = []
+    if args.sweep != "none":
+        plan = [(wl.QWEN3_30B, [1, 8, 32, 128, 512, 2048, 8192]), (wl.DSV3_EP, [1, 16, 64, 256, 1024, 4096])]
+        if args.sweep == "full":
+            plan.append((wl.DSV3_FULL, [8192]))
+        for lay, Ms in plan:
+            w = weights if lay.name == layer.name else wl.make_weights(lay, seed=0, device=dev, gen_device="cuda")
+            for M in Ms:
+                p2 = Point(lay, w, M, dev)
+                sweep.append(measure_point(p2, max(5, args.steps // 2), max(2, args.warmup // 2), flush, 0,
+                                           flags_default))
+                print(f"[sweep] {json.dumps(sweep[-1])}", file=sys.stderr, flush=True)
+                del p2
+            if lay.name != layer.name:
+                del w
+                torch.cuda.empty_cache()
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(layer, weights, min(args.tokens, 256))
+
+    t = head["ms_per_step"] * 1e-3
+    line = {
+        "metric": "block-INT8 fused-MoE tokens/s", "value": round(args.tokens / t, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": f"{layer.name} E={L.E}/{L.E_global} top{L.top_k} H={L.H} I={L.I} "
+                               f"block-INT8[128,128], M={args.tokens}",
+                   "tokens": args.tokens, "block_size_m": bs_used, "routing": L.routing},
+        "int8_tops": head["int8_tops"], "hbm_gbs": head["hbm_gbs"], "frac_hbm": head["frac_hbm"],
+        "frac_mfma": head["frac_mfma"], "stage_ms": {k: round(v, 4) for k, v in stages.items()},
+        "roofline": roofline, "cpu_baseline": cpu, "sweep": sweep,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -39,6 +39,7 @@ struct GemmArgs {
   int64_t K;
   int32_t top_k;
   int32_t n_tiles;       // workgroups along N
+  int32_t E;             // experts held by W
   int32_t mul_routed;
 };
 
@@ -52,6 +53,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   const int mb = bid / a.n_tiles, nt = bid - mb * a.n_tiles;
   if (static_cast<int64_t>(mb) * BM >= a.ntpp[0]) return;
   const int e = a.expert_ids[mb];
+  if (e >= a.E) return; // an expert_map entry outside the weight tensor: nothing to read
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, c = lane >> 4;
   const int64_t K = a.K, N = a.N;
@@ -300,7 +302,7 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   GemmArgs a{};
   a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.C = static_cast<uint16_t *>(C);
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
-  a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.E = E; a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
@@ -332,7 +334,7 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
   GemmArgs a{};
   a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.A2q = A2q; a.A2s = A2s;
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
-  a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.E = E; a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.n_tiles = static_cast<int32_t>(I / kGroup);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 31), LO_EINVAL, "moe_gemm1_silu_quant: grid too large");
