@@ -40,6 +40,8 @@ def parse_args():
     p.add_argument("--sweep", default="default", choices=["default", "none", "full"])
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--block-size-m", type=int, default=0)
+    p.add_argument("--row-major-weights", action="store_true",
+                   help="keep w1/w2 row-major instead of the load-time pre-shuffled layout")
     p.add_argument("--fused-scale", type=int, default=-1, help="-1: library default per tile, 0/1: force")
     return p.parse_args()
 
@@ -107,7 +109,7 @@ class Point:
             expert_map=self.emap, w1_scale=self.w1s, w2_scale=self.w2s, block_shape=[128, 128],
             lightop_amd_block_size_m=bs, lightop_amd_flags=flags)
 
-    def stage_times(self, steps, warmup, flush, bs=0, fused_scale=False):
+    def stage_times(self, steps, warmup, flush, bs=0, fused_scale=None):
         """Event-timed duration of each stage kernel launched on its own (ms, mean)."""
         from lightop_amd import moe
         from lightop_amd.quant import per_token_group_quant_int8
@@ -170,7 +172,7 @@ def cpu_baseline(layer, weights, M_sample, seed=0):
 
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    w1, w2, w1s, w2s = (t.cpu() for t in weights)
+    w1, w2, w1s, w2s = weights
     x, tw, ids = wl.make_inputs(layer, M_sample, seed=seed)
     emap = wl.expert_map_for(layer)
     t0 = time.perf_counter()
@@ -197,14 +199,27 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     flush = Flusher(dev)
-    flags_default = 0 if args.fused_scale <= 0 else _lib.LO_GEMM_FUSED_SCALE
+    flags_default = {-1: 0, 0: _lib.LO_GEMM_CANONICAL_ORDER, 1: _lib.LO_GEMM_FUSED_SCALE}[args.fused_scale]
+
+    from lightop_amd.moe import preshuffle_moe_weight
+
+    cpu_weights = []
+
+    def load_weights(lay, keep_cpu_copy=False):
+        """Synthetic checkpoint -> device, then the one-time load-time layout change."""
+        w1, w2, w1s, w2s = wl.make_weights(lay, seed=0, device=dev, gen_device="cuda")
+        if keep_cpu_copy:
+            cpu_weights.extend(t.cpu() for t in (w1, w2, w1s, w2s))
+        if not args.row_major_weights:
+            w1, w2 = preshuffle_moe_weight(w1), preshuffle_moe_weight(w2)
+        return w1, w2, w1s, w2s
 
     layer = wl.LAYERS[args.workload]
-    weights = wl.make_weights(layer, seed=0, device=dev, gen_device="cuda")
+    weights = load_weights(layer, keep_cpu_copy=not args.no_cpu_baseline and layer.weight_bytes < 8e9)
     pt = Point(layer, weights, args.tokens, dev)
     head = measure_point(pt, args.steps, args.warmup, flush, args.block_size_m, flags_default)
     stages, bs_used = pt.stage_times(args.steps, args.warmup, flush, args.block_size_m,
-                                     fused_scale=bool(flags_default))
+                                     fused_scale={-1: None, 0: False, 1: True}[args.fused_scale])
 
     # dominant kernel: the first grouped GEMM with its fused SiLU*mul + re-quantisation
     L = layer
@@ -230,7 +245,7 @@ def main():
         if args.sweep == "full":
             plan.append((wl.DSV3_FULL, [8192]))
         for lay, Ms in plan:
-            w = weights if lay.name == layer.name else wl.make_weights(lay, seed=0, device=dev, gen_device="cuda")
+            w = weights if lay.name == layer.name else load_weights(lay)
             for M in Ms:
                 p2 = Point(lay, w, M, dev)
                 sweep.append(measure_point(p2, max(5, args.steps // 2), max(2, args.warmup // 2), flush, 0,
@@ -242,8 +257,8 @@ def main():
                 torch.cuda.empty_cache()
 
     cpu = None
-    if not args.no_cpu_baseline:
-        cpu = cpu_baseline(layer, weights, min(args.tokens, 256))
+    if cpu_weights:
+        cpu = cpu_baseline(layer, cpu_weights, min(args.tokens, 2048))
 
     t = head["ms_per_step"] * 1e-3
     line = {

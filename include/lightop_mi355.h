@@ -39,7 +39,16 @@ enum {
   /* accumulate acc += f32(d) * (a_s * b_s) with one fused multiply-add per
    * 128-K block instead of the canonical (f32(d) * a_s) * b_s then add.  The
    * int32 partial sums are identical; the fp32 rounding differs in the last ulp. */
-  LO_GEMM_FUSED_SCALE = 1
+  LO_GEMM_FUSED_SCALE = 1,
+  /* always use the weight-streaming kernels, also where the LDS-tiled kernel applies */
+  LO_GEMM_FORCE_STREAMING = 2,
+  /* canonical (f32(d) * a_s) * b_s + acc order in every kernel.  Without this flag the
+   * LDS-tiled kernel (128-token tiles, where the scale arithmetic competes with the MFMA
+   * pipe) uses the fused-scale order; the weight-streaming kernels are canonical unless
+   * LO_GEMM_FUSED_SCALE is given. */
+  LO_GEMM_CANONICAL_ORDER = 4,
+  /* W (for the whole path: w1 and w2) is in the layout of lo_preshuffle_weight_int8 */
+  LO_GEMM_W_PRESHUFFLED = 8
 };
 
 int lo_version(void);
@@ -134,6 +143,17 @@ int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *ac
  */
 int lo_moe_sum(const void *in, void *out, const void *bias, int dtype, int64_t M, int32_t topk,
                int64_t H, float factor, lo_stream_t stream);
+
+/*
+ * Load-time weight layout for the GEMM kernels: every block of 16 rows x 128 K-bytes of
+ * W [E, N, K] is stored as [8 chunks of 16 K-bytes][16 rows][16 bytes], blocks ordered
+ * [E][K/128][N/16].  Same size as the source; N % 16 == 0, K % 128 == 0; src != dst.
+ * No counterpart on the reference's block-INT8 path (its Triton kernel reads row-major
+ * weights); comparable to the load-time shuffle of its native kernels,
+ * test/moe_w8a8/w8a8_quant.py:66-111.
+ */
+int lo_preshuffle_weight_int8(const int8_t *src, int8_t *dst, int32_t E, int64_t N, int64_t K,
+                              lo_stream_t stream);
 
 /*
  * Tile table: block_size_m (the alignment block and GEMM token tile) chosen for a

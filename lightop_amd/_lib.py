@@ -6,11 +6,12 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
-LIB_PATH = os.path.join(_CSRC, "liblightop_mi355.so")
+LIB_PATH = os.environ.get("LIGHTOP_AMD_LIB") or os.path.join(_CSRC, "liblightop_mi355.so")
 
 LO_BF16, LO_F16 = 0, 1
 LO_I32, LO_I64 = 0, 1
-LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE = 0, 1
+LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE, LO_GEMM_FORCE_STREAMING, LO_GEMM_CANONICAL_ORDER = 0, 1, 2, 4
+LO_GEMM_W_PRESHUFFLED = 8
 
 
 class LoMoeTile(ctypes.Structure):
@@ -32,6 +33,7 @@ SIGNATURES = {
                                                    c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                                    c_int64, c_int64, c_int64, c_int32, c_int64, c_int64,
                                                    c_int32, c_int32, c_int, c_int, c_void_p]),
+    "lo_preshuffle_weight_int8": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "lo_silu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float, c_void_p]),
     "lo_moe_tile_query": (c_int, [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,

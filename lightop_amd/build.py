@@ -29,12 +29,13 @@ def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def build_library(verbose: bool = False, extra_flags=()) -> str:
+def build_library(verbose: bool = False, extra_flags=(), out_path: str = LIB_PATH) -> str:
+    """Compile every .hip under csrc/ and link them into one shared library."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objs = []
 
     def compile_one(src):
-        obj = os.path.join(CSRC, src[:-4] + ".o")
+        obj = os.path.join(CSRC, src[:-4] + f".{os.getpid()}.{abs(hash(out_path)) % 99991}.o")
         cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
         res = subprocess.run(cmd, capture_output=True, text=True)
         noise = "is not a recognized feature for this target"
@@ -47,13 +48,13 @@ def build_library(verbose: bool = False, extra_flags=()) -> str:
 
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
         objs = list(ex.map(compile_one, sources()))
-    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out_path, *objs]
     res = subprocess.run(link, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
     for o in objs:
         os.remove(o)
-    return LIB_PATH
+    return out_path
 
 
 if __name__ == "__main__":

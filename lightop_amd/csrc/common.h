@@ -11,6 +11,22 @@ namespace lo {
 constexpr int kWave = 64;   // CDNA wavefront
 constexpr int kGroup = 128; // quantisation group along K and weight block edge
 
+// Order of the 2 KB blocks (16 rows x 128 K-bytes) of a pre-shuffled expert weight:
+// K-block-major, i.e. [K/128][N/16]: the blocks that neighbouring waves read at the same
+// step of their K loops are contiguous in memory.  (Row-block-major order puts them
+// K*16 bytes apart, which for K = 2048 is a 32 KB stride and piles the concurrent reads
+// onto a few memory channels.)
+#ifndef LO_SHUF_KB_MAJOR
+#define LO_SHUF_KB_MAJOR 1
+#endif
+// byte offset of block (row block nb, K block kb) inside one expert
+__host__ __device__ __forceinline__ int64_t shuf_block_off(int64_t nb, int64_t kb, int64_t NBLK, int64_t KB) {
+  return (LO_SHUF_KB_MAJOR ? kb * NBLK + nb : nb * KB + kb) * 2048;
+}
+// the two strides of that formula, for kernels that advance kb with a scalar offset
+__host__ __device__ __forceinline__ int shuf_nb_stride(int KB) { return LO_SHUF_KB_MAJOR ? 2048 : KB * 2048; }
+__host__ __device__ __forceinline__ int shuf_kb_stride(int NBLK) { return LO_SHUF_KB_MAJOR ? NBLK * 2048 : 2048; }
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));

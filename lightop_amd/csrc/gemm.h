@@ -1,0 +1,56 @@
+// Argument block and launchers shared by the grouped block-INT8 GEMM kernels.
+#pragma once
+#include "common.h"
+
+namespace lo {
+
+struct GemmArgs {
+  const int8_t *A;       // [a_rows, K]
+  const float *As;       // [a_rows, K/128]
+  const int8_t *W;       // [E, N, K]
+  const float *Ws;       // [E, NB, K/128]
+  uint16_t *C;           // plain: [num_valid, N]
+  int8_t *A2q;           // fused: [num_valid, I]
+  float *A2s;            // fused: [num_valid, I/128]
+  const float *topk_w;   // [num_valid]
+  const int32_t *sorted; // [>= m_blocks*BM]
+  const int32_t *expert_ids;
+  const int32_t *ntpp;
+  int64_t num_valid;
+  int64_t a_rows;        // rows of A / As
+  int64_t N;             // weight rows per expert (2I for the fused first GEMM)
+  int64_t K;
+  int32_t top_k;
+  int32_t n_tiles;       // workgroups along N
+  int32_t E;             // experts held by W
+  int32_t mul_routed;
+  int32_t w_shuffled;    // W is in the pre-shuffled layout (shuffle.hip)
+};
+
+__device__ __forceinline__ v4i ld16(const int8_t *p) { return *reinterpret_cast<const v4i *>(p); }
+
+// Buffer addressing: a wave-uniform 128-bit resource (base, extent) + one 32-bit lane
+// offset + one scalar offset.  The K loop then advances a scalar only, no per-lane 64-bit
+// address arithmetic, and a read past the extent returns zero instead of faulting.
+typedef __amdgpu_buffer_rsrc_t brsrc;
+__device__ __forceinline__ brsrc make_rsrc(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+constexpr int kCacheDefault = 0;
+constexpr int kCacheStream = 2; // "nt": data that is read once (weights in the streaming regime)
+template <int AUX = kCacheDefault>
+__device__ __forceinline__ v4i bld16(brsrc r, int voff, int soff) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, AUX);
+}
+__device__ __forceinline__ float bld_f32(brsrc r, int voff, int soff) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+
+// Weight-streaming kernels (gemm_ws.hip): block_size_m in {16, 32, 64, 128}.
+int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
+                   hipStream_t s);
+// LDS-tiled kernel (gemm_tile.hip): block_size_m == 128, compute-bound regime.
+int launch_gemm_tile(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
+bool gemm_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);
+
+} // namespace lo

@@ -1,0 +1,106 @@
+// C ABI of the grouped block-INT8 GEMM stages: validation and kernel choice.
+#include "gemm.h"
+
+namespace lo {
+
+static int64_t grid_m_blocks(int64_t sorted_cap, int64_t num_valid, int bs) {
+  // The sorted list can hold at most one partially filled block per slot, so when
+  // there are fewer slots than blocks the tail can never be reached (the bound of
+  // invoke_fused_moe_kernel_int8, int8.py:572-580).
+  int64_t blocks = sorted_cap / bs;
+  if (num_valid < blocks) blocks = num_valid;
+  return blocks;
+}
+
+static int validate_common(const char *who, const void *A, const void *As, const void *W,
+                           const void *Ws, const void *sorted, const void *eids, const void *ntpp,
+                           int64_t K, int32_t top_k, int32_t E, int64_t a_rows) {
+  LO_REQUIRE(A && As && W && Ws && sorted && eids && ntpp, LO_EINVAL, "%s: null pointer", who);
+  LO_REQUIRE(K > 0 && K % kGroup == 0, LO_EINVAL, "%s: K (%lld) must be a multiple of 128", who,
+             (long long)K);
+  LO_REQUIRE(top_k >= 1 && E >= 1 && a_rows >= 1, LO_EINVAL, "%s: bad top_k / E / a_rows", who);
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(A) & 15) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0,
+             LO_EINVAL, "%s: A and W must be 16-byte aligned", who);
+  // the kernels address A and one expert's weights with 32-bit byte offsets
+  LO_REQUIRE(a_rows * K < (1ll << 31), LO_ENOTSUP, "%s: A (%lld x %lld bytes) exceeds 2 GiB", who,
+             (long long)a_rows, (long long)K);
+  return LO_OK;
+}
+
+// The LDS-tiled kernel serves the 128-token tile (tokens per expert large enough for
+// the MFMA pipe to matter); everything else streams weights.
+static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int64_t m_blocks,
+                       hipStream_t s) {
+  if (!(flags & LO_GEMM_FORCE_STREAMING) && gemm_tile_supports(a, fused_act, bs))
+    return launch_gemm_tile(a, fused_act, flags, m_blocks, s);
+  return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
+}
+
+} // namespace lo
+
+extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W,
+                                      const float *Ws, void *C, int c_dtype, const float *topk_w,
+                                      const int32_t *sorted_ids, const int32_t *expert_ids,
+                                      const int32_t *num_tokens_post_pad, int64_t sorted_cap,
+                                      int64_t num_valid, int64_t a_rows, int32_t E, int64_t N,
+                                      int64_t K, int32_t top_k, int32_t block_size_m,
+                                      int mul_routed, int flags, lo_stream_t stream) {
+  using namespace lo;
+  int rc = validate_common("moe_gemm", A, As, W, Ws, sorted_ids, expert_ids, num_tokens_post_pad, K,
+                           top_k, E, a_rows);
+  if (rc) return rc;
+  LO_REQUIRE(C, LO_EINVAL, "moe_gemm: null output");
+  LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm: only bf16 output is built");
+  LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm: N (%lld) must be a multiple of 16", (long long)N);
+  LO_REQUIRE(N * K < (1ll << 31), LO_ENOTSUP, "moe_gemm: one expert's weights exceed 2 GiB");
+  LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm: mul_routed needs topk_weights");
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(C) & 7) == 0, LO_EINVAL, "moe_gemm: C must be 8-byte aligned");
+  LO_REQUIRE((num_valid + top_k - 1) / top_k <= a_rows, LO_EINVAL,
+             "moe_gemm: %lld slots / top_k %d exceed the %lld rows of A", (long long)num_valid, top_k,
+             (long long)a_rows);
+  if (num_valid == 0) return LO_OK;
+  GemmArgs a{};
+  a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.C = static_cast<uint16_t *>(C);
+  a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
+  a.E = E; a.a_rows = a_rows; a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
+  a.n_tiles = static_cast<int32_t>((N + 63) / 64);
+  const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
+  LO_REQUIRE(mblocks * a.n_tiles < (1ll << 30), LO_EINVAL, "moe_gemm: grid too large");
+  if (mblocks == 0) return LO_OK;
+  return launch_gemm(a, false, block_size_m, flags, mblocks, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lo_moe_gemm1_silu_quant_block_int8(
+    const int8_t *A, const float *As, const int8_t *W, const float *Ws, int8_t *A2q, float *A2s,
+    int c_dtype, const float *topk_w, const int32_t *sorted_ids, const int32_t *expert_ids,
+    const int32_t *num_tokens_post_pad, int64_t sorted_cap, int64_t num_valid, int64_t a_rows,
+    int32_t E, int64_t I, int64_t K, int32_t top_k, int32_t block_size_m, int mul_routed, int flags,
+    lo_stream_t stream) {
+  using namespace lo;
+  int rc = validate_common("moe_gemm1_silu_quant", A, As, W, Ws, sorted_ids, expert_ids,
+                           num_tokens_post_pad, K, top_k, E, a_rows);
+  if (rc) return rc;
+  LO_REQUIRE(A2q && A2s, LO_EINVAL, "moe_gemm1_silu_quant: null output");
+  LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm1_silu_quant: only bf16 rounding is built");
+  LO_REQUIRE(I > 0 && I % kGroup == 0, LO_EINVAL,
+             "moe_gemm1_silu_quant: intermediate size (%lld) must be a multiple of 128", (long long)I);
+  LO_REQUIRE(2 * I * K < (1ll << 31), LO_ENOTSUP, "moe_gemm1_silu_quant: one expert's weights exceed 2 GiB");
+  LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm1_silu_quant: mul_routed needs topk_weights");
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(A2q) & 3) == 0, LO_EINVAL,
+             "moe_gemm1_silu_quant: A2q must be 4-byte aligned");
+  LO_REQUIRE((num_valid + top_k - 1) / top_k <= a_rows, LO_EINVAL,
+             "moe_gemm1_silu_quant: %lld slots / top_k %d exceed the %lld rows of A",
+             (long long)num_valid, top_k, (long long)a_rows);
+  if (num_valid == 0) return LO_OK;
+  GemmArgs a{};
+  a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.A2q = A2q; a.A2s = A2s;
+  a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
+  a.E = E; a.a_rows = a_rows; a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
+  a.n_tiles = static_cast<int32_t>(I / kGroup);
+  const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
+  LO_REQUIRE(mblocks * a.n_tiles < (1ll << 31), LO_EINVAL, "moe_gemm1_silu_quant: grid too large");
+  if (mblocks == 0) return LO_OK;
+  return launch_gemm(a, true, block_size_m, flags, mblocks, static_cast<hipStream_t>(stream));
+}

@@ -13,6 +13,7 @@ _NATIVE_APIS = {
     "invoke_fused_moe_gemm1_silu_quant",
     "silu_and_mul",
     "fused_experts_workspace_bytes",
+    "preshuffle_moe_weight",
 }
 
 
@@ -34,5 +35,6 @@ __all__ = [
     "moe_align_block_size",
     "moe_align_block_size_out",
     "moe_sum",
+    "preshuffle_moe_weight",
     "silu_and_mul",
 ]

@@ -29,6 +29,35 @@ def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bo
     return as_dict(t1), as_dict(t2)
 
 
+def _scale_flags(fused_scale: Optional[bool]) -> int:
+    """None: the library's choice per kernel; True: acc += d * (a_s * b_s) everywhere;
+    False: the canonical (d * a_s) * b_s + acc everywhere."""
+    if fused_scale is None:
+        return 0
+    return _lib.LO_GEMM_FUSED_SCALE if fused_scale else _lib.LO_GEMM_CANONICAL_ORDER
+
+
+def preshuffle_moe_weight(w: torch.Tensor) -> torch.Tensor:
+    """Return expert weights ``w`` [E, N, K] (int8, row-major) in the load-time layout of the
+    gfx950 GEMM kernels: each 16-row x 128-byte block stored as [8 x 16-byte K chunks][16 rows].
+    Same shape and dtype as ``w``; the result carries ``lo_preshuffled = True`` and is what
+    ``fused_experts_impl_int8`` wants for ``w1`` / ``w2`` when full speed matters.  Do this
+    once when the checkpoint is loaded.  N % 16 == 0 and K % 128 == 0 are required."""
+    _require_cuda(w)
+    assert w.dtype == torch.int8 and w.dim() == 3 and w.is_contiguous()
+    E, N, K = w.shape
+    out = torch.empty_like(w)
+    with _on_device(w):
+        _lib.check(_lib.lib().lo_preshuffle_weight_int8(_lib.ptr(w), _lib.ptr(out), E, N, K,
+                                                        _lib.stream_of(w)))
+    out.lo_preshuffled = True
+    return out
+
+
+def _is_preshuffled(w: torch.Tensor) -> bool:
+    return bool(getattr(w, "lo_preshuffled", False))
+
+
 def _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded):
     _require_cuda(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)
     assert A.dtype == torch.int8 and B.dtype == torch.int8, "A and B must be int8"
@@ -47,7 +76,8 @@ def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tens
                                  topk_weights: Optional[torch.Tensor],
                                  sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                                  num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
-                                 top_k: int, config: Dict[str, Any], fused_scale: bool = False) -> None:
+                                 top_k: int, config: Dict[str, Any], fused_scale: Optional[bool] = None,
+                                 flags: int = 0) -> None:
     """One grouped block-INT8 GEMM stage: C[f] = bf16(sum_kb dot(A[f // top_k], B[e])_kb *
     A_scale * B_scale) (* topk_weights[f]) for every routed slot f (reference:
     invoke_fused_moe_kernel_int8, int8.py:543-626).  ``C`` is [M, topk, N] or [S, N]."""
@@ -67,7 +97,8 @@ def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tens
             _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(expert_ids),
             _lib.ptr(num_tokens_post_padded), sorted_token_ids.numel(), num_valid, A.shape[0], E, N, K,
             int(top_k), int(config["BLOCK_SIZE_M"]), 1 if mul_routed_weight else 0,
-            _lib.LO_GEMM_FUSED_SCALE if fused_scale else 0, _lib.stream_of(A)))
+            _scale_flags(fused_scale) | flags | (_lib.LO_GEMM_W_PRESHUFFLED if _is_preshuffled(B) else 0),
+            _lib.stream_of(A)))
 
 
 def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale: torch.Tensor,
@@ -75,7 +106,7 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
                                       sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                                       num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
                                       top_k: int, num_valid: int, config: Dict[str, Any],
-                                      fused_scale: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+                                      fused_scale: Optional[bool] = None, flags: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
     """First GEMM with SiLU-and-mul and the 1x128 re-quantisation in its epilogue: the
     sequence int8.py:784-823 in one kernel.  Returns (A2q [num_valid, I] int8,
     A2s [num_valid, I/128] f32); rows of slots routed to non-local experts are not written."""
@@ -96,7 +127,8 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
             _lib.LO_BF16, _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(expert_ids),
             _lib.ptr(num_tokens_post_padded), sorted_token_ids.numel(), num_valid, A.shape[0], E, I, K,
             int(top_k), int(config["BLOCK_SIZE_M"]), 1 if mul_routed_weight else 0,
-            _lib.LO_GEMM_FUSED_SCALE if fused_scale else 0, _lib.stream_of(A)))
+            _scale_flags(fused_scale) | flags | (_lib.LO_GEMM_W_PRESHUFFLED if _is_preshuffled(B) else 0),
+            _lib.stream_of(A)))
     return a2q, a2s
 
 
@@ -220,6 +252,9 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     ws_ptr = (workspace.data_ptr() + 255) // 256 * 256
     ws_avail = ws_bytes - (ws_ptr - workspace.data_ptr())
     flags = int(extra.get("lightop_amd_flags", 0))
+    assert _is_preshuffled(w1) == _is_preshuffled(w2), "preshuffle both w1 and w2 or neither"
+    if _is_preshuffled(w1) or extra.get("lightop_amd_weights_preshuffled", False):
+        flags |= _lib.LO_GEMM_W_PRESHUFFLED
     block_size_m = int(extra.get("lightop_amd_block_size_m", 0))
 
     with _on_device(hidden_states):
@@ -247,5 +282,5 @@ def ctypes_void(addr: int):
     return ctypes.c_void_p(addr)
 
 
-__all__ = ["fused_experts_impl_int8", "get_w8a8moe_json", "invoke_fused_moe_kernel_int8",
+__all__ = ["fused_experts_impl_int8", "get_w8a8moe_json", "preshuffle_moe_weight", "invoke_fused_moe_kernel_int8",
            "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes"]

@@ -196,23 +196,30 @@ def gemm_case(seed, M, k, E, Eg, N, K, small_values=False):
                                           (300, 2, 3, 3, 128, 2048)])
 @pytest.mark.parametrize("bs", BS_ALL)
 def test_gemm_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
-    from lightop_amd.moe import invoke_fused_moe_kernel_int8, moe_align_block_size
+    from lightop_amd.moe import invoke_fused_moe_kernel_int8, moe_align_block_size, preshuffle_moe_weight
 
     say(f"gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs}")
     Aq, As, W, Ws, ids, tw, emap = gemm_case(M + N + bs, M, k, E, Eg, N, K)
     rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
     S = M * k
+    # the 128-token tile has two implementations: LDS-tiled (default) and weight-streaming
+    impls = (0, 2) if bs == 128 else (0,)
+    Wd = W.to(dev)
+    Wsh = preshuffle_moe_weight(Wd)
     for mul in (False, True):
         ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, k, S, bs)
-        C = torch.full((M, k, N), 7.0, dtype=torch.bfloat16, device=dev)
-        s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
-        invoke_fused_moe_kernel_int8(Aq.to(dev), W.to(dev), C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
-                                     mul, k, {"BLOCK_SIZE_M": bs})
-        torch.cuda.synchronize()
-        assert torch.equal(C.view(S, N).cpu().view(torch.int16), ref.view(torch.int16)), f"mul_routed={mul}"
+        for force_streaming in impls:
+            for Wx in (Wd, Wsh):  # row-major and load-time pre-shuffled weights
+                C = torch.full((M, k, N), 7.0, dtype=torch.bfloat16, device=dev)
+                s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
+                invoke_fused_moe_kernel_int8(Aq.to(dev), Wx, C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
+                                             mul, k, {"BLOCK_SIZE_M": bs}, fused_scale=False, flags=force_streaming)
+                torch.cuda.synchronize()
+                assert torch.equal(C.view(S, N).cpu().view(torch.int16), ref.view(torch.int16)), \
+                    f"mul_routed={mul} flags={force_streaming} preshuffled={Wx is Wsh}"
     # fused-scale variant: same integers, fp32 rounding differs in the last place only
     C2 = torch.empty((M, k, N), dtype=torch.bfloat16, device=dev)
-    invoke_fused_moe_kernel_int8(Aq.to(dev), W.to(dev), C2, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
+    invoke_fused_moe_kernel_int8(Aq.to(dev), Wsh, C2, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
                                  True, k, {"BLOCK_SIZE_M": bs}, fused_scale=True)
     torch.cuda.synchronize()
     assert within_tolerance(C2.view(S, N), ref)
@@ -244,7 +251,7 @@ def test_gemm_int32_accumulators_exact(dev, oracle, bs):
                                           (50, 8, 4, 16, 256, 768), (200, 4, 6, 6, 384, 1024)])
 @pytest.mark.parametrize("bs", BS_ALL)
 def test_gemm1_silu_quant_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
-    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size
+    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_weight
 
     say(f"gemm1+silu+quant M={M} k={k} E={E}/{Eg} I={I} K={K} bs={bs}")
     Aq, As, W, Ws, ids, tw, emap = gemm_case(M + I + bs + 1, M, k, E, Eg, 2 * I, K)
@@ -252,22 +259,39 @@ def test_gemm1_silu_quant_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
     rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
     S = M * k
     s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
+    impls = (0, 2) if bs == 128 else (0,)
     for mul in (False, True):
         c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, k, S, bs)
         rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
-        q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), W.to(dev), As.to(dev), Ws.to(dev), tw.to(dev),
-                                                  s, e, p, mul, k, S, {"BLOCK_SIZE_M": bs})
-        torch.cuda.synchronize()
-        local = torch.ones(S, dtype=torch.bool) if emap is None else emap.long()[ids.reshape(-1).long()] >= 0
-        assert torch.equal(sc.cpu()[local], rsc[local]), f"scales differ (mul_routed={mul})"
-        assert torch.equal(q.cpu()[local], rq[local]), f"int8 activations differ (mul_routed={mul})"
+        for force_streaming in impls:
+            for Wx in (W.to(dev), preshuffle_moe_weight(W.to(dev))):
+                q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wx, As.to(dev), Ws.to(dev), tw.to(dev),
+                                                          s, e, p, mul, k, S, {"BLOCK_SIZE_M": bs}, fused_scale=False,
+                                                          flags=force_streaming)
+                torch.cuda.synchronize()
+                local = torch.ones(S, dtype=torch.bool) if emap is None else emap.long()[ids.reshape(-1).long()] >= 0
+                what = f"mul_routed={mul}, flags={force_streaming}, preshuffled={hasattr(Wx, 'lo_preshuffled')}"
+                assert torch.equal(sc.cpu()[local], rsc[local]), f"scales differ ({what})"
+                assert torch.equal(q.cpu()[local], rq[local]), f"int8 activations differ ({what})"
+
+
+def test_preshuffle_layout(dev):
+    from lightop_amd.moe import preshuffle_moe_weight
+
+    say("preshuffle layout")
+    E, N, K = 3, 48, 384
+    w = torch.arange(E * N * K, dtype=torch.int64).remainder(251).sub(125).to(torch.int8).view(E, N, K)
+    got = preshuffle_moe_weight(w.to(dev)).cpu()
+    # [E, N/16, 16 rows, K/128, 8 chunks, 16 B] -> [E, K/128, N/16, 8 chunks, 16 rows, 16 B]
+    want = w.view(E, N // 16, 16, K // 128, 8, 16).permute(0, 3, 1, 4, 2, 5).contiguous().view(E, N, K)
+    assert torch.equal(got, want)
 
 
 # ---------------------------------------------------------------- whole path ---
 
-def run_fused(dev, layer, M, seed, bs=0, flags=0, shared=False, on_input=False, inplace=False):
+def run_fused(dev, layer, M, seed, bs=0, flags=4, shared=False, on_input=False, inplace=False, preshuffle=False):
     from lightop_amd import workloads as wl
-    from lightop_amd.moe import fused_experts_impl_int8
+    from lightop_amd.moe import fused_experts_impl_int8, preshuffle_moe_weight
 
     w1, w2, w1s, w2s = wl.make_weights(layer, seed=seed)
     x, tw, ids = wl.make_inputs(layer, M, seed=seed)
@@ -276,8 +300,11 @@ def run_fused(dev, layer, M, seed, bs=0, flags=0, shared=False, on_input=False, 
     sh = torch.randn(M, layer.H, generator=g).to(torch.bfloat16) if shared else None
     cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
     xd = x.to(dev)
+    w1d, w2d = w1.to(dev), w2.to(dev)
+    if preshuffle:
+        w1d, w2d = preshuffle_moe_weight(w1d), preshuffle_moe_weight(w2d)
     out = fused_experts_impl_int8(
-        xd, w1.to(dev), w2.to(dev), tw.to(dev), ids.to(dev), cache13, inplace=inplace,
+        xd, w1d, w2d, tw.to(dev), ids.to(dev), cache13, inplace=inplace,
         apply_router_weight_on_input=on_input, use_int8_w8a8=True, global_num_experts=layer.E_global,
         expert_map=None if emap is None else emap.to(dev), w1_scale=w1s.to(dev), w2_scale=w2s.to(dev),
         block_shape=[128, 128], routed_scaling_factor=1.0 if not shared else 2.5,
@@ -289,12 +316,13 @@ def run_fused(dev, layer, M, seed, bs=0, flags=0, shared=False, on_input=False, 
 
 
 @pytest.mark.parametrize("bs", BS_ALL)
-def test_fused_experts_tiny_config_bit_exact(dev, oracle, bs):
+@pytest.mark.parametrize("preshuffle", [False, True])
+def test_fused_experts_tiny_config_bit_exact(dev, oracle, bs, preshuffle):
     """BASELINE config 1: E=8, top-2, H=1024, I=512, M=64, seed 0."""
     from lightop_amd import workloads as wl
 
-    say(f"fused tiny bs={bs}")
-    (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, wl.TINY, 64, 0, bs=bs)
+    say(f"fused tiny bs={bs} preshuffle={preshuffle}")
+    (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, wl.TINY, 64, 0, bs=bs, preshuffle=preshuffle)
     ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, bs)
     assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
