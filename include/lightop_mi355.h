@@ -48,7 +48,10 @@ enum {
    * LO_GEMM_FUSED_SCALE is given. */
   LO_GEMM_CANONICAL_ORDER = 4,
   /* W (for the whole path: w1 and w2) is in the layout of lo_preshuffle_weight_int8 */
-  LO_GEMM_W_PRESHUFFLED = 8
+  LO_GEMM_W_PRESHUFFLED = 8,
+  /* leave the output rows of blocks whose expert id is -1 untouched instead of zeroing
+   * them (the caller then reduces with an expert_mask, see lo_moe_sum) */
+  LO_GEMM_SKIP_NONLOCAL = 16
 };
 
 int lo_version(void);
@@ -78,6 +81,19 @@ int lo_moe_align_block_size(const void *topk_ids, int ids_dtype, int64_t numel,
                             int32_t *sorted_ids, int64_t sorted_cap,
                             int32_t *expert_ids, int64_t expert_ids_cap,
                             int32_t *num_tokens_post_pad, lo_stream_t stream);
+
+/*
+ * Same, and additionally writes slot_mask[numel] (one byte per slot): 1 if the slot's
+ * expert is held by this rank (expert_map[id] >= 0, or no map), else 0 - the
+ * expert_mask that lo_moe_sum takes.
+ */
+int lo_moe_align_block_size_mask(const void *topk_ids, int ids_dtype, int64_t numel,
+                                 int32_t num_experts, int32_t block_size,
+                                 const int32_t *expert_map, int ignore_invalid,
+                                 int32_t *sorted_ids, int64_t sorted_cap,
+                                 int32_t *expert_ids, int64_t expert_ids_cap,
+                                 int32_t *num_tokens_post_pad, uint8_t *slot_mask,
+                                 lo_stream_t stream);
 
 /*
  * 1x128 group quantisation of activations to int8 with fp32 scales.
@@ -140,9 +156,11 @@ int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *ac
  * Replaces op.moe_sum (csrc/pybind/export.cpp:1584-1592,
  * csrc/kernels/moe_align_sum_kernels.cu:1315-2092).  fp32 accumulation in slot
  * order; without bias one rounding (:619-633), with bias the three roundings of :886-909.
+ * expert_mask [M*topk] bytes or NULL: slots whose byte is 0 are not read and add nothing
+ * (the expert_mask argument of the reference op, :661-672).
  */
-int lo_moe_sum(const void *in, void *out, const void *bias, int dtype, int64_t M, int32_t topk,
-               int64_t H, float factor, lo_stream_t stream);
+int lo_moe_sum(const void *in, void *out, const void *bias, const uint8_t *expert_mask, int dtype,
+               int64_t M, int32_t topk, int64_t H, float factor, lo_stream_t stream);
 
 /*
  * Load-time weight layout for the GEMM kernels: every block of 16 rows x 128 K-bytes of
@@ -198,7 +216,8 @@ int lo_fused_experts_block_int8(const void *x, int dtype, int64_t M, int64_t H, 
 /*
  * Views into the workspace of the last layout computed for the same arguments, so
  * that tests can read every intermediate of lo_fused_experts_block_int8:
- * which = 0 a1q, 1 a1s, 2 sorted_ids, 3 expert_ids, 4 num_tokens_post_pad, 5 a2q, 6 a2s.
+ * which = 0 a1q, 1 a1s, 2 sorted_ids, 3 expert_ids, 4 num_tokens_post_pad, 5 a2q, 6 a2s,
+ * 7 slot mask.
  * Returns the byte offset inside the workspace or a negative error.
  */
 int64_t lo_fused_experts_workspace_offset(int which, int64_t M, int32_t top_k, int64_t H, int64_t I,

@@ -12,6 +12,7 @@ LO_BF16, LO_F16 = 0, 1
 LO_I32, LO_I64 = 0, 1
 LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE, LO_GEMM_FORCE_STREAMING, LO_GEMM_CANONICAL_ORDER = 0, 1, 2, 4
 LO_GEMM_W_PRESHUFFLED = 8
+LO_GEMM_SKIP_NONLOCAL = 16
 
 
 class LoMoeTile(ctypes.Structure):
@@ -24,6 +25,8 @@ SIGNATURES = {
     "lo_last_error": (c_char_p, []),
     "lo_moe_align_block_size": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,
                                         c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
+    "lo_moe_align_block_size_mask": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,
+                                             c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "lo_per_token_group_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_float, c_void_p,
                                               c_void_p, c_void_p]),
     "lo_moe_gemm_block_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -35,7 +38,8 @@ SIGNATURES = {
                                                    c_int32, c_int32, c_int, c_int, c_void_p]),
     "lo_preshuffle_weight_int8": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "lo_silu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
-    "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float, c_void_p]),
+    "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float,
+                           c_void_p]),
     "lo_moe_tile_query": (c_int, [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
                                   ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
     "lo_fused_experts_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),

@@ -24,7 +24,7 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
     const IdT *__restrict__ ids, int64_t numel, int num_experts, int bs,
     const int32_t *__restrict__ expert_map, int ignore_invalid, int32_t *__restrict__ sorted,
     int64_t sorted_cap, int32_t *__restrict__ expert_ids, int64_t expert_ids_cap,
-    int32_t *__restrict__ ntpp, int key_bits) {
+    int32_t *__restrict__ ntpp, int key_bits, uint8_t *__restrict__ slot_mask) {
   extern __shared__ int32_t lds[];
   const int nw = blockDim.x / kWave;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -62,6 +62,11 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
   for (int64_t t = t0; t < t1; ++t) {
     bool ok;
     int e = key_of(t * kWave + lane, ok);
+    if (slot_mask && t * kWave + lane < numel) { // is the slot's expert held by this rank?
+      bool local = ok;
+      if (ok && expert_map && !ignore_invalid) local = expert_map[e] >= 0;
+      slot_mask[t * kWave + lane] = local ? 1 : 0;
+    }
     uint64_t peers = match_any(e, key_bits, ok);
     if (ok) {
       int leader = __ffsll(static_cast<unsigned long long>(peers)) - 1;
@@ -144,6 +149,18 @@ extern "C" int lo_moe_align_block_size(const void *topk_ids, int ids_dtype, int6
                                        int32_t *sorted_ids, int64_t sorted_cap,
                                        int32_t *expert_ids, int64_t expert_ids_cap,
                                        int32_t *num_tokens_post_pad, lo_stream_t stream) {
+  return lo_moe_align_block_size_mask(topk_ids, ids_dtype, numel, num_experts, block_size, expert_map,
+                                      ignore_invalid, sorted_ids, sorted_cap, expert_ids,
+                                      expert_ids_cap, num_tokens_post_pad, nullptr, stream);
+}
+
+extern "C" int lo_moe_align_block_size_mask(const void *topk_ids, int ids_dtype, int64_t numel,
+                                            int32_t num_experts, int32_t block_size,
+                                            const int32_t *expert_map, int ignore_invalid,
+                                            int32_t *sorted_ids, int64_t sorted_cap,
+                                            int32_t *expert_ids, int64_t expert_ids_cap,
+                                            int32_t *num_tokens_post_pad, uint8_t *slot_mask,
+                                            lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(topk_ids && sorted_ids && expert_ids && num_tokens_post_pad, LO_EINVAL,
              "moe_align_block_size: null pointer");
@@ -174,11 +191,11 @@ extern "C" int lo_moe_align_block_size(const void *topk_ids, int ids_dtype, int6
     hipLaunchKernelGGL(moe_align_kernel<int32_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
                        static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,
                        expert_map, ignore_invalid, sorted_ids, sorted_cap, expert_ids,
-                       expert_ids_cap, num_tokens_post_pad, key_bits);
+                       expert_ids_cap, num_tokens_post_pad, key_bits, slot_mask);
   else
     hipLaunchKernelGGL(moe_align_kernel<int64_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
                        static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size,
                        expert_map, ignore_invalid, sorted_ids, sorted_cap, expert_ids,
-                       expert_ids_cap, num_tokens_post_pad, key_bits);
+                       expert_ids_cap, num_tokens_post_pad, key_bits, slot_mask);
   return check_launch("moe_align_block_size");
 }

@@ -37,7 +37,7 @@ static void align_caps(int64_t numel, int32_t num_experts, int32_t bs, int64_t *
 }
 
 struct WsLayout {
-  int64_t off[7];
+  int64_t off[8];
   int64_t total;
   int64_t sorted_cap, blocks_cap;
 };
@@ -47,15 +47,16 @@ static WsLayout ws_layout(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_
   WsLayout L{};
   const int64_t S = M * top_k;
   align_caps(S, num_experts, bs, &L.sorted_cap, &L.blocks_cap);
-  const int64_t sizes[7] = {M * H,                 // a1q
+  const int64_t sizes[8] = {M * H,                 // a1q
                             M * (H / kGroup) * 4,  // a1s
                             L.sorted_cap * 4,      // sorted_ids
                             L.blocks_cap * 4,      // expert_ids
                             4,                     // num_tokens_post_pad
                             S * I,                 // a2q
-                            S * (I / kGroup) * 4}; // a2s
+                            S * (I / kGroup) * 4,  // a2s
+                            S};                    // slot mask
   int64_t o = 0;
-  for (int i = 0; i < 7; ++i) {
+  for (int i = 0; i < 8; ++i) {
     L.off[i] = o;
     o += align_up(sizes[i] > 0 ? sizes[i] : 1, 256);
   }
@@ -104,7 +105,7 @@ extern "C" int64_t lo_fused_experts_workspace_offset(int which, int64_t M, int32
                                                      int64_t I, int32_t num_experts,
                                                      int32_t block_size_m) {
   using namespace lo;
-  if (which < 0 || which > 6 || block_size_m <= 0) return LO_EINVAL;
+  if (which < 0 || which > 7 || block_size_m <= 0) return LO_EINVAL;
   return ws_layout(M, top_k, H, I, num_experts, block_size_m).off[which];
 }
 
@@ -143,12 +144,15 @@ extern "C" int lo_fused_experts_block_int8(
   int32_t *ntpp = reinterpret_cast<int32_t *>(ws + L.off[4]);
   int8_t *a2q = reinterpret_cast<int8_t *>(ws + L.off[5]);
   float *a2s = reinterpret_cast<float *>(ws + L.off[6]);
+  // With an expert_map most slots may belong to other ranks: their rows of cache3 are
+  // neither zero-filled by the second GEMM nor read by the reduction.
+  uint8_t *mask = expert_map ? reinterpret_cast<uint8_t *>(ws + L.off[7]) : nullptr;
   const int64_t S = M * top_k;
 
   int rc = lo_per_token_group_quant_int8(x, dtype, M, H, 1e-10f, a1q, a1s, stream);
   if (rc) return rc;
-  rc = lo_moe_align_block_size(topk_ids, ids_dtype, S, num_experts, block_size_m, expert_map, 0,
-                               sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, stream);
+  rc = lo_moe_align_block_size_mask(topk_ids, ids_dtype, S, num_experts, block_size_m, expert_map, 0,
+                                    sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, mask, stream);
   if (rc) return rc;
   rc = lo_moe_gemm1_silu_quant_block_int8(a1q, a1s, w1, w1s, a2q, a2s, dtype, topk_w, sorted, eids,
                                           ntpp, L.sorted_cap, S, M, E, I, H, top_k, block_size_m,
@@ -156,7 +160,9 @@ extern "C" int lo_fused_experts_block_int8(
   if (rc) return rc;
   rc = lo_moe_gemm_block_int8(a2q, a2s, w2, w2s, cache3, dtype, topk_w, sorted, eids, ntpp,
                               L.sorted_cap, S, S, E, H, I, 1, block_size_m,
-                              !apply_router_weight_on_input, flags, stream);
+                              !apply_router_weight_on_input, flags | (mask ? LO_GEMM_SKIP_NONLOCAL : 0),
+                              stream);
   if (rc) return rc;
-  return lo_moe_sum(cache3, out, shared_output, dtype, M, top_k, H, routed_scaling_factor, stream);
+  return lo_moe_sum(cache3, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor,
+                    stream);
 }

@@ -50,12 +50,9 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
   return __uint_as_float(static_cast<uint32_t>(h) << 16);
 }
 
-// Round-to-nearest-even; NaN stays a quiet NaN.
+// Round-to-nearest-even (gfx950 has the conversion in hardware: v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 __device__ __forceinline__ float f16_to_f32(uint16_t h) {
@@ -78,8 +75,8 @@ template <int DT> __device__ __forceinline__ uint16_t from_f32(float f) {
 // degree-7 polynomial, exact power-of-two scaling), so that the result does not
 // depend on a math library.  Used for SiLU: g / (1 + exp(-g)).
 __device__ __forceinline__ float det_expf(float x) {
-  if (x > 88.72283f) return __uint_as_float(0x7f800000u);
-  if (x < -87.0f) return 0.0f;
+  const float x_in = x;
+  x = fminf(fmaxf(x, -87.0f), 88.72283f); // straight-line code: the ends are patched below
   float n = __builtin_rintf(x * 1.44269504088896341f);
   float r = __builtin_fmaf(n, -0.693145751953125f, x);
   r = __builtin_fmaf(n, -1.42860682030941723212e-6f, r);
@@ -95,7 +92,9 @@ __device__ __forceinline__ float det_expf(float x) {
   int h = ni / 2;
   float a = __uint_as_float(static_cast<uint32_t>(h + 127) << 23);
   float b = __uint_as_float(static_cast<uint32_t>(ni - h + 127) << 23);
-  return (p * a) * b;
+  float e = (p * a) * b;
+  e = x_in > 88.72283f ? __uint_as_float(0x7f800000u) : e;
+  return x_in < -87.0f ? 0.0f : e;
 }
 
 // act = T( T(silu(g)) * u ), everything in fp32 between the roundings.

@@ -69,6 +69,7 @@ template <int DT, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t *__restrict__ in,
                                                       uint16_t *__restrict__ out,
                                                       const uint16_t *__restrict__ bias,
+                                                      const uint8_t *__restrict__ mask,
                                                       int64_t M, int topk, int64_t H,
                                                       float factor) {
   const int64_t vec_per_row = H / 8;
@@ -79,6 +80,7 @@ __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t *__restrict
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     const uint16_t *p = in + t * topk * H + c;
     for (int j = 0; j < topk; ++j) {
+      if (mask && !mask[t * topk + j]) continue; // slot of an expert on another rank: adds 0
       const v8u16 r = *reinterpret_cast<const v8u16 *>(p + static_cast<int64_t>(j) * H);
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[i] = acc[i] + to_f32<DT>(r[i]);
@@ -144,8 +146,9 @@ extern "C" int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
   return check_launch("silu_and_mul");
 }
 
-extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, int dtype, int64_t M,
-                          int32_t topk, int64_t H, float factor, lo_stream_t stream) {
+extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uint8_t *expert_mask,
+                          int dtype, int64_t M, int32_t topk, int64_t H, float factor,
+                          lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(in && out, LO_EINVAL, "moe_sum: null pointer");
   LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "moe_sum: only bf16 is built");
@@ -160,10 +163,10 @@ extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, int dtype
   if (bias)
     hipLaunchKernelGGL((moe_sum_kernel<LO_BF16, true>), dim3(grid), dim3(256), 0, s,
                        static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),
-                       static_cast<const uint16_t *>(bias), M, topk, H, factor);
+                       static_cast<const uint16_t *>(bias), expert_mask, M, topk, H, factor);
   else
     hipLaunchKernelGGL((moe_sum_kernel<LO_BF16, false>), dim3(grid), dim3(256), 0, s,
                        static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),
-                       static_cast<const uint16_t *>(nullptr), M, topk, H, factor);
+                       static_cast<const uint16_t *>(nullptr), expert_mask, M, topk, H, factor);
   return check_launch("moe_sum");
 }

@@ -25,6 +25,7 @@ struct GemmArgs {
   int32_t E;             // experts held by W
   int32_t mul_routed;
   int32_t w_shuffled;    // W is in the pre-shuffled layout (shuffle.hip)
+  int32_t skip_nonlocal; // blocks of expert -1: leave the output rows untouched
 };
 
 __device__ __forceinline__ v4i ld16(const int8_t *p) { return *reinterpret_cast<const v4i *>(p); }
@@ -49,8 +50,9 @@ __device__ __forceinline__ float bld_f32(brsrc r, int voff, int soff) {
 // Weight-streaming kernels (gemm_ws.hip): block_size_m in {16, 32, 64, 128}.
 int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
                    hipStream_t s);
-// LDS-tiled kernel (gemm_tile.hip): block_size_m == 128, compute-bound regime.
-int launch_gemm_tile(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
+// LDS-tiled kernels (gemm_tile.hip): block_size_m 64 or 128, compute-bound regime.
+int launch_gemm_tile(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
+                     hipStream_t s);
 bool gemm_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 
 } // namespace lo

@@ -32,7 +32,7 @@ static int validate_common(const char *who, const void *A, const void *As, const
 static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int64_t m_blocks,
                        hipStream_t s) {
   if (!(flags & LO_GEMM_FORCE_STREAMING) && gemm_tile_supports(a, fused_act, bs))
-    return launch_gemm_tile(a, fused_act, flags, m_blocks, s);
+    return launch_gemm_tile(a, fused_act, bs, flags, m_blocks, s);
   return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
 }
 
@@ -64,6 +64,7 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
   a.E = E; a.a_rows = a_rows; a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
+  a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 30), LO_EINVAL, "moe_gemm: grid too large");
@@ -98,6 +99,7 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
   a.E = E; a.a_rows = a_rows; a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
+  a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.n_tiles = static_cast<int32_t>(I / kGroup);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 31), LO_EINVAL, "moe_gemm1_silu_quant: grid too large");

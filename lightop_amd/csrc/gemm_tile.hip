@@ -25,7 +25,6 @@ namespace lo {
 
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kTileM = 128;      // tokens per workgroup
 constexpr int kTileRow = 144;    // LDS row pitch in bytes: 128 + 16 keeps ds_read_b128 conflict-free
 
 // Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
@@ -50,11 +49,15 @@ __device__ __forceinline__ bool tile_of(int bid, int n_tiles, int m_blocks, int 
   return true;
 }
 
-template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF>
-__global__ __launch_bounds__(512) void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks) {
+// WT = number of 64-token halves per workgroup: 2 -> 128-token tile, 8 waves, one
+// workgroup per CU; 1 -> 64-token tile, 4 waves, two workgroups per CU that are not
+// synchronised with each other, so one computes while the other waits at its barrier.
+template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int WT>
+__global__ __launch_bounds__(256 * WT) void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks) {
+  constexpr int kTileM = 64 * WT; // tokens per workgroup
   __shared__ __attribute__((aligned(16))) int8_t sA[2][kTileM * kTileRow];
   __shared__ float sS[2][kTileM];
-  __shared__ float sRed[2][2][4][32];
+  __shared__ float sRed[WT][2][4][32];
 
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, mb, nt)) return;
@@ -64,7 +67,7 @@ __global__ __launch_bounds__(512) void moe_gemm_tile_kernel(const GemmArgs a, in
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: scalar address math
   const int wr = wave & 3;  // which 64 weight rows of the tile
-  const int wt = wave >> 2; // which 64 tokens of the tile
+  const int wt = wave >> 2; // which 64 tokens of the tile (always 0 when WT == 1)
   const int r = lane & 31, c = lane >> 5;
   const int64_t K = a.K, N = a.N;
   const int KB = static_cast<int>(K / kGroup);
@@ -92,7 +95,7 @@ __global__ __launch_bounds__(512) void moe_gemm_tile_kernel(const GemmArgs a, in
 
   if (e < 0) {
     if constexpr (!FUSED_ACT) {
-      if (wave_active) {
+      if (wave_active && !a.skip_nonlocal) {
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb)
           if (valid[tb])
@@ -132,6 +135,8 @@ __global__ __launch_bounds__(512) void moe_gemm_tile_kernel(const GemmArgs a, in
     wsrow[rb] = a.Ws + (static_cast<int64_t>(e) * NB + nr / kGroup) * KB;
   }
 
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
   v16i zero16;
 #pragma unroll
   for (int i = 0; i < 16; ++i) zero16[i] = 0;
@@ -145,23 +150,28 @@ __global__ __launch_bounds__(512) void moe_gemm_tile_kernel(const GemmArgs a, in
 
   v4i wreg[2][2][4]; // [buffer][row fragment][k-step]
   float bsc[2][2];   // [buffer][row fragment] weight-block scales, fetched with the fragments
-  v4i areg[2];
-  float sreg = 0.0f;
+  v4i areg[2][2]; // [set][16-byte piece]: token bytes in flight for two K blocks
+  float sreg[2] = {0.0f, 0.0f};
 
   // The K loop is free of branches (branches around the loads make the compiler wait for
   // all of them): a step past the end of K re-reads the last K block and stores a token
   // scale of zero, so it adds exactly 0 to every accumulator.
-  auto load_act = [&](int kb) {
+  // The token bytes of K block kb are requested two iterations before they are needed
+  // and written to LDS one iteration before: set = kb & 1 in registers, stage = kb & 1
+  // in LDS.
+  auto load_act = [&](auto SET, int kb) {
+    constexpr int st = decltype(SET)::value;
     const int kc = kb < KB ? kb : KB - 1;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) areg[j] = bld16(rA, aoff, kc * kGroup + j * 16);
-    sreg = bld_f32(rAs, asoff, kc * 4);
+    for (int j = 0; j < 2; ++j) areg[st][j] = bld16(rA, aoff, kc * kGroup + j * 16);
+    sreg[st] = bld_f32(rAs, asoff, kc * 4);
   };
-  auto store_act = [&](int stage, bool live) {
-    int8_t *d = stage ? sdst1 : sdst0;
+  auto store_act = [&](auto SET, bool live) {
+    constexpr int st = decltype(SET)::value;
+    int8_t *d = st ? sdst1 : sdst0;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) *reinterpret_cast<v4i *>(d + j * 16) = areg[j];
-    if (lq == 0) sS[stage][lt] = live ? sreg : 0.0f;
+    for (int j = 0; j < 2; ++j) *reinterpret_cast<v4i *>(d + j * 16) = areg[st][j];
+    if (lq == 0) sS[st][lt] = live ? sreg[st] : 0.0f;
   };
   auto load_w = [&](auto BUF, int kb) {
     constexpr int b = decltype(BUF)::value;
@@ -230,26 +240,25 @@ __global__ __launch_bounds__(512) void moe_gemm_tile_kernel(const GemmArgs a, in
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  using B0 = std::integral_constant<int, 0>;
-  using B1 = std::integral_constant<int, 1>;
-  load_act(0);
+  load_act(B0{}, 0);
+  load_act(B1{}, 1);
   load_w(B0{}, 0);
-  store_act(0, true);
+  store_act(B0{}, true);
   __syncthreads();
   for (int kb = 0; kb < KB; kb += 2) {
-    // even K block: compute from buffers 0, prefetch into buffers 1
-    load_act(kb + 1);
-    load_w(B1{}, kb + 1);
+    // even K block: compute from LDS stage 0 / weight buffer 0
+    load_act(B0{}, kb + 2);            // needed in two iterations
+    load_w(B1{}, kb + 1);              // needed in the next iteration
     __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMAs
     compute(B0{});
-    store_act(1, kb + 1 < KB);
+    store_act(B1{}, kb + 1 < KB);      // requested one iteration ago
     __syncthreads();
     // odd K block (a dead step when K/128 is odd: zero token scales)
-    load_act(kb + 2);
+    load_act(B1{}, kb + 3);
     load_w(B0{}, kb + 2);
     __builtin_amdgcn_sched_barrier(0);
     compute(B1{});
-    store_act(0, kb + 2 < KB);
+    store_act(B0{}, kb + 2 < KB);
     __syncthreads();
   }
 
@@ -318,12 +327,13 @@ __global__ __launch_bounds__(512) void moe_gemm_tile_kernel(const GemmArgs a, in
 }
 
 bool gemm_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
-  if (block_size_m != kTileM) return false;
+  if (block_size_m != 128 && block_size_m != 64) return false;
   if (!fused_act && a.N % 64 != 0) return false;
   return true;
 }
 
-int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int flags, int64_t m_blocks, hipStream_t s) {
+int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
+                     hipStream_t s) {
   GemmArgs a = a0;
   a.n_tiles = fused_act ? static_cast<int32_t>(a.N / 2 / kGroup) : static_cast<int32_t>((a.N + 255) / 256);
   // every chunk of 4 token blocks owns 4 * n_tiles consecutive slots on one XCD
@@ -331,12 +341,18 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
   const int64_t grid = (chunks + 7) / 8 * (4 * a.n_tiles) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
   const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
-  const dim3 g(static_cast<unsigned>(grid)), b(512);
+  const int wt = block_size_m / 64;
+  const dim3 g(static_cast<unsigned>(grid)), b(256 * wt);
   const int mbi = static_cast<int>(m_blocks);
-#define LO_TILE_LAUNCH(FA, FS)                                                                   \
-  do {                                                                                           \
-    if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, true>), g, b, 0, s, a, mbi);  \
-    else hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, false>), g, b, 0, s, a, mbi);     \
+#define LO_TILE_LAUNCH2(FA, FS, SH)                                                             \
+  do {                                                                                          \
+    if (wt == 2) hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, SH, 2>), g, b, 0, s, a, mbi); \
+    else hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, SH, 1>), g, b, 0, s, a, mbi);         \
+  } while (0)
+#define LO_TILE_LAUNCH(FA, FS)                         \
+  do {                                                 \
+    if (a.w_shuffled) LO_TILE_LAUNCH2(FA, FS, true);   \
+    else LO_TILE_LAUNCH2(FA, FS, false);               \
   } while (0)
   if (fused_act) {
     if (fast) LO_TILE_LAUNCH(true, true);
@@ -346,6 +362,7 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
     else LO_TILE_LAUNCH(false, false);
   }
 #undef LO_TILE_LAUNCH
+#undef LO_TILE_LAUNCH2
   return check_launch(fused_act ? "moe_gemm1_silu_quant(tile)" : "moe_gemm(tile)");
 }
 

@@ -76,6 +76,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
     const int64_t n0 = static_cast<int64_t>(nt) * (16 * NWAVES * RPW) + wave * (16 * RPW);
     if (n0 >= N) return;
     if (e < 0) { // expert not held by this rank: the rows are defined to be zero
+      if (a.skip_nonlocal) return;
 #pragma unroll
       for (int j = 0; j < TM; ++j)
         if (valid[j])

@@ -85,11 +85,12 @@ def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: i
 def moe_sum(input: torch.Tensor, output: torch.Tensor, bias: Optional[torch.Tensor] = None,
             expert_mask: Optional[torch.Tensor] = None, num_local_tokens: Optional[torch.Tensor] = None,
             factor: float = 1.0, expect_m: int = -1) -> None:
-    """``op.moe_sum`` (export.cpp:1584-1592): output[t] = factor * sum_k input[t, k] (+ bias[t])."""
-    if expert_mask is not None or num_local_tokens is not None:
+    """``op.moe_sum`` (export.cpp:1584-1592): output[t] = factor * sum_k input[t, k] (+ bias[t]).
+    Slots whose ``expert_mask`` entry is False are skipped."""
+    if num_local_tokens is not None:
         raise NotImplementedError(
-            "lightop_amd.op.moe_sum: expert_mask / num_local_tokens belong to the DeepEP layout, "
-            "which this build does not cover")
+            "lightop_amd.op.moe_sum: num_local_tokens belongs to the DeepEP layout, which this build "
+            "does not cover")
     del expect_m
     _require_cuda(input, output, bias)
     if input.dim() != 3:
@@ -102,7 +103,12 @@ def moe_sum(input: torch.Tensor, output: torch.Tensor, bias: Optional[torch.Tens
                            "tensor of the input dtype")
     if bias is not None and (not bias.is_contiguous() or bias.numel() != M * H or bias.dtype != input.dtype):
         raise RuntimeError("lightop_amd.op.moe_sum: bias must match output")
+    if expert_mask is not None:
+        _require_cuda(expert_mask)
+        if expert_mask.numel() != M * k or expert_mask.dtype not in (torch.bool, torch.uint8):
+            raise RuntimeError("lightop_amd.op.moe_sum: expert_mask must be a bool tensor of M*topk elements")
+        expert_mask = expert_mask.contiguous().view(torch.uint8)
     with _on_device(input):
         _lib.check(_lib.lib().lo_moe_sum(_lib.ptr(input), _lib.ptr(output), _lib.ptr(bias),
-                                         _act_dtype(input), M, k, H, float(factor),
+                                         _lib.ptr(expert_mask), _act_dtype(input), M, k, H, float(factor),
                                          _lib.stream_of(input)))
