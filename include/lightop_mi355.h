@@ -58,6 +58,15 @@ int lo_version(void);
 const char *lo_last_error(void);
 
 /*
+ * Optional one-time set-up for the current device: builds the 128 KB bf16 SiLU table
+ * that the fused GEMM epilogue looks activations up in.  The first fused-GEMM call on a
+ * device does this by itself (and synchronises the stream once); call lo_init() first
+ * when that first call would fall inside a HIP graph capture.  No counterpart in the
+ * reference.
+ */
+int lo_init(lo_stream_t stream);
+
+/*
  * Routing alignment.
  * Replaces op.moe_align_block_size (csrc/pybind/export.cpp:1593-1605,
  * csrc/kernels/moe_align_sum_kernels.cu:1210-1314) together with the

@@ -23,6 +23,7 @@ class LoMoeTile(ctypes.Structure):
 SIGNATURES = {
     "lo_version": (c_int, []),
     "lo_last_error": (c_char_p, []),
+    "lo_init": (c_int, [c_void_p]),
     "lo_moe_align_block_size": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,
                                         c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "lo_moe_align_block_size_mask": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,

@@ -58,22 +58,25 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
     return e;
   };
 
-  // pass 1: per-wave histogram
-  for (int64_t t = t0; t < t1; ++t) {
-    bool ok;
-    int e = key_of(t * kWave + lane, ok);
-    if (slot_mask && t * kWave + lane < numel) { // is the slot's expert held by this rank?
-      bool local = ok;
-      if (ok && expert_map && !ignore_invalid) local = expert_map[e] >= 0;
-      slot_mask[t * kWave + lane] = local ? 1 : 0;
+  // pass 1: per-wave histogram.  Counting does not depend on order, so LDS atomics are
+  // fine here; ids are fetched kBatch tiles at a time so that their latency overlaps.
+  constexpr int kBatch = 8;
+  for (int64_t t = t0; t < t1; t += kBatch) {
+    int ek[kBatch];
+    bool okk[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int64_t f = (t + b) * kWave + lane;
+      ek[b] = key_of((t + b < t1) ? f : numel, okk[b]);
+      if (slot_mask && t + b < t1 && f < numel) { // is the slot's expert held by this rank?
+        bool local = okk[b];
+        if (local && expert_map && !ignore_invalid) local = expert_map[ek[b]] >= 0;
+        slot_mask[f] = local ? 1 : 0;
+      }
     }
-    uint64_t peers = match_any(e, key_bits, ok);
-    if (ok) {
-      int leader = __ffsll(static_cast<unsigned long long>(peers)) - 1;
-      if (lane == leader) wcnt[wave * E + e] += __popcll(peers);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b)
+      if (okk[b]) atomicAdd(&wcnt[wave * E + ek[b]], 1);
   }
   __syncthreads();
 
@@ -122,22 +125,31 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
   for (int64_t i = P + tid; i < sorted_cap; i += blockDim.x) sorted[i] = static_cast<int32_t>(numel);
 
   // pass 3: stable scatter.  wcnt[wave][e] is the running number of slots of expert
-  // e that precede the current tile.
-  for (int64_t t = t0; t < t1; ++t) {
-    bool ok;
-    int64_t f = t * kWave + lane;
-    int e = key_of(f, ok);
-    uint64_t peers = match_any(e, key_bits, ok);
-    if (ok) {
-      int before = __popcll(peers & ((1ull << lane) - 1ull));
-      int leader = __ffsll(static_cast<unsigned long long>(peers)) - 1;
-      int base = wcnt[wave * E + e];
-      sorted[offs[e] + base + before] = static_cast<int32_t>(f);
+  // e that precede the current tile.  Ranks inside a tile come from a ballot match, the
+  // running counters are updated by one lane per expert: no atomics, fixed order.
+  for (int64_t t = t0; t < t1; t += kBatch) {
+    int ek[kBatch];
+    bool okk[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b)
+      ek[b] = key_of((t + b < t1) ? (t + b) * kWave + lane : numel, okk[b]);
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int e = ek[b];
+      const bool ok = okk[b];
+      const int64_t f = (t + b) * kWave + lane;
+      uint64_t peers = match_any(e, key_bits, ok);
+      if (ok) {
+        int before = __popcll(peers & ((1ull << lane) - 1ull));
+        int leader = __ffsll(static_cast<unsigned long long>(peers)) - 1;
+        int base = wcnt[wave * E + e];
+        sorted[offs[e] + base + before] = static_cast<int32_t>(f);
+        __builtin_amdgcn_wave_barrier();
+        if (lane == leader) wcnt[wave * E + e] = base + __popcll(peers);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      if (lane == leader) wcnt[wave * E + e] = base + __popcll(peers);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
   }
 }
 

@@ -71,8 +71,10 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k) {
   const double per_expert = static_cast<double>(M) * top_k / (num_experts > 0 ? num_experts : 1);
   if (per_expert <= 12.0) return 16;
   if (per_expert <= 24.0) return 32;
-  if (per_expert <= 96.0) return 64;
-  return 128;
+  // 64-token LDS tiles: two workgroups per CU hide each other's barrier and memory
+  // waits, which measured faster than the 128-token tile (one workgroup per CU) on
+  // every layer shape tried.
+  return 64;
 }
 
 } // namespace lo

@@ -36,6 +36,8 @@ typedef unsigned short v8u16 __attribute__((ext_vector_type(8)));
 // ---- error reporting (host) -------------------------------------------------
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
+// bf16(silu(g)) for all 65536 bf16 patterns g, built on first use (per device).
+int silu_table(hipStream_t stream, const uint16_t **table);
 
 #define LO_REQUIRE(cond, code, ...)  \
   do {                               \
@@ -103,6 +105,12 @@ template <int DT> __device__ __forceinline__ uint16_t silu_mul(uint16_t g16, uin
   float e = det_expf(-g);
   float sg = to_f32<DT>(from_f32<DT>(g / (1.0f + e)));
   return from_f32<DT>(sg * to_f32<DT>(u16));
+}
+
+// Same with the SiLU taken from the per-device table.
+__device__ __forceinline__ uint16_t silu_mul_tab(const uint16_t *__restrict__ table, uint16_t g16, uint16_t u16) {
+  const float sg = bf16_to_f32(table[g16]);
+  return f32_to_bf16(sg * bf16_to_f32(u16));
 }
 
 // q = (int8) trunc(clamp(v / s, -128, 127))

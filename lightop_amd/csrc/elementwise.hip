@@ -1,6 +1,8 @@
 // Streaming stages of the block-INT8 fused-MoE path on gfx950: 1x128 group
 // quantisation, SiLU-and-mul, and the top-k reduction.  All are HBM-bound; every
 // lane moves 16 bytes per load and a workgroup covers whole 128-element groups.
+#include <mutex>
+
 #include "common.h"
 
 namespace lo {
@@ -102,6 +104,19 @@ __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t *__restrict
   }
 }
 
+// ---- SiLU table ------------------------------------------------------------------
+// bf16(silu(g)) for every bf16 pattern g (128 KB, stays in L2).  The GEMM epilogues look
+// the activation up instead of spending ~45 vector instructions per element on
+// exp / divide / round; the entries are produced by exactly those instructions, once
+// per device.
+__device__ uint16_t g_silu_bf16_table[65536];
+
+__global__ __launch_bounds__(256) void silu_table_init_kernel(uint16_t *table) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  const float g = bf16_to_f32(static_cast<uint16_t>(i));
+  table[i] = f32_to_bf16(g / (1.0f + det_expf(-g)));
+}
+
 static int grid_for(int64_t work_items, int per_block) {
   int64_t b = (work_items + per_block - 1) / per_block;
   if (b < 1) b = 1;
@@ -109,7 +124,48 @@ static int grid_for(int64_t work_items, int per_block) {
   return static_cast<int>(b);
 }
 
+static std::mutex g_table_mutex;
+static const uint16_t *g_table_ptr[64] = {};
+
+int silu_table(hipStream_t stream, const uint16_t **out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    set_error("silu table: no current HIP device");
+    return LO_ELAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_table_mutex);
+  if (!g_table_ptr[dev]) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) {
+      set_error("the first call on a device builds the SiLU table and must not be captured: "
+                "call lo_init() (or run the op once) before capturing a graph");
+      return LO_EINVAL;
+    }
+    uint16_t *p = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(g_silu_bf16_table)) != hipSuccess || !p) {
+      set_error("silu table: hipGetSymbolAddress failed");
+      return LO_ELAUNCH;
+    }
+    hipLaunchKernelGGL(silu_table_init_kernel, dim3(256), dim3(256), 0, stream, p);
+    int rc = check_launch("silu_table_init");
+    if (rc) return rc;
+    // one-time only: other streams of this device may use the table right after
+    if (hipStreamSynchronize(stream) != hipSuccess) {
+      set_error("silu table: synchronisation failed");
+      return LO_ELAUNCH;
+    }
+    g_table_ptr[dev] = p;
+  }
+  *out = g_table_ptr[dev];
+  return LO_OK;
+}
+
 } // namespace lo
+
+extern "C" int lo_init(lo_stream_t stream) {
+  const uint16_t *t = nullptr;
+  return lo::silu_table(static_cast<hipStream_t>(stream), &t);
+}
 
 extern "C" int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t rows,
                                              int64_t cols, float eps, int8_t *q, float *s,

@@ -13,6 +13,7 @@ struct GemmArgs {
   int8_t *A2q;           // fused: [num_valid, I]
   float *A2s;            // fused: [num_valid, I/128]
   const float *topk_w;   // [num_valid]
+  const uint16_t *silu;  // fused: bf16(silu(g)) table indexed by the bf16 pattern of g
   const int32_t *sorted; // [>= m_blocks*BM]
   const int32_t *expert_ids;
   const int32_t *ntpp;

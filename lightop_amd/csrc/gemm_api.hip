@@ -101,6 +101,8 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.n_tiles = static_cast<int32_t>(I / kGroup);
+  rc = silu_table(static_cast<hipStream_t>(stream), &a.silu);
+  if (rc) return rc;
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 31), LO_EINVAL, "moe_gemm1_silu_quant: grid too large");
   if (mblocks == 0) return LO_OK;

@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256 * WT) void moe_gemm_tile_kernel(const GemmArgs 
           g = g * w;
           u = u * w;
         }
-        const uint16_t act16 = silu_mul<LO_BF16>(f32_to_bf16(g), f32_to_bf16(u));
+        const uint16_t act16 = silu_mul_tab(a.silu, f32_to_bf16(g), f32_to_bf16(u));
         actf[tb][i] = bf16_to_f32(act16);
         amax = fmaxf(amax, fabsf(actf[tb][i]));
       }

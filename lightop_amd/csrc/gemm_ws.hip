@@ -235,7 +235,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
           g = g * w;
           u = u * w;
         }
-        const uint16_t act16 = silu_mul<LO_BF16>(f32_to_bf16(g), f32_to_bf16(u));
+        const uint16_t act16 = silu_mul_tab(a.silu, f32_to_bf16(g), f32_to_bf16(u));
         actf[j][i] = bf16_to_f32(act16);
         amax = fmaxf(amax, fabsf(actf[j][i]));
       }

@@ -1,0 +1,98 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/lightop_mi355.h
+declares; argument validation that happens before any HIP call is exercised too."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "lightop_mi355.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lo_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from lightop_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from lightop_amd import build
+
+        build.build_library()
+    return _lib.lib()
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("lo_moe_align_block_size", "lo_per_token_group_quant_int8", "lo_moe_gemm_block_int8",
+                 "lo_moe_gemm1_silu_quant_block_int8", "lo_silu_and_mul", "lo_moe_sum",
+                 "lo_fused_experts_block_int8", "lo_fused_experts_workspace_bytes",
+                 "lo_preshuffle_weight_int8", "lo_moe_tile_query", "lo_last_error", "lo_version"):
+        assert must in names
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    from lightop_amd import _lib
+
+    names = declared_functions()
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature in lightop_amd/_lib.py"
+    assert sorted(_lib.SIGNATURES) == names, "ctypes table and header disagree"
+
+
+def test_header_cites_the_reference_for_every_entry_point():
+    text = open(HEADER).read()
+    for cite in ("export.cpp:1593-1605", "int8_utils.py:125-195", "int8.py:543-626", "int8.py:811",
+                 "export.cpp:1584-1592", "int8.py:220-256", "int8.py:703-888"):
+        assert cite in text
+
+
+def test_version_and_tile_table(lib):
+    from lightop_amd import _lib
+
+    assert lib.lo_version() >= 100
+    t1, t2 = _lib.LoMoeTile(), _lib.LoMoeTile()
+    # DeepSeek-V3 EP share: 256 global experts, top-8
+    sizes = {}
+    for M in (1, 16, 64, 256, 1024, 4096, 8192):
+        assert lib.lo_moe_tile_query(M, 32, 256, 8, 7168, 2048, t1, t2) == 0
+        assert t1.block_size_m == t2.block_size_m and t1.block_size_m in (16, 32, 64, 128)
+        sizes[M] = t1.block_size_m
+    assert sizes[1] == 16 and sizes[64] == 16
+    assert all(sizes[a] <= sizes[b] for a, b in zip(list(sizes)[:-1], list(sizes)[1:]))
+    assert lib.lo_moe_tile_query(-1, 32, 256, 8, 7168, 2048, t1, t2) < 0
+    assert b"moe_tile_query" in lib.lo_last_error()
+
+
+def test_workspace_sizing(lib):
+    n16 = lib.lo_fused_experts_workspace_bytes(64, 8, 7168, 2048, 256, 16)
+    n0 = lib.lo_fused_experts_workspace_bytes(64, 8, 7168, 2048, 256, 0)
+    assert 0 < n16 <= n0
+    # a1q + a2q alone
+    assert n16 >= 64 * 7168 + 64 * 8 * 2048
+    assert lib.lo_fused_experts_workspace_bytes(64, 8, 100, 2048, 256, 16) < 0
+    offs = [lib.lo_fused_experts_workspace_offset(i, 64, 8, 7168, 2048, 256, 16) for i in range(8)]
+    assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
+    assert lib.lo_fused_experts_workspace_offset(8, 64, 8, 7168, 2048, 256, 16) < 0
+
+
+def test_validation_happens_before_any_launch(lib):
+    """Null pointers and bad shapes are rejected on the host (no GPU needed)."""
+    null = ctypes.c_void_p(0)
+    assert lib.lo_moe_align_block_size(null, 0, 8, 8, 16, null, 0, null, 128, null, 8, null, null) == -1
+    assert b"null pointer" in lib.lo_last_error()
+    buf = (ctypes.c_int32 * 64)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.lo_moe_align_block_size(p, 7, 8, 8, 16, null, 0, p, 128, p, 8, p, null) == -1     # bad id dtype
+    assert lib.lo_moe_align_block_size(p, 0, 8, 8, 16, null, 0, p, 10, p, 8, p, null) == -2      # buffer too small
+    assert b"sorted_ids holds 10" in lib.lo_last_error()
+    assert lib.lo_per_token_group_quant_int8(p, 0, 1, 100, 1e-10, p, p, null) == -1              # cols % 128
+    assert lib.lo_per_token_group_quant_int8(p, 1, 1, 128, 1e-10, p, p, null) == -4              # fp16 not built
+    assert lib.lo_moe_sum(p, p, null, null, 0, 1, 8, 100, 1.0, null) == -1                       # H % 8
+    assert lib.lo_preshuffle_weight_int8(p, p, 1, 16, 128, null) == -1                           # src == dst

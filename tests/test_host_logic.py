@@ -1,0 +1,227 @@
+"""Host-side logic that needs no GPU: the Python drop-in surface, lazy flags, workload
+generators and the golden fixtures against the oracle."""
+import hashlib
+import importlib
+import inspect
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLDEN = os.path.join(HERE, "golden")
+
+
+def test_import_touches_no_gpu_and_surface_matches_the_reference():
+    import lightop_amd
+    from lightop_amd import moe, quant
+
+    assert {"fused_experts_impl_int8", "moe_align_block_size", "moe_align_block_size_out", "moe_sum"} <= set(moe.__all__)
+    assert "per_token_group_quant_int8" in quant.__all__
+    # the quant entry point stays out of the moe namespace (reference: test_quant_per_token_quant_int8.py:22-25)
+    assert "per_token_group_quant_int8" not in moe.__all__
+    assert lightop_amd.moe_sum is moe.moe_sum
+    with pytest.raises(AttributeError):
+        moe.no_such_function
+
+
+def test_signatures_match_the_reference():
+    from lightop_amd import moe, quant
+
+    sig = inspect.signature(moe.fused_experts_impl_int8)
+    names = list(sig.parameters)
+    # int8.py:628-656
+    assert names[:6] == ["hidden_states", "w1", "w2", "topk_weights", "topk_ids", "cache13"]
+    assert names[6:] == ["inplace", "activation", "apply_router_weight_on_input", "use_fp8_w8a8", "use_int8_w8a8",
+                         "use_int8_w8a16", "use_int4_w4a16", "per_channel_quant", "global_num_experts", "expert_map",
+                         "w1_scale", "w2_scale", "w1_zp", "w2_zp", "a1_scale", "a2_scale", "block_shape",
+                         "use_nn_moe", "routed_scaling_factor", "shared_output", "i_q", "i_s", "_"]
+    assert sig.parameters["inplace"].default is False and sig.parameters["activation"].default == "silu"
+    assert sig.parameters["global_num_experts"].default == -1 and sig.parameters["routed_scaling_factor"].default == 1.0
+    assert sig.parameters["_"].kind is inspect.Parameter.VAR_KEYWORD
+    # moe_align_block_size.py:17-24
+    assert list(inspect.signature(moe.moe_align_block_size).parameters) == [
+        "topk_ids", "block_size", "num_experts", "expert_map", "pad_sorted_ids", "ignore_invalid_experts"]
+    # moe/routing.py:23-35
+    assert list(inspect.signature(moe.moe_align_block_size_out).parameters) == [
+        "topk_ids", "num_experts", "block_size", "sorted_ids", "expert_ids", "num_tokens_post_pad", "expert_map",
+        "expert_mask", "num_local_tokens", "is_ep", "is_fuse_fill"]
+    # moe_align_sum.py:12-20
+    ms = inspect.signature(moe.moe_sum)
+    assert list(ms.parameters) == ["input", "output", "bias", "expert_mask", "num_local_tokens", "factor", "expect_m"]
+    assert ms.parameters["factor"].default == 1.0 and ms.parameters["expect_m"].default == -1
+    # int8_utils.py:125-130
+    qs = inspect.signature(quant.per_token_group_quant_int8)
+    assert list(qs.parameters) == ["x", "group_size", "eps", "dtype"]
+    assert qs.parameters["eps"].default == 1e-10 and qs.parameters["dtype"].default is torch.int8
+
+
+def test_out_variant_forwards_positionally(monkeypatch):
+    """moe_align_block_size_out passes its 11 arguments through unchanged
+    (reference: test/test_moe_align_block_size_out.py:11-27)."""
+    from lightop_amd.moe import routing
+
+    seen = {}
+    monkeypatch.setattr(routing.op, "moe_align_block_size", lambda *a: seen.setdefault("args", a))
+    routing.moe_align_block_size_out(1, 2, 3, 4, 5, 6, 7, 8, 9, True, False)
+    assert seen["args"] == (1, 2, 3, 4, 5, 6, 7, 8, 9, True, False)
+
+
+def test_env_flags_are_lazy(monkeypatch):
+    from lightop_amd import envs
+
+    assert envs.LMSLIM_FUSED_MOE_CHUNK_SIZE == 16 * 1024
+    monkeypatch.setenv("VLLM_FUSED_MOE_CHUNK_SIZE", "4096")
+    assert envs.LMSLIM_FUSED_MOE_CHUNK_SIZE == 4096
+    monkeypatch.setenv("LMSLIM_FUSED_MOE_CHUNK_SIZE", "512")  # the LMSLIM name wins over the alias
+    assert envs.LMSLIM_FUSED_MOE_CHUNK_SIZE == 512
+    assert envs.LMSLIM_USE_GLOBAL_MOE_CACHE is False
+    monkeypatch.setenv("LMSLIM_USE_GLOBAL_MOE_CACHE", "yes")
+    assert envs.LMSLIM_USE_GLOBAL_MOE_CACHE is True
+    with pytest.raises(AttributeError):
+        envs.NOT_A_FLAG
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    """There is no CPU fallback: a CPU tensor is an error, not a slow path."""
+    from lightop_amd import moe, quant
+
+    with pytest.raises(RuntimeError, match="GPU"):
+        quant.per_token_group_quant_int8(torch.zeros(2, 128, dtype=torch.bfloat16), 128)
+    with pytest.raises(RuntimeError, match="GPU"):
+        moe.moe_sum(torch.zeros(2, 2, 128, dtype=torch.bfloat16), torch.zeros(2, 128, dtype=torch.bfloat16))
+
+
+def test_missing_library_is_an_error(monkeypatch, tmp_path):
+    from lightop_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.lib()
+
+
+def test_product_never_imports_the_oracle():
+    """The oracle is the checker; the shipped package must not reach it in any way."""
+    root = os.path.dirname(HERE)
+    for d, _, files in os.walk(os.path.join(root, "lightop_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(d, f)).read()
+                for needle in ("import oracle", "from oracle", "oracle/", "moe_oracle", "cpu_oracle", "torch_ref"):
+                    assert needle not in text, f"{f} refers to {needle}"
+
+
+def test_tile_config_dictionary():
+    from lightop_amd.moe import get_w8a8moe_json
+
+    c1, c2 = get_w8a8moe_json(64, 32, 4096, 7168, 2048, True, [128, 128], 8, 256)
+    for c in (c1, c2):
+        assert {"BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K", "GROUP_SIZE_M", "num_warps", "num_stages"} <= set(c)
+    assert c1["BLOCK_SIZE_M"] == c2["BLOCK_SIZE_M"] == 16  # the alignment block serves both GEMMs (int8.py:767)
+
+
+# ------------------------------------------------------------------ workloads --
+
+def test_routing_generators():
+    from lightop_amd import workloads as wl
+
+    x, w, ids = wl.make_inputs(wl.QWEN3_30B, 33, seed=1)
+    assert x.shape == (33, 2048) and x.dtype == torch.bfloat16 and ids.dtype == torch.int32
+    assert torch.allclose(w.sum(-1), torch.ones(33), atol=1e-5)
+    assert all(len(set(r)) == 8 for r in ids.tolist()) and ids.max() < 128
+    x, w, ids = wl.make_inputs(wl.DSV3_EP, 50, seed=1)
+    assert torch.allclose(w.sum(-1), torch.full((50,), 2.5), atol=1e-4)
+    groups = (ids // 32)
+    assert all(len(set(r)) <= 4 for r in groups.tolist())       # top-4 of 8 groups
+    emap = wl.expert_map_for(wl.DSV3_EP)
+    assert emap[:32].tolist() == list(range(32)) and (emap[32:] == -1).all()
+    assert wl.expert_map_for(wl.QWEN3_30B) is None
+    # Zipf skew: the most loaded expert gets far more than the mean
+    _, _, idz = wl.make_inputs(wl.DSV3_FULL, 2048, seed=0)
+    counts = torch.bincount(idz.reshape(-1).long(), minlength=256)
+    assert counts.max() > 4 * counts.float().mean()
+    ops, nbytes, sloc, eact = wl.algorithmic_work(wl.DSV3_EP, ids, emap)
+    assert ops == 6 * sloc * 2048 * 7168 and eact <= 32
+    assert nbytes >= eact * 3 * 2048 * 7168
+
+
+def test_weight_generator_ranges():
+    from lightop_amd import workloads as wl
+
+    w1, w2, s1, s2 = wl.make_weights(wl.TINY, seed=0)
+    assert w1.shape == (8, 1024, 1024) and w2.shape == (8, 1024, 512) and s1.shape == (8, 8, 8) and s2.shape == (8, 8, 4)
+    assert w1.min() >= -127 and w1.max() <= 127 and (s1 > 0).all()
+    assert abs(float(torch.log(s1).mean()) - np.log(1e-3)) < 0.1
+
+
+# --------------------------------------------------------------------- golden --
+
+def _t(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    return t.view(torch.bfloat16) if dtype == "bf16" else t
+
+
+def load_small_layer():
+    z = np.load(os.path.join(GOLDEN, "small_layer.npz"))
+    bf = {"x", "shared_output", "ref_c1", "ref_act", "ref_c3", "ref_out"}
+    return {k: _t(z[k], "bf16" if k in bf else None) for k in z.files}
+
+
+def test_golden_small_layer_oracle(oracle):
+    g = load_small_layer()
+    r = oracle.fused_experts_block_int8(g["x"], g["w1"], g["w2"], g["w1_scale"], g["w2_scale"], g["topk_weights"],
+                                        g["topk_ids"], 16, global_num_experts=8, expert_map=g["expert_map"],
+                                        routed_scaling_factor=2.5, shared_output=g["shared_output"],
+                                        return_intermediates=True)
+    for k, v in r.items():
+        ref = g["ref_" + k]
+        same = torch.equal(v.view(torch.int16), ref.view(torch.int16)) if v.dtype == torch.bfloat16 else torch.equal(v, ref)
+        assert same, k
+
+
+def test_golden_tiny_config1_oracle(oracle):
+    from lightop_amd import workloads as wl
+
+    doc = json.load(open(os.path.join(GOLDEN, "tiny_config1.json")))
+    w1, w2, w1s, w2s = wl.make_weights(wl.TINY, seed=0)
+    x, tw, ids = wl.make_inputs(wl.TINY, 64, seed=0)
+
+    def sha(t):
+        a = t.contiguous().view(torch.int16).numpy() if t.dtype == torch.bfloat16 else t.contiguous().numpy()
+        return hashlib.sha256(a.tobytes()).hexdigest()
+
+    assert {"x": sha(x), "w1": sha(w1), "topk_ids": sha(ids)}.items() <= doc["inputs_sha256"].items(), \
+        "the workload generator no longer reproduces the fixture's inputs"
+    r = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
+    P = doc["num_tokens_post_pad"]
+    assert r["num_tokens_post_pad"].item() == P
+    assert r["sorted_ids"][:P].tolist() == doc["sorted_token_ids"]
+    assert r["expert_ids"][: P // 16].tolist() == doc["expert_ids"]
+    for k, h in doc["sha256"].items():
+        assert sha(r[k]) == h, k
+
+
+def test_golden_align_docstring(oracle):
+    doc = json.load(open(os.path.join(GOLDEN, "align_docstring.json")))
+    s, e, p = oracle.moe_align_block_size(torch.tensor(doc["topk_ids"], dtype=torch.int32), doc["block_size"],
+                                          doc["num_experts"])
+    assert p.item() == doc["num_tokens_post_pad"]
+    assert s[: p.item()].tolist() == doc["sorted_token_ids"] and e[:4].tolist() == doc["expert_ids"]
+
+
+def test_torch_restatement_agrees_with_oracle_on_config1(oracle):
+    """The timed CPU baseline (oracle/torch_ref.py) and the C oracle are independent
+    restatements; on BASELINE config 1 they agree within the path's tolerance."""
+    from lightop_amd import workloads as wl
+    from oracle import torch_ref
+
+    w1, w2, w1s, w2s = wl.make_weights(wl.TINY, seed=0)
+    x, tw, ids = wl.make_inputs(wl.TINY, 64, seed=0)
+    out = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 16).float()
+    ref = torch_ref.torch_w8a8_block_int8_moe(x, w1, w2, w1s, w2s, tw, ids).float()
+    err = (out - ref).abs()
+    assert err.max() <= 1e-2 * ref.abs().max()
+    assert err.sum() / ref.abs().sum() <= 2e-3 * 3
