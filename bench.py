@@ -235,7 +235,8 @@ def main():
         ach, peak, unit = g1_bytes / g1_t / 1e9, HBM_PEAK_GBS, "GB/s"
     roofline = {"bound": head["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
                 "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
-                "kernel": "moe_gemm_ws_kernel (GEMM1 + SiLU*mul + 1x128 re-quant)",
+                "kernel": ("moe_gemm_tile_kernel" if bs_used >= 64 else "moe_gemm_ws_kernel")
+                + "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)",
                 "kernel_ms": round(stages["gemm1_silu_quant"], 4),
                 "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately)"}
 
@@ -258,7 +259,7 @@ def main():
 
     cpu = None
     if cpu_weights:
-        cpu = cpu_baseline(layer, cpu_weights, min(args.tokens, 2048))
+        cpu = cpu_baseline(layer, cpu_weights, min(args.tokens, 4096))
 
     t = head["ms_per_step"] * 1e-3
     line = {

@@ -105,6 +105,23 @@ int lo_moe_align_block_size_mask(const void *topk_ids, int ids_dtype, int64_t nu
                                  lo_stream_t stream);
 
 /*
+ * Same again with a scratch buffer that lets large inputs (numel >= 8192) be aligned by
+ * many workgroups instead of one: lo_moe_align_scratch_bytes(numel, num_experts) bytes of
+ * device memory, 4-byte aligned, contents irrelevant (0 = no scratch needed).  Without
+ * scratch the single-workgroup kernel runs; the result is identical.  The reference's
+ * large-input kernels allocate a zeroed tensor themselves
+ * (csrc/kernels/moe_align_sum_kernels.cu:1175).
+ */
+int64_t lo_moe_align_scratch_bytes(int64_t numel, int32_t num_experts);
+int lo_moe_align_block_size_ws(const void *topk_ids, int ids_dtype, int64_t numel,
+                               int32_t num_experts, int32_t block_size,
+                               const int32_t *expert_map, int ignore_invalid,
+                               int32_t *sorted_ids, int64_t sorted_cap,
+                               int32_t *expert_ids, int64_t expert_ids_cap,
+                               int32_t *num_tokens_post_pad, uint8_t *slot_mask,
+                               void *scratch, int64_t scratch_bytes, lo_stream_t stream);
+
+/*
  * 1x128 group quantisation of activations to int8 with fp32 scales.
  * Replaces per_token_group_quant_int8 (python/lightop/_lmslim_native/layers/gemm/
  * int8_utils.py:125-195, Triton kernel :74-122).

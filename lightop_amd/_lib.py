@@ -28,6 +28,10 @@ SIGNATURES = {
                                         c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "lo_moe_align_block_size_mask": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,
                                              c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
+    "lo_moe_align_scratch_bytes": (c_int64, [c_int64, c_int32]),
+    "lo_moe_align_block_size_ws": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,
+                                           c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
+                                           c_int64, c_void_p]),
     "lo_per_token_group_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_float, c_void_p,
                                               c_void_p, c_void_p]),
     "lo_moe_gemm_block_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,

@@ -153,6 +153,187 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
   }
 }
 
+// ---- large inputs: the same algorithm spread over many workgroups ------------------
+// Phase 1: every workgroup counts the experts of its chunk of slots into cnt[chunk][E].
+// Phase 2: every workgroup rebuilds the padded expert offsets from cnt (a few KB from
+// L2), adds the counts of the chunks before it, and scatters its chunk exactly like the
+// single-workgroup kernel does; padding, expert ids and the tail are shared out by expert.
+// Chunks, waves, tiles and lanes are all in slot order, so the result is the same stable
+// order, bit for bit.
+template <typename IdT>
+__device__ __forceinline__ int align_key(const IdT *__restrict__ ids, int64_t f, int64_t numel, int E,
+                                         const int32_t *__restrict__ expert_map, int ignore_invalid,
+                                         bool &ok) {
+  ok = f < numel;
+  int e = 0;
+  if (ok) {
+    int64_t raw = static_cast<int64_t>(ids[f]);
+    ok = raw >= 0 && raw < E;
+    e = ok ? static_cast<int>(raw) : 0;
+    if (ok && ignore_invalid && expert_map) {
+      e = expert_map[e];
+      ok = e >= 0 && e < E;
+      if (!ok) e = 0;
+    }
+  }
+  return e;
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(256) void moe_align_count_kernel(
+    const IdT *__restrict__ ids, int64_t numel, int E, const int32_t *__restrict__ expert_map,
+    int ignore_invalid, int64_t chunk_slots, int32_t *__restrict__ cnt, uint8_t *__restrict__ slot_mask) {
+  extern __shared__ int32_t lds[];
+  for (int i = threadIdx.x; i < E; i += blockDim.x) lds[i] = 0;
+  __syncthreads();
+  const int64_t begin = blockIdx.x * chunk_slots;
+  const int64_t end = (begin + chunk_slots < numel) ? begin + chunk_slots : numel;
+  for (int64_t f0 = begin + threadIdx.x; f0 < end; f0 += 4 * blockDim.x) {
+    int ek[4];
+    bool okk[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int64_t f = f0 + static_cast<int64_t>(b) * blockDim.x;
+      ek[b] = align_key(ids, f < end ? f : numel, numel, E, expert_map, ignore_invalid, okk[b]);
+      if (slot_mask && f < end) {
+        bool local = okk[b];
+        if (local && expert_map && !ignore_invalid) local = expert_map[ek[b]] >= 0;
+        slot_mask[f] = local ? 1 : 0;
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      if (okk[b]) atomicAdd(&lds[ek[b]], 1);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < E; i += blockDim.x) cnt[static_cast<int64_t>(blockIdx.x) * E + i] = lds[i];
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(256) void moe_align_scatter_kernel(
+    const IdT *__restrict__ ids, int64_t numel, int E, int bs, const int32_t *__restrict__ expert_map,
+    int ignore_invalid, int64_t chunk_slots, const int32_t *__restrict__ cnt,
+    int32_t *__restrict__ sorted, int64_t sorted_cap, int32_t *__restrict__ expert_ids,
+    int64_t expert_ids_cap, int32_t *__restrict__ ntpp, int key_bits) {
+  extern __shared__ int32_t lds[];
+  constexpr int nw = 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int chunk = blockIdx.x, nchunks = gridDim.x;
+  int32_t *offs = lds;              // [E + 1] padded exclusive prefix
+  int32_t *total = lds + (E + 1);   // [E]
+  int32_t *cbase = total + E;       // [E] slots of expert e in earlier chunks
+  int32_t *wcnt = cbase + E;        // [nw][E]
+  __shared__ int32_t wave_sum[nw];
+
+  for (int i = tid; i < nw * E; i += blockDim.x) wcnt[i] = 0;
+  for (int base = 0; base < E; base += blockDim.x) {
+    const int e = base + tid;
+    int t = 0, b = 0;
+    if (e < E) {
+      for (int c = 0; c < nchunks; ++c) {
+        const int v = cnt[static_cast<int64_t>(c) * E + e];
+        if (c < chunk) b += v;
+        t += v;
+      }
+      total[e] = t;
+      cbase[e] = b;
+    }
+    int incl = (e < E) ? (t + bs - 1) / bs * bs : 0;
+    for (int d = 1; d < kWave; d <<= 1) {
+      int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) wave_sum[wave] = incl;
+    __syncthreads();
+    int carry = (base == 0) ? 0 : offs[base];
+    for (int w = 0; w < wave; ++w) carry += wave_sum[w];
+    if (e < E) offs[e + 1] = carry + incl;
+    if (base == 0 && tid == 0) offs[0] = 0;
+    __syncthreads();
+  }
+  const int P = offs[E];
+
+  // shared-out bookkeeping: workgroup c looks after experts c, c + nchunks, ...
+  if (chunk == 0 && tid == 0) ntpp[0] = P;
+  for (int e = chunk; e < E; e += nchunks) {
+    const int v = (expert_map && !ignore_invalid) ? expert_map[e] : e;
+    for (int b = offs[e] / bs + tid; b < offs[e + 1] / bs; b += blockDim.x) expert_ids[b] = v;
+    for (int i = offs[e] + total[e] + tid; i < offs[e + 1]; i += blockDim.x) sorted[i] = static_cast<int32_t>(numel);
+  }
+  for (int64_t b = P / bs + chunk * blockDim.x + tid; b < expert_ids_cap; b += static_cast<int64_t>(nchunks) * blockDim.x)
+    expert_ids[b] = -1;
+  for (int64_t i = P + chunk * blockDim.x + tid; i < sorted_cap; i += static_cast<int64_t>(nchunks) * blockDim.x)
+    sorted[i] = static_cast<int32_t>(numel);
+
+  // this chunk: contiguous sub-range per wave, whole 64-slot tiles
+  const int64_t begin = chunk * chunk_slots;
+  const int64_t end = (begin + chunk_slots < numel) ? begin + chunk_slots : numel;
+  const int64_t tiles = (end > begin) ? (end - begin + kWave - 1) / kWave : 0;
+  const int64_t tiles_per_wave = (tiles + nw - 1) / nw;
+  const int64_t t0 = wave * tiles_per_wave;
+  const int64_t t1 = (t0 + tiles_per_wave < tiles) ? t0 + tiles_per_wave : tiles;
+  constexpr int kBatch = 4;
+  for (int64_t t = t0; t < t1; t += kBatch) {
+    int ek[kBatch];
+    bool okk[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int64_t f = begin + (t + b) * kWave + lane;
+      ek[b] = align_key(ids, (t + b < t1 && f < end) ? f : numel, numel, E, expert_map, ignore_invalid, okk[b]);
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b)
+      if (okk[b]) atomicAdd(&wcnt[wave * E + ek[b]], 1);
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += blockDim.x) {
+    int c = 0;
+    for (int w = 0; w < nw; ++w) {
+      const int v = wcnt[w * E + e];
+      wcnt[w * E + e] = c;
+      c += v;
+    }
+  }
+  __syncthreads();
+  for (int64_t t = t0; t < t1; t += kBatch) {
+    int ek[kBatch];
+    bool okk[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int64_t f = begin + (t + b) * kWave + lane;
+      ek[b] = align_key(ids, (t + b < t1 && f < end) ? f : numel, numel, E, expert_map, ignore_invalid, okk[b]);
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int e = ek[b];
+      const bool ok = okk[b];
+      const int64_t f = begin + (t + b) * kWave + lane;
+      uint64_t peers = match_any(e, key_bits, ok);
+      if (ok) {
+        int before = __popcll(peers & ((1ull << lane) - 1ull));
+        int leader = __ffsll(static_cast<unsigned long long>(peers)) - 1;
+        int run = wcnt[wave * E + e];
+        sorted[offs[e] + cbase[e] + run + before] = static_cast<int32_t>(f);
+        __builtin_amdgcn_wave_barrier();
+        if (lane == leader) wcnt[wave * E + e] = run + __popcll(peers);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+}
+
+// chunks for the multi-workgroup path: about 1024 slots each, at most 256 chunks
+static void align_chunks(int64_t numel, int *nchunks, int64_t *chunk_slots) {
+  int64_t n = (numel + 1023) / 1024;
+  if (n > 256) n = 256;
+  if (n < 1) n = 1;
+  int64_t cs = (numel + n - 1) / n;
+  cs = (cs + 255) / 256 * 256;
+  *chunk_slots = cs;
+  *nchunks = static_cast<int>((numel + cs - 1) / cs);
+}
+
 } // namespace lo
 
 extern "C" int lo_moe_align_block_size(const void *topk_ids, int ids_dtype, int64_t numel,
@@ -173,6 +354,27 @@ extern "C" int lo_moe_align_block_size_mask(const void *topk_ids, int ids_dtype,
                                             int32_t *expert_ids, int64_t expert_ids_cap,
                                             int32_t *num_tokens_post_pad, uint8_t *slot_mask,
                                             lo_stream_t stream) {
+  return lo_moe_align_block_size_ws(topk_ids, ids_dtype, numel, num_experts, block_size, expert_map,
+                                    ignore_invalid, sorted_ids, sorted_cap, expert_ids, expert_ids_cap,
+                                    num_tokens_post_pad, slot_mask, nullptr, 0, stream);
+}
+
+extern "C" int64_t lo_moe_align_scratch_bytes(int64_t numel, int32_t num_experts) {
+  if (numel < 0 || num_experts < 1) return LO_EINVAL;
+  if (numel < 8192) return 0; // one workgroup is faster below this
+  int nchunks;
+  int64_t cs;
+  lo::align_chunks(numel, &nchunks, &cs);
+  return static_cast<int64_t>(nchunks) * num_experts * 4;
+}
+
+extern "C" int lo_moe_align_block_size_ws(const void *topk_ids, int ids_dtype, int64_t numel,
+                                          int32_t num_experts, int32_t block_size,
+                                          const int32_t *expert_map, int ignore_invalid,
+                                          int32_t *sorted_ids, int64_t sorted_cap,
+                                          int32_t *expert_ids, int64_t expert_ids_cap,
+                                          int32_t *num_tokens_post_pad, uint8_t *slot_mask,
+                                          void *scratch, int64_t scratch_bytes, lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(topk_ids && sorted_ids && expert_ids && num_tokens_post_pad, LO_EINVAL,
              "moe_align_block_size: null pointer");
@@ -191,14 +393,42 @@ extern "C" int lo_moe_align_block_size_mask(const void *topk_ids, int ids_dtype,
              "moe_align_block_size: expert_ids holds %lld, needs %lld", (long long)expert_ids_cap,
              (long long)((need + block_size - 1) / block_size));
 
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int key_bits = 1;
+  while ((1 << key_bits) < num_experts) ++key_bits;
+  const int64_t want = lo_moe_align_scratch_bytes(numel, num_experts);
+  if (want > 0 && scratch && scratch_bytes >= want && (reinterpret_cast<uintptr_t>(scratch) & 3) == 0) {
+    int nchunks;
+    int64_t cs;
+    align_chunks(numel, &nchunks, &cs);
+    int32_t *cnt = static_cast<int32_t *>(scratch);
+    const size_t lds1 = static_cast<size_t>(num_experts) * 4;
+    const size_t lds2 = (static_cast<size_t>(4 + 3) * num_experts + 1) * 4;
+    if (ids_dtype == LO_I32) {
+      hipLaunchKernelGGL(moe_align_count_kernel<int32_t>, dim3(nchunks), dim3(256), lds1, s,
+                         static_cast<const int32_t *>(topk_ids), numel, num_experts, expert_map,
+                         ignore_invalid, cs, cnt, slot_mask);
+      hipLaunchKernelGGL(moe_align_scatter_kernel<int32_t>, dim3(nchunks), dim3(256), lds2, s,
+                         static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,
+                         expert_map, ignore_invalid, cs, cnt, sorted_ids, sorted_cap, expert_ids,
+                         expert_ids_cap, num_tokens_post_pad, key_bits);
+    } else {
+      hipLaunchKernelGGL(moe_align_count_kernel<int64_t>, dim3(nchunks), dim3(256), lds1, s,
+                         static_cast<const int64_t *>(topk_ids), numel, num_experts, expert_map,
+                         ignore_invalid, cs, cnt, slot_mask);
+      hipLaunchKernelGGL(moe_align_scatter_kernel<int64_t>, dim3(nchunks), dim3(256), lds2, s,
+                         static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size,
+                         expert_map, ignore_invalid, cs, cnt, sorted_ids, sorted_cap, expert_ids,
+                         expert_ids_cap, num_tokens_post_pad, key_bits);
+    }
+    return check_launch("moe_align_block_size(multi)");
+  }
+
   // waves per workgroup: as many as the per-wave LDS counters allow (<= 60 KB)
   int nw = 16;
   while (nw > 1 && (static_cast<int64_t>(nw) + 2) * num_experts + 1 > 15360) nw >>= 1;
   if (numel <= 64 * 4) nw = nw < 4 ? nw : 4;
   size_t lds_bytes = (static_cast<size_t>(nw + 2) * num_experts + 1) * sizeof(int32_t);
-  int key_bits = 1;
-  while ((1 << key_bits) < num_experts) ++key_bits;
-  hipStream_t s = static_cast<hipStream_t>(stream);
   if (ids_dtype == LO_I32)
     hipLaunchKernelGGL(moe_align_kernel<int32_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
                        static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,

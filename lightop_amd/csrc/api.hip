@@ -37,7 +37,8 @@ static void align_caps(int64_t numel, int32_t num_experts, int32_t bs, int64_t *
 }
 
 struct WsLayout {
-  int64_t off[8];
+  int64_t off[9];
+  int64_t align_scratch;
   int64_t total;
   int64_t sorted_cap, blocks_cap;
 };
@@ -47,16 +48,18 @@ static WsLayout ws_layout(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_
   WsLayout L{};
   const int64_t S = M * top_k;
   align_caps(S, num_experts, bs, &L.sorted_cap, &L.blocks_cap);
-  const int64_t sizes[8] = {M * H,                 // a1q
+  L.align_scratch = lo_moe_align_scratch_bytes(S, num_experts);
+  const int64_t sizes[9] = {M * H,                 // a1q
                             M * (H / kGroup) * 4,  // a1s
                             L.sorted_cap * 4,      // sorted_ids
                             L.blocks_cap * 4,      // expert_ids
                             4,                     // num_tokens_post_pad
                             S * I,                 // a2q
                             S * (I / kGroup) * 4,  // a2s
-                            S};                    // slot mask
+                            S,                     // slot mask
+                            L.align_scratch};      // per-chunk expert counters of the alignment
   int64_t o = 0;
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < 9; ++i) {
     L.off[i] = o;
     o += align_up(sizes[i] > 0 ? sizes[i] : 1, 256);
   }
@@ -153,8 +156,9 @@ extern "C" int lo_fused_experts_block_int8(
 
   int rc = lo_per_token_group_quant_int8(x, dtype, M, H, 1e-10f, a1q, a1s, stream);
   if (rc) return rc;
-  rc = lo_moe_align_block_size_mask(topk_ids, ids_dtype, S, num_experts, block_size_m, expert_map, 0,
-                                    sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, mask, stream);
+  rc = lo_moe_align_block_size_ws(topk_ids, ids_dtype, S, num_experts, block_size_m, expert_map, 0,
+                                  sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, mask, ws + L.off[8],
+                                  L.align_scratch, stream);
   if (rc) return rc;
   rc = lo_moe_gemm1_silu_quant_block_int8(a1q, a1s, w1, w1s, a2q, a2s, dtype, topk_w, sorted, eids,
                                           ntpp, L.sorted_cap, S, M, E, I, H, top_k, block_size_m,

@@ -24,6 +24,7 @@ struct GemmArgs {
   int32_t top_k;
   int32_t n_tiles;       // workgroups along N
   int32_t E;             // experts held by W
+  int32_t experts_routed; // experts the routing spreads the slots over (estimate, for tile order)
   int32_t mul_routed;
   int32_t w_shuffled;    // W is in the pre-shuffled layout (shuffle.hip)
   int32_t skip_nonlocal; // blocks of expert -1: leave the output rows untouched

@@ -12,6 +12,15 @@ static int64_t grid_m_blocks(int64_t sorted_cap, int64_t num_valid, int bs) {
   return blocks;
 }
 
+// The alignment buffers are sized S + E_global * (bs - 1): recover E_global from them.
+static int32_t routed_experts(int64_t sorted_cap, int64_t num_valid, int bs, int32_t E) {
+  if (bs > 1 && sorted_cap > num_valid) {
+    const int64_t eg = (sorted_cap - num_valid) / (bs - 1);
+    if (eg >= E && eg <= 4096) return static_cast<int32_t>(eg);
+  }
+  return E;
+}
+
 static int validate_common(const char *who, const void *A, const void *As, const void *W,
                            const void *Ws, const void *sorted, const void *eids, const void *ntpp,
                            int64_t K, int32_t top_k, int32_t E, int64_t a_rows) {
@@ -62,7 +71,7 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   GemmArgs a{};
   a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.C = static_cast<uint16_t *>(C);
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
-  a.E = E; a.a_rows = a_rows; a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.E = E; a.experts_routed = routed_experts(sorted_cap, num_valid, block_size_m, E); a.a_rows = a_rows; a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
@@ -97,7 +106,7 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
   GemmArgs a{};
   a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.A2q = A2q; a.A2s = A2s;
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
-  a.E = E; a.a_rows = a_rows; a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.E = E; a.experts_routed = routed_experts(sorted_cap, num_valid, block_size_m, E); a.a_rows = a_rows; a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.n_tiles = static_cast<int32_t>(I / kGroup);

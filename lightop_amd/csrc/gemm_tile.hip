@@ -28,14 +28,15 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kTileRow = 144;    // LDS row pitch in bytes: 128 + 16 keeps ds_read_b128 conflict-free
 
 // Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
-// The logical tile list is cut into chunks of (4 token blocks x all weight tiles): the
+// The logical tile list is cut into chunks of (G token blocks x all weight tiles): the
 // tiles of a chunk share token rows, and neighbouring token blocks mostly share an
-// expert's weights.  Chunks are dealt round-robin to the XCDs, and the workgroups that
+// expert's weights; G is about one expert's worth of token blocks, so that an expert's
+// weights are fetched into one L2 only.  Chunks are dealt round-robin to the XCDs, and the workgroups that
 // an XCD receives one after the other walk through one chunk, so what is shared is
 // fetched into that XCD's L2 once; blocks of experts that are not on this rank (which
 // cluster by expert id) still spread evenly over all XCDs.
-__device__ __forceinline__ bool tile_of(int bid, int n_tiles, int m_blocks, int &mb, int &nt) {
-  constexpr int XCD = 8, G = 4;
+__device__ __forceinline__ bool tile_of(int bid, int n_tiles, int m_blocks, int G, int &mb, int &nt) {
+  constexpr int XCD = 8;
   const int xcd = bid % XCD, slot = bid / XCD;
   const int span = G * n_tiles;                      // tiles per chunk
   const int chunk = (slot / span) * XCD + xcd, in = slot % span;
@@ -53,14 +54,14 @@ __device__ __forceinline__ bool tile_of(int bid, int n_tiles, int m_blocks, int 
 // workgroup per CU; 1 -> 64-token tile, 4 waves, two workgroups per CU that are not
 // synchronised with each other, so one computes while the other waits at its barrier.
 template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int WT>
-__global__ __launch_bounds__(256 * WT) void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks) {
+__global__ __launch_bounds__(256 * WT) void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   constexpr int kTileM = 64 * WT; // tokens per workgroup
   __shared__ __attribute__((aligned(16))) int8_t sA[2][kTileM * kTileRow];
   __shared__ float sS[2][kTileM];
   __shared__ float sRed[WT][2][4][32];
 
   int mb, nt;
-  if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, mb, nt)) return;
+  if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
   if (static_cast<int64_t>(mb) * kTileM >= a.ntpp[0]) return;
   const int e = a.expert_ids[mb];
   if (e >= a.E) return;
@@ -336,9 +337,11 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int block_size_m, int f
                      hipStream_t s) {
   GemmArgs a = a0;
   a.n_tiles = fused_act ? static_cast<int32_t>(a.N / 2 / kGroup) : static_cast<int32_t>((a.N + 255) / 256);
-  // every chunk of 4 token blocks owns 4 * n_tiles consecutive slots on one XCD
-  const int64_t chunks = (m_blocks + 3) / 4;
-  const int64_t grid = (chunks + 7) / 8 * (4 * a.n_tiles) * 8;
+  // every chunk of G token blocks owns G * n_tiles consecutive slots on one XCD
+  int64_t G = a.num_valid / (static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * block_size_m);
+  G = G < 2 ? 2 : (G > 16 ? 16 : G);
+  const int64_t chunks = (m_blocks + G - 1) / G;
+  const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
   const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
   const int wt = block_size_m / 64;
@@ -346,8 +349,8 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int block_size_m, int f
   const int mbi = static_cast<int>(m_blocks);
 #define LO_TILE_LAUNCH2(FA, FS, SH)                                                             \
   do {                                                                                          \
-    if (wt == 2) hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, SH, 2>), g, b, 0, s, a, mbi); \
-    else hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, SH, 1>), g, b, 0, s, a, mbi);         \
+    if (wt == 2) hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, SH, 2>), g, b, 0, s, a, mbi, static_cast<int>(G)); \
+    else hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, SH, 1>), g, b, 0, s, a, mbi, static_cast<int>(G));         \
   } while (0)
 #define LO_TILE_LAUNCH(FA, FS)                         \
   do {                                                 \

@@ -54,12 +54,18 @@ def _align(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num
             raise RuntimeError(f"lightop_amd: {name} must be a contiguous int32 tensor")
     if expert_map is not None and (expert_map.dtype != torch.int32 or not expert_map.is_contiguous()):
         expert_map = expert_map.to(torch.int32).contiguous()
+    lib = _lib.lib()
+    # large inputs are aligned by many workgroups; their per-chunk counters live in a
+    # scratch tensor (the reference allocates one too, moe_align_sum_kernels.cu:1175)
+    nscratch = int(lib.lo_moe_align_scratch_bytes(topk_ids.numel(), int(num_experts)))
+    scratch = torch.empty(nscratch, dtype=torch.uint8, device=topk_ids.device) if nscratch > 0 else None
     with _on_device(topk_ids):
-        _lib.check(_lib.lib().lo_moe_align_block_size(
+        _lib.check(lib.lo_moe_align_block_size_ws(
             _lib.ptr(topk_ids), _ids_dtype(topk_ids), topk_ids.numel(), int(num_experts), int(block_size),
             _lib.ptr(expert_map), 1 if ignore_invalid else 0, _lib.ptr(sorted_token_ids),
             sorted_token_ids.numel(), _lib.ptr(experts_ids), experts_ids.numel(),
-            _lib.ptr(num_tokens_post_pad), _lib.stream_of(topk_ids)))
+            _lib.ptr(num_tokens_post_pad), None, _lib.ptr(scratch), max(nscratch, 0),
+            _lib.stream_of(topk_ids)))
 
 
 def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: int,

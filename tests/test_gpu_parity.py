@@ -56,13 +56,14 @@ def test_align_bit_exact(dev, oracle, S, E, bs, idt):
 
 
 @pytest.mark.parametrize("ignore", [False, True])
-def test_align_expert_map(dev, oracle, ignore):
+@pytest.mark.parametrize("tokens", [333, 4099])  # one workgroup / many workgroups
+def test_align_expert_map(dev, oracle, ignore, tokens):
     from lightop_amd.moe import moe_align_block_size
 
-    say(f"align expert_map ignore={ignore}")
+    say(f"align expert_map ignore={ignore} tokens={tokens}")
     g = torch.Generator().manual_seed(11)
     E = 256
-    ids = torch.randint(0, E, (333, 8), generator=g, dtype=torch.int32)
+    ids = torch.randint(0, E, (tokens, 8), generator=g, dtype=torch.int32)
     emap = torch.full((E,), -1, dtype=torch.int32)
     emap[64:96] = torch.arange(32, dtype=torch.int32)
     rs, re, rp = oracle.moe_align_block_size(ids, 16, E, expert_map=emap, ignore_invalid_experts=ignore)
