@@ -121,9 +121,33 @@ __device__ __forceinline__ int quant_one(float v, float s) {
   return static_cast<int>(t);
 }
 
+// The same value as quant_one(v, s) from y = 1.0f / s (one IEEE division per row instead of
+// one per element): q = RN(v*y) is within an ulp of v/s, the remainder v - q*s is exact in
+// a fused multiply-add, and RN(q + rem*y) is then the correctly rounded quotient (Markstein's
+// theorem, valid for a correctly rounded reciprocal and no under/overflow).  Quotients
+// of denormal magnitude may differ in the last bit; they truncate to 0 either way.  Not
+// valid for s = inf (a row that holds an infinity): callers take quant_one then.
+__device__ __forceinline__ int quant_one_rcp(float v, float s, float y) {
+  const float q = v * y;
+  const float rem = __builtin_fmaf(-q, s, v);
+  float t = __builtin_fmaf(rem, y, q);
+  t = fmaxf(t, -128.0f);
+  t = fminf(t, 127.0f);
+  return static_cast<int>(t);
+}
+
 __device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
   return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
          ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+}
+
+// four elements of one row -> four packed int8; y = 1.0f / s
+__device__ __forceinline__ uint32_t quant4(const float *v, float s, float y) {
+  if (s < __builtin_inff()) {
+    return pack4_i8(quant_one_rcp(v[0], s, y), quant_one_rcp(v[1], s, y), quant_one_rcp(v[2], s, y),
+                    quant_one_rcp(v[3], s, y));
+  }
+  return pack4_i8(quant_one(v[0], s), quant_one(v[1], s), quant_one(v[2], s), quant_one(v[3], s));
 }
 
 } // namespace lo

@@ -315,11 +315,10 @@ __global__ __launch_bounds__(256 * WT) void moe_gemm_tile_kernel(const GemmArgs 
                          fmaxf(sRed[wt][tb][2][r], sRed[wt][tb][3][r]));
       amax = fmaxf(amax, 1e-10f);
       const float sc = amax / 127.0f;
+      const float rsc = 1.0f / sc;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const uint32_t packed =
-            pack4_i8(quant_one(actf[tb][4 * q + 0], sc), quant_one(actf[tb][4 * q + 1], sc),
-                     quant_one(actf[tb][4 * q + 2], sc), quant_one(actf[tb][4 * q + 3], sc));
+        const uint32_t packed = quant4(&actf[tb][4 * q], sc, rsc);
         *reinterpret_cast<uint32_t *>(a.A2q + f[tb] * I + nrow[0] + 8 * q + 4 * c) = packed;
       }
       if (wr == 0 && c == 0) a.A2s[f[tb] * G + nt] = sc;

@@ -253,8 +253,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       for (int w2 = 0; w2 < NWAVES; ++w2) amax = fmaxf(amax, red[j][w2][r]);
       amax = fmaxf(amax, 1e-10f);
       const float sc = amax / 127.0f;
-      const uint32_t packed = pack4_i8(quant_one(actf[j][0], sc), quant_one(actf[j][1], sc),
-                                       quant_one(actf[j][2], sc), quant_one(actf[j][3], sc));
+      const uint32_t packed = quant4(actf[j], sc, 1.0f / sc);
       *reinterpret_cast<uint32_t *>(a.A2q + f[j] * I + nrow[0] + 4 * c) = packed;
       if (wave == 0 && c == 0) a.A2s[f[j] * G + nt] = sc;
     }
