@@ -49,6 +49,29 @@ __device__ __forceinline__ float bld_f32(brsrc r, int voff, int soff) {
   return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
 }
 
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
+// The logical tile list is cut into chunks of (G token blocks x all weight tiles): the
+// tiles of a chunk share token rows, and neighbouring token blocks mostly share an
+// expert's weights; G is about one expert's worth of token blocks, so that an expert's
+// weights are fetched into one L2 only.  Chunks are dealt round-robin to the XCDs, and the workgroups that
+// an XCD receives one after the other walk through one chunk, so what is shared is
+// fetched into that XCD's L2 once; blocks of experts that are not on this rank (which
+// cluster by expert id) still spread evenly over all XCDs.
+__device__ __forceinline__ bool tile_of(int bid, int n_tiles, int m_blocks, int G, int &mb, int &nt) {
+  constexpr int XCD = 8;
+  const int xcd = bid % XCD, slot = bid / XCD;
+  const int span = G * n_tiles;                      // tiles per chunk
+  const int chunk = (slot / span) * XCD + xcd, in = slot % span;
+  const int first = chunk * G;
+  if (first >= m_blocks) return false;
+  const int gsz = (m_blocks - first < G) ? (m_blocks - first) : G;
+  nt = in / G;
+  const int off = in - nt * G;
+  if (off >= gsz) return false;
+  mb = first + off;
+  return true;
+}
+
 // Weight-streaming kernels (gemm_ws.hip): block_size_m in {16, 32, 64, 128}.
 int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
                    hipStream_t s);
@@ -56,5 +79,8 @@ int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flag
 int launch_gemm_tile(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
                      hipStream_t s);
 bool gemm_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);
+// Activation-stationary kernel (gemm_as.hip): plain epilogue, block_size_m 64, short K.
+int launch_gemm_as(const GemmArgs &a, int flags, int64_t m_blocks, hipStream_t s);
+bool gemm_as_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 
 } // namespace lo

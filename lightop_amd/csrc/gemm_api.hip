@@ -40,8 +40,10 @@ static int validate_common(const char *who, const void *A, const void *As, const
 // the MFMA pipe to matter); everything else streams weights.
 static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int64_t m_blocks,
                        hipStream_t s) {
-  if (!(flags & LO_GEMM_FORCE_STREAMING) && gemm_tile_supports(a, fused_act, bs))
-    return launch_gemm_tile(a, fused_act, bs, flags, m_blocks, s);
+  if (!(flags & LO_GEMM_FORCE_STREAMING)) {
+    if (gemm_as_supports(a, fused_act, bs)) return launch_gemm_as(a, flags, m_blocks, s);
+    if (gemm_tile_supports(a, fused_act, bs)) return launch_gemm_tile(a, fused_act, bs, flags, m_blocks, s);
+  }
   return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
 }
 

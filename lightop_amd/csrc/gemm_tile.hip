@@ -27,29 +27,6 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kTileRow = 144;    // LDS row pitch in bytes: 128 + 16 keeps ds_read_b128 conflict-free
 
-// Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
-// The logical tile list is cut into chunks of (G token blocks x all weight tiles): the
-// tiles of a chunk share token rows, and neighbouring token blocks mostly share an
-// expert's weights; G is about one expert's worth of token blocks, so that an expert's
-// weights are fetched into one L2 only.  Chunks are dealt round-robin to the XCDs, and the workgroups that
-// an XCD receives one after the other walk through one chunk, so what is shared is
-// fetched into that XCD's L2 once; blocks of experts that are not on this rank (which
-// cluster by expert id) still spread evenly over all XCDs.
-__device__ __forceinline__ bool tile_of(int bid, int n_tiles, int m_blocks, int G, int &mb, int &nt) {
-  constexpr int XCD = 8;
-  const int xcd = bid % XCD, slot = bid / XCD;
-  const int span = G * n_tiles;                      // tiles per chunk
-  const int chunk = (slot / span) * XCD + xcd, in = slot % span;
-  const int first = chunk * G;
-  if (first >= m_blocks) return false;
-  const int gsz = (m_blocks - first < G) ? (m_blocks - first) : G;
-  nt = in / G;
-  const int off = in - nt * G;
-  if (off >= gsz) return false;
-  mb = first + off;
-  return true;
-}
-
 // WT = number of 64-token halves per workgroup: 2 -> 128-token tile, 8 waves, one
 // workgroup per CU; 1 -> 64-token tile, 4 waves, two workgroups per CU that are not
 // synchronised with each other, so one computes while the other waits at its barrier.
