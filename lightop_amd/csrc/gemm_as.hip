@@ -18,7 +18,8 @@ namespace lo {
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 template <bool FAST_SCALE, bool SHUF>
-__global__ __launch_bounds__(256) void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
                                                           int n_groups, int n_cnt) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   constexpr int kTileM = 64;

@@ -31,7 +31,8 @@ constexpr int kTileRow = 144;    // LDS row pitch in bytes: 128 + 16 keeps ds_re
 // workgroup per CU; 1 -> 64-token tile, 4 waves, two workgroups per CU that are not
 // synchronised with each other, so one computes while the other waits at its barrier.
 template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int WT>
-__global__ __launch_bounds__(256 * WT) void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
+__global__ __launch_bounds__(256 * WT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   constexpr int kTileM = 64 * WT; // tokens per workgroup
   __shared__ __attribute__((aligned(16))) int8_t sA[2][kTileM * kTileRow];
   __shared__ float sS[2][kTileM];
