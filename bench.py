@@ -24,10 +24,16 @@ import torch
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0        # MI355X dense INT8 MFMA, published (5.0 POP/s)
 
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc
-# (FETCH_SIZE and WRITE_SIZE runs, scaled by a copy kernel of known size); keyed by
-# (workload, tokens).  None until measured for that point.
-MEASURED_TRAFFIC = {}
+# HBM bytes per launch of the dominant kernel (the first grouped GEMM), measured with
+# rocprofv3 --pmc: FETCH_SIZE x 2.00 x 1024 + WRITE_SIZE x 1.00 x 1024, the factors being
+# what the same counters read for kernels of known size in the same runs (a 512 MiB fill
+# and the one-pass weight shuffle); the summaries are the files under profiles/.  Keyed
+# by (workload, tokens); None for points that were not profiled.
+MEASURED_TRAFFIC = {
+    ("qwen3-30b-a3b", 8192): 1066796118,
+    ("deepseek-v3-ep8-share", 64): 805685369,
+    ("deepseek-v3-ep8-share", 4096): 2063886851,
+}
 
 
 def parse_args():
@@ -147,8 +153,31 @@ class Point:
         return {n: sum(v) / len(v) for n, v in acc.items()}, bs
 
 
+def graph_ms(pt, steps, flush, bs, flags):
+    """Mean time (ms) of one step replayed from a HIP graph: the five launches of the path
+    without their host-side launch cost.  None if the capture is refused."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                pt.step(bs, flags)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            pt.step(bs, flags)
+        mean_ms, _, _ = time_steps(g.replay, steps, 2, flush)
+        del g
+        return mean_ms
+    except Exception as e:  # report, do not fail the benchmark
+        print(f"[graph] capture failed for M={pt.M}: {e}", file=sys.stderr, flush=True)
+        return None
+
+
 def measure_point(pt, steps, warmup, flush, bs, flags):
     mean_ms, med_ms, min_ms = time_steps(lambda: pt.step(bs, flags), steps, warmup, flush)
+    g_ms = graph_ms(pt, steps, flush, bs, flags) if pt.M <= 64 else None
     t = mean_ms * 1e-3
     L = pt.layer
     hbm = pt.bytes / t / 1e9
@@ -161,6 +190,7 @@ def measure_point(pt, steps, warmup, flush, bs, flags):
         "hbm_gbs": round(hbm, 1), "S_loc": pt.S_loc, "E_act": pt.E_act, "bound": bound,
         "roofline_frac": round((tops / INT8_PEAK_TOPS) if bound == "mfma" else (hbm / HBM_PEAK_GBS), 4),
         "frac_hbm": round(hbm / HBM_PEAK_GBS, 4), "frac_mfma": round(tops / INT8_PEAK_TOPS, 4),
+        "ms_graph_replay": None if g_ms is None else round(g_ms, 4),
     }
 
 
@@ -175,12 +205,15 @@ def cpu_baseline(layer, weights, M_sample, seed=0):
     w1, w2, w1s, w2s = weights
     x, tw, ids = wl.make_inputs(layer, M_sample, seed=seed)
     emap = wl.expert_map_for(layer)
-    t0 = time.perf_counter()
-    torch_ref.torch_w8a8_block_int8_moe(x, w1, w2, w1s, w2s, tw, ids, expert_map=emap)
-    dt = time.perf_counter() - t0
+    runs = []
+    for i in range(4):  # one warm-up, three timed
+        t0 = time.perf_counter()
+        torch_ref.torch_w8a8_block_int8_moe(x, w1, w2, w1s, w2s, tw, ids, expert_map=emap)
+        runs.append(time.perf_counter() - t0)
+    dt = statistics.median(runs[1:])
     return {"value": round(M_sample / dt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"{layer.name}, first {M_sample} tokens of the same synthetic batch, one timed run of "
-                      f"oracle/torch_ref.py ({dt:.1f} s), torch {torch.__version__} CPU"}
+            "sample": f"{layer.name}, first {M_sample} tokens of the same synthetic batch, median of three runs "
+                      f"after one warm-up of oracle/torch_ref.py ({dt:.1f} s each), torch {torch.__version__} CPU"}
 
 
 def main():
@@ -235,6 +268,7 @@ def main():
         ach, peak, unit = g1_bytes / g1_t / 1e9, HBM_PEAK_GBS, "GB/s"
     roofline = {"bound": head["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
                 "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
+                "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
                 "kernel": ("moe_gemm_tile_kernel" if bs_used >= 64 else "moe_gemm_ws_kernel")
                 + "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)",
                 "kernel_ms": round(stages["gemm1_silu_quant"], 4),
@@ -259,7 +293,7 @@ def main():
 
     cpu = None
     if cpu_weights:
-        cpu = cpu_baseline(layer, cpu_weights, min(args.tokens, 4096))
+        cpu = cpu_baseline(layer, cpu_weights, min(args.tokens, 8192))
 
     t = head["ms_per_step"] * 1e-3
     line = {
