@@ -28,8 +28,8 @@ enum {
   LO_ENOTSUP = -4   /* valid request that this build has no kernel for */
 };
 
-/* activation element types */
-enum { LO_BF16 = 0, LO_F16 = 1 };
+/* activation element types (LO_F32: router inputs only) */
+enum { LO_BF16 = 0, LO_F16 = 1, LO_F32 = 2 };
 /* index element types of topk_ids */
 enum { LO_I32 = 0, LO_I64 = 1 };
 
@@ -248,6 +248,48 @@ int lo_fused_experts_block_int8(const void *x, int dtype, int64_t M, int64_t H, 
  */
 int64_t lo_fused_experts_workspace_offset(int which, int64_t M, int32_t top_k, int64_t H, int64_t I,
                                           int32_t num_experts, int32_t block_size_m);
+
+/* ---- routers upstream of the path (they produce topk_ids / topk_weights) ---------- */
+
+/*
+ * Softmax over all experts, the topk largest, their probabilities.
+ * Replaces op.topk_softmax(topk_weights, topk_indices, token_expert_indices, gating_output,
+ * Is_renormalize) (csrc/pybind/export.cpp:546, :1437;
+ * csrc/kernels/softmax/topk_softmax_kernels.cu:1716-1790, kernel :1381-1582).
+ *
+ *   gating [num_tokens, num_experts] fp32 / fp16 / bf16 (dtype = LO_F32 / LO_F16 / LO_BF16)
+ *   topk_weights [num_tokens, topk] fp32;  topk_indices [num_tokens, topk] int32 / int64
+ *   token_expert_indices [num_tokens, topk] int32 or NULL: entry (t, j) = j * num_tokens + t
+ *   renormalize = 0: exp(x - max) / (sum over all experts + 1e-6)
+ *   renormalize = 1: exp(x - max) / (sum over the selected + 1e-6)
+ * Winners in descending order; equal scores are won by the lower expert id (the reference
+ * leaves that open).  num_experts <= 1024, topk <= 64.
+ */
+int lo_topk_softmax(const void *gating, int dtype, int64_t num_tokens, int32_t num_experts,
+                    int32_t topk, int renormalize, float *topk_weights, void *topk_indices,
+                    int idx_dtype, int32_t *token_expert_indices, lo_stream_t stream);
+
+/*
+ * Grouped sigmoid top-k with a correction bias (DeepSeek-V3 style).  Replaces
+ * op.moe_fused_gate(input, bias, num_expert_group, topk_group, topk, n_share_experts_fusion,
+ * routed_scaling_factor, apply_routed_scaling_factor_on_output, output_indices_int64)
+ * (csrc/pybind/export.cpp:566, :1508; csrc/kernels/moe_gate/moe_fused_gate.cu:76-312, :1331-1530).
+ *
+ *   s = sigmoid(input);  c = bias + s;  group score = sum of the two largest c of the group;
+ *   the topk_group best groups stay; the topk - n_share best c among them are selected
+ *   (descending, ties to the lower id); weight = s / (sum of the selected s) * scale with
+ *   scale = routed_scaling_factor if apply_... and the factor is positive, else 1.
+ *   The n_share shared experts follow with ids num_experts, num_experts + 1, ... and weight
+ *   (sum / routed_scaling_factor) / sum * scale.
+ *   input [num_tokens, num_experts], bias [num_experts]: fp32 / fp16 / bf16 each.
+ * Unlike the reference, every (num_experts <= 1024, groups <= 64, topk <= 64) combination
+ * that divides evenly is served by one kernel.
+ */
+int lo_moe_fused_gate(const void *input, int dtype, const void *bias, int bias_dtype,
+                      int64_t num_tokens, int32_t num_experts, int32_t num_expert_group,
+                      int32_t topk_group, int32_t topk, int32_t n_share_experts_fusion,
+                      double routed_scaling_factor, int apply_routed_scaling_factor_on_output,
+                      float *topk_weights, void *topk_indices, int idx_dtype, lo_stream_t stream);
 
 #ifdef __cplusplus
 }

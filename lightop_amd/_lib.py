@@ -8,7 +8,7 @@ from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.environ.get("LIGHTOP_AMD_LIB") or os.path.join(_CSRC, "liblightop_mi355.so")
 
-LO_BF16, LO_F16 = 0, 1
+LO_BF16, LO_F16, LO_F32 = 0, 1, 2
 LO_I32, LO_I64 = 0, 1
 LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE, LO_GEMM_FORCE_STREAMING, LO_GEMM_CANONICAL_ORDER = 0, 1, 2, 4
 LO_GEMM_W_PRESHUFFLED = 8
@@ -45,6 +45,10 @@ SIGNATURES = {
     "lo_silu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float,
                            c_void_p]),
+    "lo_topk_softmax": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_int, c_void_p, c_void_p, c_int,
+                                c_void_p, c_void_p]),
+    "lo_moe_fused_gate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int32, c_int32, c_int32, c_int32,
+                                  c_int32, ctypes.c_double, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "lo_moe_tile_query": (c_int, [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
                                   ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
     "lo_fused_experts_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),

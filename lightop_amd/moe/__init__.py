@@ -2,7 +2,7 @@
 from importlib import import_module
 
 from .cache import get_moe_cache
-from .routing import moe_align_block_size, moe_align_block_size_out, moe_sum
+from .routing import moe_align_block_size, moe_align_block_size_out, moe_fused_gate, moe_sum, topk_softmax
 
 # resolved on first access, like the reference's lazily imported "LMSlim native" entry points
 # (moe/__init__.py:57-78)
@@ -34,7 +34,9 @@ __all__ = [
     "invoke_fused_moe_kernel_int8",
     "moe_align_block_size",
     "moe_align_block_size_out",
+    "moe_fused_gate",
     "moe_sum",
     "preshuffle_moe_weight",
     "silu_and_mul",
+    "topk_softmax",
 ]

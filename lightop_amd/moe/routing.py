@@ -1,4 +1,4 @@
-"""Expert alignment and expert reduction (reference: python/lightop/moe/routing.py,
+"""Routers, expert alignment and expert reduction (reference: python/lightop/moe/routing.py,
 python/lightop/_lmslim_native/vllm_compat/moe_align_block_size.py,
 python/lightop/moe_align_sum.py:12-29)."""
 from __future__ import annotations
@@ -8,6 +8,10 @@ from typing import Optional, Tuple
 import torch
 
 from .. import op
+from ..moe_fused_gate import moe_fused_gate
+
+# reference: moe/routing.py:20
+topk_softmax = op.topk_softmax
 
 
 def round_up(x: int, y: int) -> int:

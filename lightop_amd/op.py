@@ -1,6 +1,6 @@
 """Flat native-op namespace (reference: the pybind module ``lightop.op``,
-csrc/pybind/export.cpp:1584-1605).  Only the two operators of the block-INT8 fused-MoE
-path exist here; both write into caller-allocated tensors and return None.
+csrc/pybind/export.cpp:1437, :1508, :1584-1605).  Only the operators of the block-INT8
+fused-MoE path and the two routers that feed it exist here.
 """
 from __future__ import annotations
 
@@ -118,3 +118,61 @@ def moe_sum(input: torch.Tensor, output: torch.Tensor, bias: Optional[torch.Tens
         _lib.check(_lib.lib().lo_moe_sum(_lib.ptr(input), _lib.ptr(output), _lib.ptr(bias),
                                          _lib.ptr(expert_mask), _act_dtype(input), M, k, H, float(factor),
                                          _lib.stream_of(input)))
+
+
+def _float_dtype(t: torch.Tensor, what: str) -> int:
+    if t.dtype == torch.float32:
+        return _lib.LO_F32
+    if t.dtype == torch.float16:
+        return _lib.LO_F16
+    if t.dtype == torch.bfloat16:
+        return _lib.LO_BF16
+    raise RuntimeError(f"lightop_amd: {what} must be float32, float16 or bfloat16, got {t.dtype}")
+
+
+def topk_softmax(topk_weights: torch.Tensor, topk_indices: torch.Tensor,
+                 token_expert_indices: Optional[torch.Tensor], gating_output: torch.Tensor,
+                 Is_renormalize: bool = False) -> None:
+    """Softmax top-k router into caller-allocated outputs (op.topk_softmax, export.cpp:546, :1437;
+    topk_softmax_kernels.cu:1716-1790).  Winners in descending order, equal logits are won by
+    the lower expert id; ``token_expert_indices[t, j] = j * num_tokens + t``."""
+    _require_cuda(topk_weights, topk_indices, token_expert_indices, gating_output)
+    if gating_output.dim() != 2 or not gating_output.is_contiguous():
+        raise RuntimeError("lightop_amd: gating_output must be a contiguous [num_tokens, num_experts] tensor")
+    T, E = gating_output.shape
+    k = topk_weights.shape[-1]
+    if topk_weights.dtype != torch.float32 or not topk_weights.is_contiguous() or topk_weights.numel() != T * k:
+        raise RuntimeError("lightop_amd: topk_weights must be a contiguous float32 [num_tokens, topk] tensor")
+    if not topk_indices.is_contiguous() or topk_indices.numel() != T * k:
+        raise RuntimeError("lightop_amd: topk_indices must be a contiguous [num_tokens, topk] tensor")
+    if token_expert_indices is not None and (token_expert_indices.dtype != torch.int32
+                                             or not token_expert_indices.is_contiguous()
+                                             or token_expert_indices.numel() != T * k):
+        raise RuntimeError("lightop_amd: token_expert_indices must be a contiguous int32 [num_tokens, topk] tensor")
+    with _on_device(gating_output):
+        _lib.check(_lib.lib().lo_topk_softmax(
+            _lib.ptr(gating_output), _float_dtype(gating_output, "gating_output"), T, E, k, int(bool(Is_renormalize)),
+            _lib.ptr(topk_weights), _lib.ptr(topk_indices), _ids_dtype(topk_indices),
+            _lib.ptr(token_expert_indices), _lib.stream_of(gating_output)))
+
+
+def moe_fused_gate(input: torch.Tensor, bias: torch.Tensor, num_expert_group: int, topk_group: int, topk: int,
+                   n_share_experts_fusion: int, routed_scaling_factor: float,
+                   apply_routed_scaling_factor_on_output: bool = True, output_indices_int64: bool = False):
+    """Grouped sigmoid top-k with correction bias; returns ``[weights f32 [T, topk], indices [T, topk]]``
+    (op.moe_fused_gate, export.cpp:566, :1508; moe_fused_gate.cu:1331-1530)."""
+    _require_cuda(input, bias)
+    if input.dim() != 2 or not input.is_contiguous():
+        raise RuntimeError("lightop_amd: input must be a contiguous [num_tokens, num_experts] tensor")
+    T, E = input.shape
+    if bias.dim() != 1 or bias.numel() != E or not bias.is_contiguous():
+        raise RuntimeError("lightop_amd: bias must be a contiguous [num_experts] tensor")
+    weights = torch.empty(T, topk, dtype=torch.float32, device=input.device)
+    indices = torch.empty(T, topk, dtype=torch.int64 if output_indices_int64 else torch.int32, device=input.device)
+    with _on_device(input):
+        _lib.check(_lib.lib().lo_moe_fused_gate(
+            _lib.ptr(input), _float_dtype(input, "input"), _lib.ptr(bias), _float_dtype(bias, "bias"), T, E,
+            int(num_expert_group), int(topk_group), int(topk), int(n_share_experts_fusion),
+            float(routed_scaling_factor), int(bool(apply_routed_scaling_factor_on_output)),
+            _lib.ptr(weights), _lib.ptr(indices), _ids_dtype(indices), _lib.stream_of(input)))
+    return [weights, indices]

@@ -130,6 +130,38 @@ def moe_sum(inp, bias=None, factor=1.0):
     return out
 
 
+def topk_softmax(gating, topk, renormalize=False):
+    """gating [T, E] (any float dtype; widened to fp32) -> weights [T,k] f32, indices [T,k] i32,
+    source_rows [T,k] i32."""
+    g = gating.to(torch.float32).contiguous()
+    T, E = g.shape
+    w = torch.empty(T, topk, dtype=torch.float32)
+    idx = torch.empty(T, topk, dtype=torch.int32)
+    src = torch.empty(T, topk, dtype=torch.int32)
+    rc = lib().orc_topk_softmax(_p(g), _i64(T), _i32(E), _i32(topk), ctypes.c_int(int(renormalize)),
+                                _p(w), _p(idx), _p(src))
+    if rc:
+        raise ValueError(f"orc_topk_softmax: rc={rc}")
+    return w, idx, src
+
+
+def moe_fused_gate(x, bias, num_expert_group, topk_group, topk, n_share_experts_fusion,
+                   routed_scaling_factor, apply_routed_scaling_factor_on_output=True):
+    """x [T, E], bias [E] (widened to fp32) -> weights [T, topk] f32, indices [T, topk] i32."""
+    g = x.to(torch.float32).contiguous()
+    b = bias.to(torch.float32).contiguous()
+    T, E = g.shape
+    w = torch.empty(T, topk, dtype=torch.float32)
+    idx = torch.empty(T, topk, dtype=torch.int32)
+    rc = lib().orc_moe_fused_gate(_p(g), _p(b), _i64(T), _i32(E), _i32(num_expert_group), _i32(topk_group),
+                                  _i32(topk), _i32(n_share_experts_fusion),
+                                  ctypes.c_double(routed_scaling_factor),
+                                  ctypes.c_int(int(apply_routed_scaling_factor_on_output)), _p(w), _p(idx))
+    if rc:
+        raise ValueError(f"orc_moe_fused_gate: rc={rc}")
+    return w, idx
+
+
 def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids, block_size_m,
                              global_num_experts=-1, expert_map=None,
                              apply_router_weight_on_input=False, routed_scaling_factor=1.0,

@@ -358,3 +358,150 @@ int orc_fused_experts_block_int8(
   if (own_c3) free(c3);
   return rc;
 }
+
+/* ------------------------------------------------------------------------- *
+ * Routers upstream of the path (they produce topk_ids / topk_weights).
+ *
+ * Reference: csrc/kernels/softmax/topk_softmax_kernels.cu:1381-1582 (generic
+ * kernel; the reference's own test, test/test_softmax_topk.py:28-66, accepts
+ * any winner among equal logits and weights within rtol 2e-5 / atol 2e-6) and
+ * csrc/kernels/moe_gate/moe_fused_gate.cu:76-312 (grouped sigmoid top-k with
+ * correction bias; test/ci_tests/test_fused_moe_gate.py:9-61 is its torch
+ * restatement, compared at rtol = atol = 1e-6 after sorting by expert id).
+ *
+ * Canonical choices where the reference leaves the result open:
+ *   - ties are won by the lower index (experts and groups), so the selection
+ *     is a stable descending order;
+ *   - exp is orc_expf;
+ *   - the sum over the selected experts runs in selection order; the full-row
+ *     softmax sum (renormalize = 0) is the 64-lane tree spelled out below.
+ * Inputs are taken as fp32 (16-bit inputs are widened first, exactly).
+ * ------------------------------------------------------------------------- */
+#define ORC_NEG (-3.402823466e+38f)
+
+/* Sum of p[0..E) the way 64 lanes do it: lane l adds p[l], p[l+64], ... in that
+ * order, then six rounds of s[l] = s[l] + s[l ^ mask], mask = 32, 16, ..., 1. */
+static float lane_tree_sum(const float *p, int32_t E) {
+  float s[64], t[64];
+  for (int l = 0; l < 64; ++l) {
+    float a = 0.0f;
+    for (int32_t i = l; i < E; i += 64) a = a + p[i];
+    s[l] = a;
+  }
+  for (int mask = 32; mask > 0; mask >>= 1) {
+    for (int l = 0; l < 64; ++l) t[l] = s[l] + s[l ^ mask];
+    memcpy(s, t, sizeof(s));
+  }
+  return s[0];
+}
+
+/* index of the largest v[i] (lowest index among equals), or -1 if E == 0 */
+static int32_t argmax_low(const float *v, int32_t E) {
+  int32_t best = -1;
+  float bv = 0.0f;
+  for (int32_t i = 0; i < E; ++i)
+    if (best < 0 || v[i] > bv) { best = i; bv = v[i]; }
+  return best;
+}
+
+/*
+ * gating[T, E] fp32 -> weights[T, k] fp32, indices[T, k] int32,
+ * source_rows[T, k] int32 (optional) = j * T + t.
+ */
+int orc_topk_softmax(const float *gating, int64_t T, int32_t E, int32_t k, int renormalize,
+                     float *weights, int32_t *indices, int32_t *source_rows) {
+  if (E < 1 || k < 1 || k > E) return -1;
+  float *v = (float *)malloc(sizeof(float) * (size_t)E);
+  float *p = (float *)malloc(sizeof(float) * (size_t)E);
+  if (!v || !p) { free(v); free(p); return -2; }
+  for (int64_t t = 0; t < T; ++t) {
+    const float *x = gating + t * E;
+    float mx = x[0];
+    for (int32_t i = 1; i < E; ++i) if (x[i] > mx) mx = x[i];
+    float scale;
+    if (renormalize) {
+      memcpy(v, x, sizeof(float) * (size_t)E);
+    } else {
+      for (int32_t i = 0; i < E; ++i) p[i] = orc_expf(x[i] - mx);
+      scale = 1.0f / (lane_tree_sum(p, E) + 1e-6f);
+      memcpy(v, p, sizeof(float) * (size_t)E);
+    }
+    float sum = 0.0f;
+    for (int32_t j = 0; j < k; ++j) {
+      const int32_t w = argmax_low(v, E);
+      const float val = renormalize ? orc_expf(v[w] - mx) : v[w];
+      v[w] = ORC_NEG;
+      weights[t * k + j] = val;
+      indices[t * k + j] = w;
+      sum = sum + val;
+      if (source_rows) source_rows[t * k + j] = (int32_t)(j * T + t);
+    }
+    if (renormalize) scale = 1.0f / (sum + 1e-6f);
+    for (int32_t j = 0; j < k; ++j) weights[t * k + j] = weights[t * k + j] * scale;
+  }
+  free(v);
+  free(p);
+  return 0;
+}
+
+/*
+ * input[T, E], bias[E] fp32 -> weights[T, topk] fp32, indices[T, topk] int32.
+ * s = 1 / (1 + exp(-x));  c = bias + s;  group score = two largest c of the group added;
+ * the topk_group best groups stay; the topk - n_share best c among them are selected;
+ * weight = s of the selected / their sum (selection order) * route scale; the shared
+ * experts E, E+1, ... follow with weight (sum / rsf) / sum * route scale.
+ */
+int orc_moe_fused_gate(const float *input, const float *bias, int64_t T, int32_t E,
+                       int32_t num_expert_group, int32_t topk_group, int32_t topk,
+                       int32_t n_share, double routed_scaling_factor, int apply_on_output,
+                       float *weights, int32_t *indices) {
+  const int32_t G = num_expert_group;
+  if (E < 1 || G < 1 || E % G || topk_group < 1 || topk_group > G || n_share < 0 || topk - n_share < 1)
+    return -1;
+  const int32_t gs = E / G, kr = topk - n_share;
+  if (kr > topk_group * gs) return -1;
+  float *s = (float *)malloc(sizeof(float) * (size_t)E);
+  float *c = (float *)malloc(sizeof(float) * (size_t)E);
+  float *gsc = (float *)malloc(sizeof(float) * (size_t)G);
+  char *keep = (char *)malloc((size_t)G);
+  if (!s || !c || !gsc || !keep) { free(s); free(c); free(gsc); free(keep); return -2; }
+  const float rsf = (float)routed_scaling_factor;
+  const float route_scale = (apply_on_output && routed_scaling_factor > 0.0) ? rsf : 1.0f;
+  for (int64_t t = 0; t < T; ++t) {
+    const float *x = input + t * E;
+    for (int32_t i = 0; i < E; ++i) {
+      s[i] = 1.0f / (1.0f + orc_expf(-x[i]));
+      c[i] = bias[i] + s[i];
+    }
+    for (int32_t g = 0; g < G; ++g) {
+      float t1 = ORC_NEG, t2 = ORC_NEG;
+      for (int32_t i = g * gs; i < (g + 1) * gs; ++i) {
+        if (c[i] > t1) { t2 = t1; t1 = c[i]; }
+        else if (c[i] > t2) t2 = c[i];
+      }
+      gsc[g] = t1 + t2;
+      keep[g] = 0;
+    }
+    for (int32_t r = 0; r < topk_group; ++r) {
+      const int32_t w = argmax_low(gsc, G);
+      keep[w] = 1;
+      gsc[w] = ORC_NEG;
+    }
+    for (int32_t i = 0; i < E; ++i) if (!keep[i / gs]) c[i] = ORC_NEG;
+    float sum = 0.0f;
+    for (int32_t j = 0; j < kr; ++j) {
+      const int32_t w = argmax_low(c, E);
+      c[w] = ORC_NEG;
+      weights[t * topk + j] = s[w];
+      indices[t * topk + j] = w;
+      sum = sum + s[w];
+    }
+    for (int32_t j = kr; j < topk; ++j) {
+      weights[t * topk + j] = sum / (routed_scaling_factor > 0.0 ? rsf : 1.0f);
+      indices[t * topk + j] = E + (j - kr);
+    }
+    for (int32_t j = 0; j < topk; ++j) weights[t * topk + j] = (weights[t * topk + j] / sum) * route_scale;
+  }
+  free(s); free(c); free(gsc); free(keep);
+  return 0;
+}
