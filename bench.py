@@ -194,6 +194,40 @@ def measure_point(pt, steps, warmup, flush, bs, flags):
     }
 
 
+def router_times(layer, M, dev, steps, warmup):
+    """Mean time (us) per call of the two routers that produce topk_ids/topk_weights, launched
+    back to back on M rows of fp32 logits over the layer's global experts (events around the
+    whole loop, so at small M this is the launch rate of the host; the kernels' own durations are
+    in profiles/router_kernels.md)."""
+    from lightop_amd.moe import moe_fused_gate, topk_softmax
+
+    E, k = layer.E_global, layer.top_k
+    logits = torch.randn(M, E, device=dev)
+    bias = torch.zeros(E, device=dev)
+    w = torch.empty(M, k, dtype=torch.float32, device=dev)
+    idx = torch.empty(M, k, dtype=torch.int32, device=dev)
+    n_group = layer.n_group if layer.routing.startswith("grouped") else 1
+    tg = layer.topk_group if layer.routing.startswith("grouped") else 1
+    fns = {"topk_softmax": lambda: topk_softmax(w, idx, None, logits, True),
+           "moe_fused_gate": lambda: moe_fused_gate(logits, bias, n_group, tg, k, 0, 2.5)}
+    out = []
+    byts = M * E * 4 + M * k * 8
+    for name, fn in fns.items():
+        for _ in range(warmup):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        us = a.elapsed_time(b) * 1e3 / steps
+        out.append({"kernel": name, "tokens": M, "experts": E, "topk": k, "us_per_call": round(us, 2),
+                    "hbm_gbs": round(byts / us / 1e3, 1)})
+    return out
+
+
 def cpu_baseline(layer, weights, M_sample, seed=0):
     """The torch-CPU restatement of the reference path on the host cores, on the first
     M_sample tokens of the benchmark's batch."""
@@ -306,7 +340,8 @@ def main():
                    "tokens": args.tokens, "block_size_m": bs_used, "routing": L.routing},
         "int8_tops": head["int8_tops"], "hbm_gbs": head["hbm_gbs"], "frac_hbm": head["frac_hbm"],
         "frac_mfma": head["frac_mfma"], "stage_ms": {k: round(v, 4) for k, v in stages.items()},
-        "roofline": roofline, "cpu_baseline": cpu, "sweep": sweep,
+        "roofline": roofline, "cpu_baseline": cpu, "routers": router_times(layer, args.tokens, dev, 50, 5),
+        "sweep": sweep,
     }
     print(json.dumps(line), flush=True)
 

@@ -19,16 +19,62 @@ template <int DT> __device__ __forceinline__ float load_as_f32(const void *p, in
   else return to_f32<DT>(static_cast<const uint16_t *>(p)[i]);
 }
 
+// Lane exchange inside a row of 16 lanes by DPP (no LDS round trip): partner = lane ^ 1,
+// lane ^ 2, then the mirror images inside 8 and inside 16 lanes.  At the step where a mirror
+// is used all lanes of the smaller unit already hold the same value, so it acts like
+// lane ^ 4 and lane ^ 8.
+template <int CTRL> __device__ __forceinline__ int dpp_i(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, dpp_i<CTRL>(__builtin_bit_cast(int, v)));
+}
+constexpr int kXor1 = 0xB1, kXor2 = 0x4E, kMirror8 = 0x141, kMirror16 = 0x140;
+__device__ __forceinline__ float lane_f(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
 // (value, index) of the best lane; ties go to the lower index, so every lane agrees
+template <int CTRL> __device__ __forceinline__ void argmax_step(float &v, int &idx) {
+  const float ov = dpp_f<CTRL>(v);
+  const int oi = dpp_i<CTRL>(idx);
+  const bool take = ov > v || (ov == v && oi < idx);
+  v = take ? ov : v;
+  idx = take ? oi : idx;
+}
 __device__ __forceinline__ void wave_argmax(float &v, int &idx) {
+  argmax_step<kXor1>(v, idx);
+  argmax_step<kXor2>(v, idx);
+  argmax_step<kMirror8>(v, idx);
+  argmax_step<kMirror16>(v, idx);
+  // the four rows, through scalar registers
+  float bv = lane_f(v, 0);
+  int bi = __builtin_amdgcn_readlane(idx, 0);
 #pragma unroll
-  for (int mask = 32; mask > 0; mask >>= 1) {
-    const float ov = __shfl_xor(v, mask);
-    const int oi = __shfl_xor(idx, mask);
-    const bool take = ov > v || (ov == v && oi < idx);
-    v = take ? ov : v;
-    idx = take ? oi : idx;
+  for (int r = 1; r < 4; ++r) {
+    const float ov = lane_f(v, 16 * r);
+    const int oi = __builtin_amdgcn_readlane(idx, 16 * r);
+    const bool take = ov > bv || (ov == bv && oi < bi);
+    bv = take ? ov : bv;
+    bi = take ? oi : bi;
   }
+  v = bv;
+  idx = bi;
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f<kXor1>(v));
+  v = fmaxf(v, dpp_f<kXor2>(v));
+  v = fmaxf(v, dpp_f<kMirror8>(v));
+  v = fmaxf(v, dpp_f<kMirror16>(v));
+  return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
+}
+// s[l] = s[l] + s[l ^ m] for m = 1, 2, 4, 8, 16, 32: the same bits in every lane
+__device__ __forceinline__ float wave_sum_tree(float v) {
+  v = v + dpp_f<kXor1>(v);
+  v = v + dpp_f<kXor2>(v);
+  v = v + dpp_f<kMirror8>(v);
+  v = v + dpp_f<kMirror16>(v);
+  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
 }
 
 // One round: the best remaining entry of the row (value, expert); the winner erases it.
@@ -62,8 +108,7 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const void *__restric
     x[j] = e < E ? load_as_f32<DT>(gating, t * E + e) : kNeg;
     mx = fmaxf(mx, x[j]);
   }
-#pragma unroll
-  for (int mask = 32; mask > 0; mask >>= 1) mx = fmaxf(mx, __shfl_xor(mx, mask));
+  mx = wave_max(mx);
   float scale = 0.0f;
   if (renormalize) {
 #pragma unroll
@@ -77,9 +122,7 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const void *__restric
       v[j] = in ? p : kNeg;
       s = s + p;
     }
-#pragma unroll
-    for (int mask = 32; mask > 0; mask >>= 1) s = s + __shfl_xor(s, mask);
-    scale = 1.0f / (s + 1e-6f);
+    scale = 1.0f / (wave_sum_tree(s) + 1e-6f);
   }
   float sum = 0.0f, mine = 0.0f;
   int mine_idx = 0;
@@ -129,28 +172,46 @@ __global__ __launch_bounds__(256) void moe_fused_gate_kernel(const void *__restr
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  // lane g < G: the two largest choice scores of group g, added
-  float gscore = kNeg;
-  if (lane < G) {
+  uint64_t keep = ~0ull;
+  if (G > 1) {
+    // lpg lanes (a power of two, at most one DPP row) share a group: each scans every lpg-th
+    // score of it, then the two largest are merged across the lpg lanes (values only, so the
+    // order of the merges does not matter)
+    int lpg = 16;
+    while (lpg * G > 64) lpg >>= 1;
+    const int g = lane / lpg, sub = lane % lpg;
     float t1 = kNeg, t2 = kNeg;
-    for (int i = lane * gs; i < (lane + 1) * gs; ++i) {
-      const float cv = sC[wv][i];
-      if (cv > t1) {
-        t2 = t1;
-        t1 = cv;
-      } else if (cv > t2) {
-        t2 = cv;
+    if (g < G)
+      for (int i = g * gs + sub; i < (g + 1) * gs; i += lpg) {
+        const float cv = sC[wv][i];
+        if (cv > t1) {
+          t2 = t1;
+          t1 = cv;
+        } else if (cv > t2) {
+          t2 = cv;
+        }
       }
+#define LO_TOP2_MERGE(CTRL)                                  \
+  do {                                                       \
+    const float o1 = dpp_f<CTRL>(t1), o2 = dpp_f<CTRL>(t2);  \
+    const float n1 = fmaxf(t1, o1);                          \
+    t2 = fmaxf(fminf(t1, o1), fmaxf(t2, o2));                \
+    t1 = n1;                                                 \
+  } while (0)
+    if (lpg > 1) LO_TOP2_MERGE(kXor1);
+    if (lpg > 2) LO_TOP2_MERGE(kXor2);
+    if (lpg > 4) LO_TOP2_MERGE(kMirror8);
+    if (lpg > 8) LO_TOP2_MERGE(kMirror16);
+#undef LO_TOP2_MERGE
+    float gscore = (g < G && sub == 0) ? t1 + t2 : kNeg;
+    keep = 0;
+    for (int r = 0; r < topk_group; ++r) {
+      float bv = gscore;
+      int bi = g;
+      wave_argmax(bv, bi);
+      keep |= 1ull << bi;
+      if (g == bi) gscore = kNeg;
     }
-    gscore = t1 + t2;
-  }
-  uint64_t keep = 0;
-  for (int r = 0; r < topk_group; ++r) {
-    float bv = gscore;
-    int bi = lane;
-    wave_argmax(bv, bi);
-    keep |= 1ull << bi;
-    if (lane == bi) gscore = kNeg;
   }
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
@@ -168,7 +229,7 @@ __global__ __launch_bounds__(256) void moe_fused_gate_kernel(const void *__restr
 #pragma unroll
     for (int q = 0; q < VPT; ++q)
       if (bidx == lane + 64 * q) sv = s[q];
-    sv = __shfl(sv, bidx & 63);
+    sv = lane_f(sv, __builtin_amdgcn_readfirstlane(bidx) & 63);
     sum = sum + sv;
     if (lane == j) {
       mine = sv;

@@ -380,7 +380,7 @@ int orc_fused_experts_block_int8(
 #define ORC_NEG (-3.402823466e+38f)
 
 /* Sum of p[0..E) the way 64 lanes do it: lane l adds p[l], p[l+64], ... in that
- * order, then six rounds of s[l] = s[l] + s[l ^ mask], mask = 32, 16, ..., 1. */
+ * order, then six rounds of s[l] = s[l] + s[l ^ mask], mask = 1, 2, ..., 32. */
 static float lane_tree_sum(const float *p, int32_t E) {
   float s[64], t[64];
   for (int l = 0; l < 64; ++l) {
@@ -388,7 +388,7 @@ static float lane_tree_sum(const float *p, int32_t E) {
     for (int32_t i = l; i < E; i += 64) a = a + p[i];
     s[l] = a;
   }
-  for (int mask = 32; mask > 0; mask >>= 1) {
+  for (int mask = 1; mask < 64; mask <<= 1) {
     for (int l = 0; l < 64; ++l) t[l] = s[l] + s[l ^ mask];
     memcpy(s, t, sizeof(s));
   }
