@@ -113,6 +113,48 @@ __device__ __forceinline__ uint16_t silu_mul_tab(const uint16_t *__restrict__ ta
   return f32_to_bf16(sg * bf16_to_f32(u16));
 }
 
+// bf16(silu(g)) has closed forms outside a narrow band of inputs: for |g| <= 0x3bb5 (about
+// 0.0055) it is bf16(g / 2), for g >= 0x40bf (about 5.97) it is g, for finite g <= 0xc2b2
+// (about -89) it is -0.  The band in between, 1788 patterns per sign, fits in LDS; NaN and
+// -inf go to the full table.  (The bounds come from the full table itself; a test drives
+// every finite bf16 gate through the kernels that use this.)
+constexpr int kSiluBandLo = 0x3bb6, kSiluBandN = 1788; // band = [lo, lo + n) on |g|
+// The band travels global -> registers early (kSiluBandPer values per thread of a 256-thread
+// workgroup) and registers -> LDS before the workgroup's first barrier.
+constexpr int kSiluBandPer = (2 * kSiluBandN + 255) / 256;
+__device__ __forceinline__ void silu_band_load(uint16_t (&regs)[kSiluBandPer], const uint16_t *__restrict__ table, int tid) {
+#pragma unroll
+  for (int j = 0; j < kSiluBandPer; ++j) {
+    int i = tid + 256 * j;
+    i = i < 2 * kSiluBandN ? i : 2 * kSiluBandN - 1;
+    const int sign = i >= kSiluBandN;
+    regs[j] = table[(sign ? 0x8000 : 0) + kSiluBandLo + (i - sign * kSiluBandN)];
+  }
+}
+__device__ __forceinline__ void silu_band_store(uint16_t *band, const uint16_t (&regs)[kSiluBandPer], int tid) {
+#pragma unroll
+  for (int j = 0; j < kSiluBandPer; ++j) {
+    const int i = tid + 256 * j;
+    if (i < 2 * kSiluBandN) band[i] = regs[j];
+  }
+}
+__device__ __forceinline__ uint16_t silu_mul_band(const uint16_t *band, const uint16_t *__restrict__ table,
+                                                  uint16_t g16, uint16_t u16) {
+  const uint32_t mag = g16 & 0x7fffu, neg = g16 >> 15;
+  const uint32_t bi = mag - kSiluBandLo;
+  uint16_t sg16;
+  if (bi < static_cast<uint32_t>(kSiluBandN)) {
+    sg16 = band[bi + neg * kSiluBandN];
+  } else if (mag < static_cast<uint32_t>(kSiluBandLo)) {
+    sg16 = f32_to_bf16(bf16_to_f32(g16) * 0.5f);
+  } else if (mag > 0x7f80u || g16 == 0xff80u) {
+    sg16 = table[g16]; // NaN, -inf
+  } else {
+    sg16 = neg ? static_cast<uint16_t>(0x8000u) : g16;
+  }
+  return f32_to_bf16(bf16_to_f32(sg16) * bf16_to_f32(u16));
+}
+
 // q = (int8) trunc(clamp(v / s, -128, 127))
 __device__ __forceinline__ int quant_one(float v, float s) {
   float t = v / s;

@@ -37,6 +37,7 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   __shared__ __attribute__((aligned(16))) int8_t sA[2][kTileM * kTileRow];
   __shared__ float sS[2][kTileM];
   __shared__ float sRed[WT][2][4][32];
+  __shared__ uint16_t sSilu[FUSED_ACT ? 2 * kSiluBandN : 2];
 
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
@@ -87,6 +88,10 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     }
     return;
   }
+
+  // the SiLU band for the epilogue: requested first, so it arrives behind the loads below
+  uint16_t band_regs[kSiluBandPer];
+  if constexpr (FUSED_ACT) silu_band_load(band_regs, a.silu, tid & 255);
 
   // cooperative gather role: thread -> (token, 32-byte quarter of the 128-byte K block)
   const int lt = tid >> 2, lq = tid & 3;
@@ -223,6 +228,8 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   load_act(B1{}, 1);
   load_w(B0{}, 0);
   store_act(B0{}, true);
+  if constexpr (FUSED_ACT)
+    if (tid < 256) silu_band_store(sSilu, band_regs, tid);
   __syncthreads();
   for (int kb = 0; kb < KB; kb += 2) {
     // even K block: compute from LDS stage 0 / weight buffer 0
@@ -277,7 +284,7 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
           g = g * w;
           u = u * w;
         }
-        const uint16_t act16 = silu_mul_tab(a.silu, f32_to_bf16(g), f32_to_bf16(u));
+        const uint16_t act16 = silu_mul_band(sSilu, a.silu, f32_to_bf16(g), f32_to_bf16(u));
         actf[tb][i] = bf16_to_f32(act16);
         amax = fmaxf(amax, fabsf(actf[tb][i]));
       }

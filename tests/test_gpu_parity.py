@@ -294,6 +294,38 @@ def test_gemm1_silu_quant_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
                 assert torch.equal(q.cpu()[local], rq[local]), f"int8 activations differ ({what})"
 
 
+@pytest.mark.parametrize("bs", [16, 64, 128])
+def test_gemm1_epilogue_every_finite_bf16_gate(dev, oracle, bs):
+    """Every bf16 value below 1e18 in magnitude as the gate of the fused epilogue (SiLU table, its LDS band and the
+    closed forms outside the band): token t's group scale is the t-th bf16 pattern and the single
+    non-zero product of its row is 1, so gate = up = that value."""
+    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size
+
+    say(f"gemm1 epilogue over all bf16 gates bs={bs}")
+    pat = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    # gate * up must stay finite: with an infinite activation the group scale is inf, the quotient
+    # NaN and its int8 image undefined (in the reference as well)
+    pat = pat[torch.isfinite(pat) & (pat.abs() < 1e18)]
+    M, I, K = pat.numel(), 128, 128
+    Aq = torch.zeros(M, K, dtype=torch.int8)
+    Aq[:, 0] = 1
+    W = torch.zeros(1, 2 * I, K, dtype=torch.int8)
+    W[0, :, 0] = 1
+    As = pat.reshape(M, 1).contiguous()
+    Ws = torch.ones(1, 2, 1)
+    ids = torch.zeros(M, 1, dtype=torch.int32)
+    tw = torch.ones(M, 1)
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, 1)
+    c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, False, 1, M, bs)
+    assert torch.equal(c1[:, 0].float(), pat)  # the construction works: gate == pattern
+    rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+    s, e, p = moe_align_block_size(ids.to(dev), bs, 1)
+    q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), W.to(dev), As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
+                                              False, 1, M, {"BLOCK_SIZE_M": bs}, fused_scale=False)
+    torch.cuda.synchronize()
+    assert torch.equal(sc.cpu(), rsc) and torch.equal(q.cpu(), rq)
+
+
 def test_preshuffle_layout(dev):
     from lightop_amd.moe import preshuffle_moe_weight
 
