@@ -122,6 +122,26 @@ int lo_moe_align_block_size_ws(const void *topk_ids, int ids_dtype, int64_t nume
                                void *scratch, int64_t scratch_bytes, lo_stream_t stream);
 
 /*
+ * Same again for batches padded to a fixed size: num_local_tokens is a device int32[1] (or
+ * NULL) and only the slots of the first num_local_tokens[0] tokens (top_k slots each) are
+ * counted and sorted; the pad value stays numel, slot_mask is 0 for the padding tokens'
+ * slots (the num_local_tokens argument of op.moe_align_block_size,
+ * csrc/pybind/export.cpp:1593-1605, csrc/kernels/moe_align_sum_kernels.cu:32-45).  With a
+ * count of 0 the reference returns without writing anything; here num_tokens_post_pad is
+ * written as 0 and the buffers are filled with their pad values, so that the GEMMs skip
+ * every block.
+ */
+int lo_moe_align_block_size_local(const void *topk_ids, int ids_dtype, int64_t numel,
+                                  int32_t num_experts, int32_t block_size,
+                                  const int32_t *expert_map, int ignore_invalid,
+                                  int32_t *sorted_ids, int64_t sorted_cap,
+                                  int32_t *expert_ids, int64_t expert_ids_cap,
+                                  int32_t *num_tokens_post_pad, uint8_t *slot_mask,
+                                  void *scratch, int64_t scratch_bytes,
+                                  const int32_t *num_local_tokens, int32_t top_k,
+                                  lo_stream_t stream);
+
+/*
  * 1x128 group quantisation of activations to int8 with fp32 scales.
  * Replaces per_token_group_quant_int8 (python/lightop/_lmslim_native/layers/gemm/
  * int8_utils.py:125-195, Triton kernel :74-122).
@@ -184,9 +204,13 @@ int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *ac
  * order; without bias one rounding (:619-633), with bias the three roundings of :886-909.
  * expert_mask [M*topk] bytes or NULL: slots whose byte is 0 are not read and add nothing
  * (the expert_mask argument of the reference op, :661-672).
+ * num_local_tokens: device int32[1] or NULL; rows t >= num_local_tokens[0] (padding tokens of
+ * a fixed-size batch) are left untouched (:644-649, :735-741; one of the reference's
+ * variants tests t > n and so also writes row n).
  */
 int lo_moe_sum(const void *in, void *out, const void *bias, const uint8_t *expert_mask, int dtype,
-               int64_t M, int32_t topk, int64_t H, float factor, lo_stream_t stream);
+               int64_t M, int32_t topk, int64_t H, float factor, const int32_t *num_local_tokens,
+               lo_stream_t stream);
 
 /*
  * Load-time weight layout for the GEMM kernels: every block of 16 rows x 128 K-bytes of

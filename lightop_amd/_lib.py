@@ -32,6 +32,9 @@ SIGNATURES = {
     "lo_moe_align_block_size_ws": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,
                                            c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                            c_int64, c_void_p]),
+    "lo_moe_align_block_size_local": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_void_p, c_int,
+                                              c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
+                                              c_int64, c_void_p, c_int32, c_void_p]),
     "lo_per_token_group_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_float, c_void_p,
                                               c_void_p, c_void_p]),
     "lo_moe_gemm_block_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -44,7 +47,7 @@ SIGNATURES = {
     "lo_preshuffle_weight_int8": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "lo_silu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float,
-                           c_void_p]),
+                           c_void_p, c_void_p]),
     "lo_topk_softmax": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_int, c_void_p, c_void_p, c_int,
                                 c_void_p, c_void_p]),
     "lo_moe_fused_gate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int32, c_int32, c_int32, c_int32,

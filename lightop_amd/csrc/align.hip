@@ -19,13 +19,28 @@ __device__ __forceinline__ uint64_t match_any(int key, int bits, bool active) {
   return peers;
 }
 
+// Only the slots of the first num_local_tokens[0] tokens are aligned when that device
+// counter is given (batches padded to a fixed size); the pad value stays the full numel
+// (csrc/kernels/moe_align_sum_kernels.cu:32-45 of the reference).
+__device__ __forceinline__ int64_t local_slots(int64_t numel, const int32_t *__restrict__ num_local_tokens,
+                                               int slots_per_token) {
+  if (!num_local_tokens) return numel;
+  const int64_t v = static_cast<int64_t>(num_local_tokens[0]) * slots_per_token;
+  return v < 0 ? 0 : (v < numel ? v : numel);
+}
+
 template <typename IdT>
 __global__ __launch_bounds__(1024) void moe_align_kernel(
     const IdT *__restrict__ ids, int64_t numel, int num_experts, int bs,
     const int32_t *__restrict__ expert_map, int ignore_invalid, int32_t *__restrict__ sorted,
     int64_t sorted_cap, int32_t *__restrict__ expert_ids, int64_t expert_ids_cap,
-    int32_t *__restrict__ ntpp, int key_bits, uint8_t *__restrict__ slot_mask) {
+    int32_t *__restrict__ ntpp, int key_bits, uint8_t *__restrict__ slot_mask,
+    const int32_t *__restrict__ num_local_tokens, int slots_per_token) {
   extern __shared__ int32_t lds[];
+  const int64_t pad_val = numel;
+  numel = local_slots(numel, num_local_tokens, slots_per_token);
+  if (slot_mask) // slots of padding tokens belong to nobody
+    for (int64_t f = numel + threadIdx.x; f < pad_val; f += blockDim.x) slot_mask[f] = 0;
   const int nw = blockDim.x / kWave;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int E = num_experts;
@@ -121,8 +136,8 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
   // padding entries: the tail of every expert's range and everything past P
   for (int e = wave; e < E; e += nw)
     for (int i = offs[e] + total[e] + lane; i < offs[e + 1]; i += kWave)
-      sorted[i] = static_cast<int32_t>(numel);
-  for (int64_t i = P + tid; i < sorted_cap; i += blockDim.x) sorted[i] = static_cast<int32_t>(numel);
+      sorted[i] = static_cast<int32_t>(pad_val);
+  for (int64_t i = P + tid; i < sorted_cap; i += blockDim.x) sorted[i] = static_cast<int32_t>(pad_val);
 
   // pass 3: stable scatter.  wcnt[wave][e] is the running number of slots of expert
   // e that precede the current tile.  Ranks inside a tile come from a ballot match, the
@@ -182,12 +197,19 @@ __device__ __forceinline__ int align_key(const IdT *__restrict__ ids, int64_t f,
 template <typename IdT>
 __global__ __launch_bounds__(256) void moe_align_count_kernel(
     const IdT *__restrict__ ids, int64_t numel, int E, const int32_t *__restrict__ expert_map,
-    int ignore_invalid, int64_t chunk_slots, int32_t *__restrict__ cnt, uint8_t *__restrict__ slot_mask) {
+    int ignore_invalid, int64_t chunk_slots, int32_t *__restrict__ cnt, uint8_t *__restrict__ slot_mask,
+    const int32_t *__restrict__ num_local_tokens, int slots_per_token) {
   extern __shared__ int32_t lds[];
   for (int i = threadIdx.x; i < E; i += blockDim.x) lds[i] = 0;
   __syncthreads();
+  const int64_t pad_val = numel;
+  numel = local_slots(numel, num_local_tokens, slots_per_token);
   const int64_t begin = blockIdx.x * chunk_slots;
   const int64_t end = (begin + chunk_slots < numel) ? begin + chunk_slots : numel;
+  if (slot_mask) { // this chunk's slots of padding tokens belong to nobody
+    const int64_t pend = (begin + chunk_slots < pad_val) ? begin + chunk_slots : pad_val;
+    for (int64_t f = (begin > numel ? begin : numel) + threadIdx.x; f < pend; f += blockDim.x) slot_mask[f] = 0;
+  }
   for (int64_t f0 = begin + threadIdx.x; f0 < end; f0 += 4 * blockDim.x) {
     int ek[4];
     bool okk[4];
@@ -214,8 +236,11 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
     const IdT *__restrict__ ids, int64_t numel, int E, int bs, const int32_t *__restrict__ expert_map,
     int ignore_invalid, int64_t chunk_slots, const int32_t *__restrict__ cnt,
     int32_t *__restrict__ sorted, int64_t sorted_cap, int32_t *__restrict__ expert_ids,
-    int64_t expert_ids_cap, int32_t *__restrict__ ntpp, int key_bits) {
+    int64_t expert_ids_cap, int32_t *__restrict__ ntpp, int key_bits,
+    const int32_t *__restrict__ num_local_tokens, int slots_per_token) {
   extern __shared__ int32_t lds[];
+  const int64_t pad_val = numel;
+  numel = local_slots(numel, num_local_tokens, slots_per_token);
   constexpr int nw = 4;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int chunk = blockIdx.x, nchunks = gridDim.x;
@@ -258,12 +283,12 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
   for (int e = chunk; e < E; e += nchunks) {
     const int v = (expert_map && !ignore_invalid) ? expert_map[e] : e;
     for (int b = offs[e] / bs + tid; b < offs[e + 1] / bs; b += blockDim.x) expert_ids[b] = v;
-    for (int i = offs[e] + total[e] + tid; i < offs[e + 1]; i += blockDim.x) sorted[i] = static_cast<int32_t>(numel);
+    for (int i = offs[e] + total[e] + tid; i < offs[e + 1]; i += blockDim.x) sorted[i] = static_cast<int32_t>(pad_val);
   }
   for (int64_t b = P / bs + chunk * blockDim.x + tid; b < expert_ids_cap; b += static_cast<int64_t>(nchunks) * blockDim.x)
     expert_ids[b] = -1;
   for (int64_t i = P + chunk * blockDim.x + tid; i < sorted_cap; i += static_cast<int64_t>(nchunks) * blockDim.x)
-    sorted[i] = static_cast<int32_t>(numel);
+    sorted[i] = static_cast<int32_t>(pad_val);
 
   // this chunk: contiguous sub-range per wave, whole 64-slot tiles
   const int64_t begin = chunk * chunk_slots;
@@ -375,7 +400,23 @@ extern "C" int lo_moe_align_block_size_ws(const void *topk_ids, int ids_dtype, i
                                           int32_t *expert_ids, int64_t expert_ids_cap,
                                           int32_t *num_tokens_post_pad, uint8_t *slot_mask,
                                           void *scratch, int64_t scratch_bytes, lo_stream_t stream) {
+  return lo_moe_align_block_size_local(topk_ids, ids_dtype, numel, num_experts, block_size, expert_map,
+                                       ignore_invalid, sorted_ids, sorted_cap, expert_ids, expert_ids_cap,
+                                       num_tokens_post_pad, slot_mask, scratch, scratch_bytes, nullptr, 1,
+                                       stream);
+}
+
+extern "C" int lo_moe_align_block_size_local(const void *topk_ids, int ids_dtype, int64_t numel,
+                                             int32_t num_experts, int32_t block_size,
+                                             const int32_t *expert_map, int ignore_invalid,
+                                             int32_t *sorted_ids, int64_t sorted_cap,
+                                             int32_t *expert_ids, int64_t expert_ids_cap,
+                                             int32_t *num_tokens_post_pad, uint8_t *slot_mask,
+                                             void *scratch, int64_t scratch_bytes,
+                                             const int32_t *num_local_tokens, int32_t top_k,
+                                             lo_stream_t stream) {
   using namespace lo;
+  LO_REQUIRE(!num_local_tokens || top_k >= 1, LO_EINVAL, "moe_align_block_size: top_k %d", top_k);
   LO_REQUIRE(topk_ids && sorted_ids && expert_ids && num_tokens_post_pad, LO_EINVAL,
              "moe_align_block_size: null pointer");
   LO_REQUIRE(ids_dtype == LO_I32 || ids_dtype == LO_I64, LO_EINVAL,
@@ -407,19 +448,19 @@ extern "C" int lo_moe_align_block_size_ws(const void *topk_ids, int ids_dtype, i
     if (ids_dtype == LO_I32) {
       hipLaunchKernelGGL(moe_align_count_kernel<int32_t>, dim3(nchunks), dim3(256), lds1, s,
                          static_cast<const int32_t *>(topk_ids), numel, num_experts, expert_map,
-                         ignore_invalid, cs, cnt, slot_mask);
+                         ignore_invalid, cs, cnt, slot_mask, num_local_tokens, top_k);
       hipLaunchKernelGGL(moe_align_scatter_kernel<int32_t>, dim3(nchunks), dim3(256), lds2, s,
                          static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,
                          expert_map, ignore_invalid, cs, cnt, sorted_ids, sorted_cap, expert_ids,
-                         expert_ids_cap, num_tokens_post_pad, key_bits);
+                         expert_ids_cap, num_tokens_post_pad, key_bits, num_local_tokens, top_k);
     } else {
       hipLaunchKernelGGL(moe_align_count_kernel<int64_t>, dim3(nchunks), dim3(256), lds1, s,
                          static_cast<const int64_t *>(topk_ids), numel, num_experts, expert_map,
-                         ignore_invalid, cs, cnt, slot_mask);
+                         ignore_invalid, cs, cnt, slot_mask, num_local_tokens, top_k);
       hipLaunchKernelGGL(moe_align_scatter_kernel<int64_t>, dim3(nchunks), dim3(256), lds2, s,
                          static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size,
                          expert_map, ignore_invalid, cs, cnt, sorted_ids, sorted_cap, expert_ids,
-                         expert_ids_cap, num_tokens_post_pad, key_bits);
+                         expert_ids_cap, num_tokens_post_pad, key_bits, num_local_tokens, top_k);
     }
     return check_launch("moe_align_block_size(multi)");
   }
@@ -433,11 +474,11 @@ extern "C" int lo_moe_align_block_size_ws(const void *topk_ids, int ids_dtype, i
     hipLaunchKernelGGL(moe_align_kernel<int32_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
                        static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,
                        expert_map, ignore_invalid, sorted_ids, sorted_cap, expert_ids,
-                       expert_ids_cap, num_tokens_post_pad, key_bits, slot_mask);
+                       expert_ids_cap, num_tokens_post_pad, key_bits, slot_mask, num_local_tokens, top_k);
   else
     hipLaunchKernelGGL(moe_align_kernel<int64_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
                        static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size,
                        expert_map, ignore_invalid, sorted_ids, sorted_cap, expert_ids,
-                       expert_ids_cap, num_tokens_post_pad, key_bits, slot_mask);
+                       expert_ids_cap, num_tokens_post_pad, key_bits, slot_mask, num_local_tokens, top_k);
   return check_launch("moe_align_block_size");
 }

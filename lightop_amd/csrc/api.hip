@@ -170,5 +170,5 @@ extern "C" int lo_fused_experts_block_int8(
                               stream);
   if (rc) return rc;
   return lo_moe_sum(cache3, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor,
-                    stream);
+                    nullptr, stream);
 }

@@ -73,8 +73,14 @@ __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t *__restrict
                                                       const uint16_t *__restrict__ bias,
                                                       const uint8_t *__restrict__ mask,
                                                       int64_t M, int topk, int64_t H,
-                                                      float factor) {
+                                                      float factor,
+                                                      const int32_t *__restrict__ num_local_tokens) {
   const int64_t vec_per_row = H / 8;
+  // rows of padding tokens (t >= num_local_tokens[0]) are left untouched
+  if (num_local_tokens) {
+    const int64_t n = num_local_tokens[0];
+    M = n < 0 ? 0 : (n < M ? n : M);
+  }
   const int64_t total = M * vec_per_row;
   for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < total;
        v += static_cast<int64_t>(gridDim.x) * blockDim.x) {
@@ -204,7 +210,7 @@ extern "C" int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
 
 extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uint8_t *expert_mask,
                           int dtype, int64_t M, int32_t topk, int64_t H, float factor,
-                          lo_stream_t stream) {
+                          const int32_t *num_local_tokens, lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(in && out, LO_EINVAL, "moe_sum: null pointer");
   LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "moe_sum: only bf16 is built");
@@ -219,10 +225,10 @@ extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uin
   if (bias)
     hipLaunchKernelGGL((moe_sum_kernel<LO_BF16, true>), dim3(grid), dim3(256), 0, s,
                        static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),
-                       static_cast<const uint16_t *>(bias), expert_mask, M, topk, H, factor);
+                       static_cast<const uint16_t *>(bias), expert_mask, M, topk, H, factor, num_local_tokens);
   else
     hipLaunchKernelGGL((moe_sum_kernel<LO_BF16, false>), dim3(grid), dim3(256), 0, s,
                        static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),
-                       static_cast<const uint16_t *>(nullptr), expert_mask, M, topk, H, factor);
+                       static_cast<const uint16_t *>(nullptr), expert_mask, M, topk, H, factor, num_local_tokens);
   return check_launch("moe_sum");
 }

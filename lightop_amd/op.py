@@ -44,8 +44,9 @@ def _act_dtype(t: torch.Tensor) -> int:
 
 
 def _align(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad,
-           expert_map, ignore_invalid):
-    _require_cuda(topk_ids, sorted_token_ids, experts_ids, num_tokens_post_pad, expert_map)
+           expert_map, ignore_invalid, expert_mask=None, num_local_tokens=None):
+    _require_cuda(topk_ids, sorted_token_ids, experts_ids, num_tokens_post_pad, expert_map, expert_mask,
+                  num_local_tokens)
     if not topk_ids.is_contiguous():
         topk_ids = topk_ids.contiguous()
     for t, name in ((sorted_token_ids, "sorted_token_ids"), (experts_ids, "experts_ids"),
@@ -54,18 +55,30 @@ def _align(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num
             raise RuntimeError(f"lightop_amd: {name} must be a contiguous int32 tensor")
     if expert_map is not None and (expert_map.dtype != torch.int32 or not expert_map.is_contiguous()):
         expert_map = expert_map.to(torch.int32).contiguous()
+    if expert_mask is not None:
+        if expert_mask.dtype not in (torch.bool, torch.uint8) or not expert_mask.is_contiguous() \
+                or expert_mask.numel() != topk_ids.numel():
+            raise RuntimeError("lightop_amd: expert_mask must be a contiguous bool tensor with one entry per slot")
+        expert_mask = expert_mask.view(torch.uint8)
+    top_k = 1
+    if num_local_tokens is not None:
+        if num_local_tokens.dtype != torch.int32 or num_local_tokens.numel() < 1:
+            raise RuntimeError("lightop_amd: num_local_tokens must be an int32 tensor with one element")
+        if topk_ids.dim() != 2:
+            raise RuntimeError("lightop_amd: num_local_tokens needs topk_ids of shape [num_tokens, topk]")
+        top_k = topk_ids.shape[1]
     lib = _lib.lib()
     # large inputs are aligned by many workgroups; their per-chunk counters live in a
     # scratch tensor (the reference allocates one too, moe_align_sum_kernels.cu:1175)
     nscratch = int(lib.lo_moe_align_scratch_bytes(topk_ids.numel(), int(num_experts)))
     scratch = torch.empty(nscratch, dtype=torch.uint8, device=topk_ids.device) if nscratch > 0 else None
     with _on_device(topk_ids):
-        _lib.check(lib.lo_moe_align_block_size_ws(
+        _lib.check(lib.lo_moe_align_block_size_local(
             _lib.ptr(topk_ids), _ids_dtype(topk_ids), topk_ids.numel(), int(num_experts), int(block_size),
             _lib.ptr(expert_map), 1 if ignore_invalid else 0, _lib.ptr(sorted_token_ids),
             sorted_token_ids.numel(), _lib.ptr(experts_ids), experts_ids.numel(),
-            _lib.ptr(num_tokens_post_pad), None, _lib.ptr(scratch), max(nscratch, 0),
-            _lib.stream_of(topk_ids)))
+            _lib.ptr(num_tokens_post_pad), _lib.ptr(expert_mask), _lib.ptr(scratch), max(nscratch, 0),
+            _lib.ptr(num_local_tokens), top_k, _lib.stream_of(topk_ids)))
 
 
 def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: int,
@@ -75,30 +88,28 @@ def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: i
                          expert_mask: Optional[torch.Tensor] = None,
                          num_local_tokens: Optional[torch.Tensor] = None,
                          Is_EP: bool = False, Is_fuse_fill: bool = True) -> None:
-    """``op.moe_align_block_size`` (export.cpp:1593-1605).  An ``expert_map`` given here is
-    applied to the ids before counting and ids mapped to -1 are dropped
-    (csrc/kernels/moe_align_sum_kernels.cu:62-90); the DeepEP-only arguments
-    ``expert_mask``, ``num_local_tokens`` and ``Is_EP`` are not part of this path."""
-    if expert_mask is not None or num_local_tokens is not None or Is_EP:
-        raise NotImplementedError(
-            "lightop_amd.op.moe_align_block_size: expert_mask / num_local_tokens / Is_EP belong to the "
-            "DeepEP layout, which this build does not cover")
+    """``op.moe_align_block_size`` (export.cpp:1593-1605; kernel semantics
+    csrc/kernels/moe_align_sum_kernels.cu:25-150).  With an ``expert_map`` the block expert ids
+    are the mapped (local) ids, -1 for experts of other ranks; ``Is_EP`` drops the slots of those
+    experts instead of keeping them as -1 blocks; ``expert_mask`` (bool, one entry per slot) is an
+    output: True where the slot's expert is on this rank; ``num_local_tokens`` (device int32[1])
+    limits the work to the first that many tokens, whose padding successors get mask False."""
     del Is_fuse_fill  # the pad value is always written
     _align(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad,
-           expert_map, ignore_invalid=True)
+           expert_map, ignore_invalid=bool(Is_EP) and expert_map is not None, expert_mask=expert_mask,
+           num_local_tokens=num_local_tokens)
 
 
 def moe_sum(input: torch.Tensor, output: torch.Tensor, bias: Optional[torch.Tensor] = None,
             expert_mask: Optional[torch.Tensor] = None, num_local_tokens: Optional[torch.Tensor] = None,
             factor: float = 1.0, expect_m: int = -1) -> None:
     """``op.moe_sum`` (export.cpp:1584-1592): output[t] = factor * sum_k input[t, k] (+ bias[t]).
-    Slots whose ``expert_mask`` entry is False are skipped."""
-    if num_local_tokens is not None:
-        raise NotImplementedError(
-            "lightop_amd.op.moe_sum: num_local_tokens belongs to the DeepEP layout, which this build "
-            "does not cover")
+    Slots whose ``expert_mask`` entry is False are skipped; rows from ``num_local_tokens[0]`` on
+    (device int32[1]) are left untouched."""
     del expect_m
-    _require_cuda(input, output, bias)
+    _require_cuda(input, output, bias, num_local_tokens)
+    if num_local_tokens is not None and (num_local_tokens.dtype != torch.int32 or num_local_tokens.numel() < 1):
+        raise RuntimeError("lightop_amd.op.moe_sum: num_local_tokens must be an int32 tensor with one element")
     if input.dim() != 3:
         raise RuntimeError("lightop_amd.op.moe_sum: input must be [num_tokens, topk, hidden]")
     if not input.is_contiguous():
@@ -117,7 +128,7 @@ def moe_sum(input: torch.Tensor, output: torch.Tensor, bias: Optional[torch.Tens
     with _on_device(input):
         _lib.check(_lib.lib().lo_moe_sum(_lib.ptr(input), _lib.ptr(output), _lib.ptr(bias),
                                          _lib.ptr(expert_mask), _act_dtype(input), M, k, H, float(factor),
-                                         _lib.stream_of(input)))
+                                         _lib.ptr(num_local_tokens), _lib.stream_of(input)))
 
 
 def _float_dtype(t: torch.Tensor, what: str) -> int:

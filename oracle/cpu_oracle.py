@@ -72,21 +72,37 @@ def align_buffer_sizes(numel: int, num_experts: int, block_size: int, pad_sorted
 
 
 def moe_align_block_size(topk_ids, block_size, num_experts, expert_map=None,
-                         pad_sorted_ids=False, ignore_invalid_experts=False):
+                         pad_sorted_ids=False, ignore_invalid_experts=False, num_local_tokens=None):
+    """With num_local_tokens only the slots of the first that many tokens are aligned; the pad
+    value and the buffer sizes stay those of the whole batch (moe_align_sum_kernels.cu:32-45)."""
     ids = topk_ids.reshape(-1).to(torch.int32).contiguous()
     S = ids.numel()
+    n_eff = S if num_local_tokens is None else max(0, min(S, int(num_local_tokens) * topk_ids.shape[-1]))
     max_pad, max_blocks = align_buffer_sizes(S, num_experts, block_size, pad_sorted_ids)
     sorted_ids = torch.empty(max_pad, dtype=torch.int32)
     expert_ids = torch.empty(max_blocks, dtype=torch.int32)
     ntpp = torch.zeros(1, dtype=torch.int32)
     emap = None if expert_map is None else expert_map.to(torch.int32).contiguous()
     rc = lib().orc_moe_align_block_size(
-        _p(ids), _i64(S), _i32(num_experts), _i32(block_size), _p(emap),
+        _p(ids[:n_eff].contiguous()), _i64(n_eff), _i32(num_experts), _i32(block_size), _p(emap),
         ctypes.c_int(1 if ignore_invalid_experts else 0), _p(sorted_ids), _i64(max_pad),
         _p(expert_ids), _i64(max_blocks), _p(ntpp))
     if rc != 0:
         raise RuntimeError("oracle moe_align_block_size: id out of range or buffer too small")
+    if n_eff != S:
+        sorted_ids[sorted_ids == n_eff] = S  # valid slot ids are below n_eff, so this only hits pads
     return sorted_ids, expert_ids, ntpp
+
+
+def align_slot_mask(topk_ids, expert_map=None, num_local_tokens=None):
+    """expert_mask output of the alignment op: True where the slot belongs to a local token and
+    its expert is on this rank (moe_align_sum_kernels.cu:73-79, :147)."""
+    ids = topk_ids.reshape(-1).long()
+    S = ids.numel()
+    n_eff = S if num_local_tokens is None else max(0, min(S, int(num_local_tokens) * topk_ids.shape[-1]))
+    mask = torch.ones(S, dtype=torch.bool) if expert_map is None else expert_map.long()[ids] >= 0
+    mask[n_eff:] = False
+    return mask
 
 
 def per_token_group_quant_int8(x, group_size=128, eps=1e-10):
@@ -122,12 +138,16 @@ def silu_and_mul(c1):
     return act
 
 
-def moe_sum(inp, bias=None, factor=1.0):
+def moe_sum(inp, bias=None, factor=1.0, num_local_tokens=None, out=None):
+    """With num_local_tokens, rows from that index on keep what ``out`` held."""
     M, k, H = inp.shape
-    out = torch.empty(M, H, dtype=torch.bfloat16)
+    res = torch.empty(M, H, dtype=torch.bfloat16)
     lib().orc_moe_sum(_p(inp.contiguous()), _i64(M), _i32(k), _i64(H),
-                      _p(None if bias is None else bias.contiguous()), ctypes.c_float(factor), _p(out))
-    return out
+                      _p(None if bias is None else bias.contiguous()), ctypes.c_float(factor), _p(res))
+    if num_local_tokens is not None:
+        n = max(0, min(M, int(num_local_tokens)))
+        res[n:] = out[n:]
+    return res
 
 
 def topk_softmax(gating, topk, renormalize=False):

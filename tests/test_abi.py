@@ -94,5 +94,5 @@ def test_validation_happens_before_any_launch(lib):
     assert b"sorted_ids holds 10" in lib.lo_last_error()
     assert lib.lo_per_token_group_quant_int8(p, 0, 1, 100, 1e-10, p, p, null) == -1              # cols % 128
     assert lib.lo_per_token_group_quant_int8(p, 1, 1, 128, 1e-10, p, p, null) == -4              # fp16 not built
-    assert lib.lo_moe_sum(p, p, null, null, 0, 1, 8, 100, 1.0, null) == -1                       # H % 8
+    assert lib.lo_moe_sum(p, p, null, null, 0, 1, 8, 100, 1.0, null, null) == -1                       # H % 8
     assert lib.lo_preshuffle_weight_int8(p, p, 1, 16, 128, null) == -1                           # src == dst

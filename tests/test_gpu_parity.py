@@ -102,6 +102,51 @@ def test_align_out_variant_and_errors(dev, oracle):
         moe_align_block_size_out(ids.to(dev), 16, 16, s[:10], e, p)
 
 
+@pytest.mark.parametrize("M,k,E", [(40, 4, 16), (3000, 8, 128)])  # one workgroup / many workgroups
+@pytest.mark.parametrize("is_ep", [False, True])
+def test_align_num_local_tokens_and_mask_output(dev, oracle, M, k, E, is_ep):
+    """op.moe_align_block_size with its padded-batch and expert-parallel arguments."""
+    from lightop_amd import op
+
+    g = torch.Generator().manual_seed(M + k)
+    ids = torch.randint(0, E, (M, k), generator=g, dtype=torch.int32)
+    emap = torch.full((E,), -1, dtype=torch.int32)
+    emap[: E // 2] = torch.arange(E // 2, dtype=torch.int32)
+    bs = 16
+    cap, nb = oracle.align_buffer_sizes(M * k, E, bs)
+    for n in (0, 1, M // 3, M):
+        say(f"align padded batch M={M} k={k} local={n} is_ep={is_ep}")
+        s = torch.full((cap,), -7, dtype=torch.int32, device=dev)
+        e = torch.full((nb,), -7, dtype=torch.int32, device=dev)
+        p = torch.full((1,), -7, dtype=torch.int32, device=dev)
+        mask = torch.ones(M * k, dtype=torch.bool, device=dev)
+        nlt = torch.tensor([n], dtype=torch.int32, device=dev)
+        op.moe_align_block_size(ids.to(dev), E, bs, s, e, p, emap.to(dev), mask, nlt, is_ep)
+        torch.cuda.synchronize()
+        rs, re, rp = oracle.moe_align_block_size(ids, bs, E, expert_map=emap, ignore_invalid_experts=is_ep,
+                                                 num_local_tokens=n)
+        assert torch.equal(p.cpu(), rp) and torch.equal(s.cpu(), rs) and torch.equal(e.cpu(), re)
+        assert torch.equal(mask.cpu(), oracle.align_slot_mask(ids, emap, n))
+
+
+def test_moe_sum_num_local_tokens(dev, oracle):
+    from lightop_amd.moe import moe_sum
+
+    say("moe_sum padded batch")
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(50, 4, 256, generator=g).to(torch.bfloat16)
+    bias = torch.randn(50, 256, generator=g).to(torch.bfloat16)
+    for n in (0, 1, 17, 50, 80):
+        for b in (None, bias):
+            prev = torch.full((50, 256), 3.0, dtype=torch.bfloat16)
+            out = prev.clone().to(dev)
+            moe_sum(x.to(dev), out, None if b is None else b.to(dev),
+                    num_local_tokens=torch.tensor([n], dtype=torch.int32, device=dev), factor=1.5)
+            torch.cuda.synchronize()
+            ref = oracle.moe_sum(x, b, 1.5, num_local_tokens=n, out=prev)
+            assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16)), f"n={n}"
+
+
 # ---------------------------------------------------------------- group quant --
 
 @pytest.mark.parametrize("rows,cols", [(1, 128), (1, 7168), (3, 2048), (64, 1024), (257, 768), (4096, 2048)])
