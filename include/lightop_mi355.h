@@ -51,7 +51,17 @@ enum {
   LO_GEMM_W_PRESHUFFLED = 8,
   /* leave the output rows of blocks whose expert id is -1 untouched instead of zeroing
    * them (the caller then reduces with an expert_mask, see lo_moe_sum) */
-  LO_GEMM_SKIP_NONLOCAL = 16
+  LO_GEMM_SKIP_NONLOCAL = 16,
+  /* W4A8 with K-group scales (BASELINE's int4 variant): W (w1 and w2 for the whole path) is
+   * packed signed int4 in the layout of lo_preshuffle_weight_int4 (LO_GEMM_W_PRESHUFFLED must
+   * be set too) and the weight scales are one per output row and 128-wide K group,
+   * Ws [E, N, K/128] instead of [E, N/128, K/128]:
+   *   acc = acc + (f32(sum_k A*w) * As[row, kb]) * Ws[e, n, kb],  w in [-8, 7].
+   * The reference's W4A8 (python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:211-401)
+   * scales per token and per channel in the epilogue instead; its nibble order (even k in
+   * the high nibble, :341, :375-377) is the one lo_preshuffle_weight_int4 reads.  Served by
+   * the weight-streaming kernels at every block_size_m. */
+  LO_GEMM_W4 = 32
 };
 
 int lo_version(void);
@@ -211,6 +221,15 @@ int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *ac
 int lo_moe_sum(const void *in, void *out, const void *bias, const uint8_t *expert_mask, int dtype,
                int64_t M, int32_t topk, int64_t H, float factor, const int32_t *num_local_tokens,
                lo_stream_t stream);
+
+/*
+ * Load-time layout of packed int4 weights for LO_GEMM_W4: src [E, N, K/2] bytes, element k of
+ * a row in byte k/2, even k in the high nibble; dst the same number of bytes, blocks of
+ * 16 rows x 128 K (1 KB) ordered [E][K/128][N/16].  N % 16 == 0, K % 128 == 0; src != dst.
+ * No counterpart in the reference (its Triton kernel reads the row-major packed tensor).
+ */
+int lo_preshuffle_weight_int4(const uint8_t *src, uint8_t *dst, int32_t E, int64_t N, int64_t K,
+                              lo_stream_t stream);
 
 /*
  * Load-time weight layout for the GEMM kernels: every block of 16 rows x 128 K-bytes of

@@ -13,6 +13,7 @@ LO_I32, LO_I64 = 0, 1
 LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE, LO_GEMM_FORCE_STREAMING, LO_GEMM_CANONICAL_ORDER = 0, 1, 2, 4
 LO_GEMM_W_PRESHUFFLED = 8
 LO_GEMM_SKIP_NONLOCAL = 16
+LO_GEMM_W4 = 32
 
 
 class LoMoeTile(ctypes.Structure):
@@ -45,6 +46,7 @@ SIGNATURES = {
                                                    c_int64, c_int64, c_int64, c_int32, c_int64, c_int64,
                                                    c_int32, c_int32, c_int, c_int, c_void_p]),
     "lo_preshuffle_weight_int8": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
+    "lo_preshuffle_weight_int4": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "lo_silu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float,
                            c_void_p, c_void_p]),

@@ -28,6 +28,7 @@ struct GemmArgs {
   int32_t mul_routed;
   int32_t w_shuffled;    // W is in the pre-shuffled layout (shuffle.hip)
   int32_t skip_nonlocal; // blocks of expert -1: leave the output rows untouched
+  int32_t w4;            // W is packed int4 (load-time layout), Ws is [E, N, K/128]
 };
 
 __device__ __forceinline__ v4i ld16(const int8_t *p) { return *reinterpret_cast<const v4i *>(p); }

@@ -40,6 +40,7 @@ static int validate_common(const char *who, const void *A, const void *As, const
 // the MFMA pipe to matter); everything else streams weights.
 static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int64_t m_blocks,
                        hipStream_t s) {
+  if (a.w4) return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s); // int4 weights: streaming kernels only
   if (!(flags & LO_GEMM_FORCE_STREAMING)) {
     if (gemm_as_supports(a, fused_act, bs)) return launch_gemm_as(a, flags, m_blocks, s);
     if (gemm_tile_supports(a, fused_act, bs)) return launch_gemm_tile(a, fused_act, bs, flags, m_blocks, s);
@@ -76,6 +77,9 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   a.E = E; a.experts_routed = routed_experts(sorted_cap, num_valid, block_size_m, E); a.a_rows = a_rows; a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
+  a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
+  LO_REQUIRE(!a.w4 || a.w_shuffled, LO_ENOTSUP,
+             "moe_gemm: int4 weights must be in the layout of lo_preshuffle_weight_int4 (LO_GEMM_W_PRESHUFFLED)");
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 30), LO_EINVAL, "moe_gemm: grid too large");
@@ -111,6 +115,10 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
   a.E = E; a.experts_routed = routed_experts(sorted_cap, num_valid, block_size_m, E); a.a_rows = a_rows; a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
+  a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
+  LO_REQUIRE(!a.w4 || a.w_shuffled, LO_ENOTSUP,
+             "moe_gemm1_silu_quant: int4 weights must be in the layout of lo_preshuffle_weight_int4 "
+             "(LO_GEMM_W_PRESHUFFLED)");
   a.n_tiles = static_cast<int32_t>(I / kGroup);
   rc = silu_table(static_cast<hipStream_t>(stream), &a.silu);
   if (rc) return rc;

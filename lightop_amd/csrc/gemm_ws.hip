@@ -38,9 +38,17 @@
 
 namespace lo {
 
-template <int TM, bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int NWAVES, int PD, int RPW>
+//
+// W4: the weights are packed signed int4 in the load-time layout of preshuffle_int4_kernel
+// (one 16-byte load per lane holds both k-steps of a 128-wide K block; two vector
+// instructions per 8 elements turn them into int8 values 16 times too large, which an
+// arithmetic shift of the exact int32 sum takes out again) and every weight row has its
+// own scale per K block, Ws [E, N, K/128].
+template <int TM, bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int NWAVES, int PD, int RPW, bool W4 = false>
 __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs a) {
+  static_assert(!W4 || SHUF, "int4 weights exist in the load-time layout only");
   constexpr int BM = 16 * TM;
+  constexpr int NS = W4 ? 4 : 1; // weight scales per 16-row fragment and lane
   // 16-row weight fragments per wave: (gate, up) when fused, else RPW consecutive ones
   constexpr int NW = FUSED_ACT ? 2 : RPW;
   // With at most 32 tokens per block an expert's weights are read by one pass only:
@@ -101,18 +109,24 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       nrow[g] = static_cast<int64_t>(nt) * (16 * NWAVES * RPW) + wave * (16 * RPW) + g * 16;
   }
   const int NB = static_cast<int>((N + kGroup - 1) / kGroup);
-  const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * N * K, static_cast<uint32_t>(N * K));
+  const int64_t wbytes = W4 ? N * K / 2 : N * K; // one expert
+  const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * wbytes, static_cast<uint32_t>(wbytes));
+  const brsrc rWs = make_rsrc(a.Ws + static_cast<int64_t>(e) * N * KB, static_cast<uint32_t>(W4 ? N * KB * 4 : 0));
   int woff[NW];
   const float *wsrow[NW];
-  const int wkstride = shuf_kb_stride(static_cast<int>(N / 16));
+  int wsoff[NW]; // W4: byte offset of the lane's first scale row
+  const int wkstride = W4 ? shuf_kb_stride(static_cast<int>(N / 16)) / 2 : shuf_kb_stride(static_cast<int>(N / 16));
 #pragma unroll
   for (int g = 0; g < NW; ++g) {
-    if constexpr (SHUF) // 2 KB blocks; one MFMA operand = 1 KB in lane order
+    if constexpr (W4) // 1 KB blocks; both k-steps of a lane in one 16-byte piece
+      woff[g] = static_cast<int>(nrow[g] / 16) * (shuf_nb_stride(KB) / 2) + lane * 16;
+    else if constexpr (SHUF) // 2 KB blocks; one MFMA operand = 1 KB in lane order
       woff[g] = static_cast<int>(nrow[g] / 16) * shuf_nb_stride(KB) + lane * 16;
     else
       woff[g] = static_cast<int>((nrow[g] + r) * K) + c * 16;
     const int64_t nclamp = nrow[g] < N ? nrow[g] : 0; // fragments past N: loads return 0, nothing is stored
     wsrow[g] = a.Ws + (static_cast<int64_t>(e) * NB + nclamp / kGroup) * KB;
+    wsoff[g] = static_cast<int>((nclamp + 4 * c) * KB * 4); // accumulator rows of this lane: 4c .. 4c+3
   }
 
   v4f acc[NW][TM];
@@ -125,26 +139,39 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   // the scales that belong to them.  The scales travel in the same ring because the
   // vector-memory counter retires in order: a scale load issued after a prefetch could
   // only be waited for by draining the prefetch as well.
-  v4i wbuf[PD][NW][2];
+  v4i wbuf[PD][NW][W4 ? 1 : 2];
   v4i abuf[PD][TM][2];
   float asbuf[PD][TM];
-  float bsbuf[PD][NW];
+  float bsbuf[PD][NW][NS];
   // The loop body is kept free of branches: a slot past the end of K re-reads the last
   // K block and gets a token scale of zero, so it adds exactly 0 to every accumulator.
   // (Branches around the loads make the compiler fall back to waiting for all of them.)
   auto issue = [&](int slot, int kb) {
     const int kc = kb < KB ? kb : KB - 1;
+    if constexpr (W4) {
+#pragma unroll
+      for (int g = 0; g < NW; ++g) wbuf[slot][g][0] = bld16<WAUX>(rW, woff[g], kc * wkstride);
+    }
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
+      if constexpr (!W4) {
 #pragma unroll
-      for (int g = 0; g < NW; ++g)
-        wbuf[slot][g][ks] = SHUF ? bld16<WAUX>(rW, woff[g], kc * wkstride + ks * 1024)
-                                 : bld16<WAUX>(rW, woff[g], kc * kGroup + ks * 64);
+        for (int g = 0; g < NW; ++g)
+          wbuf[slot][g][ks] = SHUF ? bld16<WAUX>(rW, woff[g], kc * wkstride + ks * 1024)
+                                   : bld16<WAUX>(rW, woff[g], kc * kGroup + ks * 64);
+      }
 #pragma unroll
       for (int j = 0; j < TM; ++j) abuf[slot][j][ks] = bld16(rA, aoff[j], kc * kGroup + ks * 64);
     }
 #pragma unroll
-    for (int g = 0; g < NW; ++g) bsbuf[slot][g] = wsrow[g][kc];
+    for (int g = 0; g < NW; ++g) {
+      if constexpr (W4) {
+#pragma unroll
+        for (int i = 0; i < NS; ++i) bsbuf[slot][g][i] = bld_f32(rWs, wsoff[g], (i * KB + kc) * 4);
+      } else {
+        bsbuf[slot][g][0] = wsrow[g][kc];
+      }
+    }
 #pragma unroll
     for (int j = 0; j < TM; ++j) asbuf[slot][j] = bld_f32(rAs, asoff[j], kc * 4);
   };
@@ -160,18 +187,39 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       const int kb = kb0 + p;
       v4i d[NW][TM];
 #pragma unroll
-      for (int g = 0; g < NW; ++g)
+      for (int g = 0; g < NW; ++g) {
+        v4i wop[2]; // the two k-steps of the weight fragment as MFMA operands
+        if constexpr (W4) {
+          const v4i pk = wbuf[p][g][0];
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {
+              const uint32_t word = static_cast<uint32_t>(pk[2 * ks + w]);
+              wop[ks][2 * w] = static_cast<int>((word << 4) & 0xf0f0f0f0u);
+              wop[ks][2 * w + 1] = static_cast<int>(word & 0xf0f0f0f0u);
+            }
+        } else {
+          wop[0] = wbuf[p][g][0];
+          wop[1] = wbuf[p][g][W4 ? 0 : 1];
+        }
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
           d[g][j] = v4i{0, 0, 0, 0};
 #pragma unroll
           for (int ks = 0; ks < 2; ++ks)
-            d[g][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[p][g][ks], abuf[p][j][ks],
-                                                            d[g][j], 0, 0, 0);
-        }
-      float bs[NW], as[TM];
+            d[g][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop[ks], abuf[p][j][ks], d[g][j], 0, 0, 0);
+          if constexpr (W4) {
 #pragma unroll
-      for (int g = 0; g < NW; ++g) bs[g] = bsbuf[p][g];
+            for (int i = 0; i < 4; ++i) d[g][j][i] >>= 4; // exact: every product carries the factor 16
+          }
+        }
+      }
+      float bs[NW][NS], as[TM];
+#pragma unroll
+      for (int g = 0; g < NW; ++g)
+#pragma unroll
+        for (int i = 0; i < NS; ++i) bs[g][i] = bsbuf[p][g][i];
 #pragma unroll
       for (int j = 0; j < TM; ++j) as[j] = kb < KB ? asbuf[p][j] : 0.0f; // dead slot: adds 0
       // pin the refill of this slot here: the scheduler would otherwise sink the loads
@@ -184,15 +232,14 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
 #pragma unroll
         for (int g = 0; g < NW; ++g) {
           if constexpr (FAST_SCALE) {
-            const float sc = as[j] * bs[g];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              acc[g][j][i] = __builtin_fmaf(static_cast<float>(d[g][j][i]), sc, acc[g][j][i]);
+              acc[g][j][i] = __builtin_fmaf(static_cast<float>(d[g][j][i]), as[j] * bs[g][W4 ? i : 0], acc[g][j][i]);
           } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               float t = static_cast<float>(d[g][j][i]) * as[j];
-              t = t * bs[g];
+              t = t * bs[g][W4 ? i : 0];
               acc[g][j][i] = acc[g][j][i] + t;
             }
           }
@@ -271,7 +318,9 @@ static void launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
   GemmArgs a = a0;
   if (!FUSED_ACT) a.n_tiles = static_cast<int32_t>((a.N + 16 * NWAVES * RPW - 1) / (16 * NWAVES * RPW));
   const dim3 grid(static_cast<unsigned>(m_blocks * a.n_tiles)), block(NWAVES * 64);
-  if (a.w_shuffled)
+  if (a.w4)
+    hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, true, NWAVES, PD, RPW, true>), grid, block, 0, s, a);
+  else if (a.w_shuffled)
     hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, true, NWAVES, PD, RPW>), grid, block, 0, s, a);
   else
     hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, false, NWAVES, PD, RPW>), grid, block, 0, s, a);

@@ -8,6 +8,8 @@ from .routing import moe_align_block_size, moe_align_block_size_out, moe_fused_g
 # (moe/__init__.py:57-78)
 _NATIVE_APIS = {
     "fused_experts_impl_int8",
+    "fused_experts_impl_w4a8",
+    "preshuffle_moe_weight_int4",
     "get_w8a8moe_json",
     "invoke_fused_moe_kernel_int8",
     "invoke_fused_moe_gemm1_silu_quant",
@@ -27,6 +29,7 @@ def __getattr__(name):
 
 __all__ = [
     "fused_experts_impl_int8",
+    "fused_experts_impl_w4a8",
     "fused_experts_workspace_bytes",
     "get_moe_cache",
     "get_w8a8moe_json",
@@ -37,6 +40,7 @@ __all__ = [
     "moe_fused_gate",
     "moe_sum",
     "preshuffle_moe_weight",
+    "preshuffle_moe_weight_int4",
     "silu_and_mul",
     "topk_softmax",
 ]

@@ -54,21 +54,45 @@ def preshuffle_moe_weight(w: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def preshuffle_moe_weight_int4(w_packed: torch.Tensor) -> torch.Tensor:
+    """Packed signed int4 expert weights [E, N, K/2] (two per byte along K, even k in the high
+    nibble: the reference's order, w4a8.py:341, :375-377) in the load-time layout of the gfx950
+    kernels.  Same shape and dtype; the result carries ``lo_preshuffled = True`` and
+    ``lo_int4 = True``.  N % 16 == 0 and K % 128 == 0 are required."""
+    _require_cuda(w_packed)
+    assert w_packed.dtype in (torch.int8, torch.uint8) and w_packed.dim() == 3 and w_packed.is_contiguous()
+    E, N, K2 = w_packed.shape
+    out = torch.empty_like(w_packed)
+    with _on_device(w_packed):
+        _lib.check(_lib.lib().lo_preshuffle_weight_int4(_lib.ptr(w_packed), _lib.ptr(out), E, N, 2 * K2,
+                                                        _lib.stream_of(w_packed)))
+    out.lo_preshuffled = True
+    out.lo_int4 = True
+    return out
+
+
 def _is_preshuffled(w: torch.Tensor) -> bool:
     return bool(getattr(w, "lo_preshuffled", False))
 
 
-def _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded):
+def _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded, w4=False):
     _require_cuda(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)
-    assert A.dtype == torch.int8 and B.dtype == torch.int8, "A and B must be int8"
+    assert A.dtype == torch.int8 and B.dtype in ((torch.int8, torch.uint8) if w4 else (torch.int8,)), \
+        "A must be int8, B int8 (packed int4: int8 or uint8)"
     assert A.is_contiguous() and A_scale.is_contiguous() and A_scale.dtype == torch.float32
     assert B.is_contiguous(), "weights must be contiguous [E, N, K]"
     assert B_scale.is_contiguous() and B_scale.dtype == torch.float32
     assert sorted_token_ids.stride(0) == 1 and sorted_token_ids.dtype == torch.int32
     assert expert_ids.dtype == torch.int32 and num_tokens_post_padded.dtype == torch.int32
     E, N, K = B.shape
+    if w4:
+        K *= 2
+        assert _is_preshuffled(B), "packed int4 weights must go through preshuffle_moe_weight_int4"
+        assert B_scale.shape == (E, N, K // 128), "int4 weight scales must be [E, N, K/128]"
+    else:
+        assert B_scale.shape == (E, (N + 127) // 128, K // 128), "weight scales must be [E, N/128, K/128]"
     assert A.shape[1] == K and A_scale.shape == (A.shape[0], K // 128)
-    assert B_scale.shape == (E, (N + 127) // 128, K // 128), "weight scales must be [E, N/128, K/128]"
+    return E, N, K
 
 
 def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
@@ -80,10 +104,12 @@ def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tens
                                  flags: int = 0) -> None:
     """One grouped block-INT8 GEMM stage: C[f] = bf16(sum_kb dot(A[f // top_k], B[e])_kb *
     A_scale * B_scale) (* topk_weights[f]) for every routed slot f (reference:
-    invoke_fused_moe_kernel_int8, int8.py:543-626).  ``C`` is [M, topk, N] or [S, N]."""
+    invoke_fused_moe_kernel_int8, int8.py:543-626).  ``C`` is [M, topk, N] or [S, N].
+    With ``flags=LO_GEMM_W4`` ``B`` is packed int4 from ``preshuffle_moe_weight_int4`` and
+    ``B_scale`` is [E, N, K/128] (the stage of w4a8.py:406-478 with K-group scales)."""
     assert topk_weights is not None or not mul_routed_weight
-    _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)
-    E, N, K = B.shape
+    E, N, K = _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                                 w4=bool(flags & _lib.LO_GEMM_W4))
     assert C.is_contiguous() and C.shape[-1] == N
     num_valid = C.numel() // N
     tw = None
@@ -111,8 +137,8 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
     sequence int8.py:784-823 in one kernel.  Returns (A2q [num_valid, I] int8,
     A2s [num_valid, I/128] f32); rows of slots routed to non-local experts are not written."""
     assert topk_weights is not None or not mul_routed_weight
-    _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)
-    E, N, K = B.shape
+    E, N, K = _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                                 w4=bool(flags & _lib.LO_GEMM_W4))
     I = N // 2
     a2q = torch.empty(num_valid, I, dtype=torch.int8, device=A.device)
     a2s = torch.empty(num_valid, I // 128, dtype=torch.float32, device=A.device)
@@ -228,6 +254,98 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     assert cache13.dtype == hidden_states.dtype and cache13.is_contiguous()
     assert cache13.numel() >= M * top_k_num * max(N, H), "cache13 is too small"
 
+    flags = int(extra.get("lightop_amd_flags", 0))
+    if extra.get("lightop_amd_weights_preshuffled", False):
+        flags |= _lib.LO_GEMM_W_PRESHUFFLED
+    return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
+                              apply_router_weight_on_input, global_num_experts, expert_map, w1_scale, w2_scale,
+                              routed_scaling_factor, shared_output, I, flags,
+                              int(extra.get("lightop_amd_block_size_m", 0)))
+
+
+def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
+                            w1: torch.Tensor,
+                            w2: torch.Tensor,
+                            topk_weights: torch.Tensor,
+                            topk_ids: torch.Tensor,
+                            cache13: torch.Tensor,
+                            inplace: bool = False,
+                            activation: str = "silu",
+                            apply_router_weight_on_input: bool = False,
+                            global_num_experts: int = -1,
+                            expert_map: Optional[torch.Tensor] = None,
+                            w1_scale: Optional[torch.Tensor] = None,
+                            w2_scale: Optional[torch.Tensor] = None,
+                            w1_zp: Optional[torch.Tensor] = None,
+                            w2_zp: Optional[torch.Tensor] = None,
+                            a1_scale: Optional[torch.Tensor] = None,
+                            a2_scale: Optional[torch.Tensor] = None,
+                            block_shape: Optional[List[int]] = None,
+                            use_nn_moe: Optional[bool] = False,
+                            routed_scaling_factor: Optional[float] = 1.0,
+                            shared_output: Optional[torch.Tensor] = None, **_):
+    """Fused MoE experts with packed int4 weights and int8 activations (signature of the
+    reference's fused_experts_impl_w4a8, w4a8.py:480-501).
+
+    This build implements the K-group form: ``block_shape=[1, 128]``, ``w1`` [E, 2I, H/2] and
+    ``w2`` [E, H, I/2] packed two int4 per byte along K (even k in the high nibble, the
+    reference's order) and passed through ``preshuffle_moe_weight_int4``, one fp32 scale per
+    output row and 128-wide K group (``w1_scale`` [E, 2I, H/128], ``w2_scale`` [E, H, I/128]),
+    activations quantised per 1x128 group on the fly, SiLU.  The reference's own form (scales
+    per token and per channel in the epilogue, ``block_shape=None``, w4a8.py:395) is not
+    built and raises.  The reduce is always performed.
+    """
+    extra = _
+    assert hidden_states.shape[1] == w1.shape[2] * 2, "Hidden size mismatch"  # w4a8.py:503
+    assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.stride(-1) == 1, "Stride of last dimension must be 1"
+    assert w2.stride(-1) == 1, "Stride of last dimension must be 1"
+    assert hidden_states.dtype in [torch.float32, torch.float16, torch.bfloat16]
+    if block_shape is None or list(block_shape) != [1, 128]:
+        raise NotImplementedError("lightop_amd: W4A8 is built for K-group scales, block_shape=[1, 128]")
+    if activation != "silu":
+        if activation == "gelu":
+            raise NotImplementedError("lightop_amd: the gelu activation is not built")
+        raise ValueError(f"Unsupported FusedMoe activation: {activation}")
+    if hidden_states.dtype != torch.bfloat16:
+        raise NotImplementedError("lightop_amd: hidden_states must be bfloat16")
+    if w1_zp is not None or w2_zp is not None:
+        raise NotImplementedError("lightop_amd: W4A8 zero points are not built (symmetric int4 only)")
+    assert w1_scale is not None and w2_scale is not None
+    del a1_scale, a2_scale, use_nn_moe
+    _require_cuda(hidden_states, w1, w2, topk_weights, topk_ids, cache13, w1_scale, w2_scale, expert_map,
+                  shared_output)
+    num_tokens, H = hidden_states.shape
+    E, N = w1.shape[0], w1.shape[1]
+    I = N // 2
+    assert w2.shape == (E, H, I // 2), "w2 must be packed [E, H, I/2]"
+    assert w1.is_contiguous() and w2.is_contiguous(), "expert weights must be contiguous"
+    assert w1.dtype in (torch.int8, torch.uint8) and w2.dtype == w1.dtype
+    if not (getattr(w1, "lo_int4", False) and getattr(w2, "lo_int4", False)):
+        raise RuntimeError("lightop_amd: pass w1 and w2 through preshuffle_moe_weight_int4 once at load time")
+    assert w1_scale.shape == (E, N, H // 128) and w2_scale.shape == (E, H, I // 128)
+    if global_num_experts == -1:
+        global_num_experts = E
+    M = min(num_tokens, envs.LMSLIM_FUSED_MOE_CHUNK_SIZE)
+    assert cache13.dtype == hidden_states.dtype and cache13.is_contiguous()
+    assert cache13.numel() >= M * topk_ids.shape[1] * max(N, H), "cache13 is too small"
+    flags = int(extra.get("lightop_amd_flags", 0)) | _lib.LO_GEMM_W4
+    return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
+                              apply_router_weight_on_input, global_num_experts, expert_map, w1_scale, w2_scale,
+                              routed_scaling_factor, shared_output, I, flags,
+                              int(extra.get("lightop_amd_block_size_m", 0)))
+
+
+def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace, apply_router_weight_on_input,
+                       global_num_experts, expert_map, w1_scale, w2_scale, routed_scaling_factor, shared_output,
+                       I, flags, block_size_m):
+    """Chunk loop shared by the block-INT8 and the W4A8 entry points (int8.py:703-888)."""
+    num_tokens, H = hidden_states.shape
+    E = w1.shape[0]
+    top_k_num = topk_ids.shape[1]
+    CHUNK_SIZE = envs.LMSLIM_FUSED_MOE_CHUNK_SIZE
+    M = min(num_tokens, CHUNK_SIZE)
     out_hidden_states = hidden_states if inplace else torch.empty_like(hidden_states)
     if num_tokens == 0:
         return out_hidden_states
@@ -251,11 +369,9 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=hidden_states.device)
     ws_ptr = (workspace.data_ptr() + 255) // 256 * 256
     ws_avail = ws_bytes - (ws_ptr - workspace.data_ptr())
-    flags = int(extra.get("lightop_amd_flags", 0))
     assert _is_preshuffled(w1) == _is_preshuffled(w2), "preshuffle both w1 and w2 or neither"
-    if _is_preshuffled(w1) or extra.get("lightop_amd_weights_preshuffled", False):
+    if _is_preshuffled(w1):
         flags |= _lib.LO_GEMM_W_PRESHUFFLED
-    block_size_m = int(extra.get("lightop_amd_block_size_m", 0))
 
     with _on_device(hidden_states):
         stream = _lib.stream_of(hidden_states)
@@ -282,5 +398,6 @@ def ctypes_void(addr: int):
     return ctypes.c_void_p(addr)
 
 
-__all__ = ["fused_experts_impl_int8", "get_w8a8moe_json", "preshuffle_moe_weight", "invoke_fused_moe_kernel_int8",
+__all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "preshuffle_moe_weight",
+           "preshuffle_moe_weight_int4", "invoke_fused_moe_kernel_int8",
            "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes"]

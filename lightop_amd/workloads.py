@@ -29,10 +29,11 @@ class MoeLayer:
     n_group: int = 1
     topk_group: int = 1
     routed_scaling: float = 1.0
+    weight_bits: int = 8  # 8: block-INT8 (128x128 scales); 4: packed int4, one scale per row and 128-wide K group
 
     @property
     def weight_bytes(self) -> int:
-        return self.E * 3 * self.I * self.H
+        return self.E * 3 * self.I * self.H * self.weight_bits // 8
 
 
 TINY = MoeLayer("tiny-e8", E=8, E_global=8, top_k=2, H=1024, I=512, routing="softmax")
@@ -42,14 +43,30 @@ DSV3_EP = MoeLayer("deepseek-v3-ep8-share", E=32, E_global=256, top_k=8, H=7168,
 DSV3_FULL = MoeLayer("deepseek-v3-full", E=256, E_global=256, top_k=8, H=7168, I=2048,
                      routing="grouped_sigmoid_zipf", n_group=8, topk_group=4, routed_scaling=2.5)
 
-LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL)}
+TINY_W4 = MoeLayer("tiny-e8-w4a8", E=8, E_global=8, top_k=2, H=1024, I=512, routing="softmax", weight_bits=4)
+QWEN3_235B_W4 = MoeLayer("qwen3-235b-a22b-w4a8", E=128, E_global=128, top_k=8, H=4096, I=1536, routing="softmax",
+                         weight_bits=4)
+
+LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL, TINY_W4, QWEN3_235B_W4)}
 
 
 def make_weights(layer: MoeLayer, seed: int = 0, device="cpu", gen_device: Optional[str] = None):
-    """(w1 [E,2I,H] int8, w2 [E,H,I] int8, w1_scale [E,2I/128,H/128], w2_scale [E,H/128,I/128])."""
+    """(w1 [E,2I,H] int8, w2 [E,H,I] int8, w1_scale [E,2I/128,H/128], w2_scale [E,H/128,I/128]); for a
+    4-bit layer (w1 [E,2I,H/2], w2 [E,H,I/2] uint8: int4 uniform in [-8, 7], two per byte along K, even k
+    in the high nibble; w1_scale [E,2I,H/128], w2_scale [E,H,I/128])."""
     gen_device = gen_device or "cpu"
     g = torch.Generator(device=gen_device).manual_seed(seed)
     E, H, I = layer.E, layer.H, layer.I
+    if layer.weight_bits == 4:
+        def w4(shape):  # packed bytes: both nibbles uniform, i.e. both elements uniform in [-8, 7]
+            return torch.randint(0, 256, shape, generator=g, dtype=torch.int16, device=gen_device).to(torch.uint8)
+
+        def s4(shape):
+            return torch.exp(torch.randn(shape, generator=g, dtype=torch.float32, device=gen_device) * 0.3
+                             + math.log(1e-2))
+
+        return tuple(t.to(device) for t in (w4((E, 2 * I, H // 2)), w4((E, H, I // 2)),
+                                            s4((E, 2 * I, H // 128)), s4((E, H, I // 128))))
 
     def w(shape):
         return torch.randint(-127, 128, shape, generator=g, dtype=torch.int8, device=gen_device)
@@ -123,6 +140,9 @@ def algorithmic_work(layer: MoeLayer, topk_ids: torch.Tensor, expert_map: Option
     E_act = int(torch.unique(local).numel())
     H, I = layer.H, layer.I
     M = topk_ids.shape[0]
-    per_expert = 3 * I * H + 4 * ((2 * I // 128) * (H // 128) + (H // 128) * (I // 128))
+    if layer.weight_bits == 4:  # half a byte per weight, one scale per row and K group
+        per_expert = 3 * I * H // 2 + 4 * (2 * I * (H // 128) + H * (I // 128))
+    else:
+        per_expert = 3 * I * H + 4 * ((2 * I // 128) * (H // 128) + (H // 128) * (I // 128))
     nbytes = E_act * per_expert + 2 * M * H * 2 + M * layer.top_k * 8
     return 6 * S_loc * I * H, nbytes, S_loc, E_act

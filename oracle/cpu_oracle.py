@@ -116,15 +116,36 @@ def per_token_group_quant_int8(x, group_size=128, eps=1e-10):
     return q, s
 
 
+def unpack_int4(w4):
+    """Packed signed int4 [..., K/2] (uint8 or int8; even k in the high nibble) -> int8 [..., K]."""
+    p = w4.contiguous().view(torch.uint8)
+    out = torch.empty(p.shape[:-1] + (p.shape[-1] * 2,), dtype=torch.int8)
+    lib().orc_unpack_int4(_p(p), _i64(p.numel()), _p(out))
+    return out
+
+
+def pack_int4(w):
+    """int8 values in [-8, 7], [..., K] -> packed uint8 [..., K/2] in the reference's nibble order
+    (inverse of unpack_int4; plain torch, used to build test inputs)."""
+    u = (w.to(torch.int16) & 15).to(torch.uint8)
+    return ((u[..., 0::2] << 4) | u[..., 1::2]).contiguous()
+
+
+def moe_gemm_w4a8(A, As, W4, Ws, *args, **kwargs):
+    """Grouped GEMM with packed int4 weights [E, N, K/2] and one scale per row and K group,
+    Ws [E, N, K/128]; other arguments as moe_gemm_block_int8."""
+    return moe_gemm_block_int8(A, As, unpack_int4(W4), Ws, *args, _fn="orc_moe_gemm_rowscale_int8", **kwargs)
+
+
 def moe_gemm_block_int8(A, As, W, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_routed,
-                        top_k, num_valid, block_size, dump_acc=False, out=None):
+                        top_k, num_valid, block_size, dump_acc=False, out=None, _fn="orc_moe_gemm_block_int8"):
     """One grouped-GEMM stage.  Returns C[num_valid, N] bf16 (and the int32
     per-128-block dot products when dump_acc)."""
     E, N, K = W.shape
     C = torch.zeros(num_valid, N, dtype=torch.bfloat16) if out is None else out
     acc = torch.zeros(num_valid, N, K // 128, dtype=torch.int32) if dump_acc else None
     tw = None if topk_w is None else topk_w.reshape(-1).to(torch.float32).contiguous()
-    lib().orc_moe_gemm_block_int8(
+    getattr(lib(), _fn)(
         _p(A.contiguous()), _p(As.contiguous()), _p(W.contiguous()), _p(Ws.contiguous()),
         _p(sorted_ids), _p(expert_ids), _p(ntpp), _p(tw), ctypes.c_int(1 if mul_routed else 0),
         _i32(top_k), _i64(num_valid), _i64(N), _i64(K), _i32(block_size), _p(C), _p(acc))
@@ -182,10 +203,17 @@ def moe_fused_gate(x, bias, num_expert_group, topk_group, topk, n_share_experts_
     return w, idx
 
 
+def fused_experts_w4a8(x, w1_packed, w2_packed, w1_scale, w2_scale, *args, **kwargs):
+    """Whole path with packed int4 weights ([E, 2I, H/2], [E, H, I/2]) and K-group row scales
+    ([E, 2I, H/128], [E, H, I/128]); other arguments as fused_experts_block_int8."""
+    return fused_experts_block_int8(x, unpack_int4(w1_packed), unpack_int4(w2_packed), w1_scale, w2_scale,
+                                    *args, _fn="orc_fused_experts_w4a8", **kwargs)
+
+
 def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids, block_size_m,
                              global_num_experts=-1, expert_map=None,
                              apply_router_weight_on_input=False, routed_scaling_factor=1.0,
-                             shared_output=None, return_intermediates=False):
+                             shared_output=None, return_intermediates=False, _fn="orc_fused_experts_block_int8"):
     """Whole path; with return_intermediates a dict of every stage's output."""
     M, H = x.shape
     E, N1, _ = w1.shape
@@ -208,7 +236,7 @@ def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_i
     ids = topk_ids.to(torch.int32).contiguous()
     tw = topk_weights.to(torch.float32).contiguous()
     emap = None if expert_map is None else expert_map.to(torch.int32).contiguous()
-    rc = lib().orc_fused_experts_block_int8(
+    rc = getattr(lib(), _fn)(
         _p(x.contiguous()), _i64(M), _i64(H), _i64(I), _i32(E), _i32(Eg), _i32(k),
         _p(w1.contiguous()), _p(w1_scale.contiguous()), _p(w2.contiguous()), _p(w2_scale.contiguous()),
         _p(tw), _p(ids), _p(emap), _i32(block_size_m),

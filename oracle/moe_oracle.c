@@ -171,15 +171,16 @@ void orc_group_quant_int8(const uint16_t *x, int64_t R, int64_t C, float eps,
  * per-128-block integer dot products, so that the integer part can be checked
  * on its own.
  */
-void orc_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W,
-                             const float *Ws, const int32_t *sorted,
-                             const int32_t *expert_ids,
-                             const int32_t *num_tokens_post_pad,
-                             const float *topk_w, int mul_routed, int32_t top_k,
-                             int64_t num_valid, int64_t N, int64_t K, int32_t bs,
-                             uint16_t *C, int32_t *acc_dump) {
+/* group_n = rows of W that share a scale: 128 (block-INT8) or 1 (one scale per row and K group) */
+static void gemm_core(const int8_t *A, const float *As, const int8_t *W,
+                      const float *Ws, const int32_t *sorted,
+                      const int32_t *expert_ids,
+                      const int32_t *num_tokens_post_pad,
+                      const float *topk_w, int mul_routed, int32_t top_k,
+                      int64_t num_valid, int64_t N, int64_t K, int32_t bs,
+                      uint16_t *C, int32_t *acc_dump, int64_t group_n) {
   int64_t KB = K / ORC_GROUP;
-  int64_t NB = (N + ORC_GROUP - 1) / ORC_GROUP;
+  int64_t NB = (N + group_n - 1) / group_n;
   int64_t P = num_tokens_post_pad[0];
   int64_t nblk = P / bs;
 #pragma omp parallel for schedule(dynamic, 1) collapse(2)
@@ -207,7 +208,7 @@ void orc_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W,
             d += (int32_t)a[kb * ORC_GROUP + k] * (int32_t)wn[kb * ORC_GROUP + k];
           if (acc_dump) acc_dump[(f * N + n) * KB + kb] = d;
           float t = (float)d * as[kb];
-          t = t * ws[(n / ORC_GROUP) * KB + kb];
+          t = t * ws[(n / group_n) * KB + kb];
           acc = acc + t;
         }
         if (mul_routed) acc = acc * topk_w[f];
@@ -215,6 +216,48 @@ void orc_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W,
       }
     }
   }
+}
+
+void orc_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W,
+                             const float *Ws, const int32_t *sorted,
+                             const int32_t *expert_ids,
+                             const int32_t *num_tokens_post_pad,
+                             const float *topk_w, int mul_routed, int32_t top_k,
+                             int64_t num_valid, int64_t N, int64_t K, int32_t bs,
+                             uint16_t *C, int32_t *acc_dump) {
+  gemm_core(A, As, W, Ws, sorted, expert_ids, num_tokens_post_pad, topk_w, mul_routed, top_k,
+            num_valid, N, K, bs, C, acc_dump, ORC_GROUP);
+}
+
+/*
+ * W4A8 with K-group scales: weights are signed 4-bit integers in [-8, 7], two per byte
+ * along K, with one fp32 scale per output row and 128-wide K group: Ws [E, N, K/128].
+ * Nibble order as in the reference's W4A8 kernel: element k of a row sits in byte k/2,
+ * even k in the HIGH nibble, odd k in the LOW nibble
+ * (python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341, :375-377).  The reference
+ * itself scales per token and per channel in the epilogue only (w4a8.py:395); the K-group
+ * form restated here has no reference implementation, so its parity is unpinned beyond the
+ * arithmetic it shares with the block-INT8 path:
+ *   acc = acc + (f32(sum_k A*w) * As[row, kb]) * Ws[e, n, kb]
+ */
+void orc_unpack_int4(const uint8_t *packed, int64_t n_bytes, int8_t *out) {
+  for (int64_t i = 0; i < n_bytes; ++i) {
+    const int hi = packed[i] >> 4, lo = packed[i] & 15;
+    out[2 * i] = (int8_t)(hi >= 8 ? hi - 16 : hi);
+    out[2 * i + 1] = (int8_t)(lo >= 8 ? lo - 16 : lo);
+  }
+}
+
+/* W here is already unpacked to int8 values in [-8, 7] (orc_unpack_int4) */
+void orc_moe_gemm_rowscale_int8(const int8_t *A, const float *As, const int8_t *W,
+                                const float *Ws, const int32_t *sorted,
+                                const int32_t *expert_ids,
+                                const int32_t *num_tokens_post_pad,
+                                const float *topk_w, int mul_routed, int32_t top_k,
+                                int64_t num_valid, int64_t N, int64_t K, int32_t bs,
+                                uint16_t *C, int32_t *acc_dump) {
+  gemm_core(A, As, W, Ws, sorted, expert_ids, num_tokens_post_pad, topk_w, mul_routed, top_k,
+            num_valid, N, K, bs, C, acc_dump, 1);
 }
 
 /* ------------------------------------------------------------ SiLU*mul -- */
@@ -316,7 +359,7 @@ void orc_moe_sum(const uint16_t *in, int64_t M, int32_t k, int64_t H,
  * sorted/expert_ids/ntpp are outputs too (capacities as in
  * moe_align_block_size.py:80-93).  Returns 0 or -1.
  */
-int orc_fused_experts_block_int8(
+static int fused_path(
     const uint16_t *x, int64_t M, int64_t H, int64_t I, int32_t E_local,
     int32_t num_experts_global, int32_t top_k, const int8_t *w1, const float *w1s,
     const int8_t *w2, const float *w2s, const float *topk_w, const int32_t *topk_ids,
@@ -324,7 +367,7 @@ int orc_fused_experts_block_int8(
     float routed_scaling_factor, const uint16_t *shared_output, uint16_t *out,
     int32_t *sorted, int64_t sorted_cap, int32_t *expert_ids, int64_t expert_ids_cap,
     int32_t *ntpp, int8_t *a1q, float *a1s, uint16_t *c1, uint16_t *act, int8_t *a2q,
-    float *a2s, uint16_t *c3) {
+    float *a2s, uint16_t *c3, int64_t group_n) {
   (void)E_local;
   int64_t S = M * top_k;
   int own_a1q = !a1q, own_a1s = !a1s, own_c1 = !c1, own_act = !act, own_a2q = !a2q,
@@ -341,12 +384,12 @@ int orc_fused_experts_block_int8(
   int rc = orc_moe_align_block_size(topk_ids, S, num_experts_global, bs, expert_map, 0,
                                     sorted, sorted_cap, expert_ids, expert_ids_cap, ntpp);
   if (rc == 0) {
-    orc_moe_gemm_block_int8(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
-                            apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL);
+    gemm_core(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
+              apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL, group_n);
     orc_silu_and_mul(c1, S, I, act);
     orc_group_quant_int8(act, S, I, 1e-10f, a2q, a2s);
-    orc_moe_gemm_block_int8(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
-                            !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL);
+    gemm_core(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
+              !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL, group_n);
     orc_moe_sum(c3, M, top_k, H, shared_output, routed_scaling_factor, out);
   }
   if (own_a1q) free(a1q);
@@ -357,6 +400,38 @@ int orc_fused_experts_block_int8(
   if (own_a2s) free(a2s);
   if (own_c3) free(c3);
   return rc;
+}
+
+int orc_fused_experts_block_int8(
+    const uint16_t *x, int64_t M, int64_t H, int64_t I, int32_t E_local,
+    int32_t num_experts_global, int32_t top_k, const int8_t *w1, const float *w1s,
+    const int8_t *w2, const float *w2s, const float *topk_w, const int32_t *topk_ids,
+    const int32_t *expert_map, int32_t bs, int apply_router_weight_on_input,
+    float routed_scaling_factor, const uint16_t *shared_output, uint16_t *out,
+    int32_t *sorted, int64_t sorted_cap, int32_t *expert_ids, int64_t expert_ids_cap,
+    int32_t *ntpp, int8_t *a1q, float *a1s, uint16_t *c1, uint16_t *act, int8_t *a2q,
+    float *a2s, uint16_t *c3) {
+  return fused_path(x, M, H, I, E_local, num_experts_global, top_k, w1, w1s, w2, w2s, topk_w, topk_ids,
+                    expert_map, bs, apply_router_weight_on_input, routed_scaling_factor, shared_output,
+                    out, sorted, sorted_cap, expert_ids, expert_ids_cap, ntpp, a1q, a1s, c1, act, a2q, a2s,
+                    c3, ORC_GROUP);
+}
+
+/* The same chain with W4A8 K-group weights: w1, w2 unpacked to int8 in [-8, 7]
+ * (orc_unpack_int4), w1s [E, 2I, H/128], w2s [E, H, I/128]. */
+int orc_fused_experts_w4a8(
+    const uint16_t *x, int64_t M, int64_t H, int64_t I, int32_t E_local,
+    int32_t num_experts_global, int32_t top_k, const int8_t *w1, const float *w1s,
+    const int8_t *w2, const float *w2s, const float *topk_w, const int32_t *topk_ids,
+    const int32_t *expert_map, int32_t bs, int apply_router_weight_on_input,
+    float routed_scaling_factor, const uint16_t *shared_output, uint16_t *out,
+    int32_t *sorted, int64_t sorted_cap, int32_t *expert_ids, int64_t expert_ids_cap,
+    int32_t *ntpp, int8_t *a1q, float *a1s, uint16_t *c1, uint16_t *act, int8_t *a2q,
+    float *a2s, uint16_t *c3) {
+  return fused_path(x, M, H, I, E_local, num_experts_global, top_k, w1, w1s, w2, w2s, topk_w, topk_ids,
+                    expert_map, bs, apply_router_weight_on_input, routed_scaling_factor, shared_output,
+                    out, sorted, sorted_cap, expert_ids, expert_ids_cap, ntpp, a1q, a1s, c1, act, a2q, a2s,
+                    c3, 1);
 }
 
 /* ------------------------------------------------------------------------- *
@@ -418,7 +493,7 @@ int orc_topk_softmax(const float *gating, int64_t T, int32_t E, int32_t k, int r
     const float *x = gating + t * E;
     float mx = x[0];
     for (int32_t i = 1; i < E; ++i) if (x[i] > mx) mx = x[i];
-    float scale;
+    float scale = 0.0f;
     if (renormalize) {
       memcpy(v, x, sizeof(float) * (size_t)E);
     } else {

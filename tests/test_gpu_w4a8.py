@@ -1,0 +1,166 @@
+"""GPU parity of the W4A8 (packed int4 weights, K-group scales) path, through the C ABI, bit for
+bit against the oracle in canonical order; BASELINE's int4 configuration (Qwen3-235B-A22B-shaped
+layer, M in {1, 32, 256, 2048}) on sampled tokens."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from lightop_amd import _lib
+
+    _lib.lib()
+    return torch.device("cuda:0")
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+
+
+def gemm_case(seed, M, k, E, Eg, N, K):
+    g = torch.Generator().manual_seed(seed)
+    Aq = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    As = torch.rand(M, K // 128, generator=g) * 0.05 + 0.005
+    W4 = torch.randint(0, 256, (E, N, K // 2), generator=g, dtype=torch.int16).to(torch.uint8)
+    Ws = torch.exp(torch.randn(E, N, K // 128, generator=g) * 0.3 - 4.6)
+    ids = torch.stack([torch.randperm(Eg, generator=g)[:k] for _ in range(M)]).to(torch.int32)
+    tw = torch.rand(M, k, generator=g) + 0.1
+    emap = None
+    if Eg != E:
+        emap = torch.full((Eg,), -1, dtype=torch.int32)
+        emap[:E] = torch.arange(E, dtype=torch.int32)
+    return Aq, As, W4, Ws, ids, tw, emap
+
+
+@pytest.mark.parametrize("M,k,E,Eg,N,K", [(1, 2, 4, 4, 64, 128), (5, 2, 4, 4, 256, 512), (40, 4, 8, 8, 320, 1024),
+                                          (100, 8, 4, 16, 512, 768), (300, 2, 3, 3, 128, 2048)])
+@pytest.mark.parametrize("bs", [16, 32, 64, 128])
+def test_gemm_w4a8_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
+    from lightop_amd import _lib
+    from lightop_amd.moe import invoke_fused_moe_kernel_int8, moe_align_block_size, preshuffle_moe_weight_int4
+
+    say(f"w4a8 gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs}")
+    Aq, As, W4, Ws, ids, tw, emap = gemm_case(M + N + bs, M, k, E, Eg, N, K)
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
+    s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
+    Wd = preshuffle_moe_weight_int4(W4.to(dev))
+    for mul in (False, True):
+        ref = oracle.moe_gemm_w4a8(Aq, As, W4, Ws, rs, re, rp, tw, mul, k, M * k, bs)
+        C = torch.empty((M, k, N), dtype=torch.bfloat16, device=dev)
+        invoke_fused_moe_kernel_int8(Aq.to(dev), Wd, C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, mul, k,
+                                     {"BLOCK_SIZE_M": bs}, fused_scale=False, flags=_lib.LO_GEMM_W4)
+        torch.cuda.synchronize()
+        assert torch.equal(C.cpu().view(M * k, N).view(torch.int16), ref.view(torch.int16)), f"mul_routed={mul}"
+
+
+@pytest.mark.parametrize("M,k,E,Eg,I,K", [(1, 2, 4, 4, 128, 256), (9, 2, 4, 4, 256, 512), (50, 8, 4, 16, 256, 768),
+                                          (200, 4, 6, 6, 384, 1024)])
+@pytest.mark.parametrize("bs", [16, 32, 64, 128])
+def test_gemm1_silu_quant_w4a8_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
+    from lightop_amd import _lib
+    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_weight_int4
+
+    say(f"w4a8 gemm1+silu+quant M={M} k={k} E={E}/{Eg} I={I} K={K} bs={bs}")
+    Aq, As, W4, Ws, ids, tw, emap = gemm_case(M + I + bs + 1, M, k, E, Eg, 2 * I, K)
+    Ws = Ws * 30  # bring the gate into the range where SiLU is neither 0 nor identity
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
+    S = M * k
+    s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
+    Wd = preshuffle_moe_weight_int4(W4.to(dev))
+    for mul in (False, True):
+        c1 = oracle.moe_gemm_w4a8(Aq, As, W4, Ws, rs, re, rp, tw, mul, k, S, bs)
+        rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+        q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wd, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, mul, k,
+                                                  S, {"BLOCK_SIZE_M": bs}, fused_scale=False, flags=_lib.LO_GEMM_W4)
+        torch.cuda.synchronize()
+        local = torch.ones(S, dtype=torch.bool) if emap is None else emap.long()[ids.reshape(-1).long()] >= 0
+        assert torch.equal(sc.cpu()[local], rsc[local]) and torch.equal(q.cpu()[local], rq[local]), f"mul={mul}"
+
+
+def run_path(layer, weights_dev, x, tw, ids, emap, dev, bs, flags):
+    from lightop_amd.moe import fused_experts_impl_w4a8
+
+    w1, w2, w1s, w2s = weights_dev
+    M = x.shape[0]
+    cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
+    out = fused_experts_impl_w4a8(x, w1, w2, tw, ids, cache13, global_num_experts=layer.E_global, expert_map=emap,
+                                  w1_scale=w1s, w2_scale=w2s, block_shape=[1, 128], lightop_amd_block_size_m=bs,
+                                  lightop_amd_flags=flags)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("bs", [0, 16, 64])
+@pytest.mark.parametrize("with_map", [False, True])
+def test_whole_path_tiny_bit_exact(dev, oracle, bs, with_map):
+    from lightop_amd import _lib, workloads as wl
+    from lightop_amd.moe import preshuffle_moe_weight_int4
+
+    layer = wl.TINY_W4
+    say(f"w4a8 whole path tiny bs={bs} map={with_map}")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
+    x, tw, ids = wl.make_inputs(layer, 64, seed=4)
+    emap = None
+    if with_map:
+        emap = torch.full((layer.E,), -1, dtype=torch.int32)
+        emap[:5] = torch.arange(5, dtype=torch.int32)
+    wd = (preshuffle_moe_weight_int4(w1.to(dev)), preshuffle_moe_weight_int4(w2.to(dev)), w1s.to(dev), w2s.to(dev))
+    if with_map:  # the weight tensors hold the local experts only
+        wd = (preshuffle_moe_weight_int4(w1[:5].contiguous().to(dev)),
+              preshuffle_moe_weight_int4(w2[:5].contiguous().to(dev)), w1s[:5].contiguous().to(dev),
+              w2s[:5].contiguous().to(dev))
+    out = run_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None if emap is None else emap.to(dev), dev, bs,
+                   _lib.LO_GEMM_CANONICAL_ORDER)
+    ref = oracle.fused_experts_w4a8(x, w1[:5] if with_map else w1, w2[:5] if with_map else w2,
+                                    w1s[:5] if with_map else w1s, w2s[:5] if with_map else w2s, tw, ids, 16,
+                                    global_num_experts=layer.E, expert_map=emap)
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+def test_w4a8_rejects_what_is_not_built(dev):
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import fused_experts_impl_w4a8, preshuffle_moe_weight_int4
+
+    layer = wl.TINY_W4
+    w1, w2, w1s, w2s = (t.to(dev) for t in wl.make_weights(layer, seed=0))
+    x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, 4, seed=0))
+    cache13 = torch.empty(4 * 2 * 1024, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError):  # weights not in the load-time layout
+        fused_experts_impl_w4a8(x, w1, w2, tw, ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=[1, 128])
+    w1p, w2p = preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2)
+    with pytest.raises(NotImplementedError):  # the reference's per-channel form
+        fused_experts_impl_w4a8(x, w1p, w2p, tw, ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=None)
+
+
+@pytest.mark.parametrize("M", [1, 32, 256, 2048])
+def test_baseline_int4_layer_sampled_tokens(dev, oracle, M):
+    """Qwen3-235B-A22B-shaped layer: a token's output depends on that token only, so a sample of
+    tokens goes through the oracle with just the experts it uses."""
+    from lightop_amd import _lib, workloads as wl
+    from lightop_amd.moe import preshuffle_moe_weight_int4
+
+    layer = wl.QWEN3_235B_W4
+    say(f"w4a8 {layer.name} M={M}")
+    if not hasattr(test_baseline_int4_layer_sampled_tokens, "w"):
+        w1, w2, w1s, w2s = wl.make_weights(layer, seed=0, device=dev, gen_device="cuda")
+        test_baseline_int4_layer_sampled_tokens.w = (w1, w2, w1s, w2s, preshuffle_moe_weight_int4(w1),
+                                                     preshuffle_moe_weight_int4(w2))
+    w1, w2, w1s, w2s, w1p, w2p = test_baseline_int4_layer_sampled_tokens.w
+    x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, M, seed=3))
+    tokens = torch.randperm(M, generator=torch.Generator().manual_seed(M))[: min(M, 4)].sort().values.to(dev)
+    sub_ids = ids[tokens].cpu().long()
+    used = torch.unique(sub_ids)
+    remap = torch.full((layer.E,), -1, dtype=torch.int64)
+    remap[used] = torch.arange(used.numel())
+    sel = used.to(dev)
+    ref = oracle.fused_experts_w4a8(x[tokens].cpu(), w1[sel].cpu(), w2[sel].cpu(), w1s[sel].cpu(), w2s[sel].cpu(),
+                                    tw[tokens].cpu(), remap[sub_ids].to(torch.int32), 16)
+    out = run_path(layer, (w1p, w2p, w1s, w2s), x, tw, ids, None, dev, 0, _lib.LO_GEMM_CANONICAL_ORDER)
+    assert torch.equal(out[tokens].cpu().view(torch.int16), ref.view(torch.int16))
+    out2 = run_path(layer, (w1p, w2p, w1s, w2s), x, tw, ids, None, dev, 0, 0)  # library default order
+    err = (out2.float() - out.float()).abs()
+    assert err.max() <= 1e-2 * out.float().abs().max() and err.sum() <= 2e-3 * out.float().abs().sum()
