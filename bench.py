@@ -105,11 +105,16 @@ class Point:
         self.ops, self.bytes, self.S_loc, self.E_act = ops / n, byts / n, sloc / n, eact / n
 
     def step(self, bs=0, flags=0):
-        from lightop_amd.moe import fused_experts_impl_int8
+        from lightop_amd.moe import fused_experts_impl_int8, fused_experts_impl_w4a8
 
         x, tw, ids = self.batches[self.i % len(self.batches)]
         self.i += 1
         L = self.layer
+        if L.weight_bits == 4:
+            return fused_experts_impl_w4a8(
+                x, self.w1, self.w2, tw, ids, self.cache13, global_num_experts=L.E_global, expert_map=self.emap,
+                w1_scale=self.w1s, w2_scale=self.w2s, block_shape=[1, 128], lightop_amd_block_size_m=bs,
+                lightop_amd_flags=flags)
         return fused_experts_impl_int8(
             x, self.w1, self.w2, tw, ids, self.cache13, use_int8_w8a8=True, global_num_experts=L.E_global,
             expert_map=self.emap, w1_scale=self.w1s, w2_scale=self.w2s, block_shape=[128, 128],
@@ -121,6 +126,7 @@ class Point:
         from lightop_amd.quant import per_token_group_quant_int8
 
         L = self.layer
+        wflag = _lib_flags_w4(L)
         if bs == 0:
             bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, [128, 128], L.top_k, L.E_global)[0]["BLOCK_SIZE_M"]
         cfg = {"BLOCK_SIZE_M": bs}
@@ -139,10 +145,10 @@ class Point:
             s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
             ev[2].record()
             a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
-                                                             L.top_k, S, cfg, fused_scale=fused_scale)
+                                                             L.top_k, S, cfg, fused_scale=fused_scale, flags=wflag)
             ev[3].record()
             moe.invoke_fused_moe_kernel_int8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, True, 1, cfg,
-                                             fused_scale=fused_scale)
+                                             fused_scale=fused_scale, flags=wflag)
             ev[4].record()
             moe.moe_sum(c3, out)
             ev[5].record()
@@ -173,6 +179,12 @@ def graph_ms(pt, steps, flush, bs, flags):
     except Exception as e:  # report, do not fail the benchmark
         print(f"[graph] capture failed for M={pt.M}: {e}", file=sys.stderr, flush=True)
         return None
+
+
+def _lib_flags_w4(layer):
+    from lightop_amd import _lib
+
+    return _lib.LO_GEMM_W4 if layer.weight_bits == 4 else 0
 
 
 def measure_point(pt, steps, warmup, flush, bs, flags):
@@ -239,10 +251,11 @@ def cpu_baseline(layer, weights, M_sample, seed=0):
     w1, w2, w1s, w2s = weights
     x, tw, ids = wl.make_inputs(layer, M_sample, seed=seed)
     emap = wl.expert_map_for(layer)
+    ref = torch_ref.torch_w4a8_group_moe if layer.weight_bits == 4 else torch_ref.torch_w8a8_block_int8_moe
     runs = []
     for i in range(4):  # one warm-up, three timed
         t0 = time.perf_counter()
-        torch_ref.torch_w8a8_block_int8_moe(x, w1, w2, w1s, w2s, tw, ids, expert_map=emap)
+        ref(x, w1, w2, w1s, w2s, tw, ids, expert_map=emap)
         runs.append(time.perf_counter() - t0)
     dt = statistics.median(runs[1:])
     return {"value": round(M_sample / dt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
@@ -268,7 +281,7 @@ def main():
     flush = Flusher(dev)
     flags_default = {-1: 0, 0: _lib.LO_GEMM_CANONICAL_ORDER, 1: _lib.LO_GEMM_FUSED_SCALE}[args.fused_scale]
 
-    from lightop_amd.moe import preshuffle_moe_weight
+    from lightop_amd.moe import preshuffle_moe_scale_int4, preshuffle_moe_weight, preshuffle_moe_weight_int4
 
     cpu_weights = []
 
@@ -277,7 +290,10 @@ def main():
         w1, w2, w1s, w2s = wl.make_weights(lay, seed=0, device=dev, gen_device="cuda")
         if keep_cpu_copy:
             cpu_weights.extend(t.cpu() for t in (w1, w2, w1s, w2s))
-        if not args.row_major_weights:
+        if lay.weight_bits == 4:
+            w1, w2 = preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2)
+            w1s, w2s = preshuffle_moe_scale_int4(w1s), preshuffle_moe_scale_int4(w2s)
+        elif not args.row_major_weights:
             w1, w2 = preshuffle_moe_weight(w1), preshuffle_moe_weight(w2)
         return w1, w2, w1s, w2s
 
@@ -293,8 +309,9 @@ def main():
     g1_ops = 4.0 * pt.S_loc * L.I * L.H
     # weights and block scales of the active experts once, int8 activations and their
     # group scales in (M rows) and out (S_loc rows)
-    g1_bytes = pt.E_act * (2 * L.I * L.H + 4 * (2 * L.I // 128) * (L.H // 128)) \
-        + args.tokens * (L.H + 4 * L.H // 128) + pt.S_loc * (L.I + 4 * L.I // 128)
+    g1_w = (L.I * L.H + 4 * 2 * L.I * (L.H // 128)) if L.weight_bits == 4 \
+        else (2 * L.I * L.H + 4 * (2 * L.I // 128) * (L.H // 128))
+    g1_bytes = pt.E_act * g1_w + args.tokens * (L.H + 4 * L.H // 128) + pt.S_loc * (L.I + 4 * L.I // 128)
     g1_t = stages["gemm1_silu_quant"] * 1e-3
     if head["bound"] == "mfma":
         ach, peak, unit = g1_ops / g1_t / 1e12, INT8_PEAK_TOPS, "TFLOP/s"
@@ -303,7 +320,7 @@ def main():
     roofline = {"bound": head["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
                 "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
                 "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
-                "kernel": ("moe_gemm_tile_kernel" if bs_used >= 64 else "moe_gemm_ws_kernel")
+                "kernel": ("moe_gemm_tile_kernel" if bs_used >= 64 and L.weight_bits == 8 else "moe_gemm_ws_kernel")
                 + "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)",
                 "kernel_ms": round(stages["gemm1_silu_quant"], 4),
                 "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately)"}
@@ -311,6 +328,7 @@ def main():
     sweep = []
     if args.sweep != "none":
         plan = [(wl.QWEN3_30B, [1, 8, 32, 128, 512, 2048, 8192]), (wl.DSV3_EP, [1, 16, 64, 256, 1024, 4096])]
+        plan.append((wl.QWEN3_235B_W4, [1, 32, 256, 2048]))
         if args.sweep == "full":
             plan.append((wl.DSV3_FULL, [8192]))
         for lay, Ms in plan:
@@ -336,7 +354,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": f"{layer.name} E={L.E}/{L.E_global} top{L.top_k} H={L.H} I={L.I} "
-                               f"block-INT8[128,128], M={args.tokens}",
+                               + ("W4A8 int4[1,128]" if L.weight_bits == 4 else "block-INT8[128,128]")
+                               + f", M={args.tokens}",
                    "tokens": args.tokens, "block_size_m": bs_used, "routing": L.routing},
         "int8_tops": head["int8_tops"], "hbm_gbs": head["hbm_gbs"], "frac_hbm": head["frac_hbm"],
         "frac_mfma": head["frac_mfma"], "stage_ms": {k: round(v, 4) for k, v in stages.items()},

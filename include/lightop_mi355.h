@@ -54,9 +54,10 @@ enum {
   LO_GEMM_SKIP_NONLOCAL = 16,
   /* W4A8 with K-group scales (BASELINE's int4 variant): W (w1 and w2 for the whole path) is
    * packed signed int4 in the layout of lo_preshuffle_weight_int4 (LO_GEMM_W_PRESHUFFLED must
-   * be set too) and the weight scales are one per output row and 128-wide K group,
-   * Ws [E, N, K/128] instead of [E, N/128, K/128]:
-   *   acc = acc + (f32(sum_k A*w) * As[row, kb]) * Ws[e, n, kb],  w in [-8, 7].
+   * be set too) and the weight scales are one per output row and 128-wide K group, stored
+   * K-group-major (transposed once at load time), Ws [E, K/128, N] instead of
+   * [E, N/128, K/128]; N % 4 == 0:
+   *   acc = acc + (f32(sum_k A*w) * As[row, kb]) * Ws[e, kb, n],  w in [-8, 7].
    * The reference's W4A8 (python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:211-401)
    * scales per token and per channel in the epilogue instead; its nibble order (even k in
    * the high nibble, :341, :375-377) is the one lo_preshuffle_weight_int4 reads.  Served by

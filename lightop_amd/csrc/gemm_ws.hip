@@ -43,7 +43,8 @@ namespace lo {
 // (one 16-byte load per lane holds both k-steps of a 128-wide K block; two vector
 // instructions per 8 elements turn them into int8 values 16 times too large, which an
 // arithmetic shift of the exact int32 sum takes out again) and every weight row has its
-// own scale per K block, Ws [E, N, K/128].
+// own scale per K block, stored K-group-major, Ws [E, K/128, N], so that the four rows a
+// lane accumulates are one 16-byte load.
 template <int TM, bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int NWAVES, int PD, int RPW, bool W4 = false>
 __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs a) {
   static_assert(!W4 || SHUF, "int4 weights exist in the load-time layout only");
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       woff[g] = static_cast<int>((nrow[g] + r) * K) + c * 16;
     const int64_t nclamp = nrow[g] < N ? nrow[g] : 0; // fragments past N: loads return 0, nothing is stored
     wsrow[g] = a.Ws + (static_cast<int64_t>(e) * NB + nclamp / kGroup) * KB;
-    wsoff[g] = static_cast<int>((nclamp + 4 * c) * KB * 4); // accumulator rows of this lane: 4c .. 4c+3
+    wsoff[g] = static_cast<int>((nclamp + 4 * c) * 4); // accumulator rows of this lane: 4c .. 4c+3
   }
 
   v4f acc[NW][TM];
@@ -165,9 +166,12 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
     }
 #pragma unroll
     for (int g = 0; g < NW; ++g) {
-      if constexpr (W4) {
-#pragma unroll
-        for (int i = 0; i < NS; ++i) bsbuf[slot][g][i] = bld_f32(rWs, wsoff[g], (i * KB + kc) * 4);
+      if constexpr (W4) { // scales are stored [E][K/128][N]: the lane's four rows are 16 contiguous bytes
+        const v4f sv = __builtin_bit_cast(v4f, bld16(rWs, wsoff[g], kc * static_cast<int>(N) * 4));
+        bsbuf[slot][g][0] = sv.x;
+        bsbuf[slot][g][NS > 1 ? 1 : 0] = NS > 1 ? sv.y : sv.x;
+        bsbuf[slot][g][NS > 2 ? 2 : 0] = NS > 2 ? sv.z : sv.x;
+        bsbuf[slot][g][NS > 3 ? 3 : 0] = NS > 3 ? sv.w : sv.x;
       } else {
         bsbuf[slot][g][0] = wsrow[g][kc];
       }

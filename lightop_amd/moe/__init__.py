@@ -10,6 +10,7 @@ _NATIVE_APIS = {
     "fused_experts_impl_int8",
     "fused_experts_impl_w4a8",
     "preshuffle_moe_weight_int4",
+    "preshuffle_moe_scale_int4",
     "get_w8a8moe_json",
     "invoke_fused_moe_kernel_int8",
     "invoke_fused_moe_gemm1_silu_quant",
@@ -41,6 +42,7 @@ __all__ = [
     "moe_sum",
     "preshuffle_moe_weight",
     "preshuffle_moe_weight_int4",
+    "preshuffle_moe_scale_int4",
     "silu_and_mul",
     "topk_softmax",
 ]

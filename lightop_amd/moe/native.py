@@ -71,6 +71,16 @@ def preshuffle_moe_weight_int4(w_packed: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def preshuffle_moe_scale_int4(scale: torch.Tensor) -> torch.Tensor:
+    """K-group scales of packed int4 weights, [E, N, K/128] -> [E, K/128, N] contiguous fp32 (the four
+    rows a lane accumulates become one 16-byte load).  Once at load time; the result carries
+    ``lo_kmajor = True``."""
+    assert scale.dim() == 3
+    out = scale.to(torch.float32).transpose(1, 2).contiguous()
+    out.lo_kmajor = True
+    return out
+
+
 def _is_preshuffled(w: torch.Tensor) -> bool:
     return bool(getattr(w, "lo_preshuffled", False))
 
@@ -88,7 +98,8 @@ def _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num
     if w4:
         K *= 2
         assert _is_preshuffled(B), "packed int4 weights must go through preshuffle_moe_weight_int4"
-        assert B_scale.shape == (E, N, K // 128), "int4 weight scales must be [E, N, K/128]"
+        assert getattr(B_scale, "lo_kmajor", False) and B_scale.shape == (E, K // 128, N), \
+            "int4 weight scales must go through preshuffle_moe_scale_int4 ([E, K/128, N])"
     else:
         assert B_scale.shape == (E, (N + 127) // 128, K // 128), "weight scales must be [E, N/128, K/128]"
     assert A.shape[1] == K and A_scale.shape == (A.shape[0], K // 128)
@@ -290,7 +301,8 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     This build implements the K-group form: ``block_shape=[1, 128]``, ``w1`` [E, 2I, H/2] and
     ``w2`` [E, H, I/2] packed two int4 per byte along K (even k in the high nibble, the
     reference's order) and passed through ``preshuffle_moe_weight_int4``, one fp32 scale per
-    output row and 128-wide K group (``w1_scale`` [E, 2I, H/128], ``w2_scale`` [E, H, I/128]),
+    output row and 128-wide K group (``w1_scale`` [E, 2I, H/128], ``w2_scale`` [E, H, I/128], or
+    their load-time form from ``preshuffle_moe_scale_int4``),
     activations quantised per 1x128 group on the fly, SiLU.  The reference's own form (scales
     per token and per channel in the epilogue, ``block_shape=None``, w4a8.py:395) is not
     built and raises.  The reduce is always performed.
@@ -324,7 +336,15 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     assert w1.dtype in (torch.int8, torch.uint8) and w2.dtype == w1.dtype
     if not (getattr(w1, "lo_int4", False) and getattr(w2, "lo_int4", False)):
         raise RuntimeError("lightop_amd: pass w1 and w2 through preshuffle_moe_weight_int4 once at load time")
-    assert w1_scale.shape == (E, N, H // 128) and w2_scale.shape == (E, H, I // 128)
+    # scales: [E, N, K/128] as a checkpoint holds them (transposed here, on every call) or, better,
+    # already K-group-major from preshuffle_moe_scale_int4
+    if not getattr(w1_scale, "lo_kmajor", False):
+        assert w1_scale.shape == (E, N, H // 128), "w1_scale must be [E, 2I, H/128]"
+        w1_scale = preshuffle_moe_scale_int4(w1_scale)
+    if not getattr(w2_scale, "lo_kmajor", False):
+        assert w2_scale.shape == (E, H, I // 128), "w2_scale must be [E, H, I/128]"
+        w2_scale = preshuffle_moe_scale_int4(w2_scale)
+    assert w1_scale.shape == (E, H // 128, N) and w2_scale.shape == (E, I // 128, H)
     if global_num_experts == -1:
         global_num_experts = E
     M = min(num_tokens, envs.LMSLIM_FUSED_MOE_CHUNK_SIZE)
@@ -399,5 +419,5 @@ def ctypes_void(addr: int):
 
 
 __all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "preshuffle_moe_weight",
-           "preshuffle_moe_weight_int4", "invoke_fused_moe_kernel_int8",
+           "preshuffle_moe_weight_int4", "preshuffle_moe_scale_int4", "invoke_fused_moe_kernel_int8",
            "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes"]

@@ -44,13 +44,41 @@ def native_w8a8_block_int8_matmul(A, B, As, Bs, block_size=(128, 128), output_dt
     return C.to(output_dtype)
 
 
+def unpack_int4(wp: torch.Tensor) -> torch.Tensor:
+    """Packed signed int4 [..., K/2] (even k in the high nibble, w4a8.py:341, :375-377) -> int8 [..., K]."""
+    b = wp.view(torch.uint8).to(torch.int16)
+    hi, lo = b >> 4, b & 15
+    w = torch.stack([hi, lo], dim=-1).reshape(*wp.shape[:-1], wp.shape[-1] * 2)
+    return torch.where(w >= 8, w - 16, w).to(torch.int8)
+
+
+def native_w4a8_group_matmul(A, B, As, Bs, output_dtype=torch.bfloat16):
+    """C = sum over K-blocks of (A_blk @ B_blk^T) * As[:, kb] * Bs[:, kb]; A [M,K] int8, B [N,K] int8 holding
+    int4 values, Bs [N, K/128]: one scale per output row and K group."""
+    A = A.to(torch.float32)
+    B = B.to(torch.float32)
+    M, K = A.shape
+    C = torch.zeros(M, B.shape[0], dtype=torch.float32)
+    for kb in range(K // 128):
+        C += (A[:, kb * 128:(kb + 1) * 128] @ B[:, kb * 128:(kb + 1) * 128].t()) * As[:, kb:kb + 1] * Bs[:, kb][None, :]
+    return C.to(output_dtype)
+
+
+def torch_w4a8_group_moe(x, w1_packed, w2_packed, w1_s, w2_s, topk_weight, topk_ids, expert_map=None,
+                         routed_scaling_factor: float = 1.0):
+    """The loop of torch_w8a8_block_int8_moe with packed int4 weights and K-group row scales."""
+    return torch_w8a8_block_int8_moe(x, unpack_int4(w1_packed), unpack_int4(w2_packed), w1_s, w2_s, topk_weight,
+                                     topk_ids, expert_map, routed_scaling_factor, matmul=native_w4a8_group_matmul)
+
+
 def torch_w8a8_block_int8_moe(x, w1, w2, w1_s, w2_s, topk_weight, topk_ids, expert_map=None,
-                              routed_scaling_factor: float = 1.0):
+                              routed_scaling_factor: float = 1.0, matmul=None):
     """Per-expert loop: quant -> GEMM1 -> silu*mul -> quant -> GEMM2 -> * weight -> sum over k.
 
     ``expert_map`` (global id -> local id or -1) restricts the loop to local
     experts; slots of non-local experts contribute zero.
     """
+    matmul = matmul or native_w8a8_block_int8_matmul
     M, H = x.shape
     k = topk_ids.shape[1]
     a_q, a_s = native_per_token_group_quant_int8(x)
@@ -63,11 +91,11 @@ def torch_w8a8_block_int8_moe(x, w1, w2, w1_s, w2_s, topk_weight, topk_ids, expe
         mask = local == e
         if not bool(mask.any()):
             continue
-        inter = native_w8a8_block_int8_matmul(a_q[mask], w1[e], a_s[mask], w1_s[e], output_dtype=x.dtype)
+        inter = matmul(a_q[mask], w1[e], a_s[mask], w1_s[e], output_dtype=x.dtype)
         d = inter.shape[-1] // 2
         act = F.silu(inter[..., :d]) * inter[..., d:]
         act_q, act_s = native_per_token_group_quant_int8(act.contiguous())
-        out[mask] = native_w8a8_block_int8_matmul(act_q, w2[e], act_s, w2_s[e], output_dtype=x.dtype)
+        out[mask] = matmul(act_q, w2[e], act_s, w2_s[e], output_dtype=x.dtype)
     res = (out.view(M, k, -1) * topk_weight.view(M, k, 1).to(out.dtype)).sum(dim=1)
     if routed_scaling_factor != 1.0:
         res = res * routed_scaling_factor

@@ -41,7 +41,8 @@ def gemm_case(seed, M, k, E, Eg, N, K):
 @pytest.mark.parametrize("bs", [16, 32, 64, 128])
 def test_gemm_w4a8_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
     from lightop_amd import _lib
-    from lightop_amd.moe import invoke_fused_moe_kernel_int8, moe_align_block_size, preshuffle_moe_weight_int4
+    from lightop_amd.moe import (invoke_fused_moe_kernel_int8, moe_align_block_size, preshuffle_moe_scale_int4,
+                                 preshuffle_moe_weight_int4)
 
     say(f"w4a8 gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs}")
     Aq, As, W4, Ws, ids, tw, emap = gemm_case(M + N + bs, M, k, E, Eg, N, K)
@@ -51,7 +52,7 @@ def test_gemm_w4a8_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
     for mul in (False, True):
         ref = oracle.moe_gemm_w4a8(Aq, As, W4, Ws, rs, re, rp, tw, mul, k, M * k, bs)
         C = torch.empty((M, k, N), dtype=torch.bfloat16, device=dev)
-        invoke_fused_moe_kernel_int8(Aq.to(dev), Wd, C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, mul, k,
+        invoke_fused_moe_kernel_int8(Aq.to(dev), Wd, C, As.to(dev), preshuffle_moe_scale_int4(Ws.to(dev)), tw.to(dev), s, e, p, mul, k,
                                      {"BLOCK_SIZE_M": bs}, fused_scale=False, flags=_lib.LO_GEMM_W4)
         torch.cuda.synchronize()
         assert torch.equal(C.cpu().view(M * k, N).view(torch.int16), ref.view(torch.int16)), f"mul_routed={mul}"
@@ -62,7 +63,8 @@ def test_gemm_w4a8_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
 @pytest.mark.parametrize("bs", [16, 32, 64, 128])
 def test_gemm1_silu_quant_w4a8_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
     from lightop_amd import _lib
-    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_weight_int4
+    from lightop_amd.moe import (invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_scale_int4,
+                                 preshuffle_moe_weight_int4)
 
     say(f"w4a8 gemm1+silu+quant M={M} k={k} E={E}/{Eg} I={I} K={K} bs={bs}")
     Aq, As, W4, Ws, ids, tw, emap = gemm_case(M + I + bs + 1, M, k, E, Eg, 2 * I, K)
@@ -74,7 +76,7 @@ def test_gemm1_silu_quant_w4a8_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
     for mul in (False, True):
         c1 = oracle.moe_gemm_w4a8(Aq, As, W4, Ws, rs, re, rp, tw, mul, k, S, bs)
         rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
-        q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wd, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, mul, k,
+        q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wd, As.to(dev), preshuffle_moe_scale_int4(Ws.to(dev)), tw.to(dev), s, e, p, mul, k,
                                                   S, {"BLOCK_SIZE_M": bs}, fused_scale=False, flags=_lib.LO_GEMM_W4)
         torch.cuda.synchronize()
         local = torch.ones(S, dtype=torch.bool) if emap is None else emap.long()[ids.reshape(-1).long()] >= 0
@@ -147,9 +149,11 @@ def test_baseline_int4_layer_sampled_tokens(dev, oracle, M):
     say(f"w4a8 {layer.name} M={M}")
     if not hasattr(test_baseline_int4_layer_sampled_tokens, "w"):
         w1, w2, w1s, w2s = wl.make_weights(layer, seed=0, device=dev, gen_device="cuda")
+        from lightop_amd.moe import preshuffle_moe_scale_int4
         test_baseline_int4_layer_sampled_tokens.w = (w1, w2, w1s, w2s, preshuffle_moe_weight_int4(w1),
-                                                     preshuffle_moe_weight_int4(w2))
-    w1, w2, w1s, w2s, w1p, w2p = test_baseline_int4_layer_sampled_tokens.w
+                                                     preshuffle_moe_weight_int4(w2), preshuffle_moe_scale_int4(w1s),
+                                                     preshuffle_moe_scale_int4(w2s))
+    w1, w2, w1s, w2s, w1p, w2p, w1sp, w2sp = test_baseline_int4_layer_sampled_tokens.w
     x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, M, seed=3))
     tokens = torch.randperm(M, generator=torch.Generator().manual_seed(M))[: min(M, 4)].sort().values.to(dev)
     sub_ids = ids[tokens].cpu().long()
@@ -159,8 +163,8 @@ def test_baseline_int4_layer_sampled_tokens(dev, oracle, M):
     sel = used.to(dev)
     ref = oracle.fused_experts_w4a8(x[tokens].cpu(), w1[sel].cpu(), w2[sel].cpu(), w1s[sel].cpu(), w2s[sel].cpu(),
                                     tw[tokens].cpu(), remap[sub_ids].to(torch.int32), 16)
-    out = run_path(layer, (w1p, w2p, w1s, w2s), x, tw, ids, None, dev, 0, _lib.LO_GEMM_CANONICAL_ORDER)
+    out = run_path(layer, (w1p, w2p, w1sp, w2sp), x, tw, ids, None, dev, 0, _lib.LO_GEMM_CANONICAL_ORDER)
     assert torch.equal(out[tokens].cpu().view(torch.int16), ref.view(torch.int16))
-    out2 = run_path(layer, (w1p, w2p, w1s, w2s), x, tw, ids, None, dev, 0, 0)  # library default order
+    out2 = run_path(layer, (w1p, w2p, w1sp, w2sp), x, tw, ids, None, dev, 0, 0)  # library default order
     err = (out2.float() - out.float()).abs()
     assert err.max() <= 1e-2 * out.float().abs().max() and err.sum() <= 2e-3 * out.float().abs().sum()
