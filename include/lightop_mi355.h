@@ -293,6 +293,69 @@ int lo_fused_experts_block_int8(const void *x, int dtype, int64_t M, int64_t H, 
 int64_t lo_fused_experts_workspace_offset(int which, int64_t M, int32_t top_k, int64_t H, int64_t I,
                                           int32_t num_experts, int32_t block_size_m);
 
+/* ---- per-channel W8A8 form of the same entry point ----------------------------------
+ * fused_experts_impl_int8(per_channel_quant=True, block_shape=None): one scale per token row
+ * and one per weight row, applied once after a whole-K int32 sum.
+ */
+
+/*
+ * q [rows, cols] int8, s [rows] f32: amax = max(max|x|, 1e-10), s = amax / 127,
+ * q = round-half-even(x * (127 / amax)).  Replaces per_token_quant_int8
+ * (python/lightop/_lmslim_native/layers/gemm/int8_utils.py:20-71).  cols % 8 == 0.
+ */
+int lo_per_token_quant_int8(const void *x, int x_dtype, int64_t rows, int64_t cols, int8_t *q,
+                            float *s, lo_stream_t stream);
+
+/*
+ * c1 [rows, 2I] -> q [rows, I] int8, s [rows] f32: act = T(T(silu(gate)) * up), amax = max|act|,
+ * s = amax / 127, q = round-half-even(clamp(act * (amax == 0 ? 0 : 127 / amax))).  Replaces
+ * op.fuse_silu_mul_quant(input, output, scales, num_local_tokens_tensor, topk, ...)
+ * (python/lightop/fuse_silu_mul_quant.py:45-62;
+ * csrc/kernels/gated_activation/fuse_silu_mul_quant.cu:90-133, :135-199).
+ * num_local_tokens (device int32[1] or NULL): only the first num_local_tokens[0] * top_k rows
+ * are processed.  I % 8 == 0.
+ */
+int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, int64_t I, int8_t *q, float *s,
+                           const int32_t *num_local_tokens, int32_t top_k, lo_stream_t stream);
+
+/*
+ * One grouped-GEMM stage in the per-channel form.  Replaces
+ * op.moe_gemm_w8a8(input, b_qweight, output, a_scale, b_scale, topk_weights, sorted_token_ids,
+ * experts_ids, num_tokens_post_pad, top_k, mode, delta) (python/lightop/gemmopt.py:437-457;
+ * csrc/moe_gemm/w8a8/moe_w8a8.cu:2389-2536; epilogues :156-166 and :445-470).
+ *
+ *   As [a_rows] f32, Ws [E, N] f32 (16-byte aligned); everything else as lo_moe_gemm_block_int8.
+ *   C[f, n] = T((f32(sum_k A*W) * ts) * Ws[e, n]),  ts = As[f / top_k], or
+ *   topk_w[f] * As[f / top_k] with mul_routed;  rows of expert -1 are zero.
+ *   flags: LO_GEMM_W_PRESHUFFLED, LO_GEMM_SKIP_NONLOCAL, LO_GEMM_FORCE_STREAMING.
+ * The reference picks a kernel by `mode`/`delta` from its tuning tables; here block_size_m
+ * selects it.
+ */
+int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *W, const float *Ws, void *C,
+                     int c_dtype, const float *topk_w, const int32_t *sorted_ids,
+                     const int32_t *expert_ids, const int32_t *num_tokens_post_pad,
+                     int64_t sorted_cap, int64_t num_valid, int64_t a_rows, int32_t E, int64_t N,
+                     int64_t K, int32_t top_k, int32_t block_size_m, int mul_routed, int flags,
+                     lo_stream_t stream);
+
+/*
+ * Whole path in the per-channel form: per-token quant -> align -> GEMM1 -> SiLU*mul + per-token
+ * quant -> GEMM2 -> weighted top-k reduce (the per-channel branch of int8.py:703-888; the reduce
+ * is always performed).  Arguments as lo_fused_experts_block_int8 except:
+ *   w1s [E, 2I], w2s [E, H] f32;
+ *   cache13 [M*top_k, max(2I, H)] act dtype: holds the first GEMM's output, then the second's
+ *   (the reference shares the buffer the same way, int8.py:681-682).
+ * The workspace is the one of lo_fused_experts_workspace_bytes.
+ */
+int lo_fused_experts_channel_int8(const void *x, int dtype, int64_t M, int64_t H, int64_t I,
+                                  int32_t E, int32_t num_experts, int32_t top_k, const int8_t *w1,
+                                  const float *w1s, const int8_t *w2, const float *w2s,
+                                  const float *topk_w, const void *topk_ids, int ids_dtype,
+                                  const int32_t *expert_map, int apply_router_weight_on_input,
+                                  float routed_scaling_factor, const void *shared_output,
+                                  void *cache13, void *out, void *workspace, int64_t workspace_bytes,
+                                  int32_t block_size_m, int flags, lo_stream_t stream);
+
 /* ---- routers upstream of the path (they produce topk_ids / topk_weights) ---------- */
 
 /*

@@ -58,6 +58,16 @@ SIGNATURES = {
                                   ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
     "lo_fused_experts_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
     "lo_fused_experts_workspace_offset": (c_int64, [c_int, c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
+    "lo_per_token_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),
+    "lo_fuse_silu_mul_quant": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32,
+                                       c_void_p]),
+    "lo_moe_gemm_w8a8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                 c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32,
+                                 c_int64, c_int64, c_int32, c_int32, c_int, c_int, c_void_p]),
+    "lo_fused_experts_channel_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int32, c_int32,
+                                              c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                              c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,
+                                              c_void_p, c_void_p, c_int64, c_int32, c_int, c_void_p]),
     "lo_fused_experts_block_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int32, c_int32,
                                             c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,

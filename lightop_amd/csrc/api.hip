@@ -172,3 +172,67 @@ extern "C" int lo_fused_experts_block_int8(
   return lo_moe_sum(cache3, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor,
                     nullptr, stream);
 }
+
+// The per-channel form of the same chain (int8.py:703-888 with per_channel_quant=True,
+// block_shape=None): per-token quant -> align -> moe_gemm_w8a8 -> fuse_silu_mul_quant ->
+// moe_gemm_w8a8 (routed weight in its epilogue) -> moe_sum.  cache13 holds the first GEMM's
+// output [S, 2I] and then the second's [S, H], as in the reference (int8.py:681-682).
+extern "C" int lo_fused_experts_channel_int8(
+    const void *x, int dtype, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts,
+    int32_t top_k, const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s,
+    const float *topk_w, const void *topk_ids, int ids_dtype, const int32_t *expert_map,
+    int apply_router_weight_on_input, float routed_scaling_factor, const void *shared_output,
+    void *cache13, void *out, void *workspace, int64_t workspace_bytes, int32_t block_size_m,
+    int flags, lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(x && w1 && w1s && w2 && w2s && topk_w && topk_ids && cache13 && out && workspace,
+             LO_EINVAL, "fused_experts(channel): null pointer");
+  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "fused_experts(channel): only bf16 activations are built");
+  LO_REQUIRE(M >= 0 && H >= kGroup && H % kGroup == 0 && I >= kGroup && I % kGroup == 0, LO_EINVAL,
+             "fused_experts(channel): hidden (%lld) and intermediate (%lld) sizes must be multiples of 128",
+             (long long)H, (long long)I);
+  LO_REQUIRE(E >= 1 && num_experts >= E && top_k >= 1, LO_EINVAL, "fused_experts(channel): bad expert counts");
+  LO_REQUIRE(num_experts == E || expert_map, LO_EINVAL,
+             "fused_experts(channel): global_num_experts (%d) != local experts (%d) needs an expert_map",
+             num_experts, E);
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, LO_EINVAL,
+             "fused_experts(channel): workspace must be 256-byte aligned");
+  if (M == 0) return LO_OK;
+  if (block_size_m == 0) block_size_m = pick_block_m(M, num_experts, top_k);
+  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
+             LO_EINVAL, "fused_experts(channel): block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
+  // the block layout is roomy enough: its scale segments hold one float per 128 values
+  const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
+  LO_REQUIRE(workspace_bytes >= L.total, LO_ENOSPC,
+             "fused_experts(channel): workspace holds %lld bytes, needs %lld", (long long)workspace_bytes,
+             (long long)L.total);
+  char *ws = static_cast<char *>(workspace);
+  int8_t *a1q = reinterpret_cast<int8_t *>(ws + L.off[0]);
+  float *a1s = reinterpret_cast<float *>(ws + L.off[1]);
+  int32_t *sorted = reinterpret_cast<int32_t *>(ws + L.off[2]);
+  int32_t *eids = reinterpret_cast<int32_t *>(ws + L.off[3]);
+  int32_t *ntpp = reinterpret_cast<int32_t *>(ws + L.off[4]);
+  int8_t *a2q = reinterpret_cast<int8_t *>(ws + L.off[5]);
+  float *a2s = reinterpret_cast<float *>(ws + L.off[6]);
+  uint8_t *mask = expert_map ? reinterpret_cast<uint8_t *>(ws + L.off[7]) : nullptr;
+  const int64_t S = M * top_k;
+
+  int rc = lo_per_token_quant_int8(x, dtype, M, H, a1q, a1s, stream);
+  if (rc) return rc;
+  rc = lo_moe_align_block_size_ws(topk_ids, ids_dtype, S, num_experts, block_size_m, expert_map, 0,
+                                  sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, mask, ws + L.off[8],
+                                  L.align_scratch, stream);
+  if (rc) return rc;
+  // rows of experts on other ranks are zero-filled here: the activation kernel reads every row
+  rc = lo_moe_gemm_w8a8(a1q, a1s, w1, w1s, cache13, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, M, E,
+                        2 * I, H, top_k, block_size_m, apply_router_weight_on_input, flags, stream);
+  if (rc) return rc;
+  rc = lo_fuse_silu_mul_quant(cache13, dtype, S, I, a2q, a2s, nullptr, 1, stream);
+  if (rc) return rc;
+  rc = lo_moe_gemm_w8a8(a2q, a2s, w2, w2s, cache13, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, S, E,
+                        H, I, 1, block_size_m, !apply_router_weight_on_input,
+                        flags | (mask ? LO_GEMM_SKIP_NONLOCAL : 0), stream);
+  if (rc) return rc;
+  return lo_moe_sum(cache13, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor, nullptr,
+                    stream);
+}

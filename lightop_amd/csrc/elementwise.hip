@@ -64,6 +64,102 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
   }
 }
 
+// ---- per-token int8 quantisation, plain and behind SiLU-and-mul ----------------------
+// Reference: per_token_quant_int8, python/lightop/_lmslim_native/layers/gemm/int8_utils.py:20-44
+// (amax floored at 1e-10, s = amax / 127, q = rne(x * (127 / amax))) and fuse_silu_mul_quant,
+// csrc/kernels/gated_activation/fuse_silu_mul_quant.cu:90-133 (act = bf16(bf16(silu(g)) * u),
+// no floor: a zero row gets scale 0 and multiplier 0).  One workgroup per row; a thread keeps
+// up to CH 8-value pieces of the row in registers between the amax pass and the rounding pass,
+// longer rows are read a second time.
+__device__ __forceinline__ int rne_i8(float v) {
+  v = fminf(fmaxf(v, -128.0f), 127.0f);
+  return static_cast<int>(__builtin_rintf(v)); // v_rndne_f32: ties to even
+}
+
+template <bool SILU, int CH>
+__global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restrict__ x, int64_t rows, int64_t C,
+                                                        const uint16_t *__restrict__ silu, int8_t *__restrict__ q,
+                                                        float *__restrict__ s,
+                                                        const int32_t *__restrict__ num_local_tokens, int32_t top_k) {
+  __shared__ float sRed[4];
+  __shared__ uint16_t sSilu[SILU ? 2 * kSiluBandN : 2];
+  const int tid = threadIdx.x;
+  if (num_local_tokens) { // rows of padding tokens are left untouched
+    const int64_t n = static_cast<int64_t>(num_local_tokens[0]) * top_k;
+    rows = n < 0 ? 0 : (n < rows ? n : rows);
+  }
+  if (static_cast<int64_t>(blockIdx.x) >= rows) return;
+  if constexpr (SILU) {
+    uint16_t band_regs[kSiluBandPer];
+    silu_band_load(band_regs, silu, tid);
+    silu_band_store(sSilu, band_regs, tid);
+    __syncthreads();
+  }
+  const int64_t in_stride = SILU ? 2 * C : C; // C = output columns
+  const int pieces = static_cast<int>(C / 8);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const uint16_t *xr = x + row * in_stride;
+    auto piece = [&](int p, float (&v)[8]) {
+      const v8u16 a = *reinterpret_cast<const v8u16 *>(xr + p * 8);
+      if constexpr (SILU) {
+        const v8u16 u = *reinterpret_cast<const v8u16 *>(xr + C + p * 8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = bf16_to_f32(silu_mul_band(sSilu, silu, a[i], u[i]));
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = bf16_to_f32(a[i]);
+      }
+    };
+    float keep[CH][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int p = tid + 256 * j;
+      if (p < pieces) {
+        piece(p, keep[j]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(keep[j][i]));
+      }
+    }
+    for (int p = tid + 256 * CH; p < pieces; p += 256) {
+      float v[8];
+      piece(p, v);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    }
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+    if ((tid & 63) == 0) sRed[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(sRed[0], sRed[1]), fmaxf(sRed[2], sRed[3]));
+    __syncthreads(); // sRed is reused by the next row
+    float inv;
+    if constexpr (SILU) {
+      inv = amax == 0.0f ? 0.0f : 127.0f / amax;
+    } else {
+      amax = fmaxf(amax, 1e-10f);
+      inv = 127.0f / amax;
+    }
+    if (tid == 0) s[row] = amax / 127.0f;
+    auto emit = [&](int p, const float (&v)[8]) {
+      v2i packed;
+      packed[0] = static_cast<int>(pack4_i8(rne_i8(v[0] * inv), rne_i8(v[1] * inv), rne_i8(v[2] * inv), rne_i8(v[3] * inv)));
+      packed[1] = static_cast<int>(pack4_i8(rne_i8(v[4] * inv), rne_i8(v[5] * inv), rne_i8(v[6] * inv), rne_i8(v[7] * inv)));
+      *reinterpret_cast<v2i *>(q + row * C + p * 8) = packed;
+    };
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int p = tid + 256 * j;
+      if (p < pieces) emit(p, keep[j]);
+    }
+    for (int p = tid + 256 * CH; p < pieces; p += 256) {
+      float v[8];
+      piece(p, v);
+      emit(p, v);
+    }
+  }
+}
+
 // ---- moe_sum -------------------------------------------------------------------
 // Reference: csrc/kernels/moe_align_sum_kernels.cu:604-637 (fp32 accumulation in slot
 // order, one rounding) and :886-909 (with bias: three roundings).
@@ -231,4 +327,40 @@ extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uin
                        static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),
                        static_cast<const uint16_t *>(nullptr), expert_mask, M, topk, H, factor, num_local_tokens);
   return check_launch("moe_sum");
+}
+
+extern "C" int lo_per_token_quant_int8(const void *x, int x_dtype, int64_t rows, int64_t cols, int8_t *q,
+                                       float *s, lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(x && q && s, LO_EINVAL, "per_token_quant_int8: null pointer");
+  LO_REQUIRE(x_dtype == LO_BF16, LO_ENOTSUP, "per_token_quant_int8: only bf16 input is built");
+  LO_REQUIRE(rows >= 0 && cols > 0 && cols % 8 == 0, LO_EINVAL,
+             "per_token_quant_int8: the last dimension (%lld) must be a multiple of 8", (long long)cols);
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0,
+             LO_EINVAL, "per_token_quant_int8: x must be 16-byte and q 8-byte aligned");
+  if (rows == 0) return LO_OK;
+  const unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
+  hipLaunchKernelGGL((row_quant_kernel<false, 4>), dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t *>(x), rows, cols, static_cast<const uint16_t *>(nullptr), q, s,
+                     static_cast<const int32_t *>(nullptr), 1);
+  return check_launch("per_token_quant_int8");
+}
+
+extern "C" int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, int64_t I, int8_t *q, float *s,
+                                      const int32_t *num_local_tokens, int32_t top_k, lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(c1 && q && s, LO_EINVAL, "fuse_silu_mul_quant: null pointer");
+  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "fuse_silu_mul_quant: only bf16 input is built");
+  LO_REQUIRE(rows >= 0 && I > 0 && I % 8 == 0 && top_k >= 1, LO_EINVAL,
+             "fuse_silu_mul_quant: the output width (%lld) must be a multiple of 8, top_k >= 1", (long long)I);
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0,
+             LO_EINVAL, "fuse_silu_mul_quant: input must be 16-byte and q 8-byte aligned");
+  if (rows == 0) return LO_OK;
+  const uint16_t *table = nullptr;
+  int rc = silu_table(static_cast<hipStream_t>(stream), &table);
+  if (rc) return rc;
+  const unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
+  hipLaunchKernelGGL((row_quant_kernel<true, 2>), dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t *>(c1), rows, I, table, q, s, num_local_tokens, top_k);
+  return check_launch("fuse_silu_mul_quant");
 }

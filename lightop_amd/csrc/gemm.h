@@ -28,7 +28,8 @@ struct GemmArgs {
   int32_t mul_routed;
   int32_t w_shuffled;    // W is in the pre-shuffled layout (shuffle.hip)
   int32_t skip_nonlocal; // blocks of expert -1: leave the output rows untouched
-  int32_t w4;            // W is packed int4 (load-time layout), Ws is [E, N, K/128]
+  int32_t w4;            // W is packed int4 (load-time layout), Ws is [E, K/128, N]
+  int32_t per_channel;   // As is [a_rows], Ws is [E, N]: scales applied once, after the whole-K int32 sum
 };
 
 __device__ __forceinline__ v4i ld16(const int8_t *p) { return *reinterpret_cast<const v4i *>(p); }

@@ -42,7 +42,7 @@ static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int
                        hipStream_t s) {
   if (a.w4) return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s); // int4 weights: streaming kernels only
   if (!(flags & LO_GEMM_FORCE_STREAMING)) {
-    if (gemm_as_supports(a, fused_act, bs)) return launch_gemm_as(a, flags, m_blocks, s);
+    if (!a.per_channel && gemm_as_supports(a, fused_act, bs)) return launch_gemm_as(a, flags, m_blocks, s);
     if (gemm_tile_supports(a, fused_act, bs)) return launch_gemm_tile(a, fused_act, bs, flags, m_blocks, s);
   }
   return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
@@ -126,4 +126,43 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 31), LO_EINVAL, "moe_gemm1_silu_quant: grid too large");
   if (mblocks == 0) return LO_OK;
   return launch_gemm(a, true, block_size_m, flags, mblocks, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *W, const float *Ws,
+                                void *C, int c_dtype, const float *topk_w, const int32_t *sorted_ids,
+                                const int32_t *expert_ids, const int32_t *num_tokens_post_pad,
+                                int64_t sorted_cap, int64_t num_valid, int64_t a_rows, int32_t E,
+                                int64_t N, int64_t K, int32_t top_k, int32_t block_size_m,
+                                int mul_routed, int flags, lo_stream_t stream) {
+  using namespace lo;
+  int rc = validate_common("moe_gemm_w8a8", A, As, W, Ws, sorted_ids, expert_ids, num_tokens_post_pad, K,
+                           top_k, E, a_rows);
+  if (rc) return rc;
+  LO_REQUIRE(C, LO_EINVAL, "moe_gemm_w8a8: null output");
+  LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm_w8a8: only bf16 output is built");
+  LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm_w8a8: N (%lld) must be a multiple of 16", (long long)N);
+  LO_REQUIRE(N * K < (1ll << 31), LO_ENOTSUP, "moe_gemm_w8a8: one expert's weights exceed 2 GiB");
+  LO_REQUIRE(K <= 131072, LO_ENOTSUP, "moe_gemm_w8a8: K (%lld) could overflow the int32 sum", (long long)K);
+  LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm_w8a8: mul_routed needs topk_weights");
+  LO_REQUIRE(!(flags & LO_GEMM_W4), LO_ENOTSUP, "moe_gemm_w8a8: int4 weights are not built for the per-channel form");
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(C) & 7) == 0 && (reinterpret_cast<uintptr_t>(Ws) & 15) == 0, LO_EINVAL,
+             "moe_gemm_w8a8: C must be 8-byte and the weight scales 16-byte aligned");
+  LO_REQUIRE((num_valid + top_k - 1) / top_k <= a_rows, LO_EINVAL,
+             "moe_gemm_w8a8: %lld slots / top_k %d exceed the %lld rows of A", (long long)num_valid, top_k,
+             (long long)a_rows);
+  if (num_valid == 0) return LO_OK;
+  GemmArgs a{};
+  a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.C = static_cast<uint16_t *>(C);
+  a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
+  a.E = E; a.experts_routed = routed_experts(sorted_cap, num_valid, block_size_m, E); a.a_rows = a_rows;
+  a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
+  a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
+  a.per_channel = 1;
+  a.n_tiles = static_cast<int32_t>((N + 63) / 64);
+  const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
+  LO_REQUIRE(mblocks * a.n_tiles < (1ll << 30), LO_EINVAL, "moe_gemm_w8a8: grid too large");
+  if (mblocks == 0) return LO_OK;
+  return launch_gemm(a, false, block_size_m, flags & ~(LO_GEMM_FUSED_SCALE | LO_GEMM_CANONICAL_ORDER), mblocks,
+                     static_cast<hipStream_t>(stream));
 }

@@ -45,9 +45,16 @@ namespace lo {
 // arithmetic shift of the exact int32 sum takes out again) and every weight row has its
 // own scale per K block, stored K-group-major, Ws [E, K/128, N], so that the four rows a
 // lane accumulates are one 16-byte load.
-template <int TM, bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int NWAVES, int PD, int RPW, bool W4 = false>
+//
+// PC (per-channel W8A8, reference csrc/moe_gemm/w8a8/moe_w8a8.cu:156-166, :445-470): one scale
+// per token row, As [a_rows], and one per weight row, Ws [E, N]; the int32 sum runs over the
+// whole K inside the MFMA accumulator and the scales are applied once, in the epilogue:
+// C = bf16((f32(d) * ts) * Ws[e, n]) with ts = As[row], or topk_w[f] * As[row].
+template <int TM, bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int NWAVES, int PD, int RPW, bool W4 = false,
+          bool PC = false>
 __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs a) {
   static_assert(!W4 || SHUF, "int4 weights exist in the load-time layout only");
+  static_assert(!PC || (!W4 && !FUSED_ACT), "the per-channel form is a plain int8 GEMM");
   constexpr int BM = 16 * TM;
   constexpr int NS = W4 ? 4 : 1; // weight scales per 16-row fragment and lane
   // 16-row weight fragments per wave: (gate, up) when fused, else RPW consecutive ones
@@ -76,10 +83,10 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
     valid[j] = f[j] < a.num_valid;
     const int64_t row = valid[j] ? f[j] / a.top_k : 0;
     aoff[j] = static_cast<int>(row * K) + c * 16;
-    asoff[j] = static_cast<int>(row * KB * 4);
+    asoff[j] = static_cast<int>(row * (PC ? 1 : KB) * 4);
   }
   const brsrc rA = make_rsrc(a.A, static_cast<uint32_t>(a.a_rows * K));
-  const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * KB * 4));
+  const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * (PC ? 1 : KB) * 4));
 
   if constexpr (!FUSED_ACT) {
     const int64_t n0 = static_cast<int64_t>(nt) * (16 * NWAVES * RPW) + wave * (16 * RPW);
@@ -112,7 +119,8 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   const int NB = static_cast<int>((N + kGroup - 1) / kGroup);
   const int64_t wbytes = W4 ? N * K / 2 : N * K; // one expert
   const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * wbytes, static_cast<uint32_t>(wbytes));
-  const brsrc rWs = make_rsrc(a.Ws + static_cast<int64_t>(e) * N * KB, static_cast<uint32_t>(W4 ? N * KB * 4 : 0));
+  const brsrc rWs = PC ? make_rsrc(a.Ws + static_cast<int64_t>(e) * N, static_cast<uint32_t>(N * 4))
+                       : make_rsrc(a.Ws + static_cast<int64_t>(e) * N * KB, static_cast<uint32_t>(W4 ? N * KB * 4 : 0));
   int woff[NW];
   const float *wsrow[NW];
   int wsoff[NW]; // W4: byte offset of the lane's first scale row
@@ -131,10 +139,14 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   }
 
   v4f acc[NW][TM];
+  v4i acci[NW][TM]; // PC: the whole-K int32 sums
 #pragma unroll
   for (int g = 0; g < NW; ++g)
 #pragma unroll
-    for (int j = 0; j < TM; ++j) acc[g][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < TM; ++j) {
+      acc[g][j] = v4f{0.f, 0.f, 0.f, 0.f};
+      acci[g][j] = v4i{0, 0, 0, 0};
+    }
 
   // register ring: PD K-blocks (128 bytes of K per row each) in flight, together with
   // the scales that belong to them.  The scales travel in the same ring because the
@@ -164,6 +176,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
 #pragma unroll
       for (int j = 0; j < TM; ++j) abuf[slot][j][ks] = bld16(rA, aoff[j], kc * kGroup + ks * 64);
     }
+    if constexpr (PC) return; // no scales inside the K loop
 #pragma unroll
     for (int g = 0; g < NW; ++g) {
       if constexpr (W4) { // scales are stored [E][K/128][N]: the lane's four rows are 16 contiguous bytes
@@ -209,6 +222,14 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
         }
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
+          if constexpr (PC) {
+            // a slot past the end of K holds a copy of the last K block: feed zeros instead
+            const v4i z = v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+              acci[g][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop[ks], kb < KB ? abuf[p][j][ks] : z, acci[g][j], 0, 0, 0);
+            continue;
+          }
           d[g][j] = v4i{0, 0, 0, 0};
 #pragma unroll
           for (int ks = 0; ks < 2; ++ks)
@@ -220,17 +241,20 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
         }
       }
       float bs[NW][NS], as[TM];
+      if constexpr (!PC) {
 #pragma unroll
-      for (int g = 0; g < NW; ++g)
+        for (int g = 0; g < NW; ++g)
 #pragma unroll
-        for (int i = 0; i < NS; ++i) bs[g][i] = bsbuf[p][g][i];
+          for (int i = 0; i < NS; ++i) bs[g][i] = bsbuf[p][g][i];
 #pragma unroll
-      for (int j = 0; j < TM; ++j) as[j] = kb < KB ? asbuf[p][j] : 0.0f; // dead slot: adds 0
+        for (int j = 0; j < TM; ++j) as[j] = kb < KB ? asbuf[p][j] : 0.0f; // dead slot: adds 0
+      }
       // pin the refill of this slot here: the scheduler would otherwise sink the loads
       // next to their use (to save registers) and lose the prefetch distance
       __builtin_amdgcn_sched_barrier(0);
       issue(p, kb + PD);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PC) continue;
 #pragma unroll
       for (int j = 0; j < TM; ++j) {
 #pragma unroll
@@ -252,7 +276,28 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
     }
   }
 
-  if constexpr (!FUSED_ACT) {
+  if constexpr (PC) {
+    v4f bs4[NW];
+#pragma unroll
+    for (int g = 0; g < NW; ++g) bs4[g] = __builtin_bit_cast(v4f, bld16(rWs, wsoff[g], 0));
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      if (!valid[j]) continue;
+      float ts = bld_f32(rAs, asoff[j], 0);
+      if (a.mul_routed) ts = a.topk_w[f[j]] * ts;
+#pragma unroll
+      for (int g = 0; g < NW; ++g) {
+        if (nrow[g] >= N) continue;
+        v4u16 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float t = static_cast<float>(acci[g][j][i]) * ts;
+          o[i] = f32_to_bf16(t * bs4[g][i]);
+        }
+        *reinterpret_cast<v4u16 *>(a.C + f[j] * N + nrow[g] + 4 * c) = o;
+      }
+    }
+  } else if constexpr (!FUSED_ACT) {
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
       if (!valid[j]) continue;
@@ -322,6 +367,15 @@ static void launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
   GemmArgs a = a0;
   if (!FUSED_ACT) a.n_tiles = static_cast<int32_t>((a.N + 16 * NWAVES * RPW - 1) / (16 * NWAVES * RPW));
   const dim3 grid(static_cast<unsigned>(m_blocks * a.n_tiles)), block(NWAVES * 64);
+  if constexpr (!FUSED_ACT && !FAST_SCALE) {
+    if (a.per_channel) {
+      if (a.w_shuffled)
+        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, true, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
+      else
+        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, false, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
+      return;
+    }
+  }
   if (a.w4)
     hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, true, NWAVES, PD, RPW, true>), grid, block, 0, s, a);
   else if (a.w_shuffled)
@@ -332,7 +386,7 @@ static void launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
 
 template <bool FUSED_ACT>
 static int dispatch_ws(const GemmArgs &a, int bs, int flags, int64_t m_blocks, hipStream_t s) {
-  const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0;
+  const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 && !a.per_channel;
 #define LO_WS_CASE(TMV)                                               \
   case 16 * TMV:                                                      \
     if (fast) launch_ws<TMV, FUSED_ACT, true>(a, m_blocks, s);        \

@@ -17,6 +17,7 @@ _NATIVE_APIS = {
     "silu_and_mul",
     "fused_experts_workspace_bytes",
     "preshuffle_moe_weight",
+    "moe_gemm_w8a8",
 }
 
 
@@ -39,6 +40,7 @@ __all__ = [
     "moe_align_block_size",
     "moe_align_block_size_out",
     "moe_fused_gate",
+    "moe_gemm_w8a8",
     "moe_sum",
     "preshuffle_moe_weight",
     "preshuffle_moe_weight_int4",

@@ -169,6 +169,39 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
     return a2q, a2s
 
 
+def moe_gemm_w8a8(input: torch.Tensor, b_qweight: torch.Tensor, output: torch.Tensor, a_scale: torch.Tensor,
+                  b_scale: torch.Tensor, topk_weights: Optional[torch.Tensor], sorted_token_ids: torch.Tensor,
+                  experts_ids: torch.Tensor, num_tokens_post_pad: torch.Tensor, top_k: int,
+                  config: Dict[str, Any], flags: int = 0) -> torch.Tensor:
+    """One grouped GEMM stage in the per-channel form (reference: moe_gemm_w8a8, gemmopt.py:437-457):
+    output[f] = T((sum_k input[f // top_k] * b_qweight[e]) * ts * b_scale[e]) with
+    ts = a_scale[f // top_k], times topk_weights[f] when they are given (the second stage).
+    ``a_scale`` [rows(, 1)], ``b_scale`` [E, N(, 1)]; ``config`` needs ``BLOCK_SIZE_M`` (the reference's
+    ``MODE`` / ``DELTA`` pick among its tuned kernels and are ignored)."""
+    _require_cuda(input, b_qweight, output, a_scale, b_scale, topk_weights, sorted_token_ids, experts_ids,
+                  num_tokens_post_pad)
+    assert input.dtype == torch.int8 and b_qweight.dtype == torch.int8
+    assert input.is_contiguous() and b_qweight.is_contiguous() and output.is_contiguous()
+    E, N, K = b_qweight.shape
+    assert input.shape[1] == K and output.shape[-1] == N
+    assert a_scale.dtype == torch.float32 and a_scale.is_contiguous() and a_scale.numel() == input.shape[0]
+    assert b_scale.dtype == torch.float32 and b_scale.is_contiguous() and b_scale.numel() == E * N
+    assert sorted_token_ids.dtype == torch.int32 and experts_ids.dtype == torch.int32
+    num_valid = output.numel() // N
+    tw = None
+    if topk_weights is not None:
+        tw = topk_weights if topk_weights.dtype == torch.float32 and topk_weights.is_contiguous() \
+            else topk_weights.to(torch.float32).contiguous()
+    with _on_device(input):
+        _lib.check(_lib.lib().lo_moe_gemm_w8a8(
+            _lib.ptr(input), _lib.ptr(a_scale), _lib.ptr(b_qweight), _lib.ptr(b_scale), _lib.ptr(output),
+            _act_dtype(output), _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(experts_ids),
+            _lib.ptr(num_tokens_post_pad), sorted_token_ids.numel(), num_valid, input.shape[0], E, N, K, int(top_k),
+            int(config["BLOCK_SIZE_M"]), 1 if tw is not None else 0,
+            flags | (_lib.LO_GEMM_W_PRESHUFFLED if _is_preshuffled(b_qweight) else 0), _lib.stream_of(input)))
+    return output
+
+
 def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
     """out[:, i] = T(T(silu(x[:, i])) * x[:, d + i])  (the op called at int8.py:811)."""
     _require_cuda(out, x)
@@ -218,8 +251,10 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     """Fused MoE experts with block-quantised INT8 weights (128x128 blocks, fp32 scales) and
     activations quantised per 1x128 group on the fly.
 
-    Same signature as the reference (int8.py:628-656).  This build implements the branch
-    ``use_int8_w8a8=True, block_shape=[128, 128], activation="silu"``; every other
+    Same signature as the reference (int8.py:628-656).  This build implements the branches
+    ``use_int8_w8a8=True, block_shape=[128, 128]`` and ``use_int8_w8a8=True,
+    per_channel_quant=True, block_shape=None`` (one scale per token and per weight row,
+    ``w1_scale`` [E, 2I, 1], ``w2_scale`` [E, H, 1]) with ``activation="silu"``; every other
     combination raises.  ``cache13`` is the caller's workspace (dtype of ``hidden_states``,
     at least ``min(M, CHUNK) * topk * max(2I, H)`` elements); its first ``M*topk*H``
     elements receive the second GEMM's per-slot output.  The top-k reduction is always
@@ -235,10 +270,11 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     assert w1.stride(-1) == 1, "Stride of last dimension must be 1"
     assert w2.stride(-1) == 1, "Stride of last dimension must be 1"
     assert hidden_states.dtype in [torch.float32, torch.float16, torch.bfloat16]
-    if not use_int8_w8a8 or use_fp8_w8a8 or use_int8_w8a16 or use_int4_w4a16 or per_channel_quant:
-        raise NotImplementedError("lightop_amd: only use_int8_w8a8=True with block_shape=[128, 128] is built")
-    if block_shape is None or list(block_shape) != [128, 128]:
-        raise NotImplementedError("lightop_amd: block_shape must be [128, 128]")
+    if not use_int8_w8a8 or use_fp8_w8a8 or use_int8_w8a16 or use_int4_w4a16:
+        raise NotImplementedError("lightop_amd: only use_int8_w8a8=True is built")
+    channel = bool(per_channel_quant) and block_shape is None  # int8.py:285-295: per-token x per-channel
+    if not channel and (per_channel_quant or block_shape is None or list(block_shape) != [128, 128]):
+        raise NotImplementedError("lightop_amd: block_shape must be [128, 128], or None with per_channel_quant=True")
     if activation != "silu":
         if activation == "gelu":
             raise NotImplementedError("lightop_amd: the gelu activation is not built")
@@ -256,7 +292,11 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     assert w2.shape == (E, H, I), "w2 must be [E, H, I]"
     assert w1.is_contiguous() and w2.is_contiguous(), "expert weights must be contiguous"
     assert w1.dtype == torch.int8 and w2.dtype == torch.int8
-    assert w1_scale.shape == (E, N // 128, H // 128) and w2_scale.shape == (E, H // 128, I // 128)
+    if channel:  # one scale per weight row: [E, N, 1] as the reference's tests hold them, or [E, N]
+        assert w1_scale.numel() == E * N and w2_scale.numel() == E * H, "per-channel scales must be [E, N(, 1)]"
+        w1_scale, w2_scale = w1_scale.reshape(E, N), w2_scale.reshape(E, H)
+    else:
+        assert w1_scale.shape == (E, N // 128, H // 128) and w2_scale.shape == (E, H // 128, I // 128)
     if global_num_experts == -1:
         global_num_experts = E
     top_k_num = topk_ids.shape[1]
@@ -271,7 +311,7 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
                               apply_router_weight_on_input, global_num_experts, expert_map, w1_scale, w2_scale,
                               routed_scaling_factor, shared_output, I, flags,
-                              int(extra.get("lightop_amd_block_size_m", 0)))
+                              int(extra.get("lightop_amd_block_size_m", 0)), channel=channel)
 
 
 def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
@@ -359,8 +399,8 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
 
 def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace, apply_router_weight_on_input,
                        global_num_experts, expert_map, w1_scale, w2_scale, routed_scaling_factor, shared_output,
-                       I, flags, block_size_m):
-    """Chunk loop shared by the block-INT8 and the W4A8 entry points (int8.py:703-888)."""
+                       I, flags, block_size_m, channel=False):
+    """Chunk loop shared by the block-INT8, per-channel and W4A8 entry points (int8.py:703-888)."""
     num_tokens, H = hidden_states.shape
     E = w1.shape[0]
     top_k_num = topk_ids.shape[1]
@@ -401,7 +441,8 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
             if m <= 0:
                 break
             x = hidden_states[begin:end]
-            _lib.check(lib.lo_fused_experts_block_int8(
+            entry = lib.lo_fused_experts_channel_int8 if channel else lib.lo_fused_experts_block_int8
+            _lib.check(entry(
                 _lib.ptr(x), _act_dtype(x), m, H, I, E, global_num_experts, top_k_num,
                 _lib.ptr(w1), _lib.ptr(w1_scale), _lib.ptr(w2), _lib.ptr(w2_scale),
                 _lib.ptr(topk_weights[begin:end]), _lib.ptr(topk_ids[begin:end]), _ids_dtype(topk_ids),
@@ -420,4 +461,4 @@ def ctypes_void(addr: int):
 
 __all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "preshuffle_moe_weight",
            "preshuffle_moe_weight_int4", "preshuffle_moe_scale_int4", "invoke_fused_moe_kernel_int8",
-           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes"]
+           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes", "moe_gemm_w8a8"]

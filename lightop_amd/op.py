@@ -1,6 +1,6 @@
 """Flat native-op namespace (reference: the pybind module ``lightop.op``,
 csrc/pybind/export.cpp:1437, :1508, :1584-1605).  Only the operators of the block-INT8
-fused-MoE path and the two routers that feed it exist here.
+fused-MoE path, its per-channel form and the two routers that feed it exist here.
 """
 from __future__ import annotations
 
@@ -129,6 +129,32 @@ def moe_sum(input: torch.Tensor, output: torch.Tensor, bias: Optional[torch.Tens
         _lib.check(_lib.lib().lo_moe_sum(_lib.ptr(input), _lib.ptr(output), _lib.ptr(bias),
                                          _lib.ptr(expert_mask), _act_dtype(input), M, k, H, float(factor),
                                          _lib.ptr(num_local_tokens), _lib.stream_of(input)))
+
+
+def fuse_silu_mul_quant(input: torch.Tensor, output: torch.Tensor, scales: torch.Tensor,
+                        num_local_tokens_tensor: Optional[torch.Tensor] = None, topk: int = 1, expect_m: int = -1,
+                        expert_ids: Optional[torch.Tensor] = None) -> None:
+    """``op.fuse_silu_mul_quant`` (export.cpp:1532; fuse_silu_mul_quant.cu:90-199): SiLU(gate) * up of
+    ``input`` [rows, 2d], then one int8 scale per row: ``output`` [rows, d] int8, ``scales`` [rows(, 1)] f32.
+    With ``num_local_tokens_tensor`` (device int32[1]) only the first ``n * topk`` rows are processed."""
+    del expect_m
+    if expert_ids is not None:
+        raise NotImplementedError("lightop_amd.op.fuse_silu_mul_quant: the expert_ids variant is not built")
+    _require_cuda(input, output, scales, num_local_tokens_tensor)
+    if input.dim() != 2 or not input.is_contiguous() or input.shape[1] % 16:
+        raise RuntimeError("lightop_amd.op.fuse_silu_mul_quant: input must be a contiguous [rows, 2*d] tensor, d % 8 == 0")
+    rows, d = input.shape[0], input.shape[1] // 2
+    if output.dtype != torch.int8 or not output.is_contiguous() or output.numel() != rows * d:
+        raise RuntimeError("lightop_amd.op.fuse_silu_mul_quant: output must be a contiguous int8 [rows, d] tensor")
+    if scales.dtype != torch.float32 or not scales.is_contiguous() or scales.numel() != rows:
+        raise RuntimeError("lightop_amd.op.fuse_silu_mul_quant: scales must be a contiguous float32 [rows, 1] tensor")
+    if num_local_tokens_tensor is not None and (num_local_tokens_tensor.dtype != torch.int32
+                                                or num_local_tokens_tensor.numel() < 1):
+        raise RuntimeError("lightop_amd.op.fuse_silu_mul_quant: num_local_tokens_tensor must be int32 with one element")
+    with _on_device(input):
+        _lib.check(_lib.lib().lo_fuse_silu_mul_quant(_lib.ptr(input), _act_dtype(input), rows, d, _lib.ptr(output),
+                                                     _lib.ptr(scales), _lib.ptr(num_local_tokens_tensor), int(topk),
+                                                     _lib.stream_of(input)))
 
 
 def _float_dtype(t: torch.Tensor, what: str) -> int:

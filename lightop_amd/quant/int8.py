@@ -1,5 +1,5 @@
-"""1x128 group INT8 quantisation (reference:
-python/lightop/_lmslim_native/layers/gemm/int8_utils.py:125-195)."""
+"""INT8 activation quantisation: 1x128 groups and per token (reference:
+python/lightop/_lmslim_native/layers/gemm/int8_utils.py:125-195 and :20-71)."""
 from __future__ import annotations
 
 from typing import Tuple
@@ -38,3 +38,21 @@ def per_token_group_quant_int8(
             _lib.ptr(x), _act_dtype(x), rows, cols, float(eps), _lib.ptr(x_q), _lib.ptr(x_s),
             _lib.stream_of(x)))
     return x_q, x_s
+
+
+def per_token_quant_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One scale per row of the last dimension: ``absmax = max(|x|.max(), 1e-10); s = absmax / 127;
+    q = round_half_even(x * (127 / absmax))``.  Returns ``(x_q, scales)`` with ``scales`` of shape
+    ``x.shape[:-1] + (1,)`` in fp32 (reference: per_token_quant_int8, int8_utils.py:46-71;
+    public name lightop.quant.per_token_quant_int8, python/lightop/quant/int8.py:35)."""
+    _require_cuda(x)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    x_q = torch.empty_like(x, dtype=torch.int8)
+    scales = torch.empty(x.shape[:-1] + (1,), device=x.device, dtype=torch.float32)
+    with _on_device(x):
+        _lib.check(_lib.lib().lo_per_token_quant_int8(_lib.ptr(x), _act_dtype(x), rows, cols, _lib.ptr(x_q),
+                                                      _lib.ptr(scales), _lib.stream_of(x)))
+    return x_q, scales

@@ -30,6 +30,7 @@ class MoeLayer:
     topk_group: int = 1
     routed_scaling: float = 1.0
     weight_bits: int = 8  # 8: block-INT8 (128x128 scales); 4: packed int4, one scale per row and 128-wide K group
+    quant: str = "block"  # "channel": int8 weights with one scale per row, activations one scale per token
 
     @property
     def weight_bytes(self) -> int:
@@ -47,11 +48,19 @@ TINY_W4 = MoeLayer("tiny-e8-w4a8", E=8, E_global=8, top_k=2, H=1024, I=512, rout
 QWEN3_235B_W4 = MoeLayer("qwen3-235b-a22b-w4a8", E=128, E_global=128, top_k=8, H=4096, I=1536, routing="softmax",
                          weight_bits=4)
 
-LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL, TINY_W4, QWEN3_235B_W4)}
+TINY_PC = MoeLayer("tiny-e8-channel", E=8, E_global=8, top_k=2, H=1024, I=512, routing="softmax", quant="channel")
+QWEN3_30B_PC = MoeLayer("qwen3-30b-a3b-channel", E=128, E_global=128, top_k=8, H=2048, I=768, routing="softmax",
+                        quant="channel")
+DSV3_EP_PC = MoeLayer("deepseek-v3-ep8-share-channel", E=32, E_global=256, top_k=8, H=7168, I=2048,
+                      routing="grouped_sigmoid", n_group=8, topk_group=4, routed_scaling=2.5, quant="channel")
+
+LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL, TINY_W4, QWEN3_235B_W4, TINY_PC, QWEN3_30B_PC,
+                              DSV3_EP_PC)}
 
 
 def make_weights(layer: MoeLayer, seed: int = 0, device="cpu", gen_device: Optional[str] = None):
     """(w1 [E,2I,H] int8, w2 [E,H,I] int8, w1_scale [E,2I/128,H/128], w2_scale [E,H/128,I/128]); for a
+    per-channel layer the scales are [E,2I,1] and [E,H,1]; for a
     4-bit layer (w1 [E,2I,H/2], w2 [E,H,I/2] uint8: int4 uniform in [-8, 7], two per byte along K, even k
     in the high nibble; w1_scale [E,2I,H/128], w2_scale [E,H,I/128])."""
     gen_device = gen_device or "cpu"
@@ -77,6 +86,8 @@ def make_weights(layer: MoeLayer, seed: int = 0, device="cpu", gen_device: Optio
 
     w1 = w((E, 2 * I, H))
     w2 = w((E, H, I))
+    if layer.quant == "channel":  # one scale per weight row (the reference's shape, [E, N, 1])
+        return tuple(t.to(device) for t in (w1, w2, s((E, 2 * I, 1)), s((E, H, 1))))
     w1s = s((E, 2 * I // 128, H // 128))
     w2s = s((E, H // 128, I // 128))
     return tuple(t.to(device) for t in (w1, w2, w1s, w2s))
@@ -142,6 +153,8 @@ def algorithmic_work(layer: MoeLayer, topk_ids: torch.Tensor, expert_map: Option
     M = topk_ids.shape[0]
     if layer.weight_bits == 4:  # half a byte per weight, one scale per row and K group
         per_expert = 3 * I * H // 2 + 4 * (2 * I * (H // 128) + H * (I // 128))
+    elif layer.quant == "channel":
+        per_expert = 3 * I * H + 4 * (2 * I + H)
     else:
         per_expert = 3 * I * H + 4 * ((2 * I // 128) * (H // 128) + (H // 128) * (I // 128))
     nbytes = E_act * per_expert + 2 * M * H * 2 + M * layer.top_k * 8

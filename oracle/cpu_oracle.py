@@ -116,6 +116,43 @@ def per_token_group_quant_int8(x, group_size=128, eps=1e-10):
     return q, s
 
 
+def per_token_quant_int8(x):
+    """One scale per row, round to nearest even (int8_utils.py:20-44): q [.., C] int8, s [.., 1] f32."""
+    assert x.dtype == torch.bfloat16
+    x = x.contiguous()
+    C = x.shape[-1]
+    R = x.numel() // C
+    q = torch.empty(x.shape, dtype=torch.int8)
+    s = torch.empty(x.shape[:-1] + (1,), dtype=torch.float32)
+    lib().orc_per_token_quant_int8(_p(x), _i64(R), _i64(C), _p(q), _p(s))
+    return q, s
+
+
+def fuse_silu_mul_quant(c1, return_act=False):
+    """c1 [S, 2I] bf16 -> q [S, I] int8, s [S, 1] f32 (fuse_silu_mul_quant.cu:90-133)."""
+    S, N = c1.shape
+    q = torch.empty(S, N // 2, dtype=torch.int8)
+    s = torch.empty(S, 1, dtype=torch.float32)
+    act = torch.empty(S, N // 2, dtype=torch.bfloat16) if return_act else None
+    lib().orc_fuse_silu_mul_quant(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(q), _p(s), _p(act))
+    return (q, s, act) if return_act else (q, s)
+
+
+def moe_gemm_w8a8(A, As, W, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_routed, top_k, num_valid,
+                  block_size, dump_acc=False, out=None):
+    """Per-channel grouped GEMM: As one scale per row of A, Ws [E, N(, 1)] one per weight row.
+    Returns C [num_valid, N] bf16 (and the whole-K int32 sums when dump_acc)."""
+    E, N, K = W.shape
+    C = torch.zeros(num_valid, N, dtype=torch.bfloat16) if out is None else out
+    acc = torch.zeros(num_valid, N, dtype=torch.int32) if dump_acc else None
+    tw = None if topk_w is None else topk_w.reshape(-1).to(torch.float32).contiguous()
+    lib().orc_moe_gemm_w8a8(
+        _p(A.contiguous()), _p(As.reshape(-1).contiguous()), _p(W.contiguous()), _p(Ws.reshape(E, N).contiguous()),
+        _p(sorted_ids), _p(expert_ids), _p(ntpp), _p(tw), ctypes.c_int(1 if mul_routed else 0),
+        _i32(top_k), _i64(num_valid), _i64(N), _i64(K), _i32(block_size), _p(C), _p(acc))
+    return (C, acc) if dump_acc else C
+
+
 def unpack_int4(w4):
     """Packed signed int4 [..., K/2] (uint8 or int8; even k in the high nibble) -> int8 [..., K]."""
     p = w4.contiguous().view(torch.uint8)
@@ -210,6 +247,14 @@ def fused_experts_w4a8(x, w1_packed, w2_packed, w1_scale, w2_scale, *args, **kwa
                                     *args, _fn="orc_fused_experts_w4a8", **kwargs)
 
 
+def fused_experts_channel_int8(x, w1, w2, w1_scale, w2_scale, *args, **kwargs):
+    """Whole path in the per-channel form: w1_scale [E, 2I(, 1)], w2_scale [E, H(, 1)]; the
+    intermediates a1s and a2s hold one scale per row.  Other arguments as fused_experts_block_int8."""
+    E = w1.shape[0]
+    return fused_experts_block_int8(x, w1, w2, w1_scale.reshape(E, -1), w2_scale.reshape(E, -1), *args,
+                                    _fn="orc_fused_experts_channel_int8", **kwargs)
+
+
 def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids, block_size_m,
                              global_num_experts=-1, expert_map=None,
                              apply_router_weight_on_input=False, routed_scaling_factor=1.0,
@@ -248,6 +293,9 @@ def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_i
     if rc != 0:
         raise RuntimeError("oracle fused_experts: alignment failed")
     if return_intermediates:
+        if _fn == "orc_fused_experts_channel_int8":  # one scale per row, written densely at the front
+            inter["a1s"] = inter["a1s"].reshape(-1)[:M].reshape(M, 1).clone()
+            inter["a2s"] = inter["a2s"].reshape(-1)[:S].reshape(S, 1).clone()
         inter.update(sorted_ids=sorted_ids, expert_ids=expert_ids, num_tokens_post_pad=ntpp, out=out)
         return inter
     return out

@@ -435,6 +435,155 @@ int orc_fused_experts_w4a8(
 }
 
 /* ------------------------------------------------------------------------- *
+ * Per-channel W8A8 form of the same entry point (per_channel_quant=True,
+ * block_shape=None): one scale per token row and one per weight row, applied
+ * once after an exact whole-K int32 sum.
+ *
+ * Reference:
+ *   per-token quant   python/lightop/_lmslim_native/layers/gemm/int8_utils.py:20-44
+ *   grouped GEMM      csrc/moe_gemm/w8a8/moe_w8a8.cu:156-166 (first stage),
+ *                     :445-470 (second stage, routed weight folded into the token scale);
+ *                     call sites int8.py:771-781, :845-855; wrapper gemmopt.py:437-457
+ *   SiLU*mul + quant  csrc/kernels/gated_activation/fuse_silu_mul_quant.cu:90-133
+ *                     (round to nearest even, :19-35); call site int8.py:811-813
+ *
+ * Canonical choices: bf16(silu(g)) is the correctly rounded table used for the
+ * block path (the reference kernel forms it from the hardware's approximate
+ * exp2 and reciprocal, fuse_silu_mul_quant.cu:52-66; where the two differ in the
+ * last bf16 ulp is unpinned); nearbyint is round-half-even.
+ * ------------------------------------------------------------------------- */
+
+static inline int8_t rne_int8(float v) {
+  /* the reference's clamp, fuse_silu_mul_quant.cu:19-35: fminf(127, fmaxf(-128, x)), so a NaN
+   * (0 * inf in a row of denormals, whose multiplier overflows) becomes -128 */
+  v = fminf(127.0f, fmaxf(-128.0f, v));
+  return (int8_t)(int32_t)nearbyintf(v); /* default rounding mode: half to even */
+}
+
+/* x[R, C] bf16 -> q[R, C] int8, s[R] f32:
+ *   absmax = max(max|x|, 1e-10);  s = absmax / 127;  q = rne(x * (127 / absmax)) */
+void orc_per_token_quant_int8(const uint16_t *x, int64_t R, int64_t C, int8_t *q, float *s) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < R; ++r) {
+    const uint16_t *xr = x + r * C;
+    float amax = 0.0f;
+    for (int64_t i = 0; i < C; ++i) {
+      float a = fabsf(bf16_to_f32(xr[i]));
+      if (a > amax) amax = a;
+    }
+    if (!(amax > 1e-10f)) amax = 1e-10f;
+    s[r] = amax / 127.0f;
+    const float inv = 127.0f / amax;
+    for (int64_t i = 0; i < C; ++i) q[r * C + i] = rne_int8(bf16_to_f32(xr[i]) * inv);
+  }
+}
+
+/* c1[S, 2I] bf16 -> q[S, I] int8, s[S] f32 (fuse_silu_mul_quant.cu:90-133):
+ *   act = bf16(f32(bf16(silu(g))) * u);  amax = max|act|;  s = amax / 127;
+ *   q = rne(clamp(act * (amax == 0 ? 0 : 127 / amax)))
+ * act (optional) receives the bf16 products. */
+void orc_fuse_silu_mul_quant(const uint16_t *c1, int64_t S, int64_t I, int8_t *q, float *s,
+                             uint16_t *act) {
+#pragma omp parallel for schedule(static)
+  for (int64_t f = 0; f < S; ++f) {
+    float amax = 0.0f;
+    for (int64_t i = 0; i < I; ++i) {
+      float v = fabsf(bf16_to_f32(silu_mul_one(c1[f * 2 * I + i], c1[f * 2 * I + I + i])));
+      if (v > amax) amax = v;
+    }
+    s[f] = amax / 127.0f;
+    const float inv = (amax == 0.0f) ? 0.0f : 127.0f / amax;
+    for (int64_t i = 0; i < I; ++i) {
+      const uint16_t a16 = silu_mul_one(c1[f * 2 * I + i], c1[f * 2 * I + I + i]);
+      if (act) act[f * I + i] = a16;
+      q[f * I + i] = rne_int8(bf16_to_f32(a16) * inv);
+    }
+  }
+}
+
+/*
+ *   A [*, K] int8, row of slot f is f / top_k;  As [*] f32 (one per row)
+ *   W [E, N, K] int8;                           Ws [E, N] f32 (one per weight row)
+ *   d = sum_k A*W over the whole K (int32, exact)
+ *   C[f, n] = bf16((f32(d) * ts) * Ws[e, n]),  ts = As[row], or topk_w[f] * As[row] with mul_routed
+ *   e == -1 -> C[f, :] = 0 (moe_w8a8.cu:96-118)
+ * acc_dump (optional, [num_valid, N] int32) receives d.
+ */
+void orc_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *W, const float *Ws,
+                       const int32_t *sorted, const int32_t *expert_ids,
+                       const int32_t *num_tokens_post_pad, const float *topk_w, int mul_routed,
+                       int32_t top_k, int64_t num_valid, int64_t N, int64_t K, int32_t bs,
+                       uint16_t *C, int32_t *acc_dump) {
+  int64_t P = num_tokens_post_pad[0];
+  int64_t nblk = P / bs;
+#pragma omp parallel for schedule(dynamic, 1) collapse(2)
+  for (int64_t b = 0; b < nblk; ++b) {
+    for (int32_t i = 0; i < bs; ++i) {
+      int64_t f = sorted[b * bs + i];
+      if (f >= num_valid) continue;
+      int32_t e = expert_ids[b];
+      uint16_t *c = C + f * N;
+      if (e < 0) {
+        for (int64_t n = 0; n < N; ++n) c[n] = 0;
+        continue;
+      }
+      int64_t row = f / top_k;
+      const int8_t *a = A + row * K;
+      float ts = As[row];
+      if (mul_routed) ts = topk_w[f] * ts;
+      for (int64_t n = 0; n < N; ++n) {
+        const int8_t *wn = W + ((int64_t)e * N + n) * K;
+        int32_t d = 0;
+        for (int64_t k = 0; k < K; ++k) d += (int32_t)a[k] * (int32_t)wn[k];
+        if (acc_dump) acc_dump[f * N + n] = d;
+        float t = (float)d * ts;
+        c[n] = f32_to_bf16(t * Ws[(int64_t)e * N + n]);
+      }
+    }
+  }
+}
+
+/* The chain of int8.py:703-888 on its per-channel branch, with the final reduce always
+ * performed: a1q[M,H] a1s[M]  c1[S,2I]  act[S,I]  a2q[S,I] a2s[S]  c3[S,H]. */
+int orc_fused_experts_channel_int8(
+    const uint16_t *x, int64_t M, int64_t H, int64_t I, int32_t E_local,
+    int32_t num_experts_global, int32_t top_k, const int8_t *w1, const float *w1s,
+    const int8_t *w2, const float *w2s, const float *topk_w, const int32_t *topk_ids,
+    const int32_t *expert_map, int32_t bs, int apply_router_weight_on_input,
+    float routed_scaling_factor, const uint16_t *shared_output, uint16_t *out,
+    int32_t *sorted, int64_t sorted_cap, int32_t *expert_ids, int64_t expert_ids_cap,
+    int32_t *ntpp, int8_t *a1q, float *a1s, uint16_t *c1, uint16_t *act, int8_t *a2q,
+    float *a2s, uint16_t *c3) {
+  (void)E_local;
+  int64_t S = M * top_k;
+  int own_a1q = !a1q, own_a1s = !a1s, own_c1 = !c1, own_a2q = !a2q, own_a2s = !a2s, own_c3 = !c3;
+  if (own_a1q) a1q = (int8_t *)malloc((size_t)(M * H));
+  if (own_a1s) a1s = (float *)malloc(sizeof(float) * (size_t)M);
+  if (own_c1) c1 = (uint16_t *)calloc((size_t)(S * 2 * I), 2);
+  if (own_a2q) a2q = (int8_t *)malloc((size_t)(S * I));
+  if (own_a2s) a2s = (float *)malloc(sizeof(float) * (size_t)S);
+  if (own_c3) c3 = (uint16_t *)calloc((size_t)(S * H), 2);
+  orc_per_token_quant_int8(x, M, H, a1q, a1s);
+  int rc = orc_moe_align_block_size(topk_ids, S, num_experts_global, bs, expert_map, 0,
+                                    sorted, sorted_cap, expert_ids, expert_ids_cap, ntpp);
+  if (rc == 0) {
+    orc_moe_gemm_w8a8(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
+                      apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL);
+    orc_fuse_silu_mul_quant(c1, S, I, a2q, a2s, act);
+    orc_moe_gemm_w8a8(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
+                      !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL);
+    orc_moe_sum(c3, M, top_k, H, shared_output, routed_scaling_factor, out);
+  }
+  if (own_a1q) free(a1q);
+  if (own_a1s) free(a1s);
+  if (own_c1) free(c1);
+  if (own_a2q) free(a2q);
+  if (own_a2s) free(a2s);
+  if (own_c3) free(c3);
+  return rc;
+}
+
+/* ------------------------------------------------------------------------- *
  * Routers upstream of the path (they produce topk_ids / topk_weights).
  *
  * Reference: csrc/kernels/softmax/topk_softmax_kernels.cu:1381-1582 (generic

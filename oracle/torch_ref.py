@@ -71,6 +71,51 @@ def torch_w4a8_group_moe(x, w1_packed, w2_packed, w1_s, w2_s, topk_weight, topk_
                                      topk_ids, expert_map, routed_scaling_factor, matmul=native_w4a8_group_matmul)
 
 
+def native_per_token_quant_int8(x: torch.Tensor):
+    """One scale per row, round half to even: s = absmax / 127, q = round(x * (127 / absmax))
+    (the torch form of int8_utils.py:20-44; vLLM's dynamic scaled_int8_quant, which the reference's
+    test of fuse_silu_mul_quant compares with, test/test_fuse_silu_mul_quant.py:11-14, is the same rule)."""
+    xf = x.to(torch.float32)
+    absmax = xf.abs().amax(dim=-1, keepdim=True).clamp(min=1e-10)
+    # torch evaluates `127.0 / t` as reciprocal-times-127; the rule is a true division
+    q = torch.round(xf * (torch.full_like(absmax, 127.0) / absmax)).clamp(min=-128, max=127).to(torch.int8)
+    return q, absmax / 127.0
+
+
+def native_w8a8_per_token_matmul(A, B, As, Bs, output_dtype=torch.bfloat16):
+    """C = As * (A @ B^T) * Bs: per-token scale As [M, 1], per-row weight scale Bs [N(, 1)]
+    (test/moe_w8a8/fuse_moegemm_correctness.py:825-844)."""
+    C = torch.matmul(A.to(torch.float32), B.to(torch.float32).t())  # exact below 2^24, else ~1e-7 relative
+    return (As * C * Bs.reshape(1, -1)).to(output_dtype)
+
+
+def torch_w8a8_per_column_moe(x, w1, w2, w1_s, w2_s, topk_weight, topk_ids, expert_map=None,
+                              routed_scaling_factor: float = 1.0):
+    """The per-expert loop of test/moe_w8a8/fuse_moegemm_correctness.py:847-885 (per-token activation
+    scales, per-row weight scales), with the optional ``expert_map`` of the block version."""
+    M, H = x.shape
+    k = topk_ids.shape[1]
+    a_q, a_s = native_per_token_quant_int8(x)
+    a_q = a_q.view(M, 1, H).repeat(1, k, 1).reshape(-1, H)
+    a_s = a_s.view(M, 1, 1).repeat(1, k, 1).reshape(-1, 1)
+    out = torch.zeros(M * k, w2.shape[1], dtype=x.dtype)
+    flat_ids = topk_ids.reshape(-1).long()
+    local = flat_ids if expert_map is None else expert_map.long()[flat_ids]
+    for e in range(w1.shape[0]):
+        mask = local == e
+        if not bool(mask.any()):
+            continue
+        inter = native_w8a8_per_token_matmul(a_q[mask], w1[e], a_s[mask], w1_s[e], output_dtype=x.dtype)
+        d = inter.shape[-1] // 2
+        act = F.silu(inter[..., :d]) * inter[..., d:]
+        act_q, act_s = native_per_token_quant_int8(act)
+        out[mask] = native_w8a8_per_token_matmul(act_q, w2[e], act_s, w2_s[e], output_dtype=x.dtype)
+    res = (out.view(M, k, -1) * topk_weight.view(M, k, 1).to(out.dtype)).sum(dim=1)
+    if routed_scaling_factor != 1.0:
+        res = res * routed_scaling_factor
+    return res
+
+
 def torch_w8a8_block_int8_moe(x, w1, w2, w1_s, w2_s, topk_weight, topk_ids, expert_map=None,
                               routed_scaling_factor: float = 1.0, matmul=None):
     """Per-expert loop: quant -> GEMM1 -> silu*mul -> quant -> GEMM2 -> * weight -> sum over k.
