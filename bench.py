@@ -115,6 +115,11 @@ class Point:
                 x, self.w1, self.w2, tw, ids, self.cache13, global_num_experts=L.E_global, expert_map=self.emap,
                 w1_scale=self.w1s, w2_scale=self.w2s, block_shape=[1, 128], lightop_amd_block_size_m=bs,
                 lightop_amd_flags=flags)
+        if L.quant == "channel":
+            return fused_experts_impl_int8(
+                x, self.w1, self.w2, tw, ids, self.cache13, use_int8_w8a8=True, per_channel_quant=True,
+                global_num_experts=L.E_global, expert_map=self.emap, w1_scale=self.w1s, w2_scale=self.w2s,
+                block_shape=None, lightop_amd_block_size_m=bs)
         return fused_experts_impl_int8(
             x, self.w1, self.w2, tw, ids, self.cache13, use_int8_w8a8=True, global_num_experts=L.E_global,
             expert_map=self.emap, w1_scale=self.w1s, w2_scale=self.w2s, block_shape=[128, 128],
@@ -128,11 +133,14 @@ class Point:
         L = self.layer
         wflag = _lib_flags_w4(L)
         if bs == 0:
-            bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, [128, 128], L.top_k, L.E_global)[0]["BLOCK_SIZE_M"]
+            bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, None if L.quant == "channel" else [128, 128],
+                                      L.top_k, L.E_global)[0]["BLOCK_SIZE_M"]
         cfg = {"BLOCK_SIZE_M": bs}
         S = self.M * L.top_k
         c3 = self.cache13[: S * L.H].view(self.M, L.top_k, L.H)
         out = torch.empty(self.M, L.H, dtype=torch.bfloat16, device=self.dev)
+        if L.quant == "channel":
+            return self.stage_times_channel(steps, warmup, flush, bs), bs
         names = ["quant", "align", "gemm1_silu_quant", "gemm2", "moe_sum"]
         acc = {n: [] for n in names}
         for it in range(warmup + steps):
@@ -157,6 +165,46 @@ class Point:
                 for i, n in enumerate(names):
                     acc[n].append(ev[i].elapsed_time(ev[i + 1]))
         return {n: sum(v) / len(v) for n, v in acc.items()}, bs
+
+
+def _stage_times_channel(self, steps, warmup, flush, bs):
+    """The six launches of the per-channel path, each on its own (ms, mean)."""
+    from lightop_amd import fuse_silu_mul_quant, moe
+    from lightop_amd.quant import per_token_quant_int8
+
+    L = self.layer
+    cfg = {"BLOCK_SIZE_M": bs}
+    S = self.M * L.top_k
+    c1 = self.cache13[: S * 2 * L.I].view(S, 2 * L.I)
+    c3 = self.cache13[: S * L.H].view(self.M, L.top_k, L.H)
+    out = torch.empty(self.M, L.H, dtype=torch.bfloat16, device=self.dev)
+    names = ["quant", "align", "gemm1", "silu_mul_quant", "gemm2", "moe_sum"]
+    acc = {n: [] for n in names}
+    for it in range(warmup + steps):
+        x, tw, ids = self.batches[it % len(self.batches)]
+        flush()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(7)]
+        ev[0].record()
+        a1q, a1s = per_token_quant_int8(x)
+        ev[1].record()
+        s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
+        ev[2].record()
+        moe.moe_gemm_w8a8(a1q, self.w1, c1, a1s, self.w1s, None, s, e, p, L.top_k, cfg)
+        ev[3].record()
+        a2q, a2s = fuse_silu_mul_quant(c1)
+        ev[4].record()
+        moe.moe_gemm_w8a8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, 1, cfg)
+        ev[5].record()
+        moe.moe_sum(c3, out)
+        ev[6].record()
+        if it >= warmup:
+            torch.cuda.synchronize()
+            for i, n in enumerate(names):
+                acc[n].append(ev[i].elapsed_time(ev[i + 1]))
+    return {n: sum(v) / len(v) for n, v in acc.items()}
+
+
+Point.stage_times_channel = _stage_times_channel
 
 
 def graph_ms(pt, steps, flush, bs, flags):
@@ -251,7 +299,8 @@ def cpu_baseline(layer, weights, M_sample, seed=0):
     w1, w2, w1s, w2s = weights
     x, tw, ids = wl.make_inputs(layer, M_sample, seed=seed)
     emap = wl.expert_map_for(layer)
-    ref = torch_ref.torch_w4a8_group_moe if layer.weight_bits == 4 else torch_ref.torch_w8a8_block_int8_moe
+    ref = torch_ref.torch_w4a8_group_moe if layer.weight_bits == 4 else (
+        torch_ref.torch_w8a8_per_column_moe if layer.quant == "channel" else torch_ref.torch_w8a8_block_int8_moe)
     runs = []
     for i in range(4):  # one warm-up, three timed
         t0 = time.perf_counter()
@@ -312,7 +361,11 @@ def main():
     g1_w = (L.I * L.H + 4 * 2 * L.I * (L.H // 128)) if L.weight_bits == 4 \
         else (2 * L.I * L.H + 4 * (2 * L.I // 128) * (L.H // 128))
     g1_bytes = pt.E_act * g1_w + args.tokens * (L.H + 4 * L.H // 128) + pt.S_loc * (L.I + 4 * L.I // 128)
-    g1_t = stages["gemm1_silu_quant"] * 1e-3
+    if L.quant == "channel":  # whole-row scales; bf16 [S, 2I] out instead of int8 [S, I]
+        g1_w = 2 * L.I * L.H + 4 * 2 * L.I
+        g1_bytes = pt.E_act * g1_w + args.tokens * (L.H + 4) + pt.S_loc * 2 * L.I * 2
+    g1_name = "gemm1" if L.quant == "channel" else "gemm1_silu_quant"
+    g1_t = stages[g1_name] * 1e-3
     if head["bound"] == "mfma":
         ach, peak, unit = g1_ops / g1_t / 1e12, INT8_PEAK_TOPS, "TFLOP/s"
     else:
@@ -321,14 +374,17 @@ def main():
                 "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
                 "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
                 "kernel": ("moe_gemm_tile_kernel" if bs_used >= 64 and L.weight_bits == 8 else "moe_gemm_ws_kernel")
-                + "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)",
-                "kernel_ms": round(stages["gemm1_silu_quant"], 4),
+                + ("<PC> (GEMM1, per-channel scales in the epilogue)" if L.quant == "channel"
+                   else "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)"),
+                "kernel_ms": round(stages[g1_name], 4),
                 "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately)"}
 
     sweep = []
     if args.sweep != "none":
         plan = [(wl.QWEN3_30B, [1, 8, 32, 128, 512, 2048, 8192]), (wl.DSV3_EP, [1, 16, 64, 256, 1024, 4096])]
         plan.append((wl.QWEN3_235B_W4, [1, 32, 256, 2048]))
+        plan.append((wl.QWEN3_30B_PC, [32, 512, 8192]))
+        plan.append((wl.DSV3_EP_PC, [64, 4096]))
         if args.sweep == "full":
             plan.append((wl.DSV3_FULL, [8192]))
         for lay, Ms in plan:
@@ -354,7 +410,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": f"{layer.name} E={L.E}/{L.E_global} top{L.top_k} H={L.H} I={L.I} "
-                               + ("W4A8 int4[1,128]" if L.weight_bits == 4 else "block-INT8[128,128]")
+                               + ("W4A8 int4[1,128]" if L.weight_bits == 4 else
+                                  "per-channel INT8" if L.quant == "channel" else "block-INT8[128,128]")
                                + f", M={args.tokens}",
                    "tokens": args.tokens, "block_size_m": bs_used, "routing": L.routing},
         "int8_tops": head["int8_tops"], "hbm_gbs": head["hbm_gbs"], "frac_hbm": head["frac_hbm"],

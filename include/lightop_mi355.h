@@ -258,6 +258,10 @@ typedef struct lo_moe_tile {
 
 int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k, int64_t H,
                       int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2);
+/* The same for the per-channel form (replaces get_moe_cuda_config, int8.py:735-741, and its
+ * MODE / DELTA tables). */
+int lo_moe_tile_query_channel(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k, int64_t H,
+                              int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2);
 
 /*
  * Whole path for one chunk of tokens: quant -> align -> GEMM1(+SiLU*mul+quant) -> GEMM2

@@ -160,6 +160,91 @@ __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restri
   }
 }
 
+// The same for rows of at most 512 * CH values: one wavefront per row, four rows per workgroup,
+// the row stays in registers and the reduction needs no barrier.
+template <bool SILU, int CH>
+__global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__restrict__ x, int64_t rows, int64_t C,
+                                                             const uint16_t *__restrict__ silu,
+                                                             int8_t *__restrict__ q, float *__restrict__ s,
+                                                             const int32_t *__restrict__ num_local_tokens,
+                                                             int32_t top_k) {
+  __shared__ uint16_t sSilu[SILU ? 2 * kSiluBandN : 2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (num_local_tokens) {
+    const int64_t n = static_cast<int64_t>(num_local_tokens[0]) * top_k;
+    rows = n < 0 ? 0 : (n < rows ? n : rows);
+  }
+  if (static_cast<int64_t>(blockIdx.x) * 4 >= rows) return;
+  if constexpr (SILU) {
+    uint16_t band_regs[kSiluBandPer];
+    silu_band_load(band_regs, silu, tid);
+    silu_band_store(sSilu, band_regs, tid);
+    __syncthreads();
+  }
+  const int64_t in_stride = SILU ? 2 * C : C;
+  const int pieces = static_cast<int>(C / 8);
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + wave; row < rows; row += static_cast<int64_t>(gridDim.x) * 4) {
+    const uint16_t *xr = x + row * in_stride;
+    v8u16 ga[CH], up[CH];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int p = lane + 64 * j;
+      const int pc = p < pieces ? p : 0; // lanes past the row re-read its start and are ignored
+      ga[j] = *reinterpret_cast<const v8u16 *>(xr + pc * 8);
+      if constexpr (SILU) up[j] = *reinterpret_cast<const v8u16 *>(xr + C + pc * 8);
+    }
+    float v[CH][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const bool live = lane + 64 * j < pieces;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (SILU) v[j][i] = bf16_to_f32(silu_mul_band(sSilu, silu, ga[j][i], up[j][i]));
+        else v[j][i] = bf16_to_f32(ga[j][i]);
+        amax = fmaxf(amax, live ? fabsf(v[j][i]) : 0.0f);
+      }
+    }
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+    float inv;
+    if constexpr (SILU) {
+      inv = amax == 0.0f ? 0.0f : 127.0f / amax;
+    } else {
+      amax = fmaxf(amax, 1e-10f);
+      inv = 127.0f / amax;
+    }
+    if (lane == 0) s[row] = amax / 127.0f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int p = lane + 64 * j;
+      if (p >= pieces) continue;
+      v2i packed;
+      packed[0] = static_cast<int>(pack4_i8(rne_i8(v[j][0] * inv), rne_i8(v[j][1] * inv), rne_i8(v[j][2] * inv), rne_i8(v[j][3] * inv)));
+      packed[1] = static_cast<int>(pack4_i8(rne_i8(v[j][4] * inv), rne_i8(v[j][5] * inv), rne_i8(v[j][6] * inv), rne_i8(v[j][7] * inv)));
+      *reinterpret_cast<v2i *>(q + row * C + p * 8) = packed;
+    }
+  }
+}
+
+template <bool SILU>
+static void launch_row_quant(const uint16_t *x, int64_t rows, int64_t C, const uint16_t *silu, int8_t *q, float *s,
+                             const int32_t *nlt, int32_t top_k, hipStream_t st) {
+  const int pieces = static_cast<int>(C / 8);
+  if (pieces <= 256 && rows >= 4) {
+    int64_t grid = (rows + 3) / 4;
+    if (grid > 256 * 32) grid = 256 * 32;
+    const dim3 g(static_cast<unsigned>(grid)), b(256);
+    if (pieces <= 64) hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 1>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k);
+    else if (pieces <= 128) hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 2>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k);
+    else hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 4>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k);
+    return;
+  }
+  const unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
+  hipLaunchKernelGGL((row_quant_kernel<SILU, SILU ? 2 : 4>), dim3(grid), dim3(256), 0, st, x, rows, C, silu, q, s, nlt,
+                     top_k);
+}
+
 // ---- moe_sum -------------------------------------------------------------------
 // Reference: csrc/kernels/moe_align_sum_kernels.cu:604-637 (fp32 accumulation in slot
 // order, one rounding) and :886-909 (with bias: three roundings).
@@ -339,10 +424,8 @@ extern "C" int lo_per_token_quant_int8(const void *x, int x_dtype, int64_t rows,
   LO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0,
              LO_EINVAL, "per_token_quant_int8: x must be 16-byte and q 8-byte aligned");
   if (rows == 0) return LO_OK;
-  const unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
-  hipLaunchKernelGGL((row_quant_kernel<false, 4>), dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint16_t *>(x), rows, cols, static_cast<const uint16_t *>(nullptr), q, s,
-                     static_cast<const int32_t *>(nullptr), 1);
+  launch_row_quant<false>(static_cast<const uint16_t *>(x), rows, cols, nullptr, q, s, nullptr, 1,
+                          static_cast<hipStream_t>(stream));
   return check_launch("per_token_quant_int8");
 }
 
@@ -359,8 +442,7 @@ extern "C" int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, i
   const uint16_t *table = nullptr;
   int rc = silu_table(static_cast<hipStream_t>(stream), &table);
   if (rc) return rc;
-  const unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
-  hipLaunchKernelGGL((row_quant_kernel<true, 2>), dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint16_t *>(c1), rows, I, table, q, s, num_local_tokens, top_k);
+  launch_row_quant<true>(static_cast<const uint16_t *>(c1), rows, I, table, q, s, num_local_tokens, top_k,
+                         static_cast<hipStream_t>(stream));
   return check_launch("fuse_silu_mul_quant");
 }

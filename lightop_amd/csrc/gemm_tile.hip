@@ -30,14 +30,9 @@ constexpr int kTileRow = 144;    // LDS row pitch in bytes: 128 + 16 keeps ds_re
 // WT = number of 64-token halves per workgroup: 2 -> 128-token tile, 8 waves, one
 // workgroup per CU; 1 -> 64-token tile, 4 waves, two workgroups per CU that are not
 // synchronised with each other, so one computes while the other waits at its barrier.
-//
-// PC (per-channel W8A8, reference csrc/moe_gemm/w8a8/moe_w8a8.cu:156-166, :445-470): As holds one
-// scale per token row and Ws one per weight row; the MFMA accumulator carries the int32 sum over
-// the whole K and the scales are applied once in the epilogue, so the K loop is loads and MFMAs only.
-template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int WT, bool PC = false>
+template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int WT>
 __global__ __launch_bounds__(256 * WT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
-  static_assert(!PC || !FUSED_ACT, "the per-channel form is a plain GEMM");
   constexpr int kTileM = 64 * WT; // tokens per workgroup
   __shared__ __attribute__((aligned(16))) int8_t sA[2][kTileM * kTileRow];
   __shared__ float sS[2][kTileM];
@@ -103,7 +98,7 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   const int64_t lf = a.sorted[static_cast<int64_t>(mb) * kTileM + lt];
   const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
   const brsrc rA = make_rsrc(a.A, static_cast<uint32_t>(a.a_rows * K));
-  const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * (PC ? 1 : KB) * 4));
+  const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * KB * 4));
   const int aoff = static_cast<int>(lrow * K) + lq * 32;
   const int asoff = static_cast<int>(lrow * KB * 4);
   int8_t *const sdst0 = &sA[0][lt * kTileRow + lq * 32];
@@ -130,15 +125,12 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) zero16[i] = 0;
   float acc[2][2][16]; // [token fragment][row fragment][element]
-  v16i acci[2][2];     // PC: the whole-K int32 sums
 #pragma unroll
   for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
+    for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[tb][rb][i] = 0.0f;
-      acci[tb][rb] = zero16;
-    }
 
   v4i wreg[2][2][4]; // [buffer][row fragment][k-step]
   float bsc[2][2];   // [buffer][row fragment] weight-block scales, fetched with the fragments
@@ -156,16 +148,11 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     const int kc = kb < KB ? kb : KB - 1;
 #pragma unroll
     for (int j = 0; j < 2; ++j) areg[st][j] = bld16(rA, aoff, kc * kGroup + j * 16);
-    if constexpr (!PC) sreg[st] = bld_f32(rAs, asoff, kc * 4);
+    sreg[st] = bld_f32(rAs, asoff, kc * 4);
   };
   auto store_act = [&](auto SET, bool live) {
     constexpr int st = decltype(SET)::value;
     int8_t *d = st ? sdst1 : sdst0;
-    if constexpr (PC) { // a step past the end of K must add nothing: its token bytes are zeros
-#pragma unroll
-      for (int j = 0; j < 2; ++j) *reinterpret_cast<v4i *>(d + j * 16) = live ? areg[st][j] : v4i{0, 0, 0, 0};
-      return;
-    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) *reinterpret_cast<v4i *>(d + j * 16) = areg[st][j];
     if (lq == 0) sS[st][lt] = live ? sreg[st] : 0.0f;
@@ -179,10 +166,8 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
       for (int ks = 0; ks < 4; ++ks)
         wreg[b][rb][ks] = SHUF ? bld16(rW, woff[rb], kc * wkstride + ks * 512)
                                : bld16(rW, woff[rb], kc * kGroup + ks * 16);
-    if constexpr (!PC) {
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb) bsc[b][rb] = wsrow[rb][kc];
-    }
+    for (int rb = 0; rb < 2; ++rb) bsc[b][rb] = wsrow[rb][kc];
   };
   auto fold = [&](const v16i &d, float as, float bs, float *dst) {
     if constexpr (FAST_SCALE) {
@@ -205,25 +190,6 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   auto compute = [&](auto BUF) {
     constexpr int b = decltype(BUF)::value;
     const int8_t *tile = sA[b];
-    if constexpr (PC) {
-      v4i bf[2][4];
-#pragma unroll
-      for (int tb = 0; tb < 2; ++tb) {
-        const int8_t *src = tile + (wt * 64 + tb * 32 + r) * kTileRow + (SHUF ? c * 16 : c * 64);
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-          bf[tb][ks] = *reinterpret_cast<const v4i *>(src + (SHUF ? ks * 32 : ks * 16));
-      }
-      // k-step outermost: consecutive MFMAs write different accumulators
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-        for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-          for (int rb = 0; rb < 2; ++rb)
-            acci[tb][rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[b][rb][ks], bf[tb][ks], acci[tb][rb], 0, 0, 0);
-      return;
-    }
     // The four 32x32 fragments are software-pipelined: the MFMAs of one fragment are
     // issued, then the previous fragment is folded into the fp32 accumulators while the
     // matrix pipe works.  The scheduling barriers keep the compiler from batching all
@@ -282,34 +248,7 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     __syncthreads();
   }
 
-  if constexpr (PC) {
-    if (!wave_active) return;
-    const brsrc rWs = make_rsrc(a.Ws + static_cast<int64_t>(e) * N, static_cast<uint32_t>(N * 4));
-    v4f bs4[2][4]; // scales of the 16 rows a lane holds per fragment: rows 8q + 4c + i
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        bs4[rb][q] = __builtin_bit_cast(v4f, bld16(rWs, static_cast<int>(nrow[rb] + 8 * q + 4 * c) * 4, 0));
-#pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
-      if (!valid[tb]) continue;
-      float ts = a.As[f[tb] / a.top_k];
-      if (a.mul_routed) ts = a.topk_w[f[tb]] * ts;
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          v4u16 o;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float t = static_cast<float>(acci[tb][rb][4 * q + i]) * ts;
-            o[i] = f32_to_bf16(t * bs4[rb][q][i]);
-          }
-          *reinterpret_cast<v4u16 *>(a.C + f[tb] * N + nrow[rb] + 8 * q + 4 * c) = o;
-        }
-    }
-  } else if constexpr (!FUSED_ACT) {
+  if constexpr (!FUSED_ACT) {
     if (!wave_active) return;
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
@@ -402,15 +341,7 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int block_size_m, int f
     if (a.w_shuffled) LO_TILE_LAUNCH2(FA, FS, true);   \
     else LO_TILE_LAUNCH2(FA, FS, false);               \
   } while (0)
-  if (a.per_channel) {
-    if (wt == 2) {
-      if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_tile_kernel<false, false, true, 2, true>), g, b, 0, s, a, mbi, static_cast<int>(G));
-      else hipLaunchKernelGGL((moe_gemm_tile_kernel<false, false, false, 2, true>), g, b, 0, s, a, mbi, static_cast<int>(G));
-    } else {
-      if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_tile_kernel<false, false, true, 1, true>), g, b, 0, s, a, mbi, static_cast<int>(G));
-      else hipLaunchKernelGGL((moe_gemm_tile_kernel<false, false, false, 1, true>), g, b, 0, s, a, mbi, static_cast<int>(G));
-    }
-  } else if (fused_act) {
+  if (fused_act) {
     if (fast) LO_TILE_LAUNCH(true, true);
     else LO_TILE_LAUNCH(true, false);
   } else {

@@ -49,7 +49,8 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 def test_header_cites_the_reference_for_every_entry_point():
     text = open(HEADER).read()
     for cite in ("export.cpp:1593-1605", "int8_utils.py:125-195", "int8.py:543-626", "int8.py:811",
-                 "export.cpp:1584-1592", "int8.py:220-256", "int8.py:703-888"):
+                 "export.cpp:1584-1592", "int8.py:220-256", "int8.py:703-888", "int8_utils.py:20-71",
+                 "gemmopt.py:437-457", "fuse_silu_mul_quant.cu:90-133", "w4a8.py:211-401"):
         assert cite in text
 
 
@@ -68,6 +69,10 @@ def test_version_and_tile_table(lib):
     assert all(sizes[a] <= sizes[b] for a, b in zip(list(sizes)[:-1], list(sizes)[1:]))
     assert lib.lo_moe_tile_query(-1, 32, 256, 8, 7168, 2048, t1, t2) < 0
     assert b"moe_tile_query" in lib.lo_last_error()
+    # per-channel form: same small tiles, 128 tokens once an expert sees that many
+    for M, want in ((1, 16), (64, 16), (1024, 64), (4096, 128), (8192, 128)):
+        assert lib.lo_moe_tile_query_channel(M, 32, 256, 8, 7168, 2048, t1, t2) == 0
+        assert t1.block_size_m == want and t2.block_size_m == want
 
 
 def test_workspace_sizing(lib):

@@ -462,8 +462,11 @@ def test_fused_experts_rejects_unsupported(dev):
     s1 = torch.ones(2, 2, 2, device=dev)
     s2 = torch.ones(2, 2, 1, device=dev)
     with pytest.raises(NotImplementedError):
-        fused_experts_impl_int8(x, w1, w2, tw, ids, c, use_int8_w8a8=True, per_channel_quant=True,
+        fused_experts_impl_int8(x, w1, w2, tw, ids, c, use_int8_w8a8=True, block_shape=[64, 64],
                                 w1_scale=s1, w2_scale=s2)
+    with pytest.raises(NotImplementedError):
+        fused_experts_impl_int8(x, w1, w2, tw, ids, c, use_int8_w8a8=True, use_int8_w8a16=True,
+                                block_shape=[128, 128], w1_scale=s1, w2_scale=s2)
     with pytest.raises(ValueError):
         fused_experts_impl_int8(x, w1, w2, tw, ids, c, use_int8_w8a8=True, block_shape=[128, 128],
                                 activation="relu", w1_scale=s1, w2_scale=s2)
