@@ -133,8 +133,8 @@ class Point:
         L = self.layer
         wflag = _lib_flags_w4(L)
         if bs == 0:
-            bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, None if L.quant == "channel" else [128, 128],
-                                      L.top_k, L.E_global)[0]["BLOCK_SIZE_M"]
+            shape = [1, 128] if L.weight_bits == 4 else (None if L.quant == "channel" else [128, 128])
+            bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, shape, L.top_k, L.E_global)[0]["BLOCK_SIZE_M"]
         cfg = {"BLOCK_SIZE_M": bs}
         S = self.M * L.top_k
         c3 = self.cache13[: S * L.H].view(self.M, L.top_k, L.H)
@@ -373,8 +373,9 @@ def main():
     roofline = {"bound": head["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
                 "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
                 "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
-                "kernel": ("moe_gemm_tile_kernel" if bs_used >= 64 and L.weight_bits == 8 else "moe_gemm_ws_kernel")
-                + ("<PC> (GEMM1, per-channel scales in the epilogue)" if L.quant == "channel"
+                "kernel": ("moe_gemm_ws_kernel" if bs_used < 64 else "moe_gemm_w4_tile_kernel" if L.weight_bits == 4
+                           else "moe_gemm_pc_kernel" if L.quant == "channel" else "moe_gemm_tile_kernel")
+                + (" (GEMM1, per-channel scales in the epilogue)" if L.quant == "channel"
                    else "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)"),
                 "kernel_ms": round(stages[g1_name], 4),
                 "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately)"}

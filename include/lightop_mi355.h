@@ -61,7 +61,7 @@ enum {
    * The reference's W4A8 (python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:211-401)
    * scales per token and per channel in the epilogue instead; its nibble order (even k in
    * the high nibble, :341, :375-377) is the one lo_preshuffle_weight_int4 reads.  Served by
-   * the weight-streaming kernels at every block_size_m. */
+   * an LDS-tiled kernel at block_size_m 64 and by the weight-streaming kernels otherwise. */
   LO_GEMM_W4 = 32
 };
 
@@ -258,10 +258,11 @@ typedef struct lo_moe_tile {
 
 int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k, int64_t H,
                       int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2);
-/* The same for the per-channel form (replaces get_moe_cuda_config, int8.py:735-741, and its
- * MODE / DELTA tables). */
-int lo_moe_tile_query_channel(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k, int64_t H,
-                              int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2);
+/* The same for the other forms of the path: per-channel (replaces get_moe_cuda_config,
+ * int8.py:735-741, and its MODE / DELTA tables) and W4A8 with K-group scales. */
+enum { LO_FORM_BLOCK = 0, LO_FORM_CHANNEL = 1, LO_FORM_W4 = 2 };
+int lo_moe_tile_query_form(int form, int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
+                           int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2);
 
 /*
  * Whole path for one chunk of tokens: quant -> align -> GEMM1(+SiLU*mul+quant) -> GEMM2

@@ -14,6 +14,7 @@ LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE, LO_GEMM_FORCE_STREAMING, LO_GEMM_CANONICAL
 LO_GEMM_W_PRESHUFFLED = 8
 LO_GEMM_SKIP_NONLOCAL = 16
 LO_GEMM_W4 = 32
+LO_FORM_BLOCK, LO_FORM_CHANNEL, LO_FORM_W4 = 0, 1, 2
 
 
 class LoMoeTile(ctypes.Structure):
@@ -56,8 +57,8 @@ SIGNATURES = {
                                   c_int32, ctypes.c_double, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "lo_moe_tile_query": (c_int, [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
                                   ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
-    "lo_moe_tile_query_channel": (c_int, [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
-                                          ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
+    "lo_moe_tile_query_form": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
+                                       ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
     "lo_fused_experts_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
     "lo_fused_experts_workspace_offset": (c_int64, [c_int, c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
     "lo_per_token_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),

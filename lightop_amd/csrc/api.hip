@@ -70,13 +70,16 @@ static WsLayout ws_layout(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_
 // gfx950 tile table.  The token tile (= alignment block) follows the expected number
 // of slots per expert: small tiles waste no MFMA columns on padding while the layer
 // is weight-streaming bound, larger ones amortise each pass over an expert's weights.
-static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, bool per_channel = false) {
+static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int form = LO_FORM_BLOCK) {
   const double per_expert = static_cast<double>(M) * top_k / (num_experts > 0 ? num_experts : 1);
+  // W4A8: the streaming kernel re-reads the token rows per wave, which outweighs the half-size
+  // weights early; the LDS-tiled kernel (64 tokens) wins from about 8 slots per expert.
+  if (form == LO_FORM_W4) return per_expert < 8.0 ? 16 : 64;
   if (per_expert <= 12.0) return 16;
   if (per_expert <= 24.0) return 32;
   // Per-channel form: no scale arithmetic in the K loop, so the accumulators of 128 tokens fit
   // and the larger tile halves the weight bytes requested from L2 per multiply-add.
-  if (per_channel && per_expert >= 128.0) return 128;
+  if (form == LO_FORM_CHANNEL && per_expert >= 64.0) return 128;
   // 64-token LDS tiles: two workgroups per CU hide each other's barrier and memory
   // waits, which measured faster than the 128-token tile (one workgroup per CU) on
   // every layer shape tried.
@@ -101,14 +104,15 @@ extern "C" int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts
   return LO_OK;
 }
 
-extern "C" int lo_moe_tile_query_channel(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
-                                         int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
+extern "C" int lo_moe_tile_query_form(int form, int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
+                                      int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
   using namespace lo;
-  (void)E_local;
+  if (form == LO_FORM_BLOCK) return lo_moe_tile_query(M, E_local, num_experts, top_k, H, I, gemm1, gemm2);
+  LO_REQUIRE(form == LO_FORM_CHANNEL || form == LO_FORM_W4, LO_EINVAL, "moe_tile_query_form: unknown form %d", form);
   LO_REQUIRE(M >= 0 && num_experts >= 1 && top_k >= 1 && H > 0 && I > 0, LO_EINVAL,
-             "moe_tile_query_channel: bad problem size");
-  const int32_t bm = pick_block_m(M, num_experts, top_k, true);
-  if (gemm1) *gemm1 = lo_moe_tile{bm, bm >= 64 ? 2 : 0, 4, bm >= 64 ? 256 : 64};
+             "moe_tile_query_form: bad problem size");
+  const int32_t bm = pick_block_m(M, num_experts, top_k, form);
+  if (gemm1) *gemm1 = lo_moe_tile{bm, bm >= 64 ? 2 : 0, bm >= 64 || form == LO_FORM_CHANNEL ? 4 : 8, bm >= 64 ? 256 : 64};
   if (gemm2) *gemm2 = lo_moe_tile{bm, bm >= 64 ? 2 : 0, 4, bm >= 64 ? 256 : 64};
   return LO_OK;
 }
@@ -150,7 +154,8 @@ extern "C" int lo_fused_experts_block_int8(
   LO_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, LO_EINVAL,
              "fused_experts: workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
-  if (block_size_m == 0) block_size_m = pick_block_m(M, num_experts, top_k);
+  if (block_size_m == 0)
+    block_size_m = pick_block_m(M, num_experts, top_k, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK);
   LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
              LO_EINVAL, "fused_experts: block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
   const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
@@ -213,7 +218,7 @@ extern "C" int lo_fused_experts_channel_int8(
   LO_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, LO_EINVAL,
              "fused_experts(channel): workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
-  if (block_size_m == 0) block_size_m = pick_block_m(M, num_experts, top_k, true);
+  if (block_size_m == 0) block_size_m = pick_block_m(M, num_experts, top_k, LO_FORM_CHANNEL);
   LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
              LO_EINVAL, "fused_experts(channel): block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
   // the block layout is roomy enough: its scale segments hold one float per 128 values

@@ -85,6 +85,9 @@ bool gemm_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 int launch_gemm_as(const GemmArgs &a, int flags, int64_t m_blocks, hipStream_t s);
 bool gemm_as_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 
+// W4A8 LDS-tiled kernel (gemm_w4.hip): block_size_m 64.
+int launch_gemm_w4_tile(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
+bool gemm_w4_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 // Per-channel LDS-tiled kernel (gemm_pc.hip): block_size_m 64 or 128.
 int launch_gemm_pc(const GemmArgs &a, int block_size_m, int64_t m_blocks, hipStream_t s);
 bool gemm_pc_supports(const GemmArgs &a, int block_size_m);

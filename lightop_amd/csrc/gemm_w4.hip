@@ -1,0 +1,317 @@
+// Grouped W4A8 GEMM with K-group scales for gfx950, LDS-tiled form for many tokens per expert.
+//
+// Same arithmetic as the W4 instantiations of the weight-streaming kernel (gemm_ws.hip):
+// packed int4 weights in the load-time layout of preshuffle_int4_kernel, unpacked in registers
+// to int8 values 16 times too large, v_mfma_i32_16x16x64_i8 with the weight fragment as the A
+// operand, an exact arithmetic shift of the int32 sum, then per 128-wide K block
+//   acc = acc + (f32(d) * As[token, kb]) * Ws[e, kb, row]          (one scale per weight row)
+// (nibble order: python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341, :375-377; the
+// K-group scaling itself has no counterpart in the reference, whose kernel scales once in the
+// epilogue, w4a8.py:395).
+//
+// What differs is where the tokens come from.  The streaming kernel lets every wave read its
+// token rows from global memory, which is right while a token block is 16 or 32 rows; at 64
+// tokens those reads outweigh the (half-size) weights four to one.  Here a workgroup of four
+// waves gathers the 64 token rows of the current K block once into a double-buffered,
+// row-padded LDS tile (with their group scales) and every wave multiplies its 64 weight rows
+// (four 16-row fragments, global -> registers, double buffered together with their row scales)
+// against all of them: 16 accumulators of 16x16 per wave.  With FUSED_ACT the four fragments
+// are 32 gate rows and the matching 32 up rows, and the epilogue is the SiLU(gate)*up +
+// 1x128 re-quantisation of the block-INT8 path.
+#include <type_traits>
+
+#include "gemm.h"
+
+namespace lo {
+
+constexpr int kW4Row = 144; // LDS row pitch in bytes: 128 + 16 keeps ds_read_b128 conflict-free
+
+template <bool FUSED_ACT, bool FAST_SCALE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
+  constexpr int kTileM = 64;
+  __shared__ __attribute__((aligned(16))) int8_t sA[2][kTileM * kW4Row];
+  __shared__ float sS[2][kTileM];
+  __shared__ float sRed[4][kTileM];
+  __shared__ uint16_t sSilu[FUSED_ACT ? 2 * kSiluBandN : 2];
+
+  int mb, nt;
+  if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
+  if (static_cast<int64_t>(mb) * kTileM >= a.ntpp[0]) return;
+  const int e = a.expert_ids[mb];
+  if (e >= a.E) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wr = __builtin_amdgcn_readfirstlane(tid >> 6); // which 64 weight rows of the tile
+  const int r = lane & 15, q = lane >> 4;
+  const int64_t K = a.K, N = a.N;
+  const int KB = static_cast<int>(K / kGroup);
+  const int64_t I = N / 2;
+
+  // slots of the four 16-token fragments this lane sees in the accumulator layout
+  int64_t f[4];
+  bool valid[4];
+#pragma unroll
+  for (int tf = 0; tf < 4; ++tf) {
+    f[tf] = a.sorted[static_cast<int64_t>(mb) * kTileM + tf * 16 + r];
+    valid[tf] = f[tf] < a.num_valid;
+  }
+
+  // weight rows of the wave: four 16-row fragments
+  int64_t nrow[4];
+#pragma unroll
+  for (int rf = 0; rf < 4; ++rf) {
+    if constexpr (FUSED_ACT) nrow[rf] = (rf >= 2 ? I : 0) + static_cast<int64_t>(nt) * kGroup + wr * 32 + (rf & 1) * 16;
+    else nrow[rf] = static_cast<int64_t>(nt) * 256 + wr * 64 + rf * 16;
+  }
+
+  if (e < 0) {
+    if constexpr (!FUSED_ACT) {
+      if (!a.skip_nonlocal) {
+#pragma unroll
+        for (int tf = 0; tf < 4; ++tf)
+          if (valid[tf])
+#pragma unroll
+            for (int rf = 0; rf < 4; ++rf)
+              if (nrow[rf] < N) *reinterpret_cast<v2i *>(a.C + f[tf] * N + nrow[rf] + 4 * q) = v2i{0, 0};
+      }
+    }
+    return;
+  }
+
+  uint16_t band_regs[kSiluBandPer];
+  if constexpr (FUSED_ACT) silu_band_load(band_regs, a.silu, tid);
+
+  // cooperative gather role: thread -> (token, 32-byte quarter of the 128-byte K block)
+  const int lt = tid >> 2, lq = tid & 3;
+  const int64_t lf = a.sorted[static_cast<int64_t>(mb) * kTileM + lt];
+  const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
+  const brsrc rA = make_rsrc(a.A, static_cast<uint32_t>(a.a_rows * K));
+  const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * KB * 4));
+  const int aoff = static_cast<int>(lrow * K) + lq * 32;
+  const int asoff = static_cast<int>(lrow * KB * 4);
+  int8_t *const sdst0 = &sA[0][lt * kW4Row + lq * 32];
+  int8_t *const sdst1 = &sA[1][lt * kW4Row + lq * 32];
+
+  const int64_t wbytes = N * K / 2; // one expert
+  const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * wbytes, static_cast<uint32_t>(wbytes));
+  const brsrc rWs = make_rsrc(a.Ws + static_cast<int64_t>(e) * N * KB, static_cast<uint32_t>(N * KB * 4));
+  const int wkstride = shuf_kb_stride(static_cast<int>(N / 16)) / 2;
+  int woff[4], wsoff[4];
+#pragma unroll
+  for (int rf = 0; rf < 4; ++rf) {
+    const int64_t nr = nrow[rf] < N ? nrow[rf] : 0; // fragments past N: computed on row 0, never stored
+    woff[rf] = static_cast<int>(nr / 16) * (shuf_nb_stride(KB) / 2) + lane * 16; // 1 KB blocks, lane order
+    wsoff[rf] = static_cast<int>((nr + 4 * q) * 4);                              // the lane's rows 4q .. 4q+3
+  }
+
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  v4f acc[4][4]; // [row fragment][token fragment]
+#pragma unroll
+  for (int rf = 0; rf < 4; ++rf)
+#pragma unroll
+    for (int tf = 0; tf < 4; ++tf) acc[rf][tf] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  v4i wreg[2][4]; // [buffer][row fragment]: both k-steps of a K block, packed
+  v4f bsreg[2][4]; // the row scales that go with them
+  v4i areg[2];     // token bytes on their way to LDS
+  float sreg = 0.0f;
+
+  // The K loop is free of branches: a step past the end of K re-reads the last K block and
+  // stores a token scale of zero, so it adds exactly 0 to every accumulator.
+  auto load_act = [&](int kb) {
+    const int kc = kb < KB ? kb : KB - 1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) areg[j] = bld16(rA, aoff, kc * kGroup + j * 16);
+    sreg = bld_f32(rAs, asoff, kc * 4);
+  };
+  auto store_act = [&](auto ST, bool live) {
+    constexpr int st = decltype(ST)::value;
+    int8_t *d = st ? sdst1 : sdst0;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) *reinterpret_cast<v4i *>(d + j * 16) = areg[j];
+    if (lq == 0) sS[st][lt] = live ? sreg : 0.0f;
+  };
+  auto load_w = [&](auto BUF, int kb) {
+    constexpr int b = decltype(BUF)::value;
+    const int kc = kb < KB ? kb : KB - 1;
+#pragma unroll
+    for (int rf = 0; rf < 4; ++rf) wreg[b][rf] = bld16(rW, woff[rf], kc * wkstride);
+#pragma unroll
+    for (int rf = 0; rf < 4; ++rf)
+      bsreg[b][rf] = __builtin_bit_cast(v4f, bld16(rWs, wsoff[rf], kc * static_cast<int>(N) * 4));
+  };
+  auto fold = [&](const v4i (&d)[4], const v4f &bs, const float (&as)[4], v4f (&dst)[4]) {
+#pragma unroll
+    for (int tf = 0; tf < 4; ++tf)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float x = static_cast<float>(d[tf][i] >> 4); // exact: every product carries the factor 16
+        if constexpr (FAST_SCALE) {
+          dst[tf][i] = __builtin_fmaf(x, as[tf] * bs[i], dst[tf][i]);
+        } else {
+          float t = x * as[tf];
+          t = t * bs[i];
+          dst[tf][i] = dst[tf][i] + t;
+        }
+      }
+#pragma unroll
+    for (int tf = 0; tf < 4; ++tf)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(dst[tf][i])); // keep the fold here
+  };
+  auto compute = [&](auto BUF) {
+    constexpr int b = decltype(BUF)::value;
+    const int8_t *tile = sA[b];
+    v4i bf[4][2];
+    float as[4];
+#pragma unroll
+    for (int tf = 0; tf < 4; ++tf) {
+      const int8_t *src = tile + (tf * 16 + r) * kW4Row + q * 16;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) bf[tf][ks] = *reinterpret_cast<const v4i *>(src + ks * 64);
+      as[tf] = sS[b][tf * 16 + r];
+    }
+    // software pipeline over the row fragments: the MFMAs of fragment rf are issued, then
+    // fragment rf-1 is folded into the fp32 accumulators while the matrix pipe works
+    v4i dprev[4];
+#pragma unroll
+    for (int rf = 0; rf < 4; ++rf) {
+      v4i wop[2];
+      const v4i pk = wreg[b][rf];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const uint32_t word = static_cast<uint32_t>(pk[2 * ks + w]);
+          wop[ks][2 * w] = static_cast<int>((word << 4) & 0xf0f0f0f0u);
+          wop[ks][2 * w + 1] = static_cast<int>(word & 0xf0f0f0f0u);
+        }
+      v4i d[4];
+#pragma unroll
+      for (int tf = 0; tf < 4; ++tf) {
+        d[tf] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+          d[tf] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop[ks], bf[tf][ks], d[tf], 0, 0, 0);
+      }
+      if (rf > 0) fold(dprev, bsreg[b][rf - 1], as, acc[rf - 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int tf = 0; tf < 4; ++tf) dprev[tf] = d[tf];
+    }
+    fold(dprev, bsreg[b][3], as, acc[3]);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  load_act(0);
+  load_w(B0{}, 0);
+  store_act(B0{}, true);
+  if constexpr (FUSED_ACT) silu_band_store(sSilu, band_regs, tid);
+  __syncthreads();
+  for (int kb = 0; kb < KB; kb += 2) {
+    load_act(kb + 1);
+    load_w(B1{}, kb + 1);
+    __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMAs
+    compute(B0{});
+    store_act(B1{}, kb + 1 < KB);
+    __syncthreads();
+    load_act(kb + 2);
+    load_w(B0{}, kb + 2);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(B1{});
+    store_act(B0{}, kb + 2 < KB);
+    __syncthreads();
+  }
+
+  if constexpr (!FUSED_ACT) {
+#pragma unroll
+    for (int tf = 0; tf < 4; ++tf) {
+      if (!valid[tf]) continue;
+      float w = 1.0f;
+      if (a.mul_routed) w = a.topk_w[f[tf]];
+#pragma unroll
+      for (int rf = 0; rf < 4; ++rf) {
+        if (nrow[rf] >= N) continue;
+        v4u16 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v = acc[rf][tf][i];
+          if (a.mul_routed) v = v * w;
+          o[i] = f32_to_bf16(v);
+        }
+        *reinterpret_cast<v4u16 *>(a.C + f[tf] * N + nrow[rf] + 4 * q) = o;
+      }
+    }
+  } else {
+    // acc[0..1] = gate, acc[2..3] = up for activation columns nt*128 + wr*32 + 16*g + 4q + i
+    float actf[4][2][4];
+#pragma unroll
+    for (int tf = 0; tf < 4; ++tf) {
+      float w = 1.0f;
+      if (a.mul_routed && valid[tf]) w = a.topk_w[f[tf]];
+      float amax = 0.0f;
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float gv = acc[g][tf][i], uv = acc[2 + g][tf][i];
+          if (a.mul_routed) {
+            gv = gv * w;
+            uv = uv * w;
+          }
+          const uint16_t act16 = silu_mul_band(sSilu, a.silu, f32_to_bf16(gv), f32_to_bf16(uv));
+          actf[tf][g][i] = bf16_to_f32(act16);
+          amax = fmaxf(amax, fabsf(actf[tf][g][i]));
+        }
+      amax = fmaxf(amax, __shfl_xor(amax, 16));
+      amax = fmaxf(amax, __shfl_xor(amax, 32));
+      if (q == 0) sRed[wr][tf * 16 + r] = amax;
+    }
+    __syncthreads();
+    const int64_t G = I / kGroup;
+#pragma unroll
+    for (int tf = 0; tf < 4; ++tf) {
+      if (!valid[tf]) continue;
+      const int t = tf * 16 + r;
+      float amax = fmaxf(fmaxf(sRed[0][t], sRed[1][t]), fmaxf(sRed[2][t], sRed[3][t]));
+      amax = fmaxf(amax, 1e-10f);
+      const float sc = amax / 127.0f;
+      const float rsc = 1.0f / sc;
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        const uint32_t packed = quant4(actf[tf][g], sc, rsc);
+        *reinterpret_cast<uint32_t *>(a.A2q + f[tf] * I + nrow[g] + 4 * q) = packed;
+      }
+      if (wr == 0 && q == 0) a.A2s[f[tf] * G + nt] = sc;
+    }
+  }
+}
+
+bool gemm_w4_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
+  (void)fused_act;
+  return a.w4 && a.w_shuffled && block_size_m == 64;
+}
+
+int launch_gemm_w4_tile(const GemmArgs &a0, bool fused_act, int flags, int64_t m_blocks, hipStream_t s) {
+  GemmArgs a = a0;
+  a.n_tiles = fused_act ? static_cast<int32_t>(a.N / 2 / kGroup) : static_cast<int32_t>((a.N + 255) / 256);
+  int64_t G = a.num_valid / (static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * 64);
+  G = G < 2 ? 2 : (G > 16 ? 16 : G);
+  const int64_t chunks = (m_blocks + G - 1) / G;
+  const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
+  LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm(w4): grid too large");
+  const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
+  const dim3 g(static_cast<unsigned>(grid)), b(256);
+  const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
+  if (fused_act) {
+    if (fast) hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<true, true>), g, b, 0, s, a, mbi, gi);
+    else hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<true, false>), g, b, 0, s, a, mbi, gi);
+  } else {
+    if (fast) hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<false, true>), g, b, 0, s, a, mbi, gi);
+    else hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<false, false>), g, b, 0, s, a, mbi, gi);
+  }
+  return check_launch(fused_act ? "moe_gemm1_silu_quant(w4 tile)" : "moe_gemm(w4 tile)");
+}
+
+} // namespace lo

@@ -17,12 +17,13 @@ def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bo
     int8.py:220-256, backed there by per-device JSON files).  Here the table is compiled
     into the library; the dictionaries keep the reference's keys.  ``n1`` = 2*I, ``n2`` = H,
     ``k`` = I.  ``block_shape=None`` asks for the per-channel form (the reference consults
-    get_moe_cuda_config first there, int8.py:735-741)."""
+    get_moe_cuda_config first there, int8.py:735-741), ``[1, 128]`` for W4A8 with K-group scales."""
     del use_int8_w8a8
     t1, t2 = _lib.LoMoeTile(), _lib.LoMoeTile()
     Eg = E if global_num_experts in (-1, None) else global_num_experts
-    query = _lib.lib().lo_moe_tile_query_channel if block_shape is None else _lib.lib().lo_moe_tile_query
-    _lib.check(query(m, E, Eg, topk, n2, k, t1, t2))
+    form = _lib.LO_FORM_CHANNEL if block_shape is None else (
+        _lib.LO_FORM_W4 if list(block_shape) == [1, 128] else _lib.LO_FORM_BLOCK)
+    _lib.check(_lib.lib().lo_moe_tile_query_form(form, m, E, Eg, topk, n2, k, t1, t2))
 
     def as_dict(t):
         return {"BLOCK_SIZE_M": t.block_size_m, "BLOCK_SIZE_N": t.block_n, "BLOCK_SIZE_K": 128,

@@ -1,4 +1,4 @@
-"""Tile-table tuning for the block-INT8 fused-MoE path on the GPU at hand.
+"""Tile-table tuning for the fused-MoE path (block-INT8, per-channel INT8, W4A8) on the GPU at hand.
 
     python -m lightop_amd.tune [--workload NAME | --shape E,E_global,topk,H,I] [--tokens 1,16,...]
                                [--out DIR] [--steps N]
@@ -46,7 +46,8 @@ def time_ms(fn, steps, flush):
 
 def main(argv=None):
     from lightop_amd import _lib, workloads as wl
-    from lightop_amd.moe import fused_experts_impl_int8, get_w8a8moe_json, preshuffle_moe_weight
+    from lightop_amd.moe import (fused_experts_impl_int8, fused_experts_impl_w4a8, get_w8a8moe_json,
+                                 preshuffle_moe_scale_int4, preshuffle_moe_weight, preshuffle_moe_weight_int4)
 
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--workload", default="deepseek-v3-ep8-share", help=f"one of {sorted(wl.LAYERS)}")
@@ -66,7 +67,24 @@ def main(argv=None):
     else:
         layer = wl.LAYERS[args.workload]
     w1, w2, w1s, w2s = wl.make_weights(layer, seed=0, device=dev, gen_device="cuda")
-    w1, w2 = preshuffle_moe_weight(w1), preshuffle_moe_weight(w2)
+    if layer.weight_bits == 4:
+        w1, w2 = preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2)
+        w1s, w2s = preshuffle_moe_scale_int4(w1s), preshuffle_moe_scale_int4(w2s)
+    else:
+        w1, w2 = preshuffle_moe_weight(w1), preshuffle_moe_weight(w2)
+    # which form of the path the layer asks for: block-INT8, per-channel INT8 or W4A8 with K-group scales
+    block_shape = [1, 128] if layer.weight_bits == 4 else (None if layer.quant == "channel" else [128, 128])
+
+    def run(x, tw, ids, cache13, bs):
+        if layer.weight_bits == 4:
+            return fused_experts_impl_w4a8(x, w1, w2, tw, ids, cache13, global_num_experts=layer.E_global,
+                                           expert_map=emap, w1_scale=w1s, w2_scale=w2s, block_shape=block_shape,
+                                           lightop_amd_block_size_m=bs)
+        return fused_experts_impl_int8(x, w1, w2, tw, ids, cache13, use_int8_w8a8=True,
+                                       per_channel_quant=block_shape is None, global_num_experts=layer.E_global,
+                                       expert_map=emap, w1_scale=w1s, w2_scale=w2s, block_shape=block_shape,
+                                       lightop_amd_block_size_m=bs)
+
     emap = wl.expert_map_for(layer, dev)
     flush_buf = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.int32, device=dev)
     counter = [0]
@@ -83,11 +101,9 @@ def main(argv=None):
         cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
         ms = {}
         for bs in BLOCK_SIZES:
-            ms[bs] = time_ms(lambda: fused_experts_impl_int8(
-                x, w1, w2, tw, ids, cache13, use_int8_w8a8=True, global_num_experts=layer.E_global, expert_map=emap,
-                w1_scale=w1s, w2_scale=w2s, block_shape=[128, 128], lightop_amd_block_size_m=bs), args.steps, flush)
+            ms[bs] = time_ms(lambda: run(x, tw, ids, cache13, bs), args.steps, flush)
         best = min(ms, key=ms.get)
-        c1, c2 = get_w8a8moe_json(M, layer.E, 2 * layer.I, layer.H, layer.I, True, [128, 128], layer.top_k,
+        c1, c2 = get_w8a8moe_json(M, layer.E, 2 * layer.I, layer.H, layer.I, True, block_shape, layer.top_k,
                                   layer.E_global)
         pick = c1["BLOCK_SIZE_M"]
         loss = ms[pick] / ms[best] - 1.0
@@ -102,7 +118,8 @@ def main(argv=None):
         os.makedirs(args.out, exist_ok=True)
         props = torch.cuda.get_device_properties(dev)
         devname = f"{props.gcnArchName.split(':')[0]}_{props.multi_processor_count}cu"
-        name = (f"MOE_BLOCKINT8[128,128]_E={layer.E}_N1={2 * layer.I}_N2={layer.H}_K={layer.I}_"
+        kind = "W4A8[1,128]" if layer.weight_bits == 4 else ("CHANNELINT8" if block_shape is None else "BLOCKINT8[128,128]")
+        name = (f"MOE_{kind}_E={layer.E}_N1={2 * layer.I}_N2={layer.H}_K={layer.I}_"
                 f"TOPK{layer.top_k}_{devname}.json")
         with open(os.path.join(args.out, name), "w") as f:
             json.dump({f"{2 * layer.I}_{layer.H}_{layer.I}": table}, f, indent=4)

@@ -70,9 +70,14 @@ def test_version_and_tile_table(lib):
     assert lib.lo_moe_tile_query(-1, 32, 256, 8, 7168, 2048, t1, t2) < 0
     assert b"moe_tile_query" in lib.lo_last_error()
     # per-channel form: same small tiles, 128 tokens once an expert sees that many
-    for M, want in ((1, 16), (64, 16), (1024, 64), (4096, 128), (8192, 128)):
-        assert lib.lo_moe_tile_query_channel(M, 32, 256, 8, 7168, 2048, t1, t2) == 0
+    for M, want in ((1, 16), (64, 16), (1024, 64), (2048, 128), (8192, 128)):
+        assert lib.lo_moe_tile_query_form(_lib.LO_FORM_CHANNEL, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
         assert t1.block_size_m == want and t2.block_size_m == want
+    # W4A8: streaming for a handful of slots per expert, the 64-token LDS tile from 8 on
+    for M, want in ((1, 16), (128, 16), (256, 64), (8192, 64)):
+        assert lib.lo_moe_tile_query_form(_lib.LO_FORM_W4, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
+        assert t1.block_size_m == want
+    assert lib.lo_moe_tile_query_form(7, 1, 32, 256, 8, 7168, 2048, t1, t2) < 0
 
 
 def test_workspace_sizing(lib):
