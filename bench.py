@@ -33,6 +33,8 @@ MEASURED_TRAFFIC = {
     ("qwen3-30b-a3b", 8192): 1066796118,
     ("deepseek-v3-ep8-share", 64): 805685369,
     ("deepseek-v3-ep8-share", 4096): 2063886851,
+    ("qwen3-235b-a22b-w4a8", 2048): 1638253852,
+    ("qwen3-235b-a22b-w4a8", 32): 777808537,
 }
 
 

@@ -114,23 +114,26 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
 
   v4i wreg[2][4]; // [buffer][row fragment]: both k-steps of a K block, packed
   v4f bsreg[2][4]; // the row scales that go with them
-  v4i areg[2];     // token bytes on their way to LDS
-  float sreg = 0.0f;
+  v4i areg[2][2];  // [set][16-byte piece]: token bytes in flight for two K blocks
+  float sreg[2] = {0.0f, 0.0f};
 
   // The K loop is free of branches: a step past the end of K re-reads the last K block and
   // stores a token scale of zero, so it adds exactly 0 to every accumulator.
-  auto load_act = [&](int kb) {
+  // The token bytes of K block kb are requested two iterations before they are needed and
+  // written to LDS one iteration before: set = kb & 1 in registers, stage = kb & 1 in LDS.
+  auto load_act = [&](auto ST, int kb) {
+    constexpr int st = decltype(ST)::value;
     const int kc = kb < KB ? kb : KB - 1;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) areg[j] = bld16(rA, aoff, kc * kGroup + j * 16);
-    sreg = bld_f32(rAs, asoff, kc * 4);
+    for (int j = 0; j < 2; ++j) areg[st][j] = bld16(rA, aoff, kc * kGroup + j * 16);
+    sreg[st] = bld_f32(rAs, asoff, kc * 4);
   };
   auto store_act = [&](auto ST, bool live) {
     constexpr int st = decltype(ST)::value;
     int8_t *d = st ? sdst1 : sdst0;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) *reinterpret_cast<v4i *>(d + j * 16) = areg[j];
-    if (lq == 0) sS[st][lt] = live ? sreg : 0.0f;
+    for (int j = 0; j < 2; ++j) *reinterpret_cast<v4i *>(d + j * 16) = areg[st][j];
+    if (lq == 0) sS[st][lt] = live ? sreg[st] : 0.0f;
   };
   auto load_w = [&](auto BUF, int kb) {
     constexpr int b = decltype(BUF)::value;
@@ -142,15 +145,20 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
       bsreg[b][rf] = __builtin_bit_cast(v4f, bld16(rWs, wsoff[rf], kc * static_cast<int>(N) * 4));
   };
   auto fold = [&](const v4i (&d)[4], const v4f &bs, const float (&as)[4], v4f (&dst)[4]) {
+    // every product carries the factor 16 of the unpacked nibbles: the canonical order takes it
+    // out of the exact int32 sum with a shift, the fused order puts 1/16 into the row scale
+    // (a power of two: the same value unless the scale is denormal)
+    v4f bs16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bs16[i] = bs[i] * 0.0625f;
 #pragma unroll
     for (int tf = 0; tf < 4; ++tf)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float x = static_cast<float>(d[tf][i] >> 4); // exact: every product carries the factor 16
         if constexpr (FAST_SCALE) {
-          dst[tf][i] = __builtin_fmaf(x, as[tf] * bs[i], dst[tf][i]);
+          dst[tf][i] = __builtin_fmaf(static_cast<float>(d[tf][i]), as[tf] * bs16[i], dst[tf][i]);
         } else {
-          float t = x * as[tf];
+          float t = static_cast<float>(d[tf][i] >> 4) * as[tf];
           t = t * bs[i];
           dst[tf][i] = dst[tf][i] + t;
         }
@@ -204,19 +212,20 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  load_act(0);
+  load_act(B0{}, 0);
+  load_act(B1{}, 1);
   load_w(B0{}, 0);
   store_act(B0{}, true);
   if constexpr (FUSED_ACT) silu_band_store(sSilu, band_regs, tid);
   __syncthreads();
   for (int kb = 0; kb < KB; kb += 2) {
-    load_act(kb + 1);
-    load_w(B1{}, kb + 1);
+    load_act(B0{}, kb + 2);            // needed in two iterations
+    load_w(B1{}, kb + 1);              // needed in the next iteration
     __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMAs
     compute(B0{});
-    store_act(B1{}, kb + 1 < KB);
+    store_act(B1{}, kb + 1 < KB);      // requested one iteration ago
     __syncthreads();
-    load_act(kb + 2);
+    load_act(B1{}, kb + 3);
     load_w(B0{}, kb + 2);
     __builtin_amdgcn_sched_barrier(0);
     compute(B1{});
