@@ -168,45 +168,41 @@ class Point:
                     acc[n].append(ev[i].elapsed_time(ev[i + 1]))
         return {n: sum(v) / len(v) for n, v in acc.items()}, bs
 
+    def stage_times_channel(self, steps, warmup, flush, bs):
+        """The six launches of the per-channel path, each on its own (ms, mean)."""
+        from lightop_amd import fuse_silu_mul_quant, moe
+        from lightop_amd.quant import per_token_quant_int8
 
-def _stage_times_channel(self, steps, warmup, flush, bs):
-    """The six launches of the per-channel path, each on its own (ms, mean)."""
-    from lightop_amd import fuse_silu_mul_quant, moe
-    from lightop_amd.quant import per_token_quant_int8
-
-    L = self.layer
-    cfg = {"BLOCK_SIZE_M": bs}
-    S = self.M * L.top_k
-    c1 = self.cache13[: S * 2 * L.I].view(S, 2 * L.I)
-    c3 = self.cache13[: S * L.H].view(self.M, L.top_k, L.H)
-    out = torch.empty(self.M, L.H, dtype=torch.bfloat16, device=self.dev)
-    names = ["quant", "align", "gemm1", "silu_mul_quant", "gemm2", "moe_sum"]
-    acc = {n: [] for n in names}
-    for it in range(warmup + steps):
-        x, tw, ids = self.batches[it % len(self.batches)]
-        flush()
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(7)]
-        ev[0].record()
-        a1q, a1s = per_token_quant_int8(x)
-        ev[1].record()
-        s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
-        ev[2].record()
-        moe.moe_gemm_w8a8(a1q, self.w1, c1, a1s, self.w1s, None, s, e, p, L.top_k, cfg)
-        ev[3].record()
-        a2q, a2s = fuse_silu_mul_quant(c1)
-        ev[4].record()
-        moe.moe_gemm_w8a8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, 1, cfg)
-        ev[5].record()
-        moe.moe_sum(c3, out)
-        ev[6].record()
-        if it >= warmup:
-            torch.cuda.synchronize()
-            for i, n in enumerate(names):
-                acc[n].append(ev[i].elapsed_time(ev[i + 1]))
-    return {n: sum(v) / len(v) for n, v in acc.items()}
-
-
-Point.stage_times_channel = _stage_times_channel
+        L = self.layer
+        cfg = {"BLOCK_SIZE_M": bs}
+        S = self.M * L.top_k
+        c1 = self.cache13[: S * 2 * L.I].view(S, 2 * L.I)
+        c3 = self.cache13[: S * L.H].view(self.M, L.top_k, L.H)
+        out = torch.empty(self.M, L.H, dtype=torch.bfloat16, device=self.dev)
+        names = ["quant", "align", "gemm1", "silu_mul_quant", "gemm2", "moe_sum"]
+        acc = {n: [] for n in names}
+        for it in range(warmup + steps):
+            x, tw, ids = self.batches[it % len(self.batches)]
+            flush()
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(7)]
+            ev[0].record()
+            a1q, a1s = per_token_quant_int8(x)
+            ev[1].record()
+            s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
+            ev[2].record()
+            moe.moe_gemm_w8a8(a1q, self.w1, c1, a1s, self.w1s, None, s, e, p, L.top_k, cfg)
+            ev[3].record()
+            a2q, a2s = fuse_silu_mul_quant(c1)
+            ev[4].record()
+            moe.moe_gemm_w8a8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, 1, cfg)
+            ev[5].record()
+            moe.moe_sum(c3, out)
+            ev[6].record()
+            if it >= warmup:
+                torch.cuda.synchronize()
+                for i, n in enumerate(names):
+                    acc[n].append(ev[i].elapsed_time(ev[i + 1]))
+        return {n: sum(v) / len(v) for n, v in acc.items()}
 
 
 def graph_ms(pt, steps, flush, bs, flags):

@@ -175,6 +175,53 @@ def test_whole_path_tiny_bit_exact(dev, oracle, bs, with_map, shuf):
         assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
+@pytest.mark.parametrize("M", [1, 3, 16, 77])
+@pytest.mark.parametrize("variant", ["plain", "shared", "on_input", "inplace"])
+def test_whole_path_ep_share_variants_bit_exact(dev, oracle, M, variant):
+    """An expert-parallel share (4 of 32 experts held here) with the optional arguments of the entry point."""
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import fused_experts_impl_int8
+
+    say(f"channel ep-share M={M} {variant}")
+    layer = wl.MoeLayer("ep-pc", E=4, E_global=32, top_k=8, H=512, I=256, routing="grouped_sigmoid", n_group=8,
+                        topk_group=4, routed_scaling=2.5, quant="channel")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=3)
+    x, tw, ids = wl.make_inputs(layer, M, seed=3)
+    emap = wl.expert_map_for(layer)
+    sh = torch.randn(M, layer.H, generator=torch.Generator().manual_seed(8)).to(torch.bfloat16) \
+        if variant == "shared" else None
+    cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
+    xd = x.to(dev)
+    out = fused_experts_impl_int8(
+        xd, w1.to(dev), w2.to(dev), tw.to(dev), ids.to(dev), cache13, inplace=variant == "inplace",
+        apply_router_weight_on_input=variant == "on_input", use_int8_w8a8=True, per_channel_quant=True,
+        global_num_experts=32, expert_map=emap.to(dev), w1_scale=w1s.to(dev), w2_scale=w2s.to(dev), block_shape=None,
+        routed_scaling_factor=2.5 if sh is not None else 1.0, shared_output=None if sh is None else sh.to(dev),
+        lightop_amd_block_size_m=16)
+    torch.cuda.synchronize()
+    if variant == "inplace":
+        assert out.data_ptr() == xd.data_ptr()
+    ref = oracle.fused_experts_channel_int8(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=32, expert_map=emap,
+                                            apply_router_weight_on_input=variant == "on_input",
+                                            routed_scaling_factor=2.5 if sh is not None else 1.0, shared_output=sh)
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+def test_whole_path_in_chunks(dev, oracle, monkeypatch):
+    """More tokens than LMSLIM_FUSED_MOE_CHUNK_SIZE: the chunks (int8.py:703-722) give the same rows."""
+    from lightop_amd import workloads as wl
+
+    say("channel whole path in chunks")
+    monkeypatch.setenv("LMSLIM_FUSED_MOE_CHUNK_SIZE", "40")
+    layer = wl.TINY_PC
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
+    x, tw, ids = wl.make_inputs(layer, 100, seed=6)
+    out = run_path(layer, (w1.to(dev), w2.to(dev), w1s.to(dev), w2s.to(dev)), x.to(dev), tw.to(dev), ids.to(dev),
+                   None, dev, 16)
+    ref = oracle.fused_experts_channel_int8(x, w1, w2, w1s, w2s, tw, ids, 16)
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
 def test_channel_path_rejects_mixed_arguments(dev):
     from lightop_amd import workloads as wl
     from lightop_amd.moe import fused_experts_impl_int8

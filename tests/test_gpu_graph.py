@@ -9,24 +9,33 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("M", [1, 16, 64])
-def test_graph_replays_match_eager(M):
+@pytest.mark.parametrize("form", ["block", "channel", "w4"])
+def test_graph_replays_match_eager(M, form):
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     from lightop_amd import _lib, workloads as wl
-    from lightop_amd.moe import fused_experts_impl_int8
+    from lightop_amd.moe import (fused_experts_impl_int8, fused_experts_impl_w4a8, preshuffle_moe_scale_int4,
+                                 preshuffle_moe_weight_int4)
 
     _lib.lib()
     dev = torch.device("cuda:0")
-    layer = wl.TINY
+    layer = {"block": wl.TINY, "channel": wl.TINY_PC, "w4": wl.TINY_W4}[form]
     w1, w2, w1s, w2s = wl.make_weights(layer, seed=0, device=dev)
+    if form == "w4":
+        w1, w2 = preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2)
+        w1s, w2s = preshuffle_moe_scale_int4(w1s), preshuffle_moe_scale_int4(w2s)
     x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, M, seed=5))
     cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
 
     def run():
-        return fused_experts_impl_int8(x, w1, w2, tw, ids, cache13, use_int8_w8a8=True, w1_scale=w1s,
-                                       w2_scale=w2s, block_shape=[128, 128])
+        if form == "w4":
+            return fused_experts_impl_w4a8(x, w1, w2, tw, ids, cache13, w1_scale=w1s, w2_scale=w2s,
+                                           block_shape=[1, 128])
+        return fused_experts_impl_int8(x, w1, w2, tw, ids, cache13, use_int8_w8a8=True,
+                                       per_channel_quant=form == "channel", w1_scale=w1s, w2_scale=w2s,
+                                       block_shape=None if form == "channel" else [128, 128])
 
-    print(f"[case] graph replay M={M}", flush=True)
+    print(f"[case] graph replay M={M} {form}", flush=True)
     eager = run().clone()
     torch.cuda.synchronize()
     side = torch.cuda.Stream()

@@ -56,6 +56,31 @@ def test_signatures_match_the_reference():
     qs = inspect.signature(quant.per_token_group_quant_int8)
     assert list(qs.parameters) == ["x", "group_size", "eps", "dtype"]
     assert qs.parameters["eps"].default == 1e-10 and qs.parameters["dtype"].default is torch.int8
+    # int8_utils.py:46
+    assert list(inspect.signature(quant.per_token_quant_int8).parameters) == ["x"]
+    # w4a8.py:480-501
+    w4 = inspect.signature(moe.fused_experts_impl_w4a8)
+    assert list(w4.parameters) == ["hidden_states", "w1", "w2", "topk_weights", "topk_ids", "cache13", "inplace",
+                                   "activation", "apply_router_weight_on_input", "global_num_experts", "expert_map",
+                                   "w1_scale", "w2_scale", "w1_zp", "w2_zp", "a1_scale", "a2_scale", "block_shape",
+                                   "use_nn_moe", "routed_scaling_factor", "shared_output", "_"]
+    # gemmopt.py:437-447 (a trailing private `flags` is this build's)
+    from lightop_amd import fuse_silu_mul_quant, gemmopt, moe_fused_gate as gate_mod, op
+
+    assert list(inspect.signature(gemmopt.moe_gemm_w8a8).parameters)[:11] == [
+        "input", "b_qweight", "output", "a_scale", "b_scale", "topk_weights", "sorted_token_ids", "experts_ids",
+        "num_tokens_post_pad", "top_k", "config"]
+    # fuse_silu_mul_quant.py:45-51
+    fs = inspect.signature(fuse_silu_mul_quant)
+    assert list(fs.parameters) == ["input", "num_local_tokens_tensor", "topk", "expect_m", "output", "scales",
+                                   "expert_ids"]
+    assert fs.parameters["topk"].default == 1 and fs.parameters["expect_m"].default == -1
+    # moe_fused_gate.py:10-20 and op.topk_softmax (export.cpp:1437)
+    assert list(inspect.signature(gate_mod.moe_fused_gate).parameters) == [
+        "x", "bias", "num_expert_group", "topk_group", "topk", "n_share_experts_fusion", "routed_scaling_factor",
+        "apply_routed_scaling_factor_on_output", "output_indices_int64"]
+    assert list(inspect.signature(op.topk_softmax).parameters) == [
+        "topk_weights", "topk_indices", "token_expert_indices", "gating_output", "Is_renormalize"]
 
 
 def test_out_variant_forwards_positionally(monkeypatch):
