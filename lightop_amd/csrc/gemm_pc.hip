@@ -10,7 +10,7 @@
 // wavefronts, each owning 64 weight rows (two 32-row MFMA fragments, global -> registers,
 // double buffered) against all 32*TB tokens (gathered through sorted_token_ids into a
 // double-buffered, row-padded LDS tile), i.e. 2*TB accumulators of v_mfma_i32_32x32x32_i8.
-// Two workgroups share a compute unit.
+// Two workgroups share a compute unit (three with 64-token tiles).
 #include <type_traits>
 
 #include "gemm.h"
@@ -22,8 +22,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kPcRow = 144; // LDS row pitch in bytes: 128 + 16 keeps ds_read_b128 conflict-free
 
 template <bool SHUF, int TB>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void moe_gemm_pc_kernel(const GemmArgs a, int m_blocks, int group_m) {
+__device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks, int group_m) {
   constexpr int kTileM = 32 * TB;       // tokens per workgroup
   constexpr int kThrPerTok = 256 / kTileM; // threads that gather one token row
   constexpr int kPieces = 8 / kThrPerTok;  // 16-byte pieces per thread and K block
@@ -189,6 +188,19 @@ void moe_gemm_pc_kernel(const GemmArgs a, int m_blocks, int group_m) {
   }
 }
 
+// 128 tokens: 246 registers, two waves per SIMD.  64 tokens: 162 registers, so three workgroups
+// fit a compute unit and hide each other's barrier and memory waits better than two.
+template <bool SHUF>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void moe_gemm_pc_kernel_128(const GemmArgs a, int m_blocks, int group_m) {
+  moe_gemm_pc_body<SHUF, 4>(a, m_blocks, group_m);
+}
+template <bool SHUF>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
+void moe_gemm_pc_kernel_64(const GemmArgs a, int m_blocks, int group_m) {
+  moe_gemm_pc_body<SHUF, 2>(a, m_blocks, group_m);
+}
+
 bool gemm_pc_supports(const GemmArgs &a, int block_size_m) {
   return a.per_channel && (block_size_m == 64 || block_size_m == 128) && a.N % 64 == 0;
 }
@@ -205,11 +217,11 @@ int launch_gemm_pc(const GemmArgs &a0, int block_size_m, int64_t m_blocks, hipSt
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
   if (block_size_m == 128) {
-    if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_pc_kernel<true, 4>), g, b, 0, s, a, mbi, gi);
-    else hipLaunchKernelGGL((moe_gemm_pc_kernel<false, 4>), g, b, 0, s, a, mbi, gi);
+    if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_pc_kernel_128<true>), g, b, 0, s, a, mbi, gi);
+    else hipLaunchKernelGGL((moe_gemm_pc_kernel_128<false>), g, b, 0, s, a, mbi, gi);
   } else {
-    if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_pc_kernel<true, 2>), g, b, 0, s, a, mbi, gi);
-    else hipLaunchKernelGGL((moe_gemm_pc_kernel<false, 2>), g, b, 0, s, a, mbi, gi);
+    if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_pc_kernel_64<true>), g, b, 0, s, a, mbi, gi);
+    else hipLaunchKernelGGL((moe_gemm_pc_kernel_64<false>), g, b, 0, s, a, mbi, gi);
   }
   return check_launch("moe_gemm_w8a8(tile)");
 }
