@@ -8,7 +8,7 @@ A step is one call of ``fused_experts_impl_int8`` on one batch of synthetic toke
 every input already resident in HBM.  Between steps a 512 MiB buffer is overwritten so
 that weights are streamed from HBM and not served from the 256 MB Infinity Cache; the
 step time is taken with HIP events on the launching stream and excludes that flush.
-The last line printed is one JSON object (see README / DESIGN for the fields).
+The last line printed is one JSON object (fields: metric, value, unit, ms_per_step, roofline, cpu_baseline, stage_ms, routers, sweep).
 """
 from __future__ import annotations
 
@@ -314,7 +314,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (one process, one MI355X, no collectives); "
-              f"--gpus {args.gpus} is not supported. Expert-parallel sharding is described in DESIGN.md.",
+              f"--gpus {args.gpus} is not supported. Sharding by experts is a design note only.",
               file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():

@@ -52,7 +52,7 @@ enum {
   /* leave the output rows of blocks whose expert id is -1 untouched instead of zeroing
    * them (the caller then reduces with an expert_mask, see lo_moe_sum) */
   LO_GEMM_SKIP_NONLOCAL = 16,
-  /* W4A8 with K-group scales (BASELINE's int4 variant): W (w1 and w2 for the whole path) is
+  /* W4A8 with K-group scales (the benchmark's int4 variant): W (w1 and w2 for the whole path) is
    * packed signed int4 in the layout of lo_preshuffle_weight_int4 (LO_GEMM_W_PRESHUFFLED must
    * be set too) and the weight scales are one per output row and 128-wide K group, stored
    * K-group-major (transposed once at load time), Ws [E, K/128, N] instead of

@@ -11,7 +11,7 @@ tree, checks the HIP path against fixed bytes as well as against the live oracle
   small_layer.npz    every input and every intermediate of one small fused-MoE call
                      (E=4 of 8 global, top-2, H=256, I=128, M=9, block 16, expert_map,
                      shared_output, routed_scaling_factor 2.5)
-  tiny_config1.json  BASELINE config 1 (E=8, top-2, H=1024, I=512, M=64, seed 0):
+  tiny_config1.json  the tiny benchmark configuration (E=8, top-2, H=1024, I=512, M=64, seed 0):
                      routing outputs in full, sha256 of every other stage's bytes
   align_docstring.json  the one literal known answer the reference holds
                      (moe_align_block_size.py:66-81)

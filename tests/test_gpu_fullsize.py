@@ -1,4 +1,4 @@
-"""GPU parity at BASELINE's full sizes, where the oracle cannot run the whole problem.
+"""GPU parity at the benchmark's full sizes, where the oracle cannot run the whole problem.
 
 Three kinds of checks:
   * size-independent properties of the routing alignment and the group quantisation;
@@ -126,7 +126,7 @@ def test_full_size_sampled_tokens_vs_oracle(dev, oracle, name, M, block_sizes):
 
 
 def test_full_deepseek_v3_zipf_routing(dev, oracle):
-    """BASELINE config 4 in shape (all 256 experts resident, Zipf-skewed routing, M=8192,
+    """The full DeepSeek-V3 benchmark configuration in shape (all 256 experts resident, Zipf-skewed routing, M=8192,
     block sizes 16..128); the hidden/intermediate sizes are halved so that the weights
     (2.8 GB) are generated and shuffled in seconds."""
     from lightop_amd import _lib, workloads as wl

@@ -84,7 +84,7 @@ def test_small_layer_whole_path(dev, preshuffle):
 
 
 def test_tiny_config1_digests(dev):
-    """BASELINE config 1 end to end: routing outputs in full, every other stage by digest."""
+    """The tiny benchmark configuration end to end: routing outputs in full, every other stage by digest."""
     from lightop_amd import moe, workloads as wl
     from lightop_amd.quant import per_token_group_quant_int8
 

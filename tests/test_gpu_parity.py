@@ -414,7 +414,7 @@ def run_fused(dev, layer, M, seed, bs=0, flags=4, shared=False, on_input=False, 
 @pytest.mark.parametrize("bs", BS_ALL)
 @pytest.mark.parametrize("preshuffle", [False, True])
 def test_fused_experts_tiny_config_bit_exact(dev, oracle, bs, preshuffle):
-    """BASELINE config 1: E=8, top-2, H=1024, I=512, M=64, seed 0."""
+    """The tiny benchmark configuration: E=8, top-2, H=1024, I=512, M=64, seed 0."""
     from lightop_amd import workloads as wl
 
     say(f"fused tiny bs={bs} preshuffle={preshuffle}")

@@ -239,7 +239,7 @@ def test_golden_align_docstring(oracle):
 
 def test_torch_restatement_agrees_with_oracle_on_config1(oracle):
     """The timed CPU baseline (oracle/torch_ref.py) and the C oracle are independent
-    restatements; on BASELINE config 1 they agree within the path's tolerance."""
+    restatements; on the tiny benchmark configuration they agree within the path's tolerance."""
     from lightop_amd import workloads as wl
     from oracle import torch_ref
 

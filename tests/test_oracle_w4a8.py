@@ -1,7 +1,7 @@
 """Pins of the W4A8 (packed int4 weights, K-group scales) restatement in oracle/moe_oracle.c.
 
 The reference implements W4A8 with per-token x per-channel scales applied once in the epilogue
-(python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:211-401); the K-group form of BASELINE's
+(python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:211-401); the K-group form of the benchmark's
 int4 configuration has no reference implementation, so against the reference it is
 "parity unpinned".  What is pinned here: the nibble order (the reference's, w4a8.py:341,
 :375-377) by known answers, the integer part by Python integers, the scale placement by a
