@@ -43,8 +43,8 @@ enum {
   /* always use the weight-streaming kernels, also where the LDS-tiled kernel applies */
   LO_GEMM_FORCE_STREAMING = 2,
   /* canonical (f32(d) * a_s) * b_s + acc order in every kernel.  Without this flag the
-   * LDS-tiled kernel (128-token tiles, where the scale arithmetic competes with the MFMA
-   * pipe) uses the fused-scale order; the weight-streaming kernels are canonical unless
+   * LDS-tiled kernels (64- and 128-token tiles, where the scale arithmetic competes with
+   * the MFMA pipe) use the fused-scale order; the weight-streaming kernels are canonical unless
    * LO_GEMM_FUSED_SCALE is given. */
   LO_GEMM_CANONICAL_ORDER = 4,
   /* W (for the whole path: w1 and w2) is in the layout of lo_preshuffle_weight_int8 */

@@ -36,8 +36,8 @@ static int validate_common(const char *who, const void *A, const void *As, const
   return LO_OK;
 }
 
-// The LDS-tiled kernel serves the 128-token tile (tokens per expert large enough for
-// the MFMA pipe to matter); everything else streams weights.
+// Token blocks of 64 or 128 rows go to the LDS-tiled kernels (tokens per expert large enough
+// for operand reuse to matter); smaller ones stream weights.
 static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int64_t m_blocks,
                        hipStream_t s) {
   if (a.w4) { // int4 weights: the LDS-tiled kernel at 64-token blocks, else streaming

@@ -1,7 +1,8 @@
 // Grouped block-INT8 GEMM for gfx950, LDS-tiled form for the compute-bound regime.
 //
-// Workgroup tile: 128 gathered token rows x 256 weight rows, 8 wavefronts in a 4 (rows)
-// x 2 (tokens) arrangement.  Each wave owns a 64 x 64 piece as 2 x 2 fragments of
+// Workgroup tile: 64 gathered token rows x 256 weight rows with 4 wavefronts (the default; two
+// such workgroups share a compute unit), or 128 x 256 with 8 wavefronts in a 4 (rows) x 2
+// (tokens) arrangement.  Each wave owns a 64 x 64 piece as 2 x 2 fragments of
 // v_mfma_i32_32x32x32_i8, with the weight fragment as the A operand and the token
 // fragment as the B operand; accumulators and the int32 partial sums stay in VGPRs
 // (64 + 32 registers), so two waves share a SIMD and one wave's MFMAs overlap the other
