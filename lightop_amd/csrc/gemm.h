@@ -85,6 +85,9 @@ bool gemm_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 int launch_gemm_as(const GemmArgs &a, int flags, int64_t m_blocks, hipStream_t s);
 bool gemm_as_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 
+// 128-token kernel with both operands copied global -> LDS (gemm_dma.hip): pre-shuffled int8 weights.
+int launch_gemm_dma(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
+bool gemm_dma_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 // W4A8 LDS-tiled kernel (gemm_w4.hip): block_size_m 64.
 int launch_gemm_w4_tile(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
 bool gemm_w4_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);
