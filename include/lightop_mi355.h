@@ -174,7 +174,7 @@ int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t rows, int6
  *   topk_w [num_valid] f32, used when mul_routed != 0
  *   sorted_ids / expert_ids / num_tokens_post_pad as produced by lo_moe_align_block_size
  *   with block_size == block_size_m; sorted_cap is the extent of sorted_ids.
- * K % 128 == 0, N % 16 == 0.
+ * K % 128 == 0, N % 16 == 0; A, W and C 16-byte aligned.
  */
 int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W, const float *Ws,
                            void *C, int c_dtype, const float *topk_w, const int32_t *sorted_ids,
@@ -189,7 +189,7 @@ int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W, co
  * int8.py:784-823 without materialising intermediate_cache1 / intermediate_cache2.
  *   W [E, 2I, K] (gate rows first, then up rows), Ws [E, 2I/128, K/128]
  *   A2q [num_valid, I] int8, A2s [num_valid, I/128] f32 (rows of -1 blocks untouched)
- * I % 128 == 0, K % 128 == 0.
+ * I % 128 == 0, K % 128 == 0; A, W and A2q 16-byte aligned.
  */
 int lo_moe_gemm1_silu_quant_block_int8(const int8_t *A, const float *As, const int8_t *W,
                                        const float *Ws, int8_t *A2q, float *A2s, int c_dtype,
@@ -329,7 +329,7 @@ int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, int64_t I, i
  * experts_ids, num_tokens_post_pad, top_k, mode, delta) (python/lightop/gemmopt.py:437-457;
  * csrc/moe_gemm/w8a8/moe_w8a8.cu:2389-2536; epilogues :156-166 and :445-470).
  *
- *   As [a_rows] f32, Ws [E, N] f32 (16-byte aligned); everything else as lo_moe_gemm_block_int8.
+ *   As [a_rows] f32, Ws [E, N] f32 (16-byte aligned, like C); everything else as lo_moe_gemm_block_int8.
  *   C[f, n] = T((f32(sum_k A*W) * ts) * Ws[e, n]),  ts = As[f / top_k], or
  *   topk_w[f] * As[f / top_k] with mul_routed;  rows of expert -1 are zero.
  *   flags: LO_GEMM_W_PRESHUFFLED, LO_GEMM_SKIP_NONLOCAL, LO_GEMM_FORCE_STREAMING.

@@ -74,6 +74,37 @@ __device__ __forceinline__ bool tile_of(int bid, int n_tiles, int m_blocks, int 
   return true;
 }
 
+// Output of the 32x32-MFMA kernels.  In the accumulator layout a lane (r = lane & 31, c = lane >> 5)
+// holds, of one 32-token x 64-column piece, token r and columns rb*32 + 8q + 4c + i: four
+// consecutive bf16 per (rb, q).  Stored directly that is 8 bytes to each of 64 different token
+// rows per instruction, and the texture path, which also carries the operand loads these
+// kernels are bound by, spends a cycle per row touched.  Each wave therefore turns its piece
+// around in LDS (LDS operations of one wave execute in order: no barrier) and stores whole
+// 128-byte row segments, eight rows per instruction.
+//   stg   32 * kStgPitch bytes of LDS owned by this wave
+//   o     the lane's 2 x 4 packed column quadruples
+//   slot  output row of token r, or -1 (lanes r and r + 32 agree)
+//   C     + slot * N + col0: first of the piece's 64 columns; 16-byte aligned
+constexpr int kStgPitch = 64 * 2 + 16; // bytes per staged token row: 16 mod 128 keeps both passes conflict-free
+__device__ __forceinline__ void wave_store_32x64_bf16(int8_t *stg, const v4u16 (&o)[2][4], int slot, uint16_t *C,
+                                                      int64_t N, int64_t col0, int lane) {
+  const int r = lane & 31, c = lane >> 5;
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      *reinterpret_cast<v4u16 *>(stg + r * kStgPitch + (rb * 32 + 8 * q + 4 * c) * 2) = o[rb][q];
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int tok = (lane >> 3) + 8 * j;
+    const v4i v = *reinterpret_cast<const v4i *>(stg + tok * kStgPitch + (lane & 7) * 16);
+    const int ft = __shfl(slot, tok);
+    if (ft >= 0) *reinterpret_cast<v4i *>(C + static_cast<int64_t>(ft) * N + col0 + (lane & 7) * 8) = v;
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
 // Weight-streaming kernels (gemm_ws.hip): block_size_m in {16, 32, 64, 128}.
 int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
                    hipStream_t s);

@@ -73,7 +73,7 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm: N (%lld) must be a multiple of 16", (long long)N);
   LO_REQUIRE(N * K < (1ll << 31), LO_ENOTSUP, "moe_gemm: one expert's weights exceed 2 GiB");
   LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm: mul_routed needs topk_weights");
-  LO_REQUIRE((reinterpret_cast<uintptr_t>(C) & 7) == 0, LO_EINVAL, "moe_gemm: C must be 8-byte aligned");
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(C) & 15) == 0, LO_EINVAL, "moe_gemm: C must be 16-byte aligned");
   LO_REQUIRE((num_valid + top_k - 1) / top_k <= a_rows, LO_EINVAL,
              "moe_gemm: %lld slots / top_k %d exceed the %lld rows of A", (long long)num_valid, top_k,
              (long long)a_rows);
@@ -110,8 +110,8 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
              "moe_gemm1_silu_quant: intermediate size (%lld) must be a multiple of 128", (long long)I);
   LO_REQUIRE(2 * I * K < (1ll << 31), LO_ENOTSUP, "moe_gemm1_silu_quant: one expert's weights exceed 2 GiB");
   LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm1_silu_quant: mul_routed needs topk_weights");
-  LO_REQUIRE((reinterpret_cast<uintptr_t>(A2q) & 3) == 0, LO_EINVAL,
-             "moe_gemm1_silu_quant: A2q must be 4-byte aligned");
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(A2q) & 15) == 0, LO_EINVAL,
+             "moe_gemm1_silu_quant: A2q must be 16-byte aligned");
   LO_REQUIRE((num_valid + top_k - 1) / top_k <= a_rows, LO_EINVAL,
              "moe_gemm1_silu_quant: %lld slots / top_k %d exceed the %lld rows of A",
              (long long)num_valid, top_k, (long long)a_rows);
@@ -152,8 +152,8 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   LO_REQUIRE(K <= 131072, LO_ENOTSUP, "moe_gemm_w8a8: K (%lld) could overflow the int32 sum", (long long)K);
   LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm_w8a8: mul_routed needs topk_weights");
   LO_REQUIRE(!(flags & LO_GEMM_W4), LO_ENOTSUP, "moe_gemm_w8a8: int4 weights are not built for the per-channel form");
-  LO_REQUIRE((reinterpret_cast<uintptr_t>(C) & 7) == 0 && (reinterpret_cast<uintptr_t>(Ws) & 15) == 0, LO_EINVAL,
-             "moe_gemm_w8a8: C must be 8-byte and the weight scales 16-byte aligned");
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(C) & 15) == 0 && (reinterpret_cast<uintptr_t>(Ws) & 15) == 0, LO_EINVAL,
+             "moe_gemm_w8a8: C and the weight scales must be 16-byte aligned");
   LO_REQUIRE((num_valid + top_k - 1) / top_k <= a_rows, LO_EINVAL,
              "moe_gemm_w8a8: %lld slots / top_k %d exceed the %lld rows of A", (long long)num_valid, top_k,
              (long long)a_rows);

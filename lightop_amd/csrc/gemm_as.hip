@@ -4,7 +4,7 @@
 // With K of a few hundred bytes the 64 gathered token rows of a token block fit in LDS
 // whole (64 x K bytes plus their group scales).  A workgroup loads them once and then
 // walks several 256-row weight tiles with them: the K loop needs no barrier, no LDS
-// write and no token reload, the weight prefetch runs on across tile boundaries, and the
+// write and no token reload, the weight prefetch (two K blocks deep) runs on across tile boundaries, and the
 // gather of sorted_token_ids is paid once per token block instead of once per tile.
 // Wave tile, MFMA layout, scaling order and output are those of the LDS-tiled kernel
 // (gemm_tile.hip); reference: Triton fused_moe_kernel, python/lightop/_lmslim_native/
@@ -28,6 +28,8 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
   const int pitch = K + 16; // = 16 mod 128: ds_read_b128 of 32 consecutive rows is conflict-free
   int8_t *const sA = smem;
   float *const sS = reinterpret_cast<float *>(smem + kTileM * pitch); // [KB][64]
+  // per-wave staging of 32 output rows x 64 columns (bf16), for row-contiguous stores
+  int8_t *const sStage = smem + kTileM * pitch + KB * kTileM * 4;
 
   int mb, ng;
   if (!tile_of(blockIdx.x, n_groups, m_blocks, group_m, mb, ng)) return;
@@ -110,14 +112,17 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
 
   using B0 = std::integral_constant<int, 0>;
   using B1 = std::integral_constant<int, 1>;
+  using B2 = std::integral_constant<int, 2>;
   v16i zero16;
 #pragma unroll
   for (int i = 0; i < 16; ++i) zero16[i] = 0;
   float acc[2][2][16]; // [token fragment][row fragment][element]
-  v4i wreg[2][2][4];   // [buffer][row fragment][k-step]
-  float bsc[2][2];     // [buffer][row fragment] weight-block scales, fetched with the fragments
+  // Ring of three weight buffers: a K block is short work (16 MFMAs per wave), an L2 round trip
+  // under load is not, so fragments are requested two K blocks ahead.
+  v4i wreg[3][2][4];   // [buffer][row fragment][k-step]
+  float bsc[3][2];     // [buffer][row fragment] weight-block scales, fetched with the fragments
 
-  auto load_w = [&](auto BUF, int nt, int kb) {
+  auto load_w = [&](auto BUF, int nt, int kb) __attribute__((always_inline)) {
     constexpr int b = decltype(BUF)::value;
     const int so = (nt - nt0) * wtstride + kb * wkstride;
 #pragma unroll
@@ -128,7 +133,7 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) bsc[b][rb] = bld_f32(rWs, wsoff[rb], ss);
   };
-  auto fold = [&](const v16i &d, float as, float bs, float *dst) {
+  auto fold = [&](const v16i &d, float as, float bs, float *dst) __attribute__((always_inline)) {
     if constexpr (FAST_SCALE) {
       const float sc = as * bs;
 #pragma unroll
@@ -146,7 +151,7 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
 #pragma unroll
     for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(dst[i]));
   };
-  auto compute = [&](auto BUF, int kb) {
+  auto compute = [&](auto BUF, int kb, bool live) __attribute__((always_inline)) {
     constexpr int b = decltype(BUF)::value;
     // The four 32x32 fragments are software-pipelined: the MFMAs of one fragment are
     // issued, then the previous fragment is folded into the fp32 accumulators while the
@@ -160,7 +165,7 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
       const int8_t *src = sA + (tb * 32 + r) * pitch + kb * kGroup + (SHUF ? c * 16 : c * 64);
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) bf[ks] = *reinterpret_cast<const v4i *>(src + (SHUF ? ks * 32 : ks * 16));
-      const float as = sS[kb * kTileM + tb * 32 + r];
+      const float as = live ? sS[kb * kTileM + tb * 32 + r] : 0.0f; // a step past the end adds 0
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb) {
         v16i d = zero16;
@@ -180,56 +185,70 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  if (nt_end > nt0) load_w(B0{}, nt0, 0); // before the barrier: in flight while the tokens land
-  __syncthreads();                         // the only barrier: the token block is complete
-
-  for (int nt = nt0; nt < nt_end; ++nt) {
+  // The (tile, K block) pairs form one flat sequence of steps; step s uses buffer s % 3.
+  const int total = (nt_end - nt0) * KB;
+  auto load_step = [&](auto BUF, int s) __attribute__((always_inline)) { // a step past the end re-reads the last one
+    const int sc = s < total ? s : total - 1;
+    load_w(BUF, nt0 + sc / KB, sc % KB);
+  };
+  auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[tb][rb][i] = 0.0f;
-    // K/128 is even (host check): buffer 0 always holds an even K block, and the block
-    // after an odd one is the first of the next tile (the last tile re-reads itself)
-    for (int kb = 0; kb < KB; kb += 2) {
-      load_w(B1{}, nt, kb + 1);
-      __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMAs
-      compute(B0{}, kb);
-      const bool wrap = kb + 2 >= KB;
-      const int ntn = wrap ? (nt + 1 < nt_end ? nt + 1 : nt) : nt;
-      load_w(B0{}, ntn, wrap ? 0 : kb + 2);
-      __builtin_amdgcn_sched_barrier(0);
-      compute(B1{}, kb + 1);
-    }
+  };
+  auto store_tile = [&](int nt) __attribute__((always_inline)) {
     const int64_t nrow0 = static_cast<int64_t>(nt) * 256 + wr * 64;
+    int8_t *stg = sStage + wr * (32 * kStgPitch);
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
-      if (!valid[tb]) continue;
       float w = 1.0f;
-      if (a.mul_routed) w = a.topk_w[f[tb]];
+      if (a.mul_routed && valid[tb]) w = a.topk_w[f[tb]];
+      v4u16 o[2][4];
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          v4u16 o;
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             float v = acc[tb][rb][4 * q + i];
             if (a.mul_routed) v = v * w;
-            o[i] = f32_to_bf16(v);
+            o[rb][q][i] = f32_to_bf16(v);
           }
-          *reinterpret_cast<v4u16 *>(a.C + f[tb] * N + nrow0 + rb * 32 + 8 * q + 4 * c) = o;
-        }
+      wave_store_32x64_bf16(stg, o, valid[tb] ? static_cast<int>(f[tb]) : -1, a.C, N, nrow0, lane);
     }
+  };
+  auto step = [&](auto BUF, auto NEXT, int s) __attribute__((always_inline)) {
+    load_step(NEXT, s + 2);
+    __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMAs
+    const int kb = s % KB;
+    compute(BUF, kb, s < total);
+    if (s < total && kb == KB - 1) { // a tile is complete
+      store_tile(nt0 + s / KB);
+      zero_acc();
+    }
+  };
+
+  if (total > 0) { // before the barrier: in flight while the tokens land
+    load_step(B0{}, 0);
+    load_step(B1{}, 1);
+  }
+  __syncthreads(); // the only barrier: the token block is complete
+  zero_acc();
+  for (int s = 0; s < total; s += 3) {
+    step(B0{}, B2{}, s);
+    step(B1{}, B0{}, s + 1);
+    step(B2{}, B1{}, s + 2);
   }
 }
 
-static int64_t as_lds_bytes(int64_t K) { return 64 * (K + 16) + (K / kGroup) * 64 * 4; }
+static int64_t as_lds_bytes(int64_t K) { return 64 * (K + 16) + (K / kGroup) * 64 * 4 + 4 * 32 * kStgPitch; }
 
 bool gemm_as_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
   if (fused_act || block_size_m != 64) return false;
-  if (a.N % 64 != 0 || a.K % 256 != 0) return false;
+  if (a.N % 64 != 0 || (reinterpret_cast<uintptr_t>(a.C) & 15) != 0) return false;
   if (as_lds_bytes(a.K) > 80 * 1024) return false; // two workgroups per CU
   // Pays off only when the launch is several rounds of workgroups deep even with half a
   // token block's weight tiles per workgroup; below that the per-tile kernel balances better.

@@ -251,24 +251,24 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
 
   if constexpr (!FUSED_ACT) {
     if (!wave_active) return;
+    // the K loop ended with a barrier: the token tile's LDS is free and serves as store staging
+    int8_t *stg = &sA[0][0] + wave * (32 * kStgPitch);
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
-      if (!valid[tb]) continue;
       float w = 1.0f;
-      if (a.mul_routed) w = a.topk_w[f[tb]];
+      if (a.mul_routed && valid[tb]) w = a.topk_w[f[tb]];
+      v4u16 o[2][4];
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          v4u16 o;
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             float v = acc[tb][rb][4 * q + i];
             if (a.mul_routed) v = v * w;
-            o[i] = f32_to_bf16(v);
+            o[rb][q][i] = f32_to_bf16(v);
           }
-          *reinterpret_cast<v4u16 *>(a.C + f[tb] * N + nrow[rb] + 8 * q + 4 * c) = o;
-        }
+      wave_store_32x64_bf16(stg, o, valid[tb] ? static_cast<int>(f[tb]) : -1, a.C, N, nrow[0], lane);
     }
   } else {
     // acc[.][0] = gate, acc[.][1] = up for activation columns nt*128 + wr*32 + 8q + 4c + i
@@ -294,20 +294,31 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     }
     __syncthreads();
     const int64_t G = I / kGroup;
+    // The quantised tile (kTileM tokens x 128 columns of int8) goes through LDS as well, so that
+    // it leaves as whole 128-byte rows instead of 4-byte pieces; the token tile's LDS is free.
+    constexpr int kQPitch = kGroup + 16;
+    int8_t *qst = &sA[0][0];
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
-      if (!valid[tb]) continue;
       float amax = fmaxf(fmaxf(sRed[wt][tb][0][r], sRed[wt][tb][1][r]),
                          fmaxf(sRed[wt][tb][2][r], sRed[wt][tb][3][r]));
       amax = fmaxf(amax, 1e-10f);
       const float sc = amax / 127.0f;
       const float rsc = 1.0f / sc;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t packed = quant4(&actf[tb][4 * q], sc, rsc);
-        *reinterpret_cast<uint32_t *>(a.A2q + f[tb] * I + nrow[0] + 8 * q + 4 * c) = packed;
-      }
-      if (wr == 0 && c == 0) a.A2s[f[tb] * G + nt] = sc;
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<uint32_t *>(qst + (wt * 64 + tb * 32 + r) * kQPitch + wr * 32 + 8 * q + 4 * c) =
+            quant4(&actf[tb][4 * q], sc, rsc);
+      if (valid[tb] && wr == 0 && c == 0) a.A2s[f[tb] * G + nt] = sc;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kTileM * 8 / (256 * WT); ++j) {
+      const int id = tid + 256 * WT * j, tok = id >> 3, piece = id & 7;
+      const int64_t ft = a.sorted[static_cast<int64_t>(mb) * kTileM + tok];
+      if (ft < a.num_valid)
+        *reinterpret_cast<v4i *>(a.A2q + ft * I + static_cast<int64_t>(nt) * kGroup + piece * 16) =
+            *reinterpret_cast<const v4i *>(qst + tok * kQPitch + piece * 16);
     }
   }
 }
