@@ -313,25 +313,25 @@ void moe_gemm_dma_kernel(const GemmArgs a, int m_blocks, int group_m) {
   __builtin_amdgcn_s_waitcnt(0); // no copy may still be writing LDS when the epilogue reuses it or the wave ends
 
   if constexpr (!FUSED_ACT) {
+    __syncthreads(); // every wave's copies have landed and its operand reads are done: the stages are free
     if (!wave_active) return;
+    int8_t *stg = smem + wave * (32 * kStgPitch);
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
-      if (!valid[tb]) continue;
       float w = 1.0f;
-      if (a.mul_routed) w = a.topk_w[f[tb]];
+      if (a.mul_routed && valid[tb]) w = a.topk_w[f[tb]];
+      v4u16 o[2][4];
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          v4u16 o;
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             float v = acc[tb][rb][4 * q + i];
             if (a.mul_routed) v = v * w;
-            o[i] = f32_to_bf16(v);
+            o[rb][q][i] = f32_to_bf16(v);
           }
-          *reinterpret_cast<v4u16 *>(a.C + f[tb] * N + nrow[rb] + 8 * q + 4 * c) = o;
-        }
+      wave_store_32x64_bf16(stg, o, valid[tb] ? static_cast<int>(f[tb]) : -1, a.C, N, nrow[0], lane);
     }
   } else {
     // acc[.][0] = gate, acc[.][1] = up for activation columns nt*128 + wr*32 + 8q + 4c + i
@@ -355,22 +355,32 @@ void moe_gemm_dma_kernel(const GemmArgs a, int m_blocks, int group_m) {
       amax = fmaxf(amax, __shfl_xor(amax, 32));
       if (c == 0) sRed[((wt * 2 + tb) * 4 + wr) * 32 + r] = amax;
     }
-    __syncthreads();
+    __syncthreads(); // also: every wave's copies have landed and its operand reads are done
     const int64_t G = I / kGroup;
+    // the quantised tile (128 tokens x 128 columns of int8) leaves through LDS as whole rows
+    constexpr int kQPitch = kGroup + 16;
+    int8_t *qst = smem;
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
-      if (!valid[tb]) continue;
       const float *red = sRed + (wt * 2 + tb) * 4 * 32 + r;
       float amax = fmaxf(fmaxf(red[0], red[32]), fmaxf(red[64], red[96]));
       amax = fmaxf(amax, 1e-10f);
       const float sc = amax / 127.0f;
       const float rsc = 1.0f / sc;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t packed = quant4(&actf[tb][4 * q], sc, rsc);
-        *reinterpret_cast<uint32_t *>(a.A2q + f[tb] * I + nrow[0] + 8 * q + 4 * c) = packed;
-      }
-      if (wr == 0 && c == 0) a.A2s[f[tb] * G + nt] = sc;
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<uint32_t *>(qst + (wt * 64 + tb * 32 + r) * kQPitch + wr * 32 + 8 * q + 4 * c) =
+            quant4(&actf[tb][4 * q], sc, rsc);
+      if (valid[tb] && wr == 0 && c == 0) a.A2s[f[tb] * G + nt] = sc;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kDmaTokens * 8 / 512; ++j) {
+      const int id = tid + 512 * j, tok = id >> 3, piece = id & 7;
+      const int64_t ft = a.sorted[static_cast<int64_t>(mb) * kDmaTokens + tok];
+      if (ft < a.num_valid)
+        *reinterpret_cast<v4i *>(a.A2q + ft * I + static_cast<int64_t>(nt) * kGroup + piece * 16) =
+            *reinterpret_cast<const v4i *>(qst + tok * kQPitch + piece * 16);
     }
   }
 }

@@ -168,23 +168,26 @@ __device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       bs4[rb][q] = __builtin_bit_cast(v4f, bld16(rWs, static_cast<int>(nrow[rb] + 8 * q + 4 * c) * 4, 0));
+  // the K loop ended with a barrier: the token tile's LDS is free and serves as store staging
+  int8_t *stg = &sA[0][0] + wr * (32 * kStgPitch);
 #pragma unroll
   for (int tb = 0; tb < TB; ++tb) {
-    if (!valid[tb]) continue;
-    float ts = a.As[f[tb] / a.top_k];
-    if (a.mul_routed) ts = a.topk_w[f[tb]] * ts;
+    float ts = 0.0f;
+    if (valid[tb]) {
+      ts = a.As[f[tb] / a.top_k];
+      if (a.mul_routed) ts = a.topk_w[f[tb]] * ts;
+    }
+    v4u16 o[2][4];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        v4u16 o;
+      for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float t = static_cast<float>(acc[tb][rb][4 * q + i]) * ts;
-          o[i] = f32_to_bf16(t * bs4[rb][q][i]);
+          o[rb][q][i] = f32_to_bf16(t * bs4[rb][q][i]);
         }
-        *reinterpret_cast<v4u16 *>(a.C + f[tb] * N + nrow[rb] + 8 * q + 4 * c) = o;
-      }
+    wave_store_32x64_bf16(stg, o, valid[tb] ? static_cast<int>(f[tb]) : -1, a.C, N, nrow[0], lane);
   }
 }
 

@@ -234,14 +234,17 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   }
 
   if constexpr (!FUSED_ACT) {
+    // A lane holds 4 consecutive columns of one token per fragment; stored directly that is
+    // 8 bytes to each of 64 rows per instruction.  Each wave turns a 16-token x 64-column piece
+    // around in LDS (in order within a wave: no barrier; the token tile's LDS is free after the K
+    // loop's last barrier) and stores 128-byte row segments instead.
+    int8_t *stg = &sA[0][0] + wr * (16 * kW4Row);
 #pragma unroll
     for (int tf = 0; tf < 4; ++tf) {
-      if (!valid[tf]) continue;
       float w = 1.0f;
-      if (a.mul_routed) w = a.topk_w[f[tf]];
+      if (a.mul_routed && valid[tf]) w = a.topk_w[f[tf]];
 #pragma unroll
       for (int rf = 0; rf < 4; ++rf) {
-        if (nrow[rf] >= N) continue;
         v4u16 o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -249,8 +252,20 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
           if (a.mul_routed) v = v * w;
           o[i] = f32_to_bf16(v);
         }
-        *reinterpret_cast<v4u16 *>(a.C + f[tf] * N + nrow[rf] + 4 * q) = o;
+        *reinterpret_cast<v4u16 *>(stg + r * kW4Row + (rf * 16 + 4 * q) * 2) = o;
       }
+      __builtin_amdgcn_wave_barrier();
+      const int slot = valid[tf] ? static_cast<int>(f[tf]) : -1;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int tok = (lane >> 3) + 8 * j;
+        const v4i v = *reinterpret_cast<const v4i *>(stg + tok * kW4Row + (lane & 7) * 16);
+        const int ft = __shfl(slot, tok);
+        // columns past N (a last tile narrower than 256) are never stored: N % 64 == 0 on this path
+        if (ft >= 0 && nrow[0] < N)
+          *reinterpret_cast<v4i *>(a.C + static_cast<int64_t>(ft) * N + nrow[0] + (lane & 7) * 8) = v;
+      }
+      __builtin_amdgcn_wave_barrier();
     }
   } else {
     // acc[0..1] = gate, acc[2..3] = up for activation columns nt*128 + wr*32 + 16*g + 4q + i
@@ -279,26 +294,34 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     }
     __syncthreads();
     const int64_t G = I / kGroup;
+    // the quantised tile (64 tokens x 128 columns of int8) leaves through LDS as whole rows
+    int8_t *qst = &sA[0][0];
 #pragma unroll
     for (int tf = 0; tf < 4; ++tf) {
-      if (!valid[tf]) continue;
       const int t = tf * 16 + r;
       float amax = fmaxf(fmaxf(sRed[0][t], sRed[1][t]), fmaxf(sRed[2][t], sRed[3][t]));
       amax = fmaxf(amax, 1e-10f);
       const float sc = amax / 127.0f;
       const float rsc = 1.0f / sc;
 #pragma unroll
-      for (int g = 0; g < 2; ++g) {
-        const uint32_t packed = quant4(actf[tf][g], sc, rsc);
-        *reinterpret_cast<uint32_t *>(a.A2q + f[tf] * I + nrow[g] + 4 * q) = packed;
-      }
-      if (wr == 0 && q == 0) a.A2s[f[tf] * G + nt] = sc;
+      for (int g = 0; g < 2; ++g)
+        *reinterpret_cast<uint32_t *>(qst + t * kW4Row + wr * 32 + g * 16 + 4 * q) = quant4(actf[tf][g], sc, rsc);
+      if (valid[tf] && wr == 0 && q == 0) a.A2s[f[tf] * G + nt] = sc;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kTileM * 8 / 256; ++j) {
+      const int id = tid + 256 * j, tok = id >> 3, piece = id & 7;
+      const int64_t ft = a.sorted[static_cast<int64_t>(mb) * kTileM + tok];
+      if (ft < a.num_valid)
+        *reinterpret_cast<v4i *>(a.A2q + ft * I + static_cast<int64_t>(nt) * kGroup + piece * 16) =
+            *reinterpret_cast<const v4i *>(qst + tok * kW4Row + piece * 16);
     }
   }
 }
 
 bool gemm_w4_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
-  (void)fused_act;
+  if (!fused_act && a.N % 64 != 0) return false; // a wave stores its 64 columns as one piece
   return a.w4 && a.w_shuffled && block_size_m == 64;
 }
 
