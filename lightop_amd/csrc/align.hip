@@ -30,7 +30,7 @@ __device__ __forceinline__ int64_t local_slots(int64_t numel, const int32_t *__r
 }
 
 template <typename IdT>
-__global__ __launch_bounds__(1024) void moe_align_kernel(
+__device__ __forceinline__ void moe_align_body(
     const IdT *__restrict__ ids, int64_t numel, int num_experts, int bs,
     const int32_t *__restrict__ expert_map, int ignore_invalid, int32_t *__restrict__ sorted,
     int64_t sorted_cap, int32_t *__restrict__ expert_ids, int64_t expert_ids_cap,
@@ -165,6 +165,36 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
     }
+  }
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(1024) void moe_align_kernel(
+    const IdT *__restrict__ ids, int64_t numel, int num_experts, int bs,
+    const int32_t *__restrict__ expert_map, int ignore_invalid, int32_t *__restrict__ sorted,
+    int64_t sorted_cap, int32_t *__restrict__ expert_ids, int64_t expert_ids_cap,
+    int32_t *__restrict__ ntpp, int key_bits, uint8_t *__restrict__ slot_mask,
+    const int32_t *__restrict__ num_local_tokens, int slots_per_token) {
+  moe_align_body<IdT>(ids, numel, num_experts, bs, expert_map, ignore_invalid, sorted, sorted_cap, expert_ids,
+                      expert_ids_cap, ntpp, key_bits, slot_mask, num_local_tokens, slots_per_token);
+}
+
+// Workgroup 0 aligns, the others quantise the activations: two independent stages, one launch.
+template <typename IdT>
+__global__ __launch_bounds__(1024) void quant_align_kernel(
+    const uint16_t *__restrict__ x, int64_t groups, float eps, int8_t *__restrict__ q, float *__restrict__ qs,
+    const IdT *__restrict__ ids, int64_t numel, int num_experts, int bs,
+    const int32_t *__restrict__ expert_map, int32_t *__restrict__ sorted, int64_t sorted_cap,
+    int32_t *__restrict__ expert_ids, int64_t expert_ids_cap, int32_t *__restrict__ ntpp, int key_bits,
+    uint8_t *__restrict__ slot_mask) {
+  if (blockIdx.x == 0) {
+    moe_align_body<IdT>(ids, numel, num_experts, bs, expert_map, 0, sorted, sorted_cap, expert_ids, expert_ids_cap,
+                        ntpp, key_bits, slot_mask, nullptr, 1);
+  } else {
+    const int per_block = blockDim.x >> 4; // groups a workgroup handles per pass
+    group_quant_body<LO_BF16>(x, groups, eps, q, qs,
+                              static_cast<int64_t>(blockIdx.x - 1) * per_block + (threadIdx.x >> 4),
+                              static_cast<int64_t>(gridDim.x - 1) * per_block, threadIdx.x & 15);
   }
 }
 
@@ -349,6 +379,15 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
 }
 
 // chunks for the multi-workgroup path: about 1024 slots each, at most 256 chunks
+static void single_wg_shape(int64_t numel, int32_t num_experts, int *nw, size_t *lds_bytes) {
+  // waves per workgroup: as many as the per-wave LDS counters allow (<= 60 KB)
+  int w = 16;
+  while (w > 1 && (static_cast<int64_t>(w) + 2) * num_experts + 1 > 15360) w >>= 1;
+  if (numel <= 64 * 4) w = w < 4 ? w : 4;
+  *nw = w;
+  *lds_bytes = (static_cast<size_t>(w + 2) * num_experts + 1) * sizeof(int32_t);
+}
+
 static void align_chunks(int64_t numel, int *nchunks, int64_t *chunk_slots) {
   int64_t n = (numel + 1023) / 1024;
   if (n > 256) n = 256;
@@ -357,6 +396,44 @@ static void align_chunks(int64_t numel, int *nchunks, int64_t *chunk_slots) {
   cs = (cs + 255) / 256 * 256;
   *chunk_slots = cs;
   *nchunks = static_cast<int>((numel + cs - 1) / cs);
+}
+
+int launch_quant_align(const void *x, int64_t M, int64_t H, float eps, int8_t *q, float *qs,
+                       const void *topk_ids, int ids_dtype, int64_t numel, int32_t num_experts,
+                       int32_t block_size, const int32_t *expert_map, int32_t *sorted_ids, int64_t sorted_cap,
+                       int32_t *expert_ids, int64_t expert_ids_cap, int32_t *num_tokens_post_pad,
+                       uint8_t *slot_mask, hipStream_t stream) {
+  if (lo_moe_align_scratch_bytes(numel, num_experts) > 0) return LO_ENOTSUP; // the multi-workgroup form
+  LO_REQUIRE(x && q && qs && topk_ids && sorted_ids && expert_ids && num_tokens_post_pad, LO_EINVAL,
+             "quant_align: null pointer");
+  LO_REQUIRE(H > 0 && H % kGroup == 0 && M >= 1 && numel >= 1 && num_experts >= 1 && num_experts <= 2048 &&
+                 block_size >= 1,
+             LO_EINVAL, "quant_align: bad shape");
+  int64_t need = numel + static_cast<int64_t>(num_experts) * (block_size - 1);
+  if (numel < num_experts && numel * block_size < need) need = numel * block_size;
+  LO_REQUIRE(sorted_cap >= need && expert_ids_cap >= (need + block_size - 1) / block_size, LO_ENOSPC,
+             "quant_align: alignment buffers too small");
+  int key_bits = 1;
+  while ((1 << key_bits) < num_experts) ++key_bits;
+  int nw;
+  size_t lds_bytes;
+  single_wg_shape(numel, num_experts, &nw, &lds_bytes);
+  const int64_t groups = M * (H / kGroup);
+  const int per_block = nw * kWave / 16;
+  int64_t qblocks = (groups + per_block - 1) / per_block;
+  if (qblocks > 4096) qblocks = 4096;
+  const dim3 grid(static_cast<unsigned>(1 + qblocks)), block(nw * kWave);
+  if (ids_dtype == LO_I32)
+    hipLaunchKernelGGL(quant_align_kernel<int32_t>, grid, block, lds_bytes, stream, static_cast<const uint16_t *>(x),
+                       groups, eps, q, qs, static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,
+                       expert_map, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, num_tokens_post_pad, key_bits,
+                       slot_mask);
+  else
+    hipLaunchKernelGGL(quant_align_kernel<int64_t>, grid, block, lds_bytes, stream, static_cast<const uint16_t *>(x),
+                       groups, eps, q, qs, static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size,
+                       expert_map, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, num_tokens_post_pad, key_bits,
+                       slot_mask);
+  return check_launch("quant_align");
 }
 
 } // namespace lo
@@ -465,11 +542,9 @@ extern "C" int lo_moe_align_block_size_local(const void *topk_ids, int ids_dtype
     return check_launch("moe_align_block_size(multi)");
   }
 
-  // waves per workgroup: as many as the per-wave LDS counters allow (<= 60 KB)
-  int nw = 16;
-  while (nw > 1 && (static_cast<int64_t>(nw) + 2) * num_experts + 1 > 15360) nw >>= 1;
-  if (numel <= 64 * 4) nw = nw < 4 ? nw : 4;
-  size_t lds_bytes = (static_cast<size_t>(nw + 2) * num_experts + 1) * sizeof(int32_t);
+  int nw;
+  size_t lds_bytes;
+  single_wg_shape(numel, num_experts, &nw, &lds_bytes);
   if (ids_dtype == LO_I32)
     hipLaunchKernelGGL(moe_align_kernel<int32_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
                        static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,

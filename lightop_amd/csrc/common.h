@@ -192,4 +192,44 @@ __device__ __forceinline__ uint32_t quant4(const float *v, float s, float y) {
   return pack4_i8(quant_one(v[0], s), quant_one(v[1], s), quant_one(v[2], s), quant_one(v[3], s));
 }
 
+// per_token_group_quant_int8 for the groups g = first + i * stride (reference:
+// python/lightop/_lmslim_native/layers/gemm/int8_utils.py:74-122).  16 lanes own one group of
+// 128 values (8 each); amax is reduced across those 16 lanes; the division is IEEE.
+template <int DT>
+__device__ __forceinline__ void group_quant_body(const uint16_t *__restrict__ x, int64_t groups, float eps,
+                                                 int8_t *__restrict__ q, float *__restrict__ s, int64_t first,
+                                                 int64_t stride, int sub) {
+  for (int64_t g = first; g < groups; g += stride) {
+    const v8u16 raw = *reinterpret_cast<const v8u16 *>(x + g * kGroup + sub * 8);
+    float v[8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      v[i] = to_f32<DT>(raw[i]);
+      amax = fmaxf(amax, fabsf(v[i]));
+    }
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+    amax = fmaxf(amax, eps);
+    const float sc = amax / 127.0f;
+    int qi[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qi[i] = quant_one(v[i], sc);
+    v2i packed;
+    packed[0] = static_cast<int>(pack4_i8(qi[0], qi[1], qi[2], qi[3]));
+    packed[1] = static_cast<int>(pack4_i8(qi[4], qi[5], qi[6], qi[7]));
+    *reinterpret_cast<v2i *>(q + g * kGroup + sub * 8) = packed;
+    if (sub == 0) s[g] = sc;
+  }
+}
+
+// Group quant of x [M, H] and the single-workgroup routing alignment in ONE launch (they are
+// independent; at decode sizes a launch costs as much as either).  Returns LO_ENOTSUP when the
+// alignment needs its multi-workgroup form: the caller then launches the two stages separately.
+int launch_quant_align(const void *x, int64_t M, int64_t H, float eps, int8_t *q, float *s,
+                       const void *topk_ids, int ids_dtype, int64_t numel, int32_t num_experts,
+                       int32_t block_size, const int32_t *expert_map, int32_t *sorted_ids, int64_t sorted_cap,
+                       int32_t *expert_ids, int64_t expert_ids_cap, int32_t *num_tokens_post_pad,
+                       uint8_t *slot_mask, hipStream_t stream);
+
 } // namespace lo

@@ -8,39 +8,15 @@
 namespace lo {
 
 // ---- per_token_group_quant_int8 ----------------------------------------------
-// Reference: python/lightop/_lmslim_native/layers/gemm/int8_utils.py:74-122.
-// 16 lanes own one group of 128 values (8 each); amax is reduced across those 16
-// lanes with DPP-free shuffles; the division is IEEE (x / s, never x * (1/s)).
+// Reference: python/lightop/_lmslim_native/layers/gemm/int8_utils.py:74-122; the body is
+// group_quant_body (common.h), shared with the fused quant + alignment launch.
 template <int DT>
 __global__ __launch_bounds__(256) void group_quant_kernel(const uint16_t *__restrict__ x,
                                                           int64_t groups, float eps,
                                                           int8_t *__restrict__ q,
                                                           float *__restrict__ s) {
-  const int sub = threadIdx.x & 15;
-  int64_t g = static_cast<int64_t>(blockIdx.x) * 16 + (threadIdx.x >> 4);
-  const int64_t gstride = static_cast<int64_t>(gridDim.x) * 16;
-  for (; g < groups; g += gstride) {
-    const v8u16 raw = *reinterpret_cast<const v8u16 *>(x + g * kGroup + sub * 8);
-    float v[8];
-    float amax = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      v[i] = to_f32<DT>(raw[i]);
-      amax = fmaxf(amax, fabsf(v[i]));
-    }
-#pragma unroll
-    for (int d = 1; d < 16; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
-    amax = fmaxf(amax, eps);
-    const float sc = amax / 127.0f;
-    int qi[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) qi[i] = quant_one(v[i], sc);
-    v2i packed;
-    packed[0] = static_cast<int>(pack4_i8(qi[0], qi[1], qi[2], qi[3]));
-    packed[1] = static_cast<int>(pack4_i8(qi[4], qi[5], qi[6], qi[7]));
-    *reinterpret_cast<v2i *>(q + g * kGroup + sub * 8) = packed;
-    if (sub == 0) s[g] = sc;
-  }
+  group_quant_body<DT>(x, groups, eps, q, s, static_cast<int64_t>(blockIdx.x) * 16 + (threadIdx.x >> 4),
+                       static_cast<int64_t>(gridDim.x) * 16, threadIdx.x & 15);
 }
 
 // ---- silu_and_mul --------------------------------------------------------------
