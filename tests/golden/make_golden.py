@@ -13,6 +13,8 @@ tree, checks the HIP path against fixed bytes as well as against the live oracle
                      shared_output, routed_scaling_factor 2.5)
   tiny_config1.json  the tiny benchmark configuration (E=8, top-2, H=1024, I=512, M=64, seed 0):
                      routing outputs in full, sha256 of every other stage's bytes
+  tiny_forms.json    the same tiny layer in the per-channel W8A8 form and in the W4A8 form with
+                     K-group scales (M=64, seed 0, block 16): sha256 of the inputs and of every stage
   align_docstring.json  the one literal known answer the reference holds
                      (moe_align_block_size.py:66-81)
 """
@@ -79,6 +81,24 @@ def tiny_config1():
         json.dump(doc, f, indent=1)
 
 
+def tiny_forms():
+    doc = {}
+    for name, layer, fn in (("channel", wl.TINY_PC, cpu_oracle.fused_experts_channel_int8),
+                            ("w4a8", wl.TINY_W4, cpu_oracle.fused_experts_w4a8)):
+        w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
+        x, tw, ids = wl.make_inputs(layer, 64, seed=0)
+        r = fn(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
+        doc[name] = {
+            "config": f"{layer.name}: E=8 top-2 H=1024 I=512 M=64 seed 0 block_size_m=16",
+            "inputs_sha256": {"x": sha(x), "w1": sha(w1), "w2": sha(w2), "w1_scale": sha(w1s), "w2_scale": sha(w2s),
+                              "topk_ids": sha(ids)},
+            "sha256": {k: sha(r[k]) for k in ("a1q", "a1s", "c1", "a2q", "a2s", "c3", "out")},
+            "out_first_row_bf16_bits": raw(r["out"])[0, :16].tolist(),
+        }
+    with open(os.path.join(HERE, "tiny_forms.json"), "w") as f:
+        json.dump(doc, f, indent=1)
+
+
 def align_docstring():
     doc = {"source": "python/lightop/_lmslim_native/vllm_compat/moe_align_block_size.py:66-81",
            "topk_ids": [[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]], "block_size": 4, "num_experts": 5,
@@ -91,5 +111,6 @@ def align_docstring():
 if __name__ == "__main__":
     small_layer()
     tiny_config1()
+    tiny_forms()
     align_docstring()
     print("wrote", sorted(f for f in os.listdir(HERE) if not f.endswith(".py")))

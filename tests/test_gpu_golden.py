@@ -108,3 +108,28 @@ def test_tiny_config1_digests(dev):
     assert sha(cache13[: 128 * 1024].view(128, 1024)) == doc["sha256"]["c3"]
     assert sha(out) == doc["sha256"]["out"]
     assert bits(out.cpu())[0, :16].tolist() == doc["out_first_row_bf16_bits"]
+
+
+@pytest.mark.parametrize("form", ["channel", "w4a8"])
+def test_tiny_forms_digests(dev, form):
+    """The tiny layer in the per-channel and W4A8 forms: whole path and second GEMM's output by digest."""
+    from lightop_amd import _lib, moe, workloads as wl
+
+    print(f"[case] golden tiny layer, {form}", flush=True)
+    doc = json.load(open(os.path.join(GOLDEN, "tiny_forms.json")))[form]
+    layer = {"channel": wl.TINY_PC, "w4a8": wl.TINY_W4}[form]
+    w1, w2, w1s, w2s = (t.to(dev) for t in wl.make_weights(layer, seed=0))
+    x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, 64, seed=0))
+    assert sha(x) == doc["inputs_sha256"]["x"] and sha(w1) == doc["inputs_sha256"]["w1"]
+    cache13 = torch.empty(64 * 2 * 1024, dtype=torch.bfloat16, device=dev)
+    if form == "channel":
+        out = moe.fused_experts_impl_int8(x, w1, w2, tw, ids, cache13, use_int8_w8a8=True, per_channel_quant=True,
+                                          w1_scale=w1s, w2_scale=w2s, block_shape=None, lightop_amd_block_size_m=16)
+    else:
+        out = moe.fused_experts_impl_w4a8(x, moe.preshuffle_moe_weight_int4(w1), moe.preshuffle_moe_weight_int4(w2), tw,
+                                          ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=[1, 128],
+                                          lightop_amd_block_size_m=16, lightop_amd_flags=_lib.LO_GEMM_CANONICAL_ORDER)
+    torch.cuda.synchronize()
+    assert sha(cache13[: 128 * 1024].view(128, 1024)) == doc["sha256"]["c3"]
+    assert sha(out) == doc["sha256"]["out"]
+    assert bits(out.cpu())[0, :16].tolist() == doc["out_first_row_bf16_bits"]

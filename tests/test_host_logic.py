@@ -229,6 +229,28 @@ def test_golden_tiny_config1_oracle(oracle):
         assert sha(r[k]) == h, k
 
 
+@pytest.mark.parametrize("form", ["channel", "w4a8"])
+def test_golden_tiny_forms_oracle(oracle, form):
+    """The per-channel and W4A8 forms of the tiny layer: the oracle still produces the committed digests."""
+    from lightop_amd import workloads as wl
+
+    doc = json.load(open(os.path.join(GOLDEN, "tiny_forms.json")))[form]
+    layer, fn = {"channel": (wl.TINY_PC, oracle.fused_experts_channel_int8),
+                 "w4a8": (wl.TINY_W4, oracle.fused_experts_w4a8)}[form]
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
+    x, tw, ids = wl.make_inputs(layer, 64, seed=0)
+
+    def sha(t):
+        a = t.contiguous().view(torch.int16).numpy() if t.dtype == torch.bfloat16 else t.contiguous().numpy()
+        return hashlib.sha256(a.tobytes()).hexdigest()
+
+    assert {"x": sha(x), "w1": sha(w1), "w1_scale": sha(w1s), "topk_ids": sha(ids)}.items() \
+        <= doc["inputs_sha256"].items(), "the workload generator no longer reproduces the fixture's inputs"
+    r = fn(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
+    for k, h in doc["sha256"].items():
+        assert sha(r[k]) == h, k
+
+
 def test_golden_align_docstring(oracle):
     doc = json.load(open(os.path.join(GOLDEN, "align_docstring.json")))
     s, e, p = oracle.moe_align_block_size(torch.tensor(doc["topk_ids"], dtype=torch.int32), doc["block_size"],
