@@ -70,7 +70,8 @@ static WsLayout ws_layout(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_
 // gfx950 tile table.  The token tile (= alignment block) follows the expected number
 // of slots per expert: small tiles waste no MFMA columns on padding while the layer
 // is weight-streaming bound, larger ones amortise each pass over an expert's weights.
-static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int form = LO_FORM_BLOCK) {
+static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64_t H, int form = LO_FORM_BLOCK,
+                            bool preshuffled = true) {
   const double per_expert = static_cast<double>(M) * top_k / (num_experts > 0 ? num_experts : 1);
   // W4A8: the streaming kernel re-reads the token rows per wave, which outweighs the half-size
   // weights early; the LDS-tiled kernel (64 tokens) wins from about 8 slots per expert.
@@ -80,9 +81,16 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int f
   // Per-channel form: no scale arithmetic in the K loop, so the accumulators of 128 tokens fit
   // and the larger tile halves the weight bytes requested from L2 per multiply-add.
   if (form == LO_FORM_CHANNEL && per_expert >= 64.0) return 128;
-  // 64-token LDS tiles: two workgroups per CU hide each other's barrier and memory
-  // waits, which measured faster than the 128-token tile (one workgroup per CU) on
-  // every layer shape tried.
+  // Block form, pre-shuffled weights, an expert's slots fill a 128-token block: the kernel that
+  // copies both operands straight into LDS (gemm_t128.hip) requests 40 % fewer operand bytes from
+  // L2 per multiply-add and skips the padded part of a block in steps of 32 tokens (measured:
+  // DeepSeek-V3 layer at 8192 tokens 5.41 -> 4.73 ms, its 32-expert share at 4096 tokens
+  // 0.646 -> 0.594 ms, Qwen3-30B-A3B layer at 8192 tokens 0.773 -> 0.745 ms).  With a short K
+  // its longer epilogue weighs more: at 128 slots per expert the Qwen3 layer (K = 2048) is 4 %
+  // slower with it, so the threshold there is 256.  Row-major weights stay at 64: their
+  // 128-token kernel is one phase-locked workgroup per CU and measured slower on every layer
+  // shape tried.
+  if (form == LO_FORM_BLOCK && preshuffled && per_expert >= (H >= 4096 ? 128.0 : 256.0)) return 128;
   return 64;
 }
 
@@ -98,7 +106,7 @@ extern "C" int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts
   (void)E_local;
   LO_REQUIRE(M >= 0 && num_experts >= 1 && top_k >= 1 && H > 0 && I > 0, LO_EINVAL,
              "moe_tile_query: bad problem size");
-  const int32_t bm = pick_block_m(M, num_experts, top_k);
+  const int32_t bm = pick_block_m(M, num_experts, top_k, H);
   if (gemm1) *gemm1 = lo_moe_tile{bm, 1, 8, 256};
   if (gemm2) *gemm2 = lo_moe_tile{bm, 0, 4, 64};
   return LO_OK;
@@ -111,7 +119,7 @@ extern "C" int lo_moe_tile_query_form(int form, int64_t M, int32_t E_local, int3
   LO_REQUIRE(form == LO_FORM_CHANNEL || form == LO_FORM_W4, LO_EINVAL, "moe_tile_query_form: unknown form %d", form);
   LO_REQUIRE(M >= 0 && num_experts >= 1 && top_k >= 1 && H > 0 && I > 0, LO_EINVAL,
              "moe_tile_query_form: bad problem size");
-  const int32_t bm = pick_block_m(M, num_experts, top_k, form);
+  const int32_t bm = pick_block_m(M, num_experts, top_k, H, form);
   if (gemm1) *gemm1 = lo_moe_tile{bm, bm >= 64 ? 2 : 0, bm >= 64 || form == LO_FORM_CHANNEL ? 4 : 8, bm >= 64 ? 256 : 64};
   if (gemm2) *gemm2 = lo_moe_tile{bm, bm >= 64 ? 2 : 0, 4, bm >= 64 ? 256 : 64};
   return LO_OK;
@@ -155,7 +163,8 @@ extern "C" int lo_fused_experts_block_int8(
              "fused_experts: workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
   if (block_size_m == 0)
-    block_size_m = pick_block_m(M, num_experts, top_k, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK);
+    block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
+                                (flags & LO_GEMM_W_PRESHUFFLED) != 0);
   LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
              LO_EINVAL, "fused_experts: block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
   const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
@@ -224,7 +233,7 @@ extern "C" int lo_fused_experts_channel_int8(
   LO_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, LO_EINVAL,
              "fused_experts(channel): workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
-  if (block_size_m == 0) block_size_m = pick_block_m(M, num_experts, top_k, LO_FORM_CHANNEL);
+  if (block_size_m == 0) block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_CHANNEL);
   LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
              LO_EINVAL, "fused_experts(channel): block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
   // the block layout is roomy enough: its scale segments hold one float per 128 values

@@ -155,6 +155,26 @@ __device__ __forceinline__ uint16_t silu_mul_band(const uint16_t *band, const ui
   return f32_to_bf16(bf16_to_f32(sg16) * bf16_to_f32(u16));
 }
 
+// The same lookup as straight-line code, for epilogues that push dozens of unrelated values per
+// lane through it: lanes of a wave never agree on an arm, so per-value branches only add
+// exec-mask bookkeeping and keep the LDS reads from being issued back to back.  The three
+// common arms are computed and selected; NaN and -inf gates are NOT handled here: the caller
+// ORs silu_gate_special() over its values and, if any lane of the wave saw one, redoes the
+// values with silu_mul_band().
+__device__ __forceinline__ uint16_t silu_mul_band_common(const uint16_t *band, uint16_t g16, uint16_t u16) {
+  const uint32_t mag = g16 & 0x7fffu, neg = g16 >> 15;
+  const uint32_t bi = mag - kSiluBandLo; // wraps around below the band
+  const bool inside = bi < static_cast<uint32_t>(kSiluBandN);
+  const uint16_t in_band = band[(inside ? bi : 0u) + neg * kSiluBandN];
+  const uint16_t below = f32_to_bf16(bf16_to_f32(g16) * 0.5f);
+  const uint16_t above = neg ? static_cast<uint16_t>(0x8000u) : g16;
+  const uint16_t sg16 = inside ? in_band : (mag < static_cast<uint32_t>(kSiluBandLo) ? below : above);
+  return f32_to_bf16(bf16_to_f32(sg16) * bf16_to_f32(u16));
+}
+__device__ __forceinline__ bool silu_gate_special(uint16_t g16) {
+  return (g16 & 0x7fffu) > 0x7f80u || g16 == 0xff80u; // NaN, -inf
+}
+
 // q = (int8) trunc(clamp(v / s, -128, 127))
 __device__ __forceinline__ int quant_one(float v, float s) {
   float t = v / s;

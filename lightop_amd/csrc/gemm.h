@@ -112,13 +112,13 @@ int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flag
 int launch_gemm_tile(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
                      hipStream_t s);
 bool gemm_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);
-// Activation-stationary kernel (gemm_as.hip): plain epilogue, block_size_m 64, short K.
-int launch_gemm_as(const GemmArgs &a, int flags, int64_t m_blocks, hipStream_t s);
+// Activation-stationary kernel (gemm_as.hip): plain epilogue, block_size_m 64 or 128, short K.
+int launch_gemm_as(const GemmArgs &a, int flags, int block_size_m, int64_t m_blocks, hipStream_t s);
 bool gemm_as_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 
-// 128-token kernel with both operands copied global -> LDS (gemm_dma.hip): pre-shuffled int8 weights.
-int launch_gemm_dma(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
-bool gemm_dma_supports(const GemmArgs &a, bool fused_act, int block_size_m);
+// 128-token kernel, two four-wave workgroups per compute unit (gemm_t128.hip): pre-shuffled int8 weights.
+int launch_gemm_t128(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
+bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 // W4A8 LDS-tiled kernel (gemm_w4.hip): block_size_m 64.
 int launch_gemm_w4_tile(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
 bool gemm_w4_tile_supports(const GemmArgs &a, bool fused_act, int block_size_m);

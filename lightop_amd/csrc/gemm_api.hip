@@ -48,8 +48,8 @@ static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int
   if (!(flags & LO_GEMM_FORCE_STREAMING)) {
     if (gemm_pc_supports(a, bs)) return launch_gemm_pc(a, bs, m_blocks, s);
     if (a.per_channel) return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
-    if (gemm_dma_supports(a, fused_act, bs)) return launch_gemm_dma(a, fused_act, flags, m_blocks, s);
-    if (gemm_as_supports(a, fused_act, bs)) return launch_gemm_as(a, flags, m_blocks, s);
+    if (gemm_as_supports(a, fused_act, bs)) return launch_gemm_as(a, flags, bs, m_blocks, s);
+    if (gemm_t128_supports(a, fused_act, bs)) return launch_gemm_t128(a, fused_act, flags, m_blocks, s);
     if (gemm_tile_supports(a, fused_act, bs)) return launch_gemm_tile(a, fused_act, bs, flags, m_blocks, s);
   }
   return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);

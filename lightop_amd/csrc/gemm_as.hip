@@ -20,7 +20,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 template <bool FAST_SCALE, bool SHUF>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
-                                                          int n_groups, int n_cnt) {
+                                                          int n_groups, int n_cnt, int sub_shift) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   constexpr int kTileM = 64;
   const int K = static_cast<int>(a.K);
@@ -34,9 +34,14 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
   int mb, ng;
   if (!tile_of(blockIdx.x, n_groups, m_blocks, group_m, mb, ng)) return;
   if (static_cast<int64_t>(mb) * kTileM >= a.ntpp[0]) return;
-  const int e = a.expert_ids[mb];
+  // mb counts 64-token pieces; an alignment block of 128 tokens is two of them (sub_shift = 1), and
+  // a piece that holds padding only is skipped
+  const int e = a.expert_ids[mb >> sub_shift];
   if (e >= a.E) return;
   const int tid = threadIdx.x, lane = tid & 63;
+  if (sub_shift &&
+      __builtin_amdgcn_ballot_w64(a.sorted[static_cast<int64_t>(mb) * kTileM + lane] < a.num_valid) == 0)
+    return;
   const int wr = __builtin_amdgcn_readfirstlane(tid >> 6); // which 64 weight rows of a tile
   const int r = lane & 31, c = lane >> 5;
   const int64_t N = a.N;
@@ -247,7 +252,7 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
 static int64_t as_lds_bytes(int64_t K) { return 64 * (K + 16) + (K / kGroup) * 64 * 4 + 4 * 32 * kStgPitch; }
 
 bool gemm_as_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
-  if (fused_act || block_size_m != 64) return false;
+  if (fused_act || (block_size_m != 64 && block_size_m != 128)) return false;
   if (a.N % 64 != 0 || (reinterpret_cast<uintptr_t>(a.C) & 15) != 0) return false;
   if (as_lds_bytes(a.K) > 80 * 1024) return false; // two workgroups per CU
   // Pays off only when the launch is several rounds of workgroups deep even with half a
@@ -255,7 +260,9 @@ bool gemm_as_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
   return a.num_valid / 64 + (a.experts_routed + 1) / 2 >= 1024;
 }
 
-int launch_gemm_as(const GemmArgs &a0, int flags, int64_t m_blocks, hipStream_t s) {
+int launch_gemm_as(const GemmArgs &a0, int flags, int block_size_m, int64_t m_blocks_bs, hipStream_t s) {
+  const int sub_shift = block_size_m == 128 ? 1 : 0;
+  const int64_t m_blocks = m_blocks_bs << sub_shift; // in 64-token pieces
   GemmArgs a = a0;
   const int n_tiles = static_cast<int>((a.N + 255) / 256);
   // Weight tiles per workgroup: half of them.  Fewer workgroups than that leave the
@@ -283,7 +290,7 @@ int launch_gemm_as(const GemmArgs &a0, int flags, int64_t m_blocks, hipStream_t 
       set_error("moe_gemm: cannot reserve %zu bytes of LDS", lds);                                    \
       return LO_ELAUNCH;                                                                              \
     }                                                                                                 \
-    hipLaunchKernelGGL(kern, g, b, lds, s, a, mbi, Gi, n_groups, n_cnt);                              \
+    hipLaunchKernelGGL(kern, g, b, lds, s, a, mbi, Gi, n_groups, n_cnt, sub_shift);                   \
   } while (0)
   if (fast) {
     if (a.w_shuffled) LO_AS_LAUNCH(true, true);

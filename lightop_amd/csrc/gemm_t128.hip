@@ -1,0 +1,483 @@
+// Grouped block-INT8 GEMM for gfx950, 128-token form with two independent workgroups per
+// compute unit.
+//
+// The LDS-tiled kernels are bound by the rate at which compute units pull operands out of L2:
+// bytes requested per multiply-add are 1/tokens + 1/rows of the workgroup tile.  A 128-token
+// tile needs 128 fp32 accumulators per lane when four waves share 256 weight rows, which leaves
+// no room for weight fragments double-buffered in registers (gemm_tile.hip) at two waves per
+// SIMD, and a single eight-wave workgroup per compute unit (gemm_dma.hip) runs phase-locked.
+// Here every operand byte enters the compute unit once by direct global -> LDS loads
+// (buffer_load ... lds) and costs no staging registers, so four waves hold 128 tokens x 256
+// rows in 72 KB of LDS and two such workgroups share a compute unit:
+//   weights  each wave copies its own rows: per 128-wide K block four pre-shuffled 2 KB blocks
+//            into a private 8 KB stage.  The wave reads the stage into registers at the start of
+//            a K block and refills it at once with the next K block, so the stage needs no
+//            barrier and no second copy, and is requested a whole K block ahead;
+//   tokens   128 rows x 128 bytes per K block into a two-stage ring shared by the workgroup
+//            (16-byte pieces XOR-swizzled by row, conflict-free operand reads), requested one K
+//            block ahead; one barrier per K block.  Every wave reads each token fragment once per
+//            K block and uses it against all 64 of its rows: LDS bandwidth is what this kernel
+//            runs out of first;
+//   scales   the tokens' group scales, through registers, one K block ahead; the weight-block
+//            scales of the tile's rows (two per K block) go to LDS once, before the K loop, so
+//            that the loop issues no vector-memory operation whose result it has to wait for
+//            (the wait would also drain the copies in flight).
+// A wave owns 64 rows x 128 tokens as 4 x 8 fragments of v_mfma_i32_16x16x64_i8 (weights as
+// the A operand) and folds each fragment's exact int32 sum over a K block into fp32 as the
+// 64-token kernel does (reference arithmetic: Triton fused_moe_kernel,
+// python/lightop/_lmslim_native/layers/fused_moe/int8.py:485-519; fused epilogue :811-823).
+#include <type_traits>
+
+#include "gemm.h"
+
+namespace lo {
+
+constexpr int kT = 128;                       // tokens per workgroup
+constexpr int kTWStage = 8192;                // one wave's weights for one K block
+constexpr int kTW = 4 * kTWStage;             // [wave]
+constexpr int kTAStage = kT * kGroup;         // token rows of one K block
+constexpr int kTA = 2 * kTAStage;
+constexpr int kTS = 2 * kT * 4;               // [stage][token] scales
+constexpr int kTRed = 4 * kT * 4;             // [wave][token] amax exchange of the fused epilogue
+constexpr int kTMaxKB = 128;                  // K blocks whose weight-block scales fit the table below
+constexpr int kTBs = 2 * kTMaxKB * 4;         // [fragment][K block] weight-block scales of the tile
+constexpr int kTLds = kTW + kTA + kTS + kTRed + kTBs + 2 * kSiluBandN * 2;
+constexpr int kTPitch = 144;                  // staging pitch of the epilogues: 128 + 16
+
+// Wait until all but the newest `N` vector-memory operations of this wave are complete and its
+// LDS operations have landed.  (__syncthreads() would drain every copy in flight: the compiler
+// treats a direct-to-LDS load as an LDS write that a workgroup fence must make visible.)
+template <int N>
+__device__ __forceinline__ void wait_copies() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_copies_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <bool FUSED_ACT, bool FAST_SCALE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+  int8_t *const sA = smem + kTW;
+  float *const sS = reinterpret_cast<float *>(smem + kTW + kTA);
+  float *const sRed = reinterpret_cast<float *>(smem + kTW + kTA + kTS);
+  float *const sBs = reinterpret_cast<float *>(smem + kTW + kTA + kTS + kTRed);
+  uint16_t *const sSilu = reinterpret_cast<uint16_t *>(smem + kTW + kTA + kTS + kTRed + kTBs);
+
+  int mb, nt;
+  if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
+  if (static_cast<int64_t>(mb) * kT >= a.ntpp[0]) return;
+  const int e = a.expert_ids[mb];
+  if (e >= a.E) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // which 64 weight rows of the tile
+  const int r = lane & 15, q = lane >> 4;
+  const int64_t K = a.K, N = a.N;
+  const int KB = static_cast<int>(K / kGroup);
+  const int64_t I = N / 2;
+  const int32_t *const sorted = a.sorted + static_cast<int64_t>(mb) * kT;
+
+  // first row of the wave's 64 (plain) or of its 32 gate rows (fused)
+  const int64_t nrow0 = FUSED_ACT ? static_cast<int64_t>(nt) * kGroup + wave * 32
+                                  : static_cast<int64_t>(nt) * 256 + wave * 64;
+  const bool wave_active = FUSED_ACT || nrow0 < N; // N % 64 == 0 is checked on the host
+
+  if (e < 0) {
+    if constexpr (!FUSED_ACT) {
+      if (wave_active && !a.skip_nonlocal) {
+#pragma unroll
+        for (int tb = 0; tb < 8; ++tb) {
+          const int64_t ft = sorted[tb * 16 + r];
+          if (ft < a.num_valid)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              *reinterpret_cast<v2i *>(a.C + ft * N + nrow0 + j * 16 + 4 * q) = v2i{0, 0};
+        }
+      }
+    }
+    return;
+  }
+
+  uint16_t band_regs[kSiluBandPer];
+  if constexpr (FUSED_ACT) silu_band_load(band_regs, a.silu, tid);
+
+  // ---- what this wave copies -----------------------------------------------------------------------
+  const int NBLK = static_cast<int>(N / 16);
+  const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * N * K, static_cast<uint32_t>(N * K));
+  const brsrc rA = make_rsrc(a.A, static_cast<uint32_t>(a.a_rows * K));
+  const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * KB * 4));
+  const int wkstride = shuf_kb_stride(NBLK);
+  int wvoff[2][2]; // [step half][fragment]: the 2 KB block of 16 rows x 128 K, in lane order
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int rf = 0; rf < 2; ++rf) {
+      int64_t nb;
+      if constexpr (FUSED_ACT) nb = (rf ? I / 16 : 0) + static_cast<int64_t>(nt) * 8 + wave * 2 + h;
+      else nb = static_cast<int64_t>(nt) * 16 + wave * 4 + h * 2 + rf;
+      if (nb >= NBLK) nb = 0; // rows past N: computed on block 0, never stored
+      wvoff[h][rf] = static_cast<int>(nb) * shuf_nb_stride(KB) + lane * 16;
+    }
+  int avoff[4]; // 1 KB pieces wave*4 + j of a token stage: eight token rows each
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int t = (wave * 4 + j) * 8 + (lane >> 3);
+    const int64_t lf = sorted[t];
+    const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
+    const int piece = (lane & 7) ^ (t & 7); // slot lane & 7 of row t holds piece slot ^ (t & 7)
+    avoff[j] = static_cast<int>(lrow * K) + piece * 16;
+  }
+  // A block's valid tokens come first; fragments of 16 tokens past them are skipped (a block
+  // of 128 is on average half a block of padding per expert).
+  int nst; // pipeline stages per K block: two per token fragment that holds a valid token
+  {
+    const int v0 = __builtin_popcountll(__builtin_amdgcn_ballot_w64(sorted[lane] < a.num_valid));
+    const int v1 = __builtin_popcountll(__builtin_amdgcn_ballot_w64(sorted[lane + 64] < a.num_valid));
+    const int npair = (v0 + v1 + 31) >> 5; // the K loop comes in variants of 2, 4, 6, 8 fragments
+    nst = __builtin_amdgcn_readfirstlane(4 * (npair < 1 ? 1 : npair));
+  }
+  int asoff; // thread t and thread t + 128 both carry the scale of token t
+  {
+    const int64_t lf = sorted[tid & (kT - 1)];
+    const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
+    asoff = static_cast<int>(lrow * KB * 4);
+  }
+  // weight-block scales of the tile: table row 0 / 1 = gate / up block (fused), or the first / second
+  // 128 rows of the tile (plain: waves 0, 1 / waves 2, 3).  Thread t fetches entry (t >> 7, t & 127).
+  const int NB = static_cast<int>((N + kGroup - 1) / kGroup);
+  float bs_mine = 0.0f;
+  {
+    const int which = tid >> 7, kbi = tid & (kTMaxKB - 1);
+    int64_t nblk = FUSED_ACT ? (which ? I / kGroup : 0) + nt : static_cast<int64_t>(nt) * 2 + which;
+    if (nblk >= NB) nblk = 0;
+    if (kbi < KB) bs_mine = a.Ws[(static_cast<int64_t>(e) * NB + nblk) * KB + kbi];
+  }
+  const float *const sBs0 = sBs + (FUSED_ACT ? 0 : (wave >> 1) * kTMaxKB);
+  const float *const sBs1 = sBs + (FUSED_ACT ? kTMaxKB : (wave >> 1) * kTMaxKB);
+
+  int8_t *const sWw = smem + wave * kTWStage; // [row half][fragment][k half] x 1 KB
+  // piece p of the 12 copies a wave issues per K block: 0..7 its weights, 8..11 token rows
+  auto copy_piece = [&](int p, int kb) __attribute__((always_inline)) {
+    const int kc = kb < KB ? kb : KB - 1;
+    if (p < 8) {
+      const int h = p >> 2, rf = (p >> 1) & 1, kh = p & 1;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[h][rf],
+                                               __builtin_amdgcn_readfirstlane(kc * wkstride) + kh * 1024, 0, 0);
+    } else {
+      const int j = p - 8;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rA, sA + (kb & 1) * kTAStage + wave * 4096 + j * 1024, 16, avoff[j],
+                                               __builtin_amdgcn_readfirstlane(kc) * kGroup, 0, 0);
+    }
+  };
+  auto copy_w = [&](int kb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) copy_piece(p, kb);
+  };
+  auto copy_a = [&](int kb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int p = 8; p < 12; ++p) copy_piece(p, kb);
+  };
+  auto load_scale = [&](int kb) __attribute__((always_inline)) {
+    return bld_f32(rAs, asoff, (kb < KB ? kb : KB - 1) * 4);
+  };
+
+  // ---- operand read offsets -------------------------------------------------------------------------
+  // token fragment tb, k-half kh: piece 4*kh + q of row tb*16 + r sits in slot piece ^ (r & 7)
+  int alds[2];
+#pragma unroll
+  for (int kh = 0; kh < 2; ++kh) alds[kh] = r * kGroup + (((4 * kh + q) ^ (r & 7)) * 16);
+
+  float acc[2][8][2][4]; // [step half][token fragment][fragment of the half][element]
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int tb = 0; tb < 8; ++tb)
+#pragma unroll
+      for (int rf = 0; rf < 2; ++rf)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[h][tb][rf][i] = 0.0f;
+
+  auto fold = [&](const v4i &d, float sc, float as, float bs, float *dst) __attribute__((always_inline)) {
+    if constexpr (FAST_SCALE) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[i] = __builtin_fmaf(static_cast<float>(d[i]), sc, dst[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float t = static_cast<float>(d[i]) * as;
+        t = t * bs;
+        dst[i] = dst[i] + t;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(dst[i])); // keep the fold here
+  };
+
+  // One K block: the wave's 64 rows (two halves h of two fragments) against all 128 tokens.
+  v4i w[2][2][2]; // the wave's weights of the current K block
+  auto read_w = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int rf = 0; rf < 2; ++rf)
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh)
+          w[h][rf][kh] = *reinterpret_cast<const v4i *>(sWw + ((h * 2 + rf) * 2 + kh) * 1024 + lane * 16);
+  };
+  auto kblock = [&](auto NST, int kb) __attribute__((always_inline)) {
+    constexpr int nst_c = decltype(NST)::value; // stages of this variant: 4, 8, 12 or 16
+    const int8_t *ta = sA + (kb & 1) * kTAStage;
+    const float *ts = sS + (kb & 1) * kT;
+    v4i bf[2][2];
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) bf[0][kh] = *reinterpret_cast<const v4i *>(ta + alds[kh]);
+    float as_t[2];
+    as_t[0] = ts[r];
+    const float bs0 = sBs0[kb], bs1 = sBs1[kb];
+    // The weight stage was read into registers before the barrier, so it is free; it and the other
+    // token stage are refilled with the next K block, two copies per pipeline stage so that the
+    // texture path never sees a burst that this wave (or the other workgroup's) queues behind.
+    const v4i cinit = {0, 0, 0, 0};
+    v4i dprev[2];
+    float as_p = 0.0f;
+    auto fold_stage = [&](int st) __attribute__((always_inline)) { // fold the fragments of stage st
+      const int tb = st >> 1, h = st & 1;
+      const float sc0 = as_p * bs0, sc1 = as_p * bs1;
+      fold(dprev[0], sc0, as_p, bs0, acc[h][tb][0]);
+      fold(dprev[1], sc1, as_p, bs1, acc[h][tb][1]);
+    };
+    // pipeline stage (tb, h): its MFMAs are issued, then the previous stage's fragments are folded
+    // while the matrix pipe works; the operands of token fragment tb + 1 are requested in (tb, 0)
+#pragma unroll
+    for (int st = 0; st < 16; ++st) {
+      const int tb = st >> 1, h = st & 1;
+      const int cur = tb & 1, nxt = cur ^ 1;
+      if (nst_c >= 8 && st < 6) {
+        copy_piece(2 * st, kb + 1);
+        copy_piece(2 * st + 1, kb + 1);
+      }
+      if (nst_c < 8 && st < 4) {
+        copy_piece(3 * st, kb + 1);
+        copy_piece(3 * st + 1, kb + 1);
+        copy_piece(3 * st + 2, kb + 1);
+      }
+      if (st < nst_c) {
+        if (h == 0 && st + 2 < nst_c) {
+#pragma unroll
+          for (int kh = 0; kh < 2; ++kh)
+            bf[nxt][kh] = *reinterpret_cast<const v4i *>(ta + (tb + 1) * 16 * kGroup + alds[kh]);
+          as_t[nxt] = ts[(tb + 1) * 16 + r];
+        }
+        v4i d[2];
+#pragma unroll
+        for (int rf = 0; rf < 2; ++rf)
+          d[rf] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[h][rf][0], bf[cur][0], cinit, 0, 0, 0);
+#pragma unroll
+        for (int rf = 0; rf < 2; ++rf)
+          d[rf] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[h][rf][1], bf[cur][1], d[rf], 0, 0, 0);
+        if (st > 0) fold_stage(st - 1);
+        if (h == 0 && st + 2 < nst_c) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (nst_c >= 8 ? (g < 2 && st < 6) : (g < 3 && st < 4)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        dprev[0] = d[0];
+        dprev[1] = d[1];
+        as_p = as_t[cur];
+      }
+    }
+    fold_stage(nst_c - 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // the next K block's weights have had a whole K block to arrive; reading them here puts the
+    // LDS latency under the barrier instead of in front of the first MFMA
+    wait_copies<0>();
+    read_w();
+  };
+
+  // ---- prologue ------------------------------------------------------------------------------------------
+  float s_now = load_scale(0), s_pending = load_scale(1);
+  __builtin_amdgcn_sched_barrier(0);
+  copy_a(0);
+  copy_w(0);
+  __builtin_amdgcn_sched_barrier(0);
+  if (tid < kT) sS[tid] = s_now;
+  sBs[tid] = bs_mine;
+  if constexpr (FUSED_ACT) silu_band_store(sSilu, band_regs, tid);
+  wait_copies<0>();
+  read_w();
+
+  auto k_loop = [&](auto NST) __attribute__((always_inline)) {
+    for (int kb = 0; kb < KB; ++kb) {
+      // every copy this wave requested a K block ago has landed; after the barrier so have everyone
+      // else's token rows, and nobody still reads the token stage and the scales of K block kb-1,
+      // which are refilled below
+      wait_copies_barrier<0>();
+      if (tid < kT) sS[((kb + 1) & 1) * kT + tid] = kb + 1 < KB ? s_pending : 0.0f;
+      s_pending = load_scale(kb + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      kblock(NST, kb);
+    }
+  };
+  // one K loop per number of token fragments that hold valid tokens (wave-uniform choice)
+  if (nst > 12) k_loop(std::integral_constant<int, 16>{});
+  else if (nst > 8) k_loop(std::integral_constant<int, 12>{});
+  else if (nst > 4) k_loop(std::integral_constant<int, 8>{});
+  else k_loop(std::integral_constant<int, 4>{});
+  wait_copies<0>(); // no copy may still be writing LDS when the epilogue reuses it or the wave ends
+  if constexpr (!FUSED_ACT) {
+    if (!wave_active) return;
+    // A lane holds 4 consecutive columns of one token per fragment.  Each wave turns a 16-token x
+    // 64-column piece around in its own (now idle) weight ring and stores 128-byte row segments.
+    int8_t *stg = sWw;
+#pragma unroll
+    for (int tb = 0; tb < 8; ++tb) {
+      if (2 * tb >= nst) continue;
+      const int64_t ft = sorted[tb * 16 + r];
+      const bool valid = ft < a.num_valid;
+      float wgt = 1.0f;
+      if (a.mul_routed && valid) wgt = a.topk_w[ft];
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int rf = 0; rf < 2; ++rf) {
+          v4u16 o;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float v = acc[h][tb][rf][i];
+            if (a.mul_routed) v = v * wgt;
+            o[i] = f32_to_bf16(v);
+          }
+          *reinterpret_cast<v4u16 *>(stg + r * kTPitch + (h * 32 + rf * 16 + 4 * q) * 2) = o;
+        }
+      __builtin_amdgcn_wave_barrier();
+      const int slot = valid ? static_cast<int>(ft) : -1;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int tok = (lane >> 3) + 8 * j;
+        const v4i v = *reinterpret_cast<const v4i *>(stg + tok * kTPitch + (lane & 7) * 16);
+        const int fs = __shfl(slot, tok);
+        if (fs >= 0) *reinterpret_cast<v4i *>(a.C + static_cast<int64_t>(fs) * N + nrow0 + (lane & 7) * 8) = v;
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  } else {
+    // acc[h][tb][0] = gate, acc[h][tb][1] = up for activation columns nt*128 + wave*32 + 16h + 4q + i
+    float actf[8][2][4];
+    if (a.mul_routed) { // router weight on the first GEMM's output: rare, kept out of the main pass
+#pragma unroll
+      for (int tb = 0; tb < 8; ++tb) {
+        const int64_t ft = sorted[tb * 16 + r];
+        const float wgt = ft < a.num_valid ? a.topk_w[ft] : 1.0f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int rf = 0; rf < 2; ++rf)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[h][tb][rf][i] = acc[h][tb][rf][i] * wgt;
+      }
+    }
+#pragma unroll
+    for (int tb = 0; tb < 8; ++tb) {
+      if (2 * tb >= nst) continue;
+      uint16_t g16[2][4], u16[2][4];
+      bool special = false;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          g16[h][i] = f32_to_bf16(acc[h][tb][0][i]);
+          u16[h][i] = f32_to_bf16(acc[h][tb][1][i]);
+          special |= silu_gate_special(g16[h][i]);
+          actf[tb][h][i] = bf16_to_f32(silu_mul_band_common(sSilu, g16[h][i], u16[h][i]));
+        }
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(special) != 0, 0)) { // a NaN or -inf gate in the wave
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            actf[tb][h][i] = bf16_to_f32(silu_mul_band(sSilu, a.silu, g16[h][i], u16[h][i]));
+      }
+      float amax = 0.0f;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) amax = fmaxf(amax, fabsf(actf[tb][h][i]));
+      amax = fmaxf(amax, __shfl_xor(amax, 16));
+      amax = fmaxf(amax, __shfl_xor(amax, 32));
+      if (q == 0) sRed[wave * kT + tb * 16 + r] = amax;
+    }
+    __syncthreads(); // also: every wave is done with the token stages
+    const int64_t G = I / kGroup;
+    // the quantised tile (128 tokens x 128 columns of int8) leaves through LDS as whole rows
+    int8_t *qst = sA;
+#pragma unroll
+    for (int tb = 0; tb < 8; ++tb) {
+      if (2 * tb >= nst) continue;
+      const int t = tb * 16 + r;
+      float amax = fmaxf(fmaxf(sRed[t], sRed[kT + t]), fmaxf(sRed[2 * kT + t], sRed[3 * kT + t]));
+      amax = fmaxf(amax, 1e-10f);
+      const float sc = amax / 127.0f;
+      const float rsc = 1.0f / sc;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        *reinterpret_cast<uint32_t *>(qst + t * kTPitch + wave * 32 + h * 16 + 4 * q) = quant4(actf[tb][h], sc, rsc);
+      if (wave == 0 && q == 0) {
+        const int64_t ft = sorted[t];
+        if (ft < a.num_valid) a.A2s[ft * G + nt] = sc;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kT * 8 / 256; ++j) {
+      const int id = tid + 256 * j, tok = id >> 3, piece = id & 7;
+      const int64_t ft = sorted[tok];
+      if (ft < a.num_valid)
+        *reinterpret_cast<v4i *>(a.A2q + ft * I + static_cast<int64_t>(nt) * kGroup + piece * 16) =
+            *reinterpret_cast<const v4i *>(qst + tok * kTPitch + piece * 16);
+    }
+  }
+}
+
+bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
+  if (block_size_m != 128 || !a.w_shuffled || a.w4 || a.per_channel) return false;
+  if (!fused_act && a.N % 64 != 0) return false;
+  return a.K / kGroup <= kTMaxKB;
+}
+
+int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_blocks, hipStream_t s) {
+  GemmArgs a = a0;
+  a.n_tiles = fused_act ? static_cast<int32_t>(a.N / 2 / kGroup) : static_cast<int32_t>((a.N + 255) / 256);
+  int64_t G = a.num_valid / (static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * kT);
+  G = G < 2 ? 2 : (G > 16 ? 16 : G);
+  const int64_t chunks = (m_blocks + G - 1) / G;
+  const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
+  LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
+  const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
+  const dim3 g(static_cast<unsigned>(grid)), b(256);
+  const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
+#define LO_T128_LAUNCH(FA, FS)                                                                                  \
+  do {                                                                                                          \
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_gemm_t128_kernel<FA, FS>),                      \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kTLds) != hipSuccess) {                 \
+      set_error("moe_gemm(t128): cannot reserve %d bytes of LDS", kTLds);                                       \
+      return LO_ELAUNCH;                                                                                        \
+    }                                                                                                           \
+    hipLaunchKernelGGL((moe_gemm_t128_kernel<FA, FS>), g, b, kTLds, s, a, mbi, gi);                             \
+  } while (0)
+  if (fused_act) {
+    if (fast) LO_T128_LAUNCH(true, true);
+    else LO_T128_LAUNCH(true, false);
+  } else {
+    if (fast) LO_T128_LAUNCH(false, true);
+    else LO_T128_LAUNCH(false, false);
+  }
+#undef LO_T128_LAUNCH
+  return check_launch(fused_act ? "moe_gemm1_silu_quant(t128)" : "moe_gemm(t128)");
+}
+
+} // namespace lo

@@ -365,8 +365,78 @@ def test_gemm1_epilogue_every_finite_bf16_gate(dev, oracle, bs):
     assert torch.equal(c1[:, 0].float(), pat)  # the construction works: gate == pattern
     rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
     s, e, p = moe_align_block_size(ids.to(dev), bs, 1)
-    q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), W.to(dev), As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
-                                              False, 1, M, {"BLOCK_SIZE_M": bs}, fused_scale=False)
+    from lightop_amd.moe import preshuffle_moe_weight
+    for Wx in (W.to(dev), preshuffle_moe_weight(W.to(dev))):  # the two layouts have kernels of their own
+        for fused_scale in (False, True):  # unit weight scales: both orders give the same values
+            q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wx, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
+                                                      False, 1, M, {"BLOCK_SIZE_M": bs}, fused_scale=fused_scale)
+            torch.cuda.synchronize()
+            assert torch.equal(sc.cpu(), rsc) and torch.equal(q.cpu(), rq)
+
+
+@pytest.mark.parametrize("bs", [64, 128])
+def test_gemm1_epilogue_nan_and_inf_gates(dev, oracle, bs):
+    """Gates that are NaN or infinite leave the fast lookup: rows that hold one, next to ordinary
+    rows in the same wavefront.  The activation's scale is then inf or NaN; what is pinned is that
+    the ordinary rows are untouched and the special rows agree with the oracle where it is finite."""
+    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_weight
+
+    say(f"gemm1 epilogue, NaN and inf gates bs={bs}")
+    M, I, K = 200, 128, 128
+    g = torch.Generator().manual_seed(3)
+    Aq = torch.zeros(M, K, dtype=torch.int8)
+    Aq[:, 0] = 1
+    W = torch.zeros(1, 2 * I, K, dtype=torch.int8)
+    W[0, :, 0] = 1
+    vals = torch.randn(M, generator=g) * 3
+    vals[5], vals[70], vals[71], vals[150] = float("inf"), float("-inf"), float("nan"), float("-inf")
+    As = vals.reshape(M, 1).contiguous()
+    Ws = torch.ones(1, 2, 1)
+    ids = torch.zeros(M, 1, dtype=torch.int32)
+    tw = torch.ones(M, 1)
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, 1)
+    c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, False, 1, M, bs)
+    rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+    s, e, p = moe_align_block_size(ids.to(dev), bs, 1)
+    ordinary = torch.isfinite(vals)
+    for Wx in (W.to(dev), preshuffle_moe_weight(W.to(dev))):
+        q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wx, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
+                                                  False, 1, M, {"BLOCK_SIZE_M": bs}, fused_scale=False)
+        torch.cuda.synchronize()
+        assert torch.equal(sc.cpu()[ordinary], rsc[ordinary]) and torch.equal(q.cpu()[ordinary], rq[ordinary])
+        special = ~ordinary
+        same_class = (torch.isnan(sc.cpu()[special]) == torch.isnan(rsc[special])) & \
+                     (torch.isinf(sc.cpu()[special]) == torch.isinf(rsc[special]))
+        assert same_class.all()
+
+
+@pytest.mark.parametrize("count", [1, 31, 32, 33, 64, 65, 96, 97, 127, 128, 129, 200])
+def test_gemm_128_token_blocks_fill_levels(dev, oracle, count):
+    """128-token blocks holding 1 ... 128 valid tokens: the K loop of the 128-token kernel comes in
+    variants by the number of 32-token pieces in use, and padded pieces are skipped."""
+    from lightop_amd.moe import (invoke_fused_moe_gemm1_silu_quant, invoke_fused_moe_kernel_int8,
+                                 moe_align_block_size, preshuffle_moe_weight)
+
+    say(f"128-token blocks, {count} tokens on expert 0")
+    bs, E, I, K = 128, 2, 128, 384
+    M = count + 3
+    Aq, As, W, Ws, _, tw, _ = gemm_case(count, M, 1, E, E, 2 * I, K)
+    Ws = Ws * 30
+    ids = torch.ones(M, 1, dtype=torch.int32)
+    ids[torch.randperm(M, generator=torch.Generator().manual_seed(count))[:count]] = 0
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, E)
+    s, e, p = moe_align_block_size(ids.to(dev), bs, E)
+    Wsh = preshuffle_moe_weight(W.to(dev))
+    ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, True, 1, M, bs)
+    C = torch.full((M, 1, 2 * I), 7.0, dtype=torch.bfloat16, device=dev)
+    invoke_fused_moe_kernel_int8(Aq.to(dev), Wsh, C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, True, 1,
+                                 {"BLOCK_SIZE_M": bs}, fused_scale=False)
+    torch.cuda.synchronize()
+    assert torch.equal(C.view(M, -1).cpu().view(torch.int16), ref.view(torch.int16))
+    c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, False, 1, M, bs)
+    rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+    q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wsh, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, False, 1,
+                                              M, {"BLOCK_SIZE_M": bs}, fused_scale=False)
     torch.cuda.synchronize()
     assert torch.equal(sc.cpu(), rsc) and torch.equal(q.cpu(), rq)
 
