@@ -372,7 +372,9 @@ def main():
                 "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
                 "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
                 "kernel": ("moe_gemm_ws_kernel" if bs_used < 64 else "moe_gemm_w4_tile_kernel" if L.weight_bits == 4
-                           else "moe_gemm_pc_kernel" if L.quant == "channel" else "moe_gemm_tile_kernel")
+                           else "moe_gemm_pc_kernel" if L.quant == "channel"
+                           else "moe_gemm_t128_kernel" if bs_used == 128 and not args.row_major_weights
+                           else "moe_gemm_tile_kernel")
                 + (" (GEMM1, per-channel scales in the epilogue)" if L.quant == "channel"
                    else "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)"),
                 "kernel_ms": round(stages[g1_name], 4),

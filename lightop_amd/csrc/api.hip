@@ -76,21 +76,29 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   // W4A8: the streaming kernel re-reads the token rows per wave, which outweighs the half-size
   // weights early; the LDS-tiled kernel (64 tokens) wins from about 8 slots per expert.
   if (form == LO_FORM_W4) return per_expert < 8.0 ? 16 : 64;
+  // Block form with pre-shuffled weights: the kernel that copies both operands straight into LDS
+  // (gemm_t128.hip, 128-token blocks, padded parts of a block skipped in steps of 32 tokens) takes
+  // over from the weight-streaming kernels as soon as an expert sees a handful of tokens - with
+  // about one token block per expert it streams the weights with the non-temporal hint and keeps
+  // far more bytes in flight per compute unit than the register-fed kernels - and stays ahead of
+  // the 64-token LDS tiles except around 128 slots per expert on a short K, where its longer
+  // epilogue weighs most.  Measured (us, whole path, 16 / 32 / 64 / 128): Qwen3-30B-A3B layer at
+  // 128 tokens 133 / 139 / 186 / 139, at 256: 190 / 160 / 190 / 146, at 1024: 505 / 414 / 224 /
+  // 191, at 2048: 878 / 690 / 267 / 285, at 8192: - / - / 682 / 645; DeepSeek-V3 share of 32
+  // experts at 128 tokens 248 / 262 / 315 / 241, at 2048: 1034 / 810 / 427 / 336, at 8192:
+  // - / - / 928 / 776.
+  if (form == LO_FORM_BLOCK && preshuffled) {
+    if (per_expert < (H >= 4096 ? 4.0 : 12.0)) return 16;
+    if (H < 4096 && per_expert >= 96.0 && per_expert < 192.0) return 64;
+    return 128;
+  }
   if (per_expert <= 12.0) return 16;
   if (per_expert <= 24.0) return 32;
   // Per-channel form: no scale arithmetic in the K loop, so the accumulators of 128 tokens fit
   // and the larger tile halves the weight bytes requested from L2 per multiply-add.
   if (form == LO_FORM_CHANNEL && per_expert >= 64.0) return 128;
-  // Block form, pre-shuffled weights, an expert's slots fill a 128-token block: the kernel that
-  // copies both operands straight into LDS (gemm_t128.hip) requests 40 % fewer operand bytes from
-  // L2 per multiply-add and skips the padded part of a block in steps of 32 tokens (measured:
-  // DeepSeek-V3 layer at 8192 tokens 5.41 -> 4.73 ms, its 32-expert share at 4096 tokens
-  // 0.646 -> 0.594 ms, Qwen3-30B-A3B layer at 8192 tokens 0.773 -> 0.745 ms).  With a short K
-  // its longer epilogue weighs more: at 128 slots per expert the Qwen3 layer (K = 2048) is 4 %
-  // slower with it, so the threshold there is 256.  Row-major weights stay at 64: their
-  // 128-token kernel is one phase-locked workgroup per CU and measured slower on every layer
-  // shape tried.
-  if (form == LO_FORM_BLOCK && preshuffled && per_expert >= (H >= 4096 ? 128.0 : 256.0)) return 128;
+  // Row-major block-form weights: 64-token LDS tiles, two workgroups per CU; their 128-token
+  // kernel is one phase-locked workgroup per CU and measured slower on every layer shape tried.
   return 64;
 }
 

@@ -56,7 +56,7 @@ __device__ __forceinline__ void wait_copies_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-template <bool FUSED_ACT, bool FAST_SCALE>
+template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -120,6 +120,17 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
       if (nb >= NBLK) nb = 0; // rows past N: computed on block 0, never stored
       wvoff[h][rf] = static_cast<int>(nb) * shuf_nb_stride(KB) + lane * 16;
     }
+  // STREAM: about one token block per expert, so a weight byte is used by one workgroup only and is
+  // requested with the streaming hint (it does not displace the token rows and scales in L2;
+  // first GEMM of the DeepSeek-V3 share at 1024 tokens 213 -> 160 us).  With several token blocks
+  // per expert the blocks share the weights through L2 and the hint costs 7 %.
+  constexpr int kWAux = STREAM ? kCacheStream : kCacheDefault;
+  // The first K block's weights depend on the expert only: they are requested before the token
+  // ids are read, so that the two dependent round trips of the tile's start-up overlap.
+  int8_t *const sWw = smem + wave * kTWStage; // [row half][fragment][k half] x 1 KB
+#pragma unroll
+  for (int p = 0; p < 8; ++p)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 2][(p >> 1) & 1], (p & 1) * 1024, 0, kWAux);
   int avoff[4]; // 1 KB pieces wave*4 + j of a token stage: eight token rows each
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -157,23 +168,18 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   const float *const sBs0 = sBs + (FUSED_ACT ? 0 : (wave >> 1) * kTMaxKB);
   const float *const sBs1 = sBs + (FUSED_ACT ? kTMaxKB : (wave >> 1) * kTMaxKB);
 
-  int8_t *const sWw = smem + wave * kTWStage; // [row half][fragment][k half] x 1 KB
   // piece p of the 12 copies a wave issues per K block: 0..7 its weights, 8..11 token rows
   auto copy_piece = [&](int p, int kb) __attribute__((always_inline)) {
     const int kc = kb < KB ? kb : KB - 1;
     if (p < 8) {
       const int h = p >> 2, rf = (p >> 1) & 1, kh = p & 1;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[h][rf],
-                                               __builtin_amdgcn_readfirstlane(kc * wkstride) + kh * 1024, 0, 0);
+                                               __builtin_amdgcn_readfirstlane(kc * wkstride) + kh * 1024, 0, kWAux);
     } else {
       const int j = p - 8;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rA, sA + (kb & 1) * kTAStage + wave * 4096 + j * 1024, 16, avoff[j],
                                                __builtin_amdgcn_readfirstlane(kc) * kGroup, 0, 0);
     }
-  };
-  auto copy_w = [&](int kb) __attribute__((always_inline)) {
-#pragma unroll
-    for (int p = 0; p < 8; ++p) copy_piece(p, kb);
   };
   auto copy_a = [&](int kb) __attribute__((always_inline)) {
 #pragma unroll
@@ -303,7 +309,6 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   float s_now = load_scale(0), s_pending = load_scale(1);
   __builtin_amdgcn_sched_barrier(0);
   copy_a(0);
-  copy_w(0);
   __builtin_amdgcn_sched_barrier(0);
   if (tid < kT) sS[tid] = s_now;
   sBs[tid] = bs_mine;
@@ -460,22 +465,30 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
   const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
-#define LO_T128_LAUNCH(FA, FS)                                                                                  \
+#define LO_T128_LAUNCH(FA, FS, ST)                                                                              \
   do {                                                                                                          \
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_gemm_t128_kernel<FA, FS>),                      \
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_gemm_t128_kernel<FA, FS, ST>),                  \
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTLds) != hipSuccess) {                 \
       set_error("moe_gemm(t128): cannot reserve %d bytes of LDS", kTLds);                                       \
       return LO_ELAUNCH;                                                                                        \
     }                                                                                                           \
-    hipLaunchKernelGGL((moe_gemm_t128_kernel<FA, FS>), g, b, kTLds, s, a, mbi, gi);                             \
+    hipLaunchKernelGGL((moe_gemm_t128_kernel<FA, FS, ST>), g, b, kTLds, s, a, mbi, gi);                         \
   } while (0)
+#define LO_T128_PICK(FA, FS)                                                                                    \
+  do {                                                                                                          \
+    if (stream) LO_T128_LAUNCH(FA, FS, true);                                                                   \
+    else LO_T128_LAUNCH(FA, FS, false);                                                                         \
+  } while (0)
+  // one token block per expert, by and large: the slots spread over the routed experts fill half a block
+  const bool stream = a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * (kT / 2);
   if (fused_act) {
-    if (fast) LO_T128_LAUNCH(true, true);
-    else LO_T128_LAUNCH(true, false);
+    if (fast) LO_T128_PICK(true, true);
+    else LO_T128_PICK(true, false);
   } else {
-    if (fast) LO_T128_LAUNCH(false, true);
-    else LO_T128_LAUNCH(false, false);
+    if (fast) LO_T128_PICK(false, true);
+    else LO_T128_PICK(false, false);
   }
+#undef LO_T128_PICK
 #undef LO_T128_LAUNCH
   return check_launch(fused_act ? "moe_gemm1_silu_quant(t128)" : "moe_gemm(t128)");
 }
