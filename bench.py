@@ -30,9 +30,10 @@ INT8_PEAK_TOPS = 5000.0        # MI355X dense INT8 MFMA, published (5.0 POP/s)
 # and the one-pass weight shuffle); the summaries are the files under profiles/.  Keyed
 # by (workload, tokens); None for points that were not profiled.
 MEASURED_TRAFFIC = {
-    ("qwen3-30b-a3b", 8192): 1068738454,
-    ("deepseek-v3-ep8-share", 64): 806088083,
-    ("deepseek-v3-ep8-share", 4096): 2052578268,
+    ("qwen3-30b-a3b", 8192): 1013504732,
+    ("deepseek-v3-ep8-share", 64): 806106492,
+    ("deepseek-v3-ep8-share", 1024): 961590003,
+    ("deepseek-v3-ep8-share", 4096): 1296022956,
     ("qwen3-235b-a22b-w4a8", 2048): 1633723174,
     ("qwen3-235b-a22b-w4a8", 32): 777707628,
 }
