@@ -140,14 +140,16 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     const int piece = (lane & 7) ^ (t & 7); // slot lane & 7 of row t holds piece slot ^ (t & 7)
     avoff[j] = static_cast<int>(lrow * K) + piece * 16;
   }
-  // A block's valid tokens come first; fragments of 16 tokens past them are skipped (a block
-  // of 128 is on average half a block of padding per expert).
-  int nst; // pipeline stages per K block: two per token fragment that holds a valid token
+  // The alignment puts a block's valid tokens first, so a block of 128 is on average half a block
+  // of padding per expert: token fragments past the last valid token are skipped, in steps of
+  // 32 tokens (taken from the position of the last valid token, not from their number, so that
+  // a caller's own sorted ids with gaps are still computed in full).
+  int nst; // pipeline stages per K block: four per 32 tokens in use
   {
-    const int v0 = __builtin_popcountll(__builtin_amdgcn_ballot_w64(sorted[lane] < a.num_valid));
-    const int v1 = __builtin_popcountll(__builtin_amdgcn_ballot_w64(sorted[lane + 64] < a.num_valid));
-    const int npair = (v0 + v1 + 31) >> 5; // the K loop comes in variants of 2, 4, 6, 8 fragments
-    nst = __builtin_amdgcn_readfirstlane(4 * (npair < 1 ? 1 : npair));
+    const uint64_t v0 = __builtin_amdgcn_ballot_w64(sorted[lane] < a.num_valid);
+    const uint64_t v1 = __builtin_amdgcn_ballot_w64(sorted[lane + 64] < a.num_valid);
+    const int last = v1 ? 127 - __builtin_clzll(v1) : (v0 ? 63 - __builtin_clzll(v0) : 0);
+    nst = __builtin_amdgcn_readfirstlane(4 * ((last >> 5) + 1)); // the K loop comes in variants of 2, 4, 6, 8 fragments
   }
   int asoff; // thread t and thread t + 128 both carry the scale of token t
   {

@@ -69,6 +69,12 @@ def test_version_and_tile_table(lib):
     assert all(sizes[a] <= sizes[b] for a, b in zip(list(sizes)[:-1], list(sizes)[1:]))
     assert lib.lo_moe_tile_query(-1, 32, 256, 8, 7168, 2048, t1, t2) < 0
     assert b"moe_tile_query" in lib.lo_last_error()
+    # the block-form table as the tuning harness last derived it (pre-shuffled weights): 128-token
+    # blocks from a handful of slots per expert on, 64 around 128 slots per expert on a short K
+    for M, want in ((64, 16), (128, 128), (1024, 128), (4096, 128)):
+        assert lib.lo_moe_tile_query(M, 32, 256, 8, 7168, 2048, t1, t2) == 0 and t1.block_size_m == want
+    for M, want in ((128, 16), (192, 128), (1024, 128), (1536, 64), (2048, 64), (3072, 128), (8192, 128)):
+        assert lib.lo_moe_tile_query(M, 128, 128, 8, 2048, 768, t1, t2) == 0 and t1.block_size_m == want
     # per-channel form: same small tiles, 128 tokens once an expert sees that many
     for M, want in ((1, 16), (64, 16), (1024, 64), (2048, 128), (8192, 128)):
         assert lib.lo_moe_tile_query_form(_lib.LO_FORM_CHANNEL, M, 32, 256, 8, 7168, 2048, t1, t2) == 0

@@ -410,6 +410,39 @@ def test_gemm1_epilogue_nan_and_inf_gates(dev, oracle, bs):
         assert same_class.all()
 
 
+@pytest.mark.parametrize("bs", [64, 128])
+def test_gemm_sorted_ids_with_gaps(dev, oracle, bs):
+    """A caller's own sorted ids need not keep a block's valid slots at its front: padding entries
+    anywhere inside a block (here: a random permutation of every block) must give the same rows."""
+    from lightop_amd.moe import (invoke_fused_moe_gemm1_silu_quant, invoke_fused_moe_kernel_int8,
+                                 preshuffle_moe_weight)
+
+    say(f"sorted ids with gaps bs={bs}")
+    M, k, E, I, K = 150, 2, 3, 128, 384
+    Aq, As, W, Ws, ids, tw, _ = gemm_case(11 + bs, M, k, E, E, 2 * I, K)
+    Ws = Ws * 30
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, E)
+    g = torch.Generator().manual_seed(bs)
+    P = int(rp)
+    rs = rs.clone()
+    for b in range(P // bs):
+        rs[b * bs:(b + 1) * bs] = rs[b * bs:(b + 1) * bs][torch.randperm(bs, generator=g)]
+    S = M * k
+    ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, True, k, S, bs)
+    c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, False, k, S, bs)
+    rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+    s, e, p = rs.to(dev), re.to(dev), rp.to(dev)
+    for Wx in (W.to(dev), preshuffle_moe_weight(W.to(dev))):
+        C = torch.full((M, k, 2 * I), 7.0, dtype=torch.bfloat16, device=dev)
+        invoke_fused_moe_kernel_int8(Aq.to(dev), Wx, C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, True, k,
+                                     {"BLOCK_SIZE_M": bs}, fused_scale=False)
+        q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wx, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, False,
+                                                  k, S, {"BLOCK_SIZE_M": bs}, fused_scale=False)
+        torch.cuda.synchronize()
+        assert torch.equal(C.view(S, -1).cpu().view(torch.int16), ref.view(torch.int16))
+        assert torch.equal(sc.cpu(), rsc) and torch.equal(q.cpu(), rq)
+
+
 @pytest.mark.parametrize("count", [1, 31, 32, 33, 64, 65, 96, 97, 127, 128, 129, 200])
 def test_gemm_128_token_blocks_fill_levels(dev, oracle, count):
     """128-token blocks holding 1 ... 128 valid tokens: the K loop of the 128-token kernel comes in
