@@ -34,8 +34,8 @@ MEASURED_TRAFFIC = {
     ("deepseek-v3-ep8-share", 64): 806106492,
     ("deepseek-v3-ep8-share", 1024): 961590003,
     ("deepseek-v3-ep8-share", 4096): 1296022956,
-    ("qwen3-235b-a22b-w4a8", 2048): 1633723174,
-    ("qwen3-235b-a22b-w4a8", 32): 777707628,
+    ("qwen3-235b-a22b-w4a8", 2048): 1341367804,
+    ("qwen3-235b-a22b-w4a8", 32): 777774457,
 }
 
 
@@ -372,7 +372,9 @@ def main():
     roofline = {"bound": head["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
                 "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
                 "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
-                "kernel": ("moe_gemm_ws_kernel" if bs_used < 64 else "moe_gemm_w4_tile_kernel" if L.weight_bits == 4
+                "kernel": ("moe_gemm_ws_kernel" if bs_used < 64
+                           else "moe_gemm_t128_kernel<W4>" if L.weight_bits == 4 and bs_used == 128
+                           else "moe_gemm_w4_tile_kernel" if L.weight_bits == 4
                            else "moe_gemm_pc_kernel" if L.quant == "channel"
                            else "moe_gemm_t128_kernel" if bs_used == 128 and not args.row_major_weights
                            else "moe_gemm_tile_kernel")

@@ -41,6 +41,8 @@ static int validate_common(const char *who, const void *A, const void *As, const
 static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int64_t m_blocks,
                        hipStream_t s) {
   if (a.w4) { // int4 weights: the LDS-tiled kernel at 64-token blocks, else streaming
+    if (!(flags & LO_GEMM_FORCE_STREAMING) && gemm_t128_supports(a, fused_act, bs))
+      return launch_gemm_t128(a, fused_act, flags, m_blocks, s);
     if (!(flags & LO_GEMM_FORCE_STREAMING) && gemm_w4_tile_supports(a, fused_act, bs))
       return launch_gemm_w4_tile(a, fused_act, flags, m_blocks, s);
     return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);

@@ -56,7 +56,7 @@ __device__ __forceinline__ void wait_copies_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM>
+template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM, bool W4>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -105,10 +105,14 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 
   // ---- what this wave copies -----------------------------------------------------------------------
   const int NBLK = static_cast<int>(N / 16);
-  const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * N * K, static_cast<uint32_t>(N * K));
+  // W4: packed int4 weights in their load-time layout (1 KB per 16 rows x 128 K, the lane's two
+  // k-steps in one 16-byte piece) and one scale per weight row and K block, [E, K/128, N]
+  const int64_t wbytes = W4 ? N * K / 2 : N * K; // one expert
+  const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * wbytes, static_cast<uint32_t>(wbytes));
+  const brsrc rWs = make_rsrc(a.Ws + static_cast<int64_t>(e) * N * KB, static_cast<uint32_t>(N * KB * 4));
   const brsrc rA = make_rsrc(a.A, static_cast<uint32_t>(a.a_rows * K));
   const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * KB * 4));
-  const int wkstride = shuf_kb_stride(NBLK);
+  const int wkstride = W4 ? shuf_kb_stride(NBLK) / 2 : shuf_kb_stride(NBLK);
   int wvoff[2][2]; // [step half][fragment]: the 2 KB block of 16 rows x 128 K, in lane order
 #pragma unroll
   for (int h = 0; h < 2; ++h)
@@ -118,8 +122,17 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
       if constexpr (FUSED_ACT) nb = (rf ? I / 16 : 0) + static_cast<int64_t>(nt) * 8 + wave * 2 + h;
       else nb = static_cast<int64_t>(nt) * 16 + wave * 4 + h * 2 + rf;
       if (nb >= NBLK) nb = 0; // rows past N: computed on block 0, never stored
-      wvoff[h][rf] = static_cast<int>(nb) * shuf_nb_stride(KB) + lane * 16;
+      wvoff[h][rf] = static_cast<int>(nb) * (W4 ? shuf_nb_stride(KB) / 2 : shuf_nb_stride(KB)) + lane * 16;
     }
+  // W4: lane l copies the scale of row l of the wave's 64 (fused: 32 gate rows, then the 32 up rows)
+  int wsvoff = 0;
+  if constexpr (W4) {
+    int64_t row;
+    if constexpr (FUSED_ACT) row = (lane < 32 ? 0 : I - 32) + static_cast<int64_t>(nt) * kGroup + wave * 32 + lane;
+    else row = static_cast<int64_t>(nt) * 256 + wave * 64 + lane;
+    if (row >= N) row = 0;
+    wsvoff = static_cast<int>(row * 4);
+  }
   // STREAM: about one token block per expert, so a weight byte is used by one workgroup only and is
   // requested with the streaming hint (it does not displace the token rows and scales in L2;
   // first GEMM of the DeepSeek-V3 share at 1024 tokens 213 -> 160 us).  With several token blocks
@@ -127,10 +140,18 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   constexpr int kWAux = STREAM ? kCacheStream : kCacheDefault;
   // The first K block's weights depend on the expert only: they are requested before the token
   // ids are read, so that the two dependent round trips of the tile's start-up overlap.
-  int8_t *const sWw = smem + wave * kTWStage; // [row half][fragment][k half] x 1 KB
+  int8_t *const sWw = smem + wave * kTWStage; // int8: [row half][fragment][k half] x 1 KB; W4: [row half][fragment] x 1 KB, row scales
+  if constexpr (W4) {
 #pragma unroll
-  for (int p = 0; p < 8; ++p)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 2][(p >> 1) & 1], (p & 1) * 1024, 0, kWAux);
+    for (int p = 0; p < 4; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 1][p & 1], 0, 0, kWAux);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rWs, sWw + 4096, 4, wsvoff, 0, 0, 0);
+  } else {
+#pragma unroll
+    for (int p = 0; p < 8; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 2][(p >> 1) & 1], (p & 1) * 1024, 0,
+                                               kWAux);
+  }
   int avoff[4]; // 1 KB pieces wave*4 + j of a token stage: eight token rows each
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -165,7 +186,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     const int which = tid >> 7, kbi = tid & (kTMaxKB - 1);
     int64_t nblk = FUSED_ACT ? (which ? I / kGroup : 0) + nt : static_cast<int64_t>(nt) * 2 + which;
     if (nblk >= NB) nblk = 0;
-    if (kbi < KB) bs_mine = a.Ws[(static_cast<int64_t>(e) * NB + nblk) * KB + kbi];
+    if (!W4 && kbi < KB) bs_mine = a.Ws[(static_cast<int64_t>(e) * NB + nblk) * KB + kbi];
   }
   const float *const sBs0 = sBs + (FUSED_ACT ? 0 : (wave >> 1) * kTMaxKB);
   const float *const sBs1 = sBs + (FUSED_ACT ? kTMaxKB : (wave >> 1) * kTMaxKB);
@@ -174,9 +195,18 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   auto copy_piece = [&](int p, int kb) __attribute__((always_inline)) {
     const int kc = kb < KB ? kb : KB - 1;
     if (p < 8) {
-      const int h = p >> 2, rf = (p >> 1) & 1, kh = p & 1;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[h][rf],
-                                               __builtin_amdgcn_readfirstlane(kc * wkstride) + kh * 1024, 0, kWAux);
+      if constexpr (W4) { // four weight pieces, the row scales, three empty slots
+        if (p < 4)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 1][p & 1],
+                                                   __builtin_amdgcn_readfirstlane(kc * wkstride), 0, kWAux);
+        else if (p == 4)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rWs, sWw + 4096, 4, wsvoff,
+                                                   __builtin_amdgcn_readfirstlane(kc) * static_cast<int>(N) * 4, 0, 0);
+      } else {
+        const int h = p >> 2, rf = (p >> 1) & 1, kh = p & 1;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[h][rf],
+                                                 __builtin_amdgcn_readfirstlane(kc * wkstride) + kh * 1024, 0, kWAux);
+      }
     } else {
       const int j = p - 8;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rA, sA + (kb & 1) * kTAStage + wave * 4096 + j * 1024, 16, avoff[j],
@@ -207,6 +237,23 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[h][tb][rf][i] = 0.0f;
 
+  // W4: every product carries the factor 16 of the unpacked nibbles; the canonical order takes it out
+  // of the exact int32 sum with a shift, the fused order puts 1/16 into the row scale (a power of
+  // two: the same value unless the scale is denormal).  One scale per weight row: bs4[i] for row 4q + i.
+  auto fold4 = [&](const v4i &d, float as, const v4f &bs4, float *dst) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (FAST_SCALE) {
+        dst[i] = __builtin_fmaf(static_cast<float>(d[i]), as * bs4[i], dst[i]); // bs4 already holds scale / 16
+      } else {
+        float t = static_cast<float>(d[i] >> 4) * as;
+        t = t * bs4[i];
+        dst[i] = dst[i] + t;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(dst[i])); // keep the fold here
+  };
   auto fold = [&](const v4i &d, float sc, float as, float bs, float *dst) __attribute__((always_inline)) {
     if constexpr (FAST_SCALE) {
 #pragma unroll
@@ -225,14 +272,36 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 
   // One K block: the wave's 64 rows (two halves h of two fragments) against all 128 tokens.
   v4i w[2][2][2]; // the wave's weights of the current K block
+  v4f wsc[2][2];  // W4: the scales of the lane's rows 4q .. 4q+3 of each fragment
   auto read_w = [&]() __attribute__((always_inline)) {
+    if constexpr (W4) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+      for (int h = 0; h < 2; ++h)
 #pragma unroll
-      for (int rf = 0; rf < 2; ++rf)
+        for (int rf = 0; rf < 2; ++rf) {
+          const v4i pk = *reinterpret_cast<const v4i *>(sWw + (h * 2 + rf) * 1024 + lane * 16);
 #pragma unroll
-        for (int kh = 0; kh < 2; ++kh)
-          w[h][rf][kh] = *reinterpret_cast<const v4i *>(sWw + ((h * 2 + rf) * 2 + kh) * 1024 + lane * 16);
+          for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+              const uint32_t word = static_cast<uint32_t>(pk[2 * ks + x]);
+              w[h][rf][ks][2 * x] = static_cast<int>((word << 4) & 0xf0f0f0f0u);
+              w[h][rf][ks][2 * x + 1] = static_cast<int>(word & 0xf0f0f0f0u);
+            }
+          // rows of fragment (h, rf) among the wave's 64: fused 32*rf + 16*h, plain 32*h + 16*rf
+          const int row0 = (FUSED_ACT ? 32 * rf + 16 * h : 32 * h + 16 * rf) + 4 * q;
+          wsc[h][rf] = *reinterpret_cast<const v4f *>(sWw + 4096 + row0 * 4);
+          if constexpr (FAST_SCALE) wsc[h][rf] = wsc[h][rf] * 0.0625f;
+        }
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int rf = 0; rf < 2; ++rf)
+#pragma unroll
+          for (int kh = 0; kh < 2; ++kh)
+            w[h][rf][kh] = *reinterpret_cast<const v4i *>(sWw + ((h * 2 + rf) * 2 + kh) * 1024 + lane * 16);
+    }
   };
   auto kblock = [&](auto NST, int kb) __attribute__((always_inline)) {
     constexpr int nst_c = decltype(NST)::value; // stages of this variant: 4, 8, 12 or 16
@@ -243,18 +312,28 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     for (int kh = 0; kh < 2; ++kh) bf[0][kh] = *reinterpret_cast<const v4i *>(ta + alds[kh]);
     float as_t[2];
     as_t[0] = ts[r];
-    const float bs0 = sBs0[kb], bs1 = sBs1[kb];
+    const float bs0 = W4 ? 0.0f : sBs0[kb], bs1 = W4 ? 0.0f : sBs1[kb];
+
     // The weight stage was read into registers before the barrier, so it is free; it and the other
     // token stage are refilled with the next K block, two copies per pipeline stage so that the
     // texture path never sees a burst that this wave (or the other workgroup's) queues behind.
     const v4i cinit = {0, 0, 0, 0};
     v4i dprev[2];
     float as_p = 0.0f;
+    float sc0 = 0.0f, sc1 = 0.0f; // scale products of the token fragment being folded (both row halves)
     auto fold_stage = [&](int st) __attribute__((always_inline)) { // fold the fragments of stage st
       const int tb = st >> 1, h = st & 1;
-      const float sc0 = as_p * bs0, sc1 = as_p * bs1;
+      if constexpr (W4) {
+        fold4(dprev[0], as_p, wsc[h][0], acc[h][tb][0]);
+        fold4(dprev[1], as_p, wsc[h][1], acc[h][tb][1]);
+        return;
+      }
+      if (FAST_SCALE && h == 0) {
+        sc0 = as_p * bs0;
+        sc1 = FUSED_ACT ? as_p * bs1 : sc0;
+      }
       fold(dprev[0], sc0, as_p, bs0, acc[h][tb][0]);
-      fold(dprev[1], sc1, as_p, bs1, acc[h][tb][1]);
+      fold(dprev[1], sc1, as_p, FUSED_ACT ? bs1 : bs0, acc[h][tb][1]);
     };
     // pipeline stage (tb, h): its MFMAs are issued, then the previous stage's fragments are folded
     // while the matrix pipe works; the operands of token fragment tb + 1 are requested in (tb, 0)
@@ -291,7 +370,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
         for (int g = 0; g < 4; ++g) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           if (nst_c >= 8 ? (g < 2 && st < 6) : (g < 3 && st < 4)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, W4 ? 7 : 5, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
         dprev[0] = d[0];
@@ -451,7 +530,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 }
 
 bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
-  if (block_size_m != 128 || !a.w_shuffled || a.w4 || a.per_channel) return false;
+  if (block_size_m != 128 || !a.w_shuffled || a.per_channel) return false;
   if (!fused_act && a.N % 64 != 0) return false;
   return a.K / kGroup <= kTMaxKB;
 }
@@ -467,19 +546,24 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
   const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
-#define LO_T128_LAUNCH(FA, FS, ST)                                                                              \
+#define LO_T128_LAUNCH(FA, FS, ST, W)                                                                           \
   do {                                                                                                          \
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_gemm_t128_kernel<FA, FS, ST>),                  \
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_gemm_t128_kernel<FA, FS, ST, W>),               \
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTLds) != hipSuccess) {                 \
       set_error("moe_gemm(t128): cannot reserve %d bytes of LDS", kTLds);                                       \
       return LO_ELAUNCH;                                                                                        \
     }                                                                                                           \
-    hipLaunchKernelGGL((moe_gemm_t128_kernel<FA, FS, ST>), g, b, kTLds, s, a, mbi, gi);                         \
+    hipLaunchKernelGGL((moe_gemm_t128_kernel<FA, FS, ST, W>), g, b, kTLds, s, a, mbi, gi);                      \
   } while (0)
 #define LO_T128_PICK(FA, FS)                                                                                    \
   do {                                                                                                          \
-    if (stream) LO_T128_LAUNCH(FA, FS, true);                                                                   \
-    else LO_T128_LAUNCH(FA, FS, false);                                                                         \
+    if (a.w4) {                                                                                                 \
+      if (stream) LO_T128_LAUNCH(FA, FS, true, true);                                                           \
+      else LO_T128_LAUNCH(FA, FS, false, true);                                                                 \
+    } else {                                                                                                    \
+      if (stream) LO_T128_LAUNCH(FA, FS, true, false);                                                          \
+      else LO_T128_LAUNCH(FA, FS, false, false);                                                                \
+    }                                                                                                           \
   } while (0)
   // one token block per expert, by and large: the slots spread over the routed experts fill half a block
   const bool stream = a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * (kT / 2);
