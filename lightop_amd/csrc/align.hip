@@ -49,6 +49,10 @@ __device__ __forceinline__ void moe_align_body(
   int32_t *wcnt = total + E;         // [nw][E] per-wave counts, later running bases
 
   for (int i = tid; i < nw * E; i += blockDim.x) wcnt[i] = 0;
+  // Every entry of sorted[] starts as padding (one coalesced sweep while the ids are on their way);
+  // the scatter of pass 3 then overwrites the valid ones.  The workgroup barriers in between
+  // order the two stores to an entry.
+  for (int64_t i = tid; i < sorted_cap; i += blockDim.x) sorted[i] = static_cast<int32_t>(pad_val);
   __syncthreads();
 
   // Each wave owns a contiguous range of slot ids, rounded to whole 64-id tiles.
@@ -57,33 +61,48 @@ __device__ __forceinline__ void moe_align_body(
   const int64_t t0 = wave * tiles_per_wave;
   const int64_t t1 = (t0 + tiles_per_wave < tiles) ? t0 + tiles_per_wave : tiles;
 
-  auto key_of = [&](int64_t f, bool &ok) -> int {
-    ok = f < numel;
-    int e = 0;
-    if (ok) {
-      int64_t raw = static_cast<int64_t>(ids[f]);
-      ok = raw >= 0 && raw < E;
-      e = ok ? static_cast<int>(raw) : 0;
-      if (ok && ignore_invalid && expert_map) {
-        e = expert_map[e];
-        ok = e >= 0 && e < E;
-        if (!ok) e = 0;
-      }
+  // Raw ids of a batch of tiles are fetched back to back (no branch between the loads: an index
+  // past the end re-reads slot 0 and is discarded), then turned into keys.
+  constexpr int kBatch = 8;
+  auto load_raw = [&](int64_t t, int64_t (&raw)[kBatch]) {
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int64_t f = (t + b) * kWave + lane;
+      raw[b] = static_cast<int64_t>(ids[(t + b < t1 && f < numel) ? f : 0]);
+    }
+  };
+  auto key_of = [&](int64_t raw, bool in_range, bool &ok) -> int {
+    ok = in_range && raw >= 0 && raw < E;
+    int e = ok ? static_cast<int>(raw) : 0;
+    if (ignore_invalid && expert_map) { // keys are local expert ids
+      const int m = expert_map[e];
+      ok = ok && m >= 0 && m < E;
+      e = ok ? m : 0;
     }
     return e;
   };
 
-  // pass 1: per-wave histogram.  Counting does not depend on order, so LDS atomics are
-  // fine here; ids are fetched kBatch tiles at a time so that their latency overlaps.
-  constexpr int kBatch = 8;
+  // pass 1: per-wave histogram.  Counting does not depend on order, so LDS atomics are fine
+  // here.  The keys of the wave's first batch stay in registers for pass 3 (up to 8192 slots
+  // on 16 waves that is all of them).
+  int ek0[kBatch];
+  bool ok0[kBatch];
+#pragma unroll
+  for (int b = 0; b < kBatch; ++b) {
+    ek0[b] = 0;
+    ok0[b] = false;
+  }
   for (int64_t t = t0; t < t1; t += kBatch) {
+    int64_t raw[kBatch];
+    load_raw(t, raw);
     int ek[kBatch];
     bool okk[kBatch];
 #pragma unroll
     for (int b = 0; b < kBatch; ++b) {
       const int64_t f = (t + b) * kWave + lane;
-      ek[b] = key_of((t + b < t1) ? f : numel, okk[b]);
-      if (slot_mask && t + b < t1 && f < numel) { // is the slot's expert held by this rank?
+      const bool in_range = t + b < t1 && f < numel;
+      ek[b] = key_of(raw[b], in_range, okk[b]);
+      if (slot_mask && in_range) { // is the slot's expert held by this rank?
         bool local = okk[b];
         if (local && expert_map && !ignore_invalid) local = expert_map[ek[b]] >= 0;
         slot_mask[f] = local ? 1 : 0;
@@ -92,6 +111,13 @@ __device__ __forceinline__ void moe_align_body(
 #pragma unroll
     for (int b = 0; b < kBatch; ++b)
       if (okk[b]) atomicAdd(&wcnt[wave * E + ek[b]], 1);
+    if (t == t0) {
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        ek0[b] = ek[b];
+        ok0[b] = okk[b];
+      }
+    }
   }
   __syncthreads();
 
@@ -133,11 +159,6 @@ __device__ __forceinline__ void moe_align_body(
   }
   for (int64_t b = P / bs + tid; b < expert_ids_cap; b += blockDim.x) expert_ids[b] = -1;
 
-  // padding entries: the tail of every expert's range and everything past P
-  for (int e = wave; e < E; e += nw)
-    for (int i = offs[e] + total[e] + lane; i < offs[e + 1]; i += kWave)
-      sorted[i] = static_cast<int32_t>(pad_val);
-  for (int64_t i = P + tid; i < sorted_cap; i += blockDim.x) sorted[i] = static_cast<int32_t>(pad_val);
 
   // pass 3: stable scatter.  wcnt[wave][e] is the running number of slots of expert
   // e that precede the current tile.  Ranks inside a tile come from a ballot match, the
@@ -145,11 +166,22 @@ __device__ __forceinline__ void moe_align_body(
   for (int64_t t = t0; t < t1; t += kBatch) {
     int ek[kBatch];
     bool okk[kBatch];
+    if (t == t0) {
 #pragma unroll
-    for (int b = 0; b < kBatch; ++b)
-      ek[b] = key_of((t + b < t1) ? (t + b) * kWave + lane : numel, okk[b]);
+      for (int b = 0; b < kBatch; ++b) {
+        ek[b] = ek0[b];
+        okk[b] = ok0[b];
+      }
+    } else {
+      int64_t raw[kBatch];
+      load_raw(t, raw);
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b)
+        ek[b] = key_of(raw[b], t + b < t1 && (t + b) * kWave + lane < numel, okk[b]);
+    }
 #pragma unroll
     for (int b = 0; b < kBatch; ++b) {
+      if (t + b >= t1) break; // wave-uniform
       const int e = ek[b];
       const bool ok = okk[b];
       const int64_t f = (t + b) * kWave + lane;
@@ -162,7 +194,9 @@ __device__ __forceinline__ void moe_align_body(
         __builtin_amdgcn_wave_barrier();
         if (lane == leader) wcnt[wave * E + e] = base + __popcll(peers);
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      // the counters are LDS words touched by this wave only, and a wave's LDS operations
+      // execute in order: the next tile sees them without waiting for the global stores
+      asm volatile("" ::: "memory");
       __builtin_amdgcn_wave_barrier();
     }
   }
@@ -379,11 +413,12 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
 }
 
 // chunks for the multi-workgroup path: about 1024 slots each, at most 256 chunks
-static void single_wg_shape(int64_t numel, int32_t num_experts, int *nw, size_t *lds_bytes) {
+static void single_wg_shape(int64_t numel, int64_t sorted_cap, int32_t num_experts, int *nw, size_t *lds_bytes) {
   // waves per workgroup: as many as the per-wave LDS counters allow (<= 60 KB)
   int w = 16;
   while (w > 1 && (static_cast<int64_t>(w) + 2) * num_experts + 1 > 15360) w >>= 1;
-  if (numel <= 64 * 4) w = w < 4 ? w : 4;
+  // a handful of slots need few waves - unless the padded buffer they have to fill is long
+  if (numel <= 64 * 4 && sorted_cap <= 4096) w = w < 4 ? w : 4;
   *nw = w;
   *lds_bytes = (static_cast<size_t>(w + 2) * num_experts + 1) * sizeof(int32_t);
 }
@@ -417,7 +452,7 @@ int launch_quant_align(const void *x, int64_t M, int64_t H, float eps, int8_t *q
   while ((1 << key_bits) < num_experts) ++key_bits;
   int nw;
   size_t lds_bytes;
-  single_wg_shape(numel, num_experts, &nw, &lds_bytes);
+  single_wg_shape(numel, sorted_cap, num_experts, &nw, &lds_bytes);
   const int64_t groups = M * (H / kGroup);
   const int per_block = nw * kWave / 16;
   int64_t qblocks = (groups + per_block - 1) / per_block;
@@ -544,7 +579,7 @@ extern "C" int lo_moe_align_block_size_local(const void *topk_ids, int ids_dtype
 
   int nw;
   size_t lds_bytes;
-  single_wg_shape(numel, num_experts, &nw, &lds_bytes);
+  single_wg_shape(numel, sorted_cap, num_experts, &nw, &lds_bytes);
   if (ids_dtype == LO_I32)
     hipLaunchKernelGGL(moe_align_kernel<int32_t>, dim3(1), dim3(nw * kWave), lds_bytes, s,
                        static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,
