@@ -243,17 +243,16 @@ template <typename IdT>
 __device__ __forceinline__ int align_key(const IdT *__restrict__ ids, int64_t f, int64_t numel, int E,
                                          const int32_t *__restrict__ expert_map, int ignore_invalid,
                                          bool &ok) {
-  ok = f < numel;
-  int e = 0;
-  if (ok) {
-    int64_t raw = static_cast<int64_t>(ids[f]);
-    ok = raw >= 0 && raw < E;
-    e = ok ? static_cast<int>(raw) : 0;
-    if (ok && ignore_invalid && expert_map) {
-      e = expert_map[e];
-      ok = e >= 0 && e < E;
-      if (!ok) e = 0;
-    }
+  // no branch around the load (an index past the end re-reads slot 0 and is discarded), so that
+  // the loads of a batch of tiles are issued back to back
+  const bool in_range = f < numel;
+  const int64_t raw = static_cast<int64_t>(ids[in_range ? f : 0]);
+  ok = in_range && raw >= 0 && raw < E;
+  int e = ok ? static_cast<int>(raw) : 0;
+  if (ignore_invalid && expert_map) {
+    const int m = expert_map[e];
+    ok = ok && m >= 0 && m < E;
+    e = ok ? m : 0;
   }
   return e;
 }
@@ -262,11 +261,16 @@ template <typename IdT>
 __global__ __launch_bounds__(256) void moe_align_count_kernel(
     const IdT *__restrict__ ids, int64_t numel, int E, const int32_t *__restrict__ expert_map,
     int ignore_invalid, int64_t chunk_slots, int32_t *__restrict__ cnt, uint8_t *__restrict__ slot_mask,
-    const int32_t *__restrict__ num_local_tokens, int slots_per_token) {
+    const int32_t *__restrict__ num_local_tokens, int slots_per_token, int32_t *__restrict__ sorted,
+    int64_t sorted_cap) {
   extern __shared__ int32_t lds[];
   for (int i = threadIdx.x; i < E; i += blockDim.x) lds[i] = 0;
   __syncthreads();
   const int64_t pad_val = numel;
+  // every entry of sorted[] starts as padding; the second launch overwrites the valid ones
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < sorted_cap;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    sorted[i] = static_cast<int32_t>(pad_val);
   numel = local_slots(numel, num_local_tokens, slots_per_token);
   const int64_t begin = blockIdx.x * chunk_slots;
   const int64_t end = (begin + chunk_slots < numel) ? begin + chunk_slots : numel;
@@ -303,7 +307,6 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
     int64_t expert_ids_cap, int32_t *__restrict__ ntpp, int key_bits,
     const int32_t *__restrict__ num_local_tokens, int slots_per_token) {
   extern __shared__ int32_t lds[];
-  const int64_t pad_val = numel;
   numel = local_slots(numel, num_local_tokens, slots_per_token);
   constexpr int nw = 4;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -315,18 +318,32 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
   __shared__ int32_t wave_sum[nw];
 
   for (int i = tid; i < nw * E; i += blockDim.x) wcnt[i] = 0;
+  for (int i = tid; i < E; i += blockDim.x) total[i] = cbase[i] = 0;
+  __syncthreads();
+  // per expert: slots in all chunks and in the chunks before this one (coalesced sweep over
+  // cnt[chunk][expert]; integer sums, so the order of the LDS atomics does not matter)
+  constexpr int kSweep = 16; // loads in flight per thread: the sweep is a few round trips, not one per entry
+  for (int idx0 = tid; idx0 < nchunks * E; idx0 += kSweep * blockDim.x) {
+    int v[kSweep];
+#pragma unroll
+    for (int u = 0; u < kSweep; ++u) {
+      const int idx = idx0 + u * blockDim.x;
+      v[u] = cnt[idx < nchunks * E ? idx : 0];
+    }
+#pragma unroll
+    for (int u = 0; u < kSweep; ++u) {
+      const int idx = idx0 + u * blockDim.x;
+      const int c = idx / E, e = idx - c * E;
+      if (idx < nchunks * E && v[u]) {
+        atomicAdd(&total[e], v[u]);
+        if (c < chunk) atomicAdd(&cbase[e], v[u]);
+      }
+    }
+  }
+  __syncthreads();
   for (int base = 0; base < E; base += blockDim.x) {
     const int e = base + tid;
-    int t = 0, b = 0;
-    if (e < E) {
-      for (int c = 0; c < nchunks; ++c) {
-        const int v = cnt[static_cast<int64_t>(c) * E + e];
-        if (c < chunk) b += v;
-        t += v;
-      }
-      total[e] = t;
-      cbase[e] = b;
-    }
+    const int t = (e < E) ? total[e] : 0;
     int incl = (e < E) ? (t + bs - 1) / bs * bs : 0;
     for (int d = 1; d < kWave; d <<= 1) {
       int up = __shfl_up(incl, d);
@@ -344,15 +361,12 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
 
   // shared-out bookkeeping: workgroup c looks after experts c, c + nchunks, ...
   if (chunk == 0 && tid == 0) ntpp[0] = P;
-  for (int e = chunk; e < E; e += nchunks) {
+  for (int e = chunk + tid * nchunks; e < E; e += nchunks * blockDim.x) { // one thread per expert: the map reads overlap
     const int v = (expert_map && !ignore_invalid) ? expert_map[e] : e;
-    for (int b = offs[e] / bs + tid; b < offs[e + 1] / bs; b += blockDim.x) expert_ids[b] = v;
-    for (int i = offs[e] + total[e] + tid; i < offs[e + 1]; i += blockDim.x) sorted[i] = static_cast<int32_t>(pad_val);
+    for (int b = offs[e] / bs; b < offs[e + 1] / bs; ++b) expert_ids[b] = v;
   }
   for (int64_t b = P / bs + chunk * blockDim.x + tid; b < expert_ids_cap; b += static_cast<int64_t>(nchunks) * blockDim.x)
     expert_ids[b] = -1;
-  for (int64_t i = P + chunk * blockDim.x + tid; i < sorted_cap; i += static_cast<int64_t>(nchunks) * blockDim.x)
-    sorted[i] = static_cast<int32_t>(pad_val);
 
   // this chunk: contiguous sub-range per wave, whole 64-slot tiles
   const int64_t begin = chunk * chunk_slots;
@@ -362,6 +376,13 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
   const int64_t t0 = wave * tiles_per_wave;
   const int64_t t1 = (t0 + tiles_per_wave < tiles) ? t0 + tiles_per_wave : tiles;
   constexpr int kBatch = 4;
+  int ek0[kBatch]; // keys of the wave's first batch, kept for the scatter below
+  bool ok0[kBatch];
+#pragma unroll
+  for (int b = 0; b < kBatch; ++b) {
+    ek0[b] = 0;
+    ok0[b] = false;
+  }
   for (int64_t t = t0; t < t1; t += kBatch) {
     int ek[kBatch];
     bool okk[kBatch];
@@ -373,6 +394,13 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
 #pragma unroll
     for (int b = 0; b < kBatch; ++b)
       if (okk[b]) atomicAdd(&wcnt[wave * E + ek[b]], 1);
+    if (t == t0) {
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        ek0[b] = ek[b];
+        ok0[b] = okk[b];
+      }
+    }
   }
   __syncthreads();
   for (int e = tid; e < E; e += blockDim.x) {
@@ -387,13 +415,22 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
   for (int64_t t = t0; t < t1; t += kBatch) {
     int ek[kBatch];
     bool okk[kBatch];
+    if (t == t0) {
 #pragma unroll
-    for (int b = 0; b < kBatch; ++b) {
-      const int64_t f = begin + (t + b) * kWave + lane;
-      ek[b] = align_key(ids, (t + b < t1 && f < end) ? f : numel, numel, E, expert_map, ignore_invalid, okk[b]);
+      for (int b = 0; b < kBatch; ++b) {
+        ek[b] = ek0[b];
+        okk[b] = ok0[b];
+      }
+    } else {
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        const int64_t f = begin + (t + b) * kWave + lane;
+        ek[b] = align_key(ids, (t + b < t1 && f < end) ? f : numel, numel, E, expert_map, ignore_invalid, okk[b]);
+      }
     }
 #pragma unroll
     for (int b = 0; b < kBatch; ++b) {
+      if (t + b >= t1) break; // wave-uniform
       const int e = ek[b];
       const bool ok = okk[b];
       const int64_t f = begin + (t + b) * kWave + lane;
@@ -406,7 +443,7 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
         __builtin_amdgcn_wave_barrier();
         if (lane == leader) wcnt[wave * E + e] = run + __popcll(peers);
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      asm volatile("" ::: "memory"); // a wave's LDS operations execute in order: no wait for the global stores
       __builtin_amdgcn_wave_barrier();
     }
   }
@@ -560,7 +597,7 @@ extern "C" int lo_moe_align_block_size_local(const void *topk_ids, int ids_dtype
     if (ids_dtype == LO_I32) {
       hipLaunchKernelGGL(moe_align_count_kernel<int32_t>, dim3(nchunks), dim3(256), lds1, s,
                          static_cast<const int32_t *>(topk_ids), numel, num_experts, expert_map,
-                         ignore_invalid, cs, cnt, slot_mask, num_local_tokens, top_k);
+                         ignore_invalid, cs, cnt, slot_mask, num_local_tokens, top_k, sorted_ids, sorted_cap);
       hipLaunchKernelGGL(moe_align_scatter_kernel<int32_t>, dim3(nchunks), dim3(256), lds2, s,
                          static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size,
                          expert_map, ignore_invalid, cs, cnt, sorted_ids, sorted_cap, expert_ids,
@@ -568,7 +605,7 @@ extern "C" int lo_moe_align_block_size_local(const void *topk_ids, int ids_dtype
     } else {
       hipLaunchKernelGGL(moe_align_count_kernel<int64_t>, dim3(nchunks), dim3(256), lds1, s,
                          static_cast<const int64_t *>(topk_ids), numel, num_experts, expert_map,
-                         ignore_invalid, cs, cnt, slot_mask, num_local_tokens, top_k);
+                         ignore_invalid, cs, cnt, slot_mask, num_local_tokens, top_k, sorted_ids, sorted_cap);
       hipLaunchKernelGGL(moe_align_scatter_kernel<int64_t>, dim3(nchunks), dim3(256), lds2, s,
                          static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size,
                          expert_map, ignore_invalid, cs, cnt, sorted_ids, sorted_cap, expert_ids,
