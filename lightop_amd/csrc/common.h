@@ -232,12 +232,11 @@ __device__ __forceinline__ void group_quant_body(const uint16_t *__restrict__ x,
     for (int d = 1; d < 16; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
     amax = fmaxf(amax, eps);
     const float sc = amax / 127.0f;
-    int qi[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) qi[i] = quant_one(v[i], sc);
+    // one IEEE reciprocal per group, then the correctly rounded quotient per value (quant4)
+    const float rsc = 1.0f / sc;
     v2i packed;
-    packed[0] = static_cast<int>(pack4_i8(qi[0], qi[1], qi[2], qi[3]));
-    packed[1] = static_cast<int>(pack4_i8(qi[4], qi[5], qi[6], qi[7]));
+    packed[0] = static_cast<int>(quant4(&v[0], sc, rsc));
+    packed[1] = static_cast<int>(quant4(&v[4], sc, rsc));
     *reinterpret_cast<v2i *>(q + g * kGroup + sub * 8) = packed;
     if (sub == 0) s[g] = sc;
   }
