@@ -224,7 +224,12 @@ static void launch_row_quant(const uint16_t *x, int64_t rows, int64_t C, const u
 // ---- moe_sum -------------------------------------------------------------------
 // Reference: csrc/kernels/moe_align_sum_kernels.cu:604-637 (fp32 accumulation in slot
 // order, one rounding) and :886-909 (with bias: three roundings).
-template <int DT, bool HAS_BIAS>
+// TOPK > 0: the slot count is a compile-time constant, so the mask bytes and then the rows of
+// the unmasked slots are requested back to back and waited for once (with a run-time count every
+// mask byte and every row is a round trip of its own).  A masked slot adds
+// +0.0f instead of being skipped, which is the same value: the sum starts at +0.0f and can
+// never become -0.0f.  TOPK = 0 keeps the run-time loop.
+template <int DT, bool HAS_BIAS, int TOPK>
 __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t *__restrict__ in,
                                                       uint16_t *__restrict__ out,
                                                       const uint16_t *__restrict__ bias,
@@ -244,11 +249,27 @@ __global__ __launch_bounds__(256) void moe_sum_kernel(const uint16_t *__restrict
     const int64_t t = v / vec_per_row, c = (v % vec_per_row) * 8;
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     const uint16_t *p = in + t * topk * H + c;
-    for (int j = 0; j < topk; ++j) {
-      if (mask && !mask[t * topk + j]) continue; // slot of an expert on another rank: adds 0
-      const v8u16 r = *reinterpret_cast<const v8u16 *>(p + static_cast<int64_t>(j) * H);
+    if constexpr (TOPK > 0) {
+      bool on[TOPK];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = acc[i] + to_f32<DT>(r[i]);
+      for (int j = 0; j < TOPK; ++j) on[j] = !mask || mask[t * TOPK + j] != 0;
+      v8u16 r[TOPK];
+#pragma unroll
+      for (int j = 0; j < TOPK; ++j) {
+        r[j] = v8u16{0, 0, 0, 0, 0, 0, 0, 0};
+        if (on[j]) r[j] = *reinterpret_cast<const v8u16 *>(p + static_cast<int64_t>(j) * H);
+      }
+#pragma unroll
+      for (int j = 0; j < TOPK; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = acc[i] + to_f32<DT>(r[j][i]);
+    } else {
+      for (int j = 0; j < topk; ++j) {
+        if (mask && !mask[t * topk + j]) continue; // slot of an expert on another rank: adds 0
+        const v8u16 r = *reinterpret_cast<const v8u16 *>(p + static_cast<int64_t>(j) * H);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = acc[i] + to_f32<DT>(r[i]);
+      }
     }
     v8u16 o;
     if constexpr (HAS_BIAS) {
@@ -379,14 +400,25 @@ extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uin
   if (M == 0) return LO_OK;
   const int grid = grid_for(M * (H / 8), 256);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (bias)
-    hipLaunchKernelGGL((moe_sum_kernel<LO_BF16, true>), dim3(grid), dim3(256), 0, s,
-                       static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),
-                       static_cast<const uint16_t *>(bias), expert_mask, M, topk, H, factor, num_local_tokens);
-  else
-    hipLaunchKernelGGL((moe_sum_kernel<LO_BF16, false>), dim3(grid), dim3(256), 0, s,
-                       static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),
-                       static_cast<const uint16_t *>(nullptr), expert_mask, M, topk, H, factor, num_local_tokens);
+#define LO_SUM_LAUNCH(HB, TK)                                                                        \
+  hipLaunchKernelGGL((moe_sum_kernel<LO_BF16, HB, TK>), dim3(grid), dim3(256), 0, s,                \
+                     static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),               \
+                     static_cast<const uint16_t *>(bias), expert_mask, M, topk, H, factor, num_local_tokens)
+#define LO_SUM_PICK(TK)                                                                              \
+  do {                                                                                               \
+    if (bias) LO_SUM_LAUNCH(true, TK);                                                               \
+    else LO_SUM_LAUNCH(false, TK);                                                                   \
+  } while (0)
+  switch (topk) { // the usual router widths get the unrolled form
+    case 1: LO_SUM_PICK(1); break;
+    case 2: LO_SUM_PICK(2); break;
+    case 4: LO_SUM_PICK(4); break;
+    case 6: LO_SUM_PICK(6); break;
+    case 8: LO_SUM_PICK(8); break;
+    default: LO_SUM_PICK(0); break;
+  }
+#undef LO_SUM_PICK
+#undef LO_SUM_LAUNCH
   return check_launch("moe_sum");
 }
 
