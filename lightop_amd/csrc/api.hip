@@ -74,12 +74,12 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
                             bool preshuffled = true) {
   const double per_expert = static_cast<double>(M) * top_k / (num_experts > 0 ? num_experts : 1);
   // W4A8: the streaming kernel re-reads the token rows per wave, which outweighs the half-size
-  // weights early; the LDS-tiled kernel (64 tokens) wins from about 8 slots per expert.
+  // weights early; the LDS-tiled kernel (64 tokens) wins above about 8 slots per expert.
   // From 48 slots per expert on the 128-token kernel takes over (measured, 64 / 128: 475 / 394 us at
   // 1024 tokens of the Qwen3-235B-A22B-shaped layer, 720 / 660 at 2048, 1227 / 1074 at 4096; equal
   // or 3 % behind up to 512 tokens, where a K block of half-size weights is shorter than the memory
   // round trip it would have to hide).
-  if (form == LO_FORM_W4) return per_expert < 8.0 ? 16 : (per_expert < 48.0 ? 64 : 128);
+  if (form == LO_FORM_W4) return per_expert <= 8.0 ? 16 : (per_expert < 48.0 ? 64 : 128);
   // Block form with pre-shuffled weights: the kernel that copies both operands straight into LDS
   // (gemm_t128.hip, 128-token blocks, padded parts of a block skipped in steps of 32 tokens) takes
   // over from the weight-streaming kernels as soon as an expert sees a handful of tokens - with

@@ -135,7 +135,11 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       woff[g] = static_cast<int>((nrow[g] + r) * K) + c * 16;
     const int64_t nclamp = nrow[g] < N ? nrow[g] : 0; // fragments past N: loads return 0, nothing is stored
     wsrow[g] = a.Ws + (static_cast<int64_t>(e) * NB + nclamp / kGroup) * KB;
-    wsoff[g] = static_cast<int>((nclamp + 4 * c) * 4); // accumulator rows of this lane: 4c .. 4c+3
+    // accumulator rows of this lane: 4c .. 4c+3.  Inside the K loop (W4) a lane fetches only the
+    // scale of row 4c + (lane & 3) - a 4-byte load costs the texture path a quarter of a 16-byte
+    // one, and these kernels issue as many scale loads as weight loads - and gets the other
+    // three from its quad neighbours when the scales are used.
+    wsoff[g] = static_cast<int>((nclamp + 4 * c + ((W4 && !PC) ? (lane & 3) : 0)) * 4);
   }
 
   v4f acc[NW][TM];
@@ -155,7 +159,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   v4i wbuf[PD][NW][W4 ? 1 : 2];
   v4i abuf[PD][TM][2];
   float asbuf[PD][TM];
-  float bsbuf[PD][NW][NS];
+  float bsbuf[PD][NW][1]; // W4: the scale of row 4c + (lane & 3); the quad holds the lane's four
   // The loop body is kept free of branches: a slot past the end of K re-reads the last
   // K block and gets a token scale of zero, so it adds exactly 0 to every accumulator.
   // (Branches around the loads make the compiler fall back to waiting for all of them.)
@@ -179,12 +183,8 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
     if constexpr (PC) return; // no scales inside the K loop
 #pragma unroll
     for (int g = 0; g < NW; ++g) {
-      if constexpr (W4) { // scales are stored [E][K/128][N]: the lane's four rows are 16 contiguous bytes
-        const v4f sv = __builtin_bit_cast(v4f, bld16(rWs, wsoff[g], kc * static_cast<int>(N) * 4));
-        bsbuf[slot][g][0] = sv.x;
-        bsbuf[slot][g][NS > 1 ? 1 : 0] = NS > 1 ? sv.y : sv.x;
-        bsbuf[slot][g][NS > 2 ? 2 : 0] = NS > 2 ? sv.z : sv.x;
-        bsbuf[slot][g][NS > 3 ? 3 : 0] = NS > 3 ? sv.w : sv.x;
+      if constexpr (W4) { // scales are stored [E][K/128][N]
+        bsbuf[slot][g][0] = bld_f32(rWs, wsoff[g], kc * static_cast<int>(N) * 4);
       } else {
         bsbuf[slot][g][0] = wsrow[g][kc];
       }
@@ -243,9 +243,17 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       float bs[NW][NS], as[TM];
       if constexpr (!PC) {
 #pragma unroll
-        for (int g = 0; g < NW; ++g)
-#pragma unroll
-          for (int i = 0; i < NS; ++i) bs[g][i] = bsbuf[p][g][i];
+        for (int g = 0; g < NW; ++g) {
+          if constexpr (W4) { // quad broadcasts: lane i of the quad holds row 4c + i
+            const int raw = __builtin_bit_cast(int, bsbuf[p][g][0]);
+            bs[g][0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0x00, 0xf, 0xf, false));
+            bs[g][NS > 1 ? 1 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0x55, 0xf, 0xf, false));
+            bs[g][NS > 2 ? 2 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0xaa, 0xf, 0xf, false));
+            bs[g][NS > 3 ? 3 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0xff, 0xf, 0xf, false));
+          } else {
+            bs[g][0] = bsbuf[p][g][0];
+          }
+        }
 #pragma unroll
         for (int j = 0; j < TM; ++j) as[j] = kb < KB ? asbuf[p][j] : 0.0f; // dead slot: adds 0
       }

@@ -80,7 +80,7 @@ def test_version_and_tile_table(lib):
         assert lib.lo_moe_tile_query_form(_lib.LO_FORM_CHANNEL, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
         assert t1.block_size_m == want and t2.block_size_m == want
     # W4A8: streaming for a handful of slots per expert, the 64-token LDS tile from 8 on, 128 tokens from 48 on
-    for M, want in ((1, 16), (128, 16), (256, 64), (1024, 64), (2048, 128), (8192, 128)):
+    for M, want in ((1, 16), (128, 16), (256, 16), (512, 64), (1024, 64), (2048, 128), (8192, 128)):
         assert lib.lo_moe_tile_query_form(_lib.LO_FORM_W4, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
         assert t1.block_size_m == want
     assert lib.lo_moe_tile_query_form(7, 1, 32, 256, 8, 7168, 2048, t1, t2) < 0
