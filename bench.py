@@ -34,8 +34,8 @@ MEASURED_TRAFFIC = {
     ("deepseek-v3-ep8-share", 64): 806123059,
     ("deepseek-v3-ep8-share", 1024): 961596966,
     ("deepseek-v3-ep8-share", 4096): 1295378508,
-    ("qwen3-235b-a22b-w4a8", 2048): 1340958217,
-    ("qwen3-235b-a22b-w4a8", 32): 777716435,
+    ("qwen3-235b-a22b-w4a8", 2048): 1341109180,
+    ("qwen3-235b-a22b-w4a8", 32): 778618758,
 }
 
 
