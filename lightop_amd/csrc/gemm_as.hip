@@ -100,7 +100,9 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
 
   const int NB = static_cast<int>((N + kGroup - 1) / kGroup);
   const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * N * K, static_cast<uint32_t>(N * K));
-  const brsrc rWs = make_rsrc(a.Ws + static_cast<int64_t>(e) * NB * KB, static_cast<uint32_t>(NB * KB * 4));
+  // the offset in 32 bits: a 64-bit multiply is a vector instruction, and a descriptor that has
+  // been through vector registers costs a readfirstlane loop at every load
+  const brsrc rWs = make_rsrc(a.Ws + e * NB * KB, static_cast<uint32_t>(NB * KB * 4));
   // lane offsets inside tile nt0; a later tile and the K block go into the scalar offset
   int woff[2], wsoff[2];
   const int wkstride = SHUF ? shuf_kb_stride(static_cast<int>(N / 16)) : kGroup;
@@ -191,10 +193,18 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
   };
 
   // The (tile, K block) pairs form one flat sequence of steps; step s uses buffer s % 3.
+  // Positions in that sequence are kept as (tile, K block) counters: a division by KB per step
+  // is a long scalar dependency chain in front of the loads.
   const int total = (nt_end - nt0) * KB;
-  auto load_step = [&](auto BUF, int s) __attribute__((always_inline)) { // a step past the end re-reads the last one
-    const int sc = s < total ? s : total - 1;
-    load_w(BUF, nt0 + sc / KB, sc % KB);
+  int l_nt = nt0, l_kb = 0; // the next step to load
+  int c_nt = nt0, c_kb = 0; // the next step to compute
+  auto load_step = [&](auto BUF) __attribute__((always_inline)) { // a step past the end re-reads the last one
+    const bool past = l_nt >= nt_end;
+    load_w(BUF, past ? nt_end - 1 : l_nt, past ? KB - 1 : l_kb);
+    if (++l_kb == KB) {
+      l_kb = 0;
+      ++l_nt;
+    }
   };
   auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
@@ -218,34 +228,36 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
         for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            float v = acc[tb][rb][4 * q + i];
-            if (a.mul_routed) v = v * w;
-            o[rb][q][i] = f32_to_bf16(v);
+            o[rb][q][i] = f32_to_bf16(acc[tb][rb][4 * q + i] * w); // w = 1 leaves every value as it is
           }
       wave_store_32x64_bf16(stg, o, valid[tb] ? static_cast<int>(f[tb]) : -1, a.C, N, nrow0, lane);
     }
   };
-  auto step = [&](auto BUF, auto NEXT, int s) __attribute__((always_inline)) {
-    load_step(NEXT, s + 2);
+  auto step = [&](auto BUF, auto NEXT) __attribute__((always_inline)) {
+    load_step(NEXT);
     __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMAs
-    const int kb = s % KB;
-    compute(BUF, kb, s < total);
-    if (s < total && kb == KB - 1) { // a tile is complete
-      store_tile(nt0 + s / KB);
+    const bool live = c_nt < nt_end;
+    compute(BUF, c_kb, live);
+    if (live && c_kb == KB - 1) { // a tile is complete
+      store_tile(c_nt);
       zero_acc();
+    }
+    if (++c_kb == KB) {
+      c_kb = 0;
+      ++c_nt;
     }
   };
 
   if (total > 0) { // before the barrier: in flight while the tokens land
-    load_step(B0{}, 0);
-    load_step(B1{}, 1);
+    load_step(B0{});
+    load_step(B1{});
   }
   __syncthreads(); // the only barrier: the token block is complete
   zero_acc();
   for (int s = 0; s < total; s += 3) {
-    step(B0{}, B2{}, s);
-    step(B1{}, B0{}, s + 1);
-    step(B2{}, B1{}, s + 2);
+    step(B0{}, B2{});
+    step(B1{}, B0{});
+    step(B2{}, B1{});
   }
 }
 
