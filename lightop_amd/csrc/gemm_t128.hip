@@ -41,7 +41,8 @@ constexpr int kTS = 2 * kT * 4;               // [stage][token] scales
 constexpr int kTRed = 4 * kT * 4;             // [wave][token] amax exchange of the fused epilogue
 constexpr int kTMaxKB = 128;                  // K blocks whose weight-block scales fit the table below
 constexpr int kTBs = 2 * kTMaxKB * 4;         // [fragment][K block] weight-block scales of the tile
-constexpr int kTLds = kTW + kTA + kTS + kTRed + kTBs + 2 * kSiluBandN * 2;
+constexpr int kTIds = kT * 4;                  // the tile's sorted ids, for the epilogues
+constexpr int kTLds = kTW + kTA + kTS + kTRed + kTBs + kTIds + 2 * kSiluBandN * 2;
 constexpr int kTPitch = 144;                  // staging pitch of the epilogues: 128 + 16
 
 // Wait until all but the newest `N` vector-memory operations of this wave are complete and its
@@ -64,7 +65,8 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   float *const sS = reinterpret_cast<float *>(smem + kTW + kTA);
   float *const sRed = reinterpret_cast<float *>(smem + kTW + kTA + kTS);
   float *const sBs = reinterpret_cast<float *>(smem + kTW + kTA + kTS + kTRed);
-  uint16_t *const sSilu = reinterpret_cast<uint16_t *>(smem + kTW + kTA + kTS + kTRed + kTBs);
+  int32_t *const sIds = reinterpret_cast<int32_t *>(smem + kTW + kTA + kTS + kTRed + kTBs);
+  uint16_t *const sSilu = reinterpret_cast<uint16_t *>(smem + kTW + kTA + kTS + kTRed + kTBs + kTIds);
 
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
@@ -177,6 +179,9 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     const int64_t lf = sorted[tid & (kT - 1)];
     const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
     asoff = static_cast<int>(lrow * KB * 4);
+    // The epilogues take the ids from LDS: a global load in each of their exec-masked blocks is a
+    // full memory round trip that nothing overlaps.
+    if (tid < kT) sIds[tid] = static_cast<int32_t>(lf);
   }
   // weight-block scales of the tile: table row 0 / 1 = gate / up block (fused), or the first / second
   // 128 rows of the tile (plain: waves 0, 1 / waves 2, 3).  Thread t fetches entry (t >> 7, t & 127).
@@ -303,15 +308,31 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
             w[h][rf][kh] = *reinterpret_cast<const v4i *>(sWw + ((h * 2 + rf) * 2 + kh) * 1024 + lane * 16);
     }
   };
+  // Full tiles meet at the barrier two stages before the end of a K block instead of at its start:
+  // by then every copy for the next K block has had eight stages to land and nobody reads this K
+  // block's token stage or scales any more, so the next block's first operands are read from LDS
+  // under the last two stages and no wave stands waiting for LDS right after a barrier.
+  float s_pending;   // token scales on their way from global memory to sS
+  v4i bf_first[2];   // first token fragment of the next K block
+  float as_first = 0.0f;
   auto kblock = [&](auto NST, int kb) __attribute__((always_inline)) {
     constexpr int nst_c = decltype(NST)::value; // stages of this variant: 4, 8, 12 or 16
+    constexpr bool kEarly = nst_c == 16 && !W4;
     const int8_t *ta = sA + (kb & 1) * kTAStage;
     const float *ts = sS + (kb & 1) * kT;
     v4i bf[2][2];
-#pragma unroll
-    for (int kh = 0; kh < 2; ++kh) bf[0][kh] = *reinterpret_cast<const v4i *>(ta + alds[kh]);
     float as_t[2];
-    as_t[0] = ts[r];
+    if constexpr (kEarly) {
+      // this wave's reads of the weight stage are complete before copies are aimed at it again
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      bf[0][0] = bf_first[0];
+      bf[0][1] = bf_first[1];
+      as_t[0] = as_first;
+    } else {
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) bf[0][kh] = *reinterpret_cast<const v4i *>(ta + alds[kh]);
+      as_t[0] = ts[r];
+    }
     const float bs0 = W4 ? 0.0f : sBs0[kb], bs1 = W4 ? 0.0f : sBs1[kb];
 
     // The weight stage was read into registers before the barrier, so it is free; it and the other
@@ -351,6 +372,12 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
         copy_piece(3 * st + 2, kb + 1);
       }
       if (st < nst_c) {
+        if (kEarly && st == 14) {
+          wait_copies_barrier<0>();
+          if (tid < kT) sS[(kb & 1) * kT + tid] = kb + 2 < KB ? s_pending : 0.0f;
+          s_pending = load_scale(kb + 3);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         if (h == 0 && st + 2 < nst_c) {
 #pragma unroll
           for (int kh = 0; kh < 2; ++kh)
@@ -364,6 +391,19 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
         for (int rf = 0; rf < 2; ++rf)
           d[rf] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[h][rf][1], bf[cur][1], d[rf], 0, 0, 0);
+        if (kEarly && st >= 14) { // the next K block's operands of this half, over the ones just used
+#pragma unroll
+          for (int rf = 0; rf < 2; ++rf)
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh)
+              w[h][rf][kh] = *reinterpret_cast<const v4i *>(sWw + ((h * 2 + rf) * 2 + kh) * 1024 + lane * 16);
+          if (st == 14) {
+            const int8_t *tan = sA + ((kb + 1) & 1) * kTAStage;
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) bf_first[kh] = *reinterpret_cast<const v4i *>(tan + alds[kh]);
+            as_first = sS[((kb + 1) & 1) * kT + r];
+          }
+        }
         if (st > 0) fold_stage(st - 1);
         if (h == 0 && st + 2 < nst_c) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
 #pragma unroll
@@ -372,6 +412,8 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
           if (nst_c >= 8 ? (g < 2 && st < 6) : (g < 3 && st < 4)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x002, W4 ? 7 : 5, 0);
         }
+        if (kEarly && st == 14) __builtin_amdgcn_sched_group_barrier(0x100, 7, 0);
+        if (kEarly && st == 15) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
         __builtin_amdgcn_sched_barrier(0);
         dprev[0] = d[0];
         dprev[1] = d[1];
@@ -380,14 +422,17 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     }
     fold_stage(nst_c - 1);
     __builtin_amdgcn_sched_barrier(0);
-    // the next K block's weights have had a whole K block to arrive; reading them here puts the
-    // LDS latency under the barrier instead of in front of the first MFMA
-    wait_copies<0>();
-    read_w();
+    if constexpr (!kEarly) {
+      // the next K block's weights have had a whole K block to arrive; reading them here puts the
+      // LDS latency under the barrier instead of in front of the first MFMA
+      wait_copies<0>();
+      read_w();
+    }
   };
 
   // ---- prologue ------------------------------------------------------------------------------------------
-  float s_now = load_scale(0), s_pending = load_scale(1);
+  float s_now = load_scale(0);
+  s_pending = load_scale(1);
   __builtin_amdgcn_sched_barrier(0);
   copy_a(0);
   __builtin_amdgcn_sched_barrier(0);
@@ -398,6 +443,17 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   read_w();
 
   auto k_loop = [&](auto NST) __attribute__((always_inline)) {
+    if constexpr (decltype(NST)::value == 16 && !W4) {
+      wait_copies_barrier<0>(); // K block 0 is complete in LDS
+      if (tid < kT) sS[kT + tid] = 1 < KB ? s_pending : 0.0f;
+      s_pending = load_scale(2);
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) bf_first[kh] = *reinterpret_cast<const v4i *>(sA + alds[kh]);
+      as_first = sS[r];
+      __builtin_amdgcn_sched_barrier(0);
+      for (int kb = 0; kb < KB; ++kb) kblock(NST, kb);
+      return;
+    }
     for (int kb = 0; kb < KB; ++kb) {
       // every copy this wave requested a K block ago has landed; after the barrier so have everyone
       // else's token rows, and nobody still reads the token stage and the scales of K block kb-1,
@@ -423,7 +479,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
     for (int tb = 0; tb < 8; ++tb) {
       if (2 * tb >= nst) continue;
-      const int64_t ft = sorted[tb * 16 + r];
+      const int64_t ft = sIds[tb * 16 + r];
       const bool valid = ft < a.num_valid;
       float wgt = 1.0f;
       if (a.mul_routed && valid) wgt = a.topk_w[ft];
@@ -457,7 +513,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     if (a.mul_routed) { // router weight on the first GEMM's output: rare, kept out of the main pass
 #pragma unroll
       for (int tb = 0; tb < 8; ++tb) {
-        const int64_t ft = sorted[tb * 16 + r];
+        const int64_t ft = sIds[tb * 16 + r];
         const float wgt = ft < a.num_valid ? a.topk_w[ft] : 1.0f;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
@@ -467,9 +523,11 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
             for (int i = 0; i < 4; ++i) acc[h][tb][rf][i] = acc[h][tb][rf][i] * wgt;
       }
     }
+    // Token fragments are in use in pairs (nst is a multiple of four stages).  A pair shares one
+    // wave-uniform branch, so the LDS lookups of its two fragments are in flight together.
 #pragma unroll
     for (int tb = 0; tb < 8; ++tb) {
-      if (2 * tb >= nst) continue;
+      if (2 * (tb & ~1) >= nst) continue; // the same condition for both fragments of a pair
       uint16_t g16[2][4], u16[2][4];
       bool special = false;
 #pragma unroll
@@ -501,19 +559,27 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     const int64_t G = I / kGroup;
     // the quantised tile (128 tokens x 128 columns of int8) leaves through LDS as whole rows
     int8_t *qst = sA;
+    // scales of all eight fragments first, outside the branches on nst: the reads are in bounds
+    // either way, and one batch of LDS reads and divisions replaces eight dependent chains
+    float sc_all[8], rsc_all[8];
 #pragma unroll
     for (int tb = 0; tb < 8; ++tb) {
-      if (2 * tb >= nst) continue;
       const int t = tb * 16 + r;
       float amax = fmaxf(fmaxf(sRed[t], sRed[kT + t]), fmaxf(sRed[2 * kT + t], sRed[3 * kT + t]));
       amax = fmaxf(amax, 1e-10f);
-      const float sc = amax / 127.0f;
-      const float rsc = 1.0f / sc;
+      sc_all[tb] = amax / 127.0f;
+      rsc_all[tb] = 1.0f / sc_all[tb];
+    }
+#pragma unroll
+    for (int tb = 0; tb < 8; ++tb) {
+      if (2 * (tb & ~1) >= nst) continue;
+      const int t = tb * 16 + r;
+      const float sc = sc_all[tb], rsc = rsc_all[tb];
 #pragma unroll
       for (int h = 0; h < 2; ++h)
         *reinterpret_cast<uint32_t *>(qst + t * kTPitch + wave * 32 + h * 16 + 4 * q) = quant4(actf[tb][h], sc, rsc);
-      if (wave == 0 && q == 0) {
-        const int64_t ft = sorted[t];
+      if (wave == (tb & 3) && q == 0) { // every wave holds every token's scale: the stores are shared out
+        const int64_t ft = sIds[t];
         if (ft < a.num_valid) a.A2s[ft * G + nt] = sc;
       }
     }
@@ -521,7 +587,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
     for (int j = 0; j < kT * 8 / 256; ++j) {
       const int id = tid + 256 * j, tok = id >> 3, piece = id & 7;
-      const int64_t ft = sorted[tok];
+      const int64_t ft = sIds[tok];
       if (ft < a.num_valid)
         *reinterpret_cast<v4i *>(a.A2q + ft * I + static_cast<int64_t>(nt) * kGroup + piece * 16) =
             *reinterpret_cast<const v4i *>(qst + tok * kTPitch + piece * 16);
