@@ -257,19 +257,20 @@ __device__ __forceinline__ int align_key(const IdT *__restrict__ ids, int64_t f,
   return e;
 }
 
+// (nblocks: the workgroups that count, blockIdx.x 0 .. nblocks-1; the grid may hold others)
 template <typename IdT>
-__global__ __launch_bounds__(256) void moe_align_count_kernel(
+__device__ __forceinline__ void moe_align_count_body(
     const IdT *__restrict__ ids, int64_t numel, int E, const int32_t *__restrict__ expert_map,
     int ignore_invalid, int64_t chunk_slots, int32_t *__restrict__ cnt, uint8_t *__restrict__ slot_mask,
     const int32_t *__restrict__ num_local_tokens, int slots_per_token, int32_t *__restrict__ sorted,
-    int64_t sorted_cap) {
+    int64_t sorted_cap, int nblocks) {
   extern __shared__ int32_t lds[];
   for (int i = threadIdx.x; i < E; i += blockDim.x) lds[i] = 0;
   __syncthreads();
   const int64_t pad_val = numel;
   // every entry of sorted[] starts as padding; the second launch overwrites the valid ones
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < sorted_cap;
-       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+       i += static_cast<int64_t>(nblocks) * blockDim.x)
     sorted[i] = static_cast<int32_t>(pad_val);
   numel = local_slots(numel, num_local_tokens, slots_per_token);
   const int64_t begin = blockIdx.x * chunk_slots;
@@ -297,6 +298,34 @@ __global__ __launch_bounds__(256) void moe_align_count_kernel(
   }
   __syncthreads();
   for (int i = threadIdx.x; i < E; i += blockDim.x) cnt[static_cast<int64_t>(blockIdx.x) * E + i] = lds[i];
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(256) void moe_align_count_kernel(
+    const IdT *__restrict__ ids, int64_t numel, int E, const int32_t *__restrict__ expert_map,
+    int ignore_invalid, int64_t chunk_slots, int32_t *__restrict__ cnt, uint8_t *__restrict__ slot_mask,
+    const int32_t *__restrict__ num_local_tokens, int slots_per_token, int32_t *__restrict__ sorted,
+    int64_t sorted_cap) {
+  moe_align_count_body<IdT>(ids, numel, E, expert_map, ignore_invalid, chunk_slots, cnt, slot_mask, num_local_tokens,
+                            slots_per_token, sorted, sorted_cap, static_cast<int>(gridDim.x));
+}
+
+// The first nchunks workgroups count, the others quantise the activations: the quantisation does
+// not depend on the alignment, and on its own launch it would only wait for the counting to end.
+template <typename IdT>
+__global__ __launch_bounds__(256) void quant_align_count_kernel(
+    const uint16_t *__restrict__ x, int64_t groups, float eps, int8_t *__restrict__ q, float *__restrict__ qs,
+    const IdT *__restrict__ ids, int64_t numel, int E, const int32_t *__restrict__ expert_map,
+    int64_t chunk_slots, int32_t *__restrict__ cnt, uint8_t *__restrict__ slot_mask, int32_t *__restrict__ sorted,
+    int64_t sorted_cap, int nchunks) {
+  if (static_cast<int>(blockIdx.x) < nchunks) {
+    moe_align_count_body<IdT>(ids, numel, E, expert_map, 0, chunk_slots, cnt, slot_mask, nullptr, 1, sorted,
+                              sorted_cap, nchunks);
+  } else {
+    group_quant_body<LO_BF16>(x, groups, eps, q, qs,
+                              static_cast<int64_t>(blockIdx.x - nchunks) * 16 + (threadIdx.x >> 4),
+                              static_cast<int64_t>(gridDim.x - nchunks) * 16, threadIdx.x & 15);
+  }
 }
 
 template <typename IdT>
@@ -474,8 +503,10 @@ int launch_quant_align(const void *x, int64_t M, int64_t H, float eps, int8_t *q
                        const void *topk_ids, int ids_dtype, int64_t numel, int32_t num_experts,
                        int32_t block_size, const int32_t *expert_map, int32_t *sorted_ids, int64_t sorted_cap,
                        int32_t *expert_ids, int64_t expert_ids_cap, int32_t *num_tokens_post_pad,
-                       uint8_t *slot_mask, hipStream_t stream) {
-  if (lo_moe_align_scratch_bytes(numel, num_experts) > 0) return LO_ENOTSUP; // the multi-workgroup form
+                       uint8_t *slot_mask, void *scratch, int64_t scratch_bytes, hipStream_t stream) {
+  const int64_t want = lo_moe_align_scratch_bytes(numel, num_experts);
+  if (want > 0 && !(scratch && scratch_bytes >= want && (reinterpret_cast<uintptr_t>(scratch) & 3) == 0))
+    return LO_ENOTSUP; // the multi-workgroup form needs its counters
   LO_REQUIRE(x && q && qs && topk_ids && sorted_ids && expert_ids && num_tokens_post_pad, LO_EINVAL,
              "quant_align: null pointer");
   LO_REQUIRE(H > 0 && H % kGroup == 0 && M >= 1 && numel >= 1 && num_experts >= 1 && num_experts <= 2048 &&
@@ -487,10 +518,39 @@ int launch_quant_align(const void *x, int64_t M, int64_t H, float eps, int8_t *q
              "quant_align: alignment buffers too small");
   int key_bits = 1;
   while ((1 << key_bits) < num_experts) ++key_bits;
+  const int64_t groups = M * (H / kGroup);
+  if (want > 0) { // many slots: counting + quantisation, then the scatter
+    int nchunks;
+    int64_t cs;
+    align_chunks(numel, &nchunks, &cs);
+    int32_t *cnt = static_cast<int32_t *>(scratch);
+    const size_t lds1 = static_cast<size_t>(num_experts) * 4;
+    const size_t lds2 = (static_cast<size_t>(4 + 3) * num_experts + 1) * 4;
+    int64_t qb = (groups + 15) / 16;
+    if (qb > 8192) qb = 8192;
+    const dim3 grid1(static_cast<unsigned>(nchunks + qb));
+    if (ids_dtype == LO_I32) {
+      hipLaunchKernelGGL(quant_align_count_kernel<int32_t>, grid1, dim3(256), lds1, stream,
+                         static_cast<const uint16_t *>(x), groups, eps, q, qs, static_cast<const int32_t *>(topk_ids),
+                         numel, num_experts, expert_map, cs, cnt, slot_mask, sorted_ids, sorted_cap, nchunks);
+      hipLaunchKernelGGL(moe_align_scatter_kernel<int32_t>, dim3(nchunks), dim3(256), lds2, stream,
+                         static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size, expert_map, 0, cs,
+                         cnt, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, num_tokens_post_pad, key_bits,
+                         nullptr, 1);
+    } else {
+      hipLaunchKernelGGL(quant_align_count_kernel<int64_t>, grid1, dim3(256), lds1, stream,
+                         static_cast<const uint16_t *>(x), groups, eps, q, qs, static_cast<const int64_t *>(topk_ids),
+                         numel, num_experts, expert_map, cs, cnt, slot_mask, sorted_ids, sorted_cap, nchunks);
+      hipLaunchKernelGGL(moe_align_scatter_kernel<int64_t>, dim3(nchunks), dim3(256), lds2, stream,
+                         static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size, expert_map, 0, cs,
+                         cnt, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, num_tokens_post_pad, key_bits,
+                         nullptr, 1);
+    }
+    return check_launch("quant_align(multi)");
+  }
   int nw;
   size_t lds_bytes;
   single_wg_shape(numel, sorted_cap, num_experts, &nw, &lds_bytes);
-  const int64_t groups = M * (H / kGroup);
   const int per_block = nw * kWave / 16;
   int64_t qblocks = (groups + per_block - 1) / per_block;
   if (qblocks > 4096) qblocks = 4096;

@@ -195,10 +195,10 @@ extern "C" int lo_fused_experts_block_int8(
   uint8_t *mask = expert_map ? reinterpret_cast<uint8_t *>(ws + L.off[7]) : nullptr;
   const int64_t S = M * top_k;
 
-  // at decode sizes the quantisation and the alignment share one launch
+  // the quantisation rides in the alignment's launch
   int rc = launch_quant_align(x, M, H, 1e-10f, a1q, a1s, topk_ids, ids_dtype, S, num_experts, block_size_m,
-                              expert_map, sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, mask,
-                              static_cast<hipStream_t>(stream));
+                              expert_map, sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, mask, ws + L.off[8],
+                              L.align_scratch, static_cast<hipStream_t>(stream));
   if (rc == LO_ENOTSUP) {
     rc = lo_per_token_group_quant_int8(x, dtype, M, H, 1e-10f, a1q, a1s, stream);
     if (rc) return rc;

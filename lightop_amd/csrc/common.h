@@ -242,13 +242,15 @@ __device__ __forceinline__ void group_quant_body(const uint16_t *__restrict__ x,
   }
 }
 
-// Group quant of x [M, H] and the single-workgroup routing alignment in ONE launch (they are
-// independent; at decode sizes a launch costs as much as either).  Returns LO_ENOTSUP when the
-// alignment needs its multi-workgroup form: the caller then launches the two stages separately.
+// Group quant of x [M, H] and the routing alignment with the quantisation riding in the
+// alignment's (first) launch: they are independent, and at decode sizes a launch costs as much
+// as either.  scratch: the multi-workgroup alignment's counters (lo_moe_align_scratch_bytes);
+// returns LO_ENOTSUP when they are needed and missing - the caller then launches the two stages
+// separately.
 int launch_quant_align(const void *x, int64_t M, int64_t H, float eps, int8_t *q, float *s,
                        const void *topk_ids, int ids_dtype, int64_t numel, int32_t num_experts,
                        int32_t block_size, const int32_t *expert_map, int32_t *sorted_ids, int64_t sorted_cap,
                        int32_t *expert_ids, int64_t expert_ids_cap, int32_t *num_tokens_post_pad,
-                       uint8_t *slot_mask, hipStream_t stream);
+                       uint8_t *slot_mask, void *scratch, int64_t scratch_bytes, hipStream_t stream);
 
 } // namespace lo
