@@ -443,15 +443,18 @@ def test_gemm_sorted_ids_with_gaps(dev, oracle, bs):
         assert torch.equal(sc.cpu(), rsc) and torch.equal(q.cpu(), rq)
 
 
-@pytest.mark.parametrize("count", [1, 31, 32, 33, 64, 65, 96, 97, 127, 128, 129, 200])
-def test_gemm_128_token_blocks_fill_levels(dev, oracle, count):
+@pytest.mark.parametrize("count,K", [(c, 384) for c in (1, 31, 32, 33, 64, 65, 96, 97, 127, 128, 129, 200)] +
+                         [(c, k) for k in (128, 256, 1024) for c in (40, 128, 250)])
+def test_gemm_128_token_blocks_fill_levels(dev, oracle, count, K):
     """128-token blocks holding 1 ... 128 valid tokens: the K loop of the 128-token kernel comes in
-    variants by the number of 32-token pieces in use, and padded pieces are skipped."""
+    variants by the number of 32-token pieces in use, and padded pieces are skipped.  One, two and
+    eight K blocks as well: the full-tile variant reads a K block's first operands during the
+    previous one and keeps the token scales two K blocks ahead."""
     from lightop_amd.moe import (invoke_fused_moe_gemm1_silu_quant, invoke_fused_moe_kernel_int8,
                                  moe_align_block_size, preshuffle_moe_weight)
 
-    say(f"128-token blocks, {count} tokens on expert 0")
-    bs, E, I, K = 128, 2, 128, 384
+    say(f"128-token blocks, {count} tokens on expert 0, K = {K}")
+    bs, E, I = 128, 2, 128
     M = count + 3
     Aq, As, W, Ws, _, tw, _ = gemm_case(count, M, 1, E, E, 2 * I, K)
     Ws = Ws * 30
