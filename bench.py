@@ -30,12 +30,12 @@ INT8_PEAK_TOPS = 5000.0        # MI355X dense INT8 MFMA, published (5.0 POP/s)
 # and the one-pass weight shuffle); the summaries are the files under profiles/.  Keyed
 # by (workload, tokens); None for points that were not profiled.
 MEASURED_TRAFFIC = {
-    ("qwen3-30b-a3b", 8192): 995679209,
-    ("deepseek-v3-ep8-share", 64): 806207971,
-    ("deepseek-v3-ep8-share", 1024): 961497196,
-    ("deepseek-v3-ep8-share", 4096): 1317125689,
-    ("qwen3-235b-a22b-w4a8", 2048): 1343139868,
-    ("qwen3-235b-a22b-w4a8", 32): 778633980,
+    ("qwen3-30b-a3b", 8192): 996929299,
+    ("deepseek-v3-ep8-share", 64): 806096515,
+    ("deepseek-v3-ep8-share", 1024): 961461529,
+    ("deepseek-v3-ep8-share", 4096): 1319223705,
+    ("qwen3-235b-a22b-w4a8", 2048): 1344825392,
+    ("qwen3-235b-a22b-w4a8", 32): 778527510,
 }
 
 
