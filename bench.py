@@ -8,7 +8,11 @@ A step is one call of ``fused_experts_impl_int8`` on one batch of synthetic toke
 every input already resident in HBM.  Between steps a 512 MiB buffer is overwritten so
 that weights are streamed from HBM and not served from the 256 MB Infinity Cache; the
 step time is taken with HIP events on the launching stream and excludes that flush.
-The last line printed is one JSON object (fields: metric, value, unit, ms_per_step, roofline, cpu_baseline, stage_ms, routers, sweep).
+ms_per_step is the median of the timed steps (mean and min are reported next to it).  The
+headline is timed in the library's default arithmetic (canonical scale order, the mode the GPU
+parity tests compare bit for bit with the CPU checker); ms_per_step_fused_scale is the same call
+with LO_GEMM_FUSED_SCALE.  The last line printed is one JSON object (fields: metric, value, unit,
+ms_per_step, roofline, cpu_baseline, stage_ms, routers, sweep).
 """
 from __future__ import annotations
 
@@ -24,25 +28,39 @@ import torch
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0        # MI355X dense INT8 MFMA, published (5.0 POP/s)
 
-# HBM bytes per launch of the dominant kernel (the first grouped GEMM), measured with
-# rocprofv3 --pmc: FETCH_SIZE x 2.00 x 1024 + WRITE_SIZE x 1.00 x 1024, the factors being
-# what the same counters read for kernels of known size in the same runs (a 512 MiB fill
-# and the one-pass weight shuffle); the summaries are the files under profiles/.  Keyed
-# by (workload, tokens); None for points that were not profiled.
-MEASURED_TRAFFIC = {
-    ("qwen3-30b-a3b", 8192): 996929299,
-    ("deepseek-v3-ep8-share", 64): 806096515,
-    ("deepseek-v3-ep8-share", 1024): 961461529,
-    ("deepseek-v3-ep8-share", 4096): 1319223705,
-    ("qwen3-235b-a22b-w4a8", 2048): 1344825392,
-    ("qwen3-235b-a22b-w4a8", 32): 778527510,
-}
+PROFILES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+
+
+def profile_record(workload, tokens):
+    """What the committed rocprofv3 summary under profiles/ says about the dominant kernel of
+    (workload, tokens): a line `bench-key: workload=... tokens=... kernel=... avg_us=... median_us=...
+    min_us=... traffic_bytes=...` in one of the .md files (traffic_bytes = FETCH_SIZE x 2.00 x 1024 +
+    WRITE_SIZE x 1.00 x 1024 per dispatch, the factors calibrated in the same runs on kernels of known
+    size).  None if that point was not profiled: nothing is made up here."""
+    try:
+        names = sorted(os.listdir(PROFILES))
+    except OSError:
+        return None
+    for name in names:
+        if not name.endswith(".md"):
+            continue
+        for line in open(os.path.join(PROFILES, name)):
+            if not line.startswith("bench-key:"):
+                continue
+            kv = dict(tok.split("=", 1) for tok in line[len("bench-key:"):].split() if "=" in tok)
+            if kv.get("workload") == workload and kv.get("tokens") == str(tokens):
+                rec = {"file": f"profiles/{name}", "kernel": kv.get("kernel")}
+                for k in ("avg_us", "median_us", "min_us"):
+                    rec[k] = float(kv[k]) if k in kv else None
+                rec["traffic_bytes"] = int(kv["traffic_bytes"]) if "traffic_bytes" in kv else None
+                return rec
+    return None
 
 
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--workload", default="qwen3-30b-a3b")
     p.add_argument("--tokens", type=int, default=8192)
@@ -51,7 +69,9 @@ def parse_args():
     p.add_argument("--block-size-m", type=int, default=0)
     p.add_argument("--row-major-weights", action="store_true",
                    help="keep w1/w2 row-major instead of the load-time pre-shuffled layout")
-    p.add_argument("--fused-scale", type=int, default=-1, help="-1: library default per tile, 0/1: force")
+    p.add_argument("--fused-scale", type=int, default=0,
+                   help="0: canonical scale order (the library default, bit-exact against the CPU checker); "
+                        "1: fused-scale order (LO_GEMM_FUSED_SCALE, tolerance-matched)")
     return p.parse_args()
 
 
@@ -89,14 +109,14 @@ def time_steps(fn, steps, warmup, flush):
 class Point:
     """One (layer, M) measurement: whole path plus the two GEMM kernels on their own."""
 
-    def __init__(self, layer, weights, M, dev, seed=0):
+    def __init__(self, layer, weights, M, dev, seed=0, emap=None, pool=None):
         from lightop_amd import workloads as wl
 
         self.layer, self.M, self.dev = layer, M, dev
         self.w1, self.w2, self.w1s, self.w2s = weights
-        self.emap = wl.expert_map_for(layer, dev)
+        self.emap = wl.expert_map_for(layer, dev) if emap is None else emap
         # a pool of different batches so that consecutive steps hit different experts
-        pool = 8 if M <= 64 else 2
+        pool = pool or (8 if M <= 64 else 2)
         self.batches = [tuple(t.to(dev) for t in wl.make_inputs(layer, M, seed=seed + i)) for i in range(pool)]
         self.cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
         self.i = 0
@@ -129,7 +149,7 @@ class Point:
             lightop_amd_block_size_m=bs, lightop_amd_flags=flags)
 
     def stage_times(self, steps, warmup, flush, bs=0, fused_scale=None):
-        """Event-timed duration of each stage kernel launched on its own (ms, mean)."""
+        """Event-timed duration of each stage kernel launched on its own (ms, median)."""
         from lightop_amd import moe
         from lightop_amd.quant import per_token_group_quant_int8
 
@@ -146,6 +166,10 @@ class Point:
             return self.stage_times_channel(steps, warmup, flush, bs), bs
         names = ["quant", "align", "gemm1_silu_quant", "gemm2", "moe_sum"]
         acc = {n: [] for n in names}
+        # With an expert_map the whole path leaves the rows of other ranks' slots untouched and
+        # reduces over the slot mask of the alignment: the stages on their own do the same here.
+        ep = self.emap is not None
+        g2flag = wflag | (_lib_skip_nonlocal() if ep else 0)
         for it in range(warmup + steps):
             x, tw, ids = self.batches[it % len(self.batches)]
             flush()
@@ -153,24 +177,31 @@ class Point:
             ev[0].record()
             a1q, a1s = per_token_group_quant_int8(x, 128)
             ev[1].record()
-            s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
+            if ep:
+                s, e, p = _align_buffers(ids, bs, L.E_global)
+                mask = torch.empty(S, dtype=torch.bool, device=self.dev)
+                moe.moe_align_block_size_out(ids, L.E_global, bs, s, e, p, self.emap, mask)
+            else:
+                mask = None
+                s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
             ev[2].record()
             a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
-                                                             L.top_k, S, cfg, fused_scale=fused_scale, flags=wflag)
+                                                             L.top_k, S, cfg, fused_scale=fused_scale, flags=wflag,
+                                                             global_num_experts=L.E_global)
             ev[3].record()
             moe.invoke_fused_moe_kernel_int8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, True, 1, cfg,
-                                             fused_scale=fused_scale, flags=wflag)
+                                             fused_scale=fused_scale, flags=g2flag, global_num_experts=L.E_global)
             ev[4].record()
-            moe.moe_sum(c3, out)
+            moe.moe_sum(c3, out, expert_mask=mask)
             ev[5].record()
             if it >= warmup:
                 torch.cuda.synchronize()
                 for i, n in enumerate(names):
                     acc[n].append(ev[i].elapsed_time(ev[i + 1]))
-        return {n: sum(v) / len(v) for n, v in acc.items()}, bs
+        return {n: statistics.median(v) for n, v in acc.items()}, bs
 
     def stage_times_channel(self, steps, warmup, flush, bs):
-        """The six launches of the per-channel path, each on its own (ms, mean)."""
+        """The six launches of the per-channel path, each on its own (ms, median)."""
         from lightop_amd import fuse_silu_mul_quant, moe
         from lightop_amd.quant import per_token_quant_int8
 
@@ -191,11 +222,12 @@ class Point:
             ev[1].record()
             s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
             ev[2].record()
-            moe.moe_gemm_w8a8(a1q, self.w1, c1, a1s, self.w1s, None, s, e, p, L.top_k, cfg)
+            moe.moe_gemm_w8a8(a1q, self.w1, c1, a1s, self.w1s, None, s, e, p, L.top_k, cfg,
+                              global_num_experts=L.E_global)
             ev[3].record()
             a2q, a2s = fuse_silu_mul_quant(c1)
             ev[4].record()
-            moe.moe_gemm_w8a8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, 1, cfg)
+            moe.moe_gemm_w8a8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, 1, cfg, global_num_experts=L.E_global)
             ev[5].record()
             moe.moe_sum(c3, out)
             ev[6].record()
@@ -203,7 +235,7 @@ class Point:
                 torch.cuda.synchronize()
                 for i, n in enumerate(names):
                     acc[n].append(ev[i].elapsed_time(ev[i + 1]))
-        return {n: sum(v) / len(v) for n, v in acc.items()}
+        return {n: statistics.median(v) for n, v in acc.items()}
 
 
 def graph_ms(pt, steps, flush, bs, flags):
@@ -234,23 +266,68 @@ def _lib_flags_w4(layer):
     return _lib.LO_GEMM_W4 if layer.weight_bits == 4 else 0
 
 
+def _lib_skip_nonlocal():
+    from lightop_amd import _lib
+
+    return _lib.LO_GEMM_SKIP_NONLOCAL
+
+
+def _align_buffers(ids, bs, num_experts):
+    """Output buffers of the alignment, sized as moe_align_block_size sizes them."""
+    numel = ids.numel()
+    cap = numel + num_experts * (bs - 1)
+    if numel < num_experts:
+        cap = min(numel * bs, cap)
+    dev = ids.device
+    return (torch.empty(cap, dtype=torch.int32, device=dev), torch.empty((cap + bs - 1) // bs, dtype=torch.int32, device=dev),
+            torch.empty(1, dtype=torch.int32, device=dev))
+
+
 def measure_point(pt, steps, warmup, flush, bs, flags):
     mean_ms, med_ms, min_ms = time_steps(lambda: pt.step(bs, flags), steps, warmup, flush)
     g_ms = graph_ms(pt, steps, flush, bs, flags) if pt.M <= 64 else None
-    t = mean_ms * 1e-3
+    t = med_ms * 1e-3
     L = pt.layer
     hbm = pt.bytes / t / 1e9
     tops = pt.ops / t / 1e12
     t_hbm, t_mfma = pt.bytes / (HBM_PEAK_GBS * 1e9), pt.ops / (INT8_PEAK_TOPS * 1e12)
     bound = "mfma" if t_mfma > t_hbm else "hbm"
     return {
-        "workload": L.name, "tokens": pt.M, "ms_per_step": round(mean_ms, 4), "ms_median": round(med_ms, 4),
+        "workload": L.name, "tokens": pt.M, "ms_per_step": round(med_ms, 4), "ms_mean": round(mean_ms, 4),
         "ms_min": round(min_ms, 4), "tokens_per_s": round(pt.M / t, 1), "int8_tops": round(tops, 2),
         "hbm_gbs": round(hbm, 1), "S_loc": pt.S_loc, "E_act": pt.E_act, "bound": bound,
         "roofline_frac": round((tops / INT8_PEAK_TOPS) if bound == "mfma" else (hbm / HBM_PEAK_GBS), 4),
         "frac_hbm": round(hbm / HBM_PEAK_GBS, 4), "frac_mfma": round(tops / INT8_PEAK_TOPS, 4),
         "ms_graph_replay": None if g_ms is None else round(g_ms, 4),
     }
+
+
+def expert_buckets(layer, weights, M, dev, steps, warmup, flush, flags):
+    """Skewed routing: the experts split into those whose share of the batch is compute-bound (more
+    slots than half the ridge point, 2 * slots op/B >= 629 op/B) and those that stream their weights
+    for a handful of tokens.  Each bucket is timed on its own by running the whole path with an
+    expert_map that hides the other bucket (those slots become -1 blocks and are skipped), and set
+    against its own roofline."""
+    from lightop_amd import workloads as wl
+
+    ridge_slots = INT8_PEAK_TOPS * 1e12 / (HBM_PEAK_GBS * 1e9) / 2.0
+    ids = wl.make_inputs(layer, M, seed=0)[2]
+    counts = torch.bincount(ids.reshape(-1).long(), minlength=layer.E_global)
+    out = []
+    for name, sel in (("compute-bound experts", counts >= ridge_slots), ("weight-streaming experts", counts < ridge_slots)):
+        if not bool(sel.any()):
+            continue
+        emap = torch.where(sel, torch.arange(layer.E_global), torch.full((layer.E_global,), -1)).to(torch.int32)
+        pt = Point(layer, weights, M, dev, emap=emap.to(dev), pool=1)
+        mean_ms, med_ms, min_ms = time_steps(lambda: pt.step(0, flags), steps, warmup, flush)
+        t = med_ms * 1e-3
+        out.append({"bucket": name, "experts": int(sel.sum()), "slots": int(counts[sel].sum()),
+                    "slots_per_expert_min": int(counts[sel].min()), "slots_per_expert_max": int(counts[sel].max()),
+                    "ms": round(med_ms, 4), "int8_tops": round(pt.ops / t / 1e12, 1),
+                    "hbm_gbs": round(pt.bytes / t / 1e9, 1), "frac_mfma": round(pt.ops / t / 1e12 / INT8_PEAK_TOPS, 4),
+                    "frac_hbm": round(pt.bytes / t / 1e9 / HBM_PEAK_GBS, 4)})
+        del pt
+    return out
 
 
 def router_times(layer, M, dev, steps, warmup):
@@ -327,7 +404,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     flush = Flusher(dev)
-    flags_default = {-1: 0, 0: _lib.LO_GEMM_CANONICAL_ORDER, 1: _lib.LO_GEMM_FUSED_SCALE}[args.fused_scale]
+    flags_default = _lib.LO_GEMM_FUSED_SCALE if args.fused_scale == 1 else 0
+    flags_other = 0 if args.fused_scale == 1 else _lib.LO_GEMM_FUSED_SCALE
 
     from lightop_amd.moe import preshuffle_moe_scale_int4, preshuffle_moe_weight, preshuffle_moe_weight_int4
 
@@ -349,8 +427,16 @@ def main():
     weights = load_weights(layer, keep_cpu_copy=not args.no_cpu_baseline and layer.weight_bytes < 8e9)
     pt = Point(layer, weights, args.tokens, dev)
     head = measure_point(pt, args.steps, args.warmup, flush, args.block_size_m, flags_default)
+    # the other scale order, for comparison (block form only: the per-channel form has one order)
+    other = None
+    if layer.quant != "channel":
+        other = time_steps(lambda: pt.step(args.block_size_m, flags_other), args.steps, args.warmup, flush)
     stages, bs_used = pt.stage_times(args.steps, args.warmup, flush, args.block_size_m,
-                                     fused_scale={-1: None, 0: False, 1: True}[args.fused_scale])
+                                     fused_scale=args.fused_scale == 1)
+    shape = [1, 128] if layer.weight_bits == 4 else (None if layer.quant == "channel" else [128, 128])
+    from lightop_amd import moe as _moe
+    tile1, tile2 = _moe.get_w8a8moe_json(args.tokens, layer.E, 2 * layer.I, layer.H, layer.I, True, shape, layer.top_k,
+                                         layer.E_global, preshuffled=not args.row_major_weights)
 
     # dominant kernel: the first grouped GEMM with its fused SiLU*mul + re-quantisation
     L = layer
@@ -369,19 +455,21 @@ def main():
         ach, peak, unit = g1_ops / g1_t / 1e12, INT8_PEAK_TOPS, "TFLOP/s"
     else:
         ach, peak, unit = g1_bytes / g1_t / 1e9, HBM_PEAK_GBS, "GB/s"
+    prof = profile_record(layer.name, args.tokens)
+    # the tile query names the kernel the stage call launched (unless the block size was forced)
+    kname = tile1["kernel_name"] if args.block_size_m in (0, tile1["BLOCK_SIZE_M"]) else f"block_size_m={bs_used}"
     roofline = {"bound": head["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
-                "frac": round(ach / peak, 4), "traffic": MEASURED_TRAFFIC.get((layer.name, args.tokens)),
+                "frac": round(ach / peak, 4), "traffic": None if prof is None else prof["traffic_bytes"],
                 "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
-                "kernel": ("moe_gemm_ws_kernel" if bs_used < 64
-                           else "moe_gemm_t128_kernel<W4>" if L.weight_bits == 4 and bs_used == 128
-                           else "moe_gemm_w4_tile_kernel" if L.weight_bits == 4
-                           else "moe_gemm_pc_kernel" if L.quant == "channel"
-                           else "moe_gemm_t128_kernel" if bs_used == 128 and not args.row_major_weights
-                           else "moe_gemm_tile_kernel")
-                + (" (GEMM1, per-channel scales in the epilogue)" if L.quant == "channel"
-                   else "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)"),
+                "kernel": kname + (" (GEMM1, per-channel scales in the epilogue)" if L.quant == "channel"
+                                   else "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)"),
                 "kernel_ms": round(stages[g1_name], 4),
-                "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately)"}
+                "scale_order": "fused" if args.fused_scale == 1 else "canonical",
+                "profile": None if prof is None else prof["file"],
+                "profile_kernel_us": None if prof is None else {k: prof[k] for k in ("avg_us", "median_us", "min_us")},
+                "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately); kernel_ms is the "
+                        "median of HIP-event timings of the stage launched on its own; traffic and "
+                        "profile_kernel_us are read from the committed rocprofv3 summary named in `profile`"}
 
     sweep = []
     if args.sweep != "none":
@@ -389,14 +477,15 @@ def main():
         plan.append((wl.QWEN3_235B_W4, [1, 32, 256, 2048]))
         plan.append((wl.QWEN3_30B_PC, [32, 512, 8192]))
         plan.append((wl.DSV3_EP_PC, [64, 4096]))
-        if args.sweep == "full":
-            plan.append((wl.DSV3_FULL, [8192]))
+        plan.append((wl.DSV3_FULL, [8192]))  # all 256 experts resident (11.3 GB), Zipf-skewed routing
+        sw_steps, sw_warm = max(10, args.steps // 2), max(2, args.warmup // 2)
         for lay, Ms in plan:
             w = weights if lay.name == layer.name else load_weights(lay)
             for M in Ms:
                 p2 = Point(lay, w, M, dev)
-                sweep.append(measure_point(p2, max(5, args.steps // 2), max(2, args.warmup // 2), flush, 0,
-                                           flags_default))
+                sweep.append(measure_point(p2, sw_steps, sw_warm, flush, 0, flags_default))
+                if lay.routing.endswith("zipf"):
+                    sweep[-1]["expert_buckets"] = expert_buckets(lay, w, M, dev, sw_steps, sw_warm, flush, flags_default)
                 print(f"[sweep] {json.dumps(sweep[-1])}", file=sys.stderr, flush=True)
                 del p2
             if lay.name != layer.name:
@@ -411,13 +500,18 @@ def main():
     line = {
         "metric": "block-INT8 fused-MoE tokens/s", "value": round(args.tokens / t, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "ms_per_step_mean": head["ms_mean"], "ms_per_step_min": head["ms_min"],
+        "scale_order": "fused" if args.fused_scale == 1 else "canonical",
+        ("ms_per_step_canonical" if args.fused_scale == 1 else "ms_per_step_fused_scale"):
+            None if other is None else round(other[1], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": f"{layer.name} E={L.E}/{L.E_global} top{L.top_k} H={L.H} I={L.I} "
                                + ("W4A8 int4[1,128]" if L.weight_bits == 4 else
                                   "per-channel INT8" if L.quant == "channel" else "block-INT8[128,128]")
                                + f", M={args.tokens}",
-                   "tokens": args.tokens, "block_size_m": bs_used, "routing": L.routing},
+                   "tokens": args.tokens, "block_size_m": bs_used, "routing": L.routing,
+                   "gemm1_kernel": tile1["kernel_name"], "gemm2_kernel": tile2["kernel_name"]},
         "int8_tops": head["int8_tops"], "hbm_gbs": head["hbm_gbs"], "frac_hbm": head["frac_hbm"],
         "frac_mfma": head["frac_mfma"], "stage_ms": {k: round(v, 4) for k, v in stages.items()},
         "roofline": roofline, "cpu_baseline": cpu, "routers": router_times(layer, args.tokens, dev, 50, 5),

@@ -36,16 +36,17 @@ enum { LO_I32 = 0, LO_I64 = 1 };
 /* flags of lo_moe_gemm_block_int8 / lo_fused_experts_block_int8 */
 enum {
   LO_GEMM_DEFAULT = 0,
-  /* accumulate acc += f32(d) * (a_s * b_s) with one fused multiply-add per
-   * 128-K block instead of the canonical (f32(d) * a_s) * b_s then add.  The
-   * int32 partial sums are identical; the fp32 rounding differs in the last ulp. */
+  /* accumulate acc = fma(f32(d), a_s * b_s, acc) per 128-K block instead of the canonical
+   * acc = acc + (f32(d) * a_s) * b_s, which every kernel computes by default.  The int32
+   * partial sums are identical; the fp32 rounding differs in the last ulp, so outputs (and the
+   * re-quantised int8 activations between the GEMMs) are no longer bit-identical to the
+   * canonical ones, only within the path's tolerance.  Halves the scale arithmetic of the
+   * compute-bound kernels. */
   LO_GEMM_FUSED_SCALE = 1,
   /* always use the weight-streaming kernels, also where the LDS-tiled kernel applies */
   LO_GEMM_FORCE_STREAMING = 2,
-  /* canonical (f32(d) * a_s) * b_s + acc order in every kernel.  Without this flag the
-   * LDS-tiled kernels (64- and 128-token tiles, where the scale arithmetic competes with
-   * the MFMA pipe) use the fused-scale order; the weight-streaming kernels are canonical unless
-   * LO_GEMM_FUSED_SCALE is given. */
+  /* canonical order in every kernel: the default, kept as an explicit flag; it wins over
+   * LO_GEMM_FUSED_SCALE. */
   LO_GEMM_CANONICAL_ORDER = 4,
   /* W (for the whole path: w1 and w2) is in the layout of lo_preshuffle_weight_int8 */
   LO_GEMM_W_PRESHUFFLED = 8,
@@ -173,15 +174,19 @@ int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t rows, int6
  *   C  [num_valid, N] c_dtype, row f;  rows of blocks whose expert id is -1 are zeroed
  *   topk_w [num_valid] f32, used when mul_routed != 0
  *   sorted_ids / expert_ids / num_tokens_post_pad as produced by lo_moe_align_block_size
- *   with block_size == block_size_m; sorted_cap is the extent of sorted_ids.
+ *   with block_size == block_size_m (16, 32, 64 or 128); sorted_cap is the extent of sorted_ids
+ *   (any extent >= the alignment's own works, e.g. one rounded up by the caller).
+ *   E: experts held by W.  num_experts: experts the routing spreads the slots over (the
+ *   num_experts given to the alignment; 0 = E).  It only steers scheduling choices (tile order,
+ *   cache hints), never the result.
  * K % 128 == 0, N % 16 == 0; A, W and C 16-byte aligned.
  */
 int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W, const float *Ws,
                            void *C, int c_dtype, const float *topk_w, const int32_t *sorted_ids,
                            const int32_t *expert_ids, const int32_t *num_tokens_post_pad,
                            int64_t sorted_cap, int64_t num_valid, int64_t a_rows, int32_t E,
-                           int64_t N, int64_t K, int32_t top_k, int32_t block_size_m,
-                           int mul_routed, int flags, lo_stream_t stream);
+                           int32_t num_experts, int64_t N, int64_t K, int32_t top_k,
+                           int32_t block_size_m, int mul_routed, int flags, lo_stream_t stream);
 
 /*
  * First grouped GEMM with the activation fused into its epilogue:
@@ -196,9 +201,10 @@ int lo_moe_gemm1_silu_quant_block_int8(const int8_t *A, const float *As, const i
                                        const float *topk_w, const int32_t *sorted_ids,
                                        const int32_t *expert_ids,
                                        const int32_t *num_tokens_post_pad, int64_t sorted_cap,
-                                       int64_t num_valid, int64_t a_rows, int32_t E, int64_t I,
-                                       int64_t K, int32_t top_k, int32_t block_size_m,
-                                       int mul_routed, int flags, lo_stream_t stream);
+                                       int64_t num_valid, int64_t a_rows, int32_t E,
+                                       int32_t num_experts, int64_t I, int64_t K, int32_t top_k,
+                                       int32_t block_size_m, int mul_routed, int flags,
+                                       lo_stream_t stream);
 
 /*
  * SiLU-and-mul: act[f, i] = T( T(silu(c1[f, i])) * c1[f, I + i] ).
@@ -251,18 +257,34 @@ int lo_preshuffle_weight_int8(const int8_t *src, int8_t *dst, int32_t E, int64_t
  */
 typedef struct lo_moe_tile {
   int32_t block_size_m; /* 16, 32, 64 or 128 */
-  int32_t kernel;       /* implementation id, for reporting */
-  int32_t waves;        /* wavefronts per workgroup */
-  int32_t block_n;      /* weight rows per workgroup */
+  int32_t kernel;       /* LO_KERNEL_*: the kernel the stage entry points launch for this problem */
+  int32_t waves;        /* wavefronts per workgroup of that kernel */
+  int32_t block_n;      /* weight rows per workgroup of that kernel */
 } lo_moe_tile;
 
+/* kernel families (lo_moe_tile.kernel) */
+enum {
+  LO_KERNEL_WS = 0,      /* weight-streaming, no LDS in the K loop (token blocks of 16 / 32) */
+  LO_KERNEL_TILE = 1,    /* LDS-tiled, weights register-fed (row-major weights, 64 / 128 tokens) */
+  LO_KERNEL_PC = 2,      /* per-channel LDS-tiled */
+  LO_KERNEL_AS = 3,      /* activation-stationary second GEMM (short K) */
+  LO_KERNEL_T128 = 4,    /* 128 tokens, both operands copied global -> LDS (pre-shuffled weights) */
+  LO_KERNEL_W4_TILE = 5  /* packed-int4 LDS-tiled, 64 tokens */
+};
+
+/* Block form with weights in the load-time layout (flags = LO_GEMM_W_PRESHUFFLED). */
 int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k, int64_t H,
                       int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2);
-/* The same for the other forms of the path: per-channel (replaces get_moe_cuda_config,
- * int8.py:735-741, and its MODE / DELTA tables) and W4A8 with K-group scales. */
+/* The same for every form of the path: block, per-channel (replaces get_moe_cuda_config,
+ * int8.py:735-741, and its MODE / DELTA tables) and W4A8 with K-group scales.  flags: the
+ * LO_GEMM_* flags the call will carry (LO_GEMM_W_PRESHUFFLED decides between the row-major
+ * and the load-time weight layout, LO_GEMM_FORCE_STREAMING is honoured; LO_GEMM_W4 is implied
+ * by the form).  The answer is what lo_fused_experts_* picks with block_size_m = 0 and what the
+ * stage entry points launch when given that block_size_m. */
 enum { LO_FORM_BLOCK = 0, LO_FORM_CHANNEL = 1, LO_FORM_W4 = 2 };
-int lo_moe_tile_query_form(int form, int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
-                           int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2);
+int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_local, int32_t num_experts,
+                           int32_t top_k, int64_t H, int64_t I, lo_moe_tile *gemm1,
+                           lo_moe_tile *gemm2);
 
 /*
  * Whole path for one chunk of tokens: quant -> align -> GEMM1(+SiLU*mul+quant) -> GEMM2
@@ -274,7 +296,8 @@ int lo_moe_tile_query_form(int form, int64_t M, int32_t E_local, int32_t num_exp
  *   cache3 [M*top_k, H] act dtype: the caller's cache13 workspace (second GEMM's output)
  *   shared_output [M, H] or NULL;  out [M, H]
  *   workspace: lo_fused_experts_workspace_bytes(...) bytes of device memory, 256-byte aligned
- *   block_size_m: 0 = take it from the tile table
+ *   block_size_m: 0 = take it from the tile table (lo_fused_experts_workspace_bytes(.., 0) is
+ *   large enough for whatever the table picks and for every explicit block size)
  */
 int64_t lo_fused_experts_workspace_bytes(int64_t M, int32_t top_k, int64_t H, int64_t I,
                                          int32_t num_experts, int32_t block_size_m);
@@ -339,9 +362,9 @@ int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, int64_t I, i
 int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *W, const float *Ws, void *C,
                      int c_dtype, const float *topk_w, const int32_t *sorted_ids,
                      const int32_t *expert_ids, const int32_t *num_tokens_post_pad,
-                     int64_t sorted_cap, int64_t num_valid, int64_t a_rows, int32_t E, int64_t N,
-                     int64_t K, int32_t top_k, int32_t block_size_m, int mul_routed, int flags,
-                     lo_stream_t stream);
+                     int64_t sorted_cap, int64_t num_valid, int64_t a_rows, int32_t E,
+                     int32_t num_experts, int64_t N, int64_t K, int32_t top_k, int32_t block_size_m,
+                     int mul_routed, int flags, lo_stream_t stream);
 
 /*
  * Whole path in the per-channel form: per-token quant -> align -> GEMM1 -> SiLU*mul + per-token

@@ -15,6 +15,10 @@ LO_GEMM_W_PRESHUFFLED = 8
 LO_GEMM_SKIP_NONLOCAL = 16
 LO_GEMM_W4 = 32
 LO_FORM_BLOCK, LO_FORM_CHANNEL, LO_FORM_W4 = 0, 1, 2
+LO_KERNEL_WS, LO_KERNEL_TILE, LO_KERNEL_PC, LO_KERNEL_AS, LO_KERNEL_T128, LO_KERNEL_W4_TILE = 0, 1, 2, 3, 4, 5
+KERNEL_NAMES = {LO_KERNEL_WS: "moe_gemm_ws_kernel", LO_KERNEL_TILE: "moe_gemm_tile_kernel",
+                LO_KERNEL_PC: "moe_gemm_pc_kernel", LO_KERNEL_AS: "moe_gemm_as_kernel",
+                LO_KERNEL_T128: "moe_gemm_t128_kernel", LO_KERNEL_W4_TILE: "moe_gemm_w4_tile_kernel"}
 
 
 class LoMoeTile(ctypes.Structure):
@@ -40,11 +44,11 @@ SIGNATURES = {
     "lo_per_token_group_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_float, c_void_p,
                                               c_void_p, c_void_p]),
     "lo_moe_gemm_block_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                       c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32,
+                                       c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32,
                                        c_int64, c_int64, c_int32, c_int32, c_int, c_int, c_void_p]),
     "lo_moe_gemm1_silu_quant_block_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                    c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                                                   c_int64, c_int64, c_int64, c_int32, c_int64, c_int64,
+                                                   c_int64, c_int64, c_int64, c_int32, c_int32, c_int64, c_int64,
                                                    c_int32, c_int32, c_int, c_int, c_void_p]),
     "lo_preshuffle_weight_int8": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "lo_preshuffle_weight_int4": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
@@ -57,7 +61,7 @@ SIGNATURES = {
                                   c_int32, ctypes.c_double, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "lo_moe_tile_query": (c_int, [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
                                   ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
-    "lo_moe_tile_query_form": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
+    "lo_moe_tile_query_form": (c_int, [c_int, c_int, c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
                                        ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
     "lo_fused_experts_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
     "lo_fused_experts_workspace_offset": (c_int64, [c_int, c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
@@ -65,7 +69,7 @@ SIGNATURES = {
     "lo_fuse_silu_mul_quant": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32,
                                        c_void_p]),
     "lo_moe_gemm_w8a8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                 c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32,
+                                 c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32,
                                  c_int64, c_int64, c_int32, c_int32, c_int, c_int, c_void_p]),
     "lo_fused_experts_channel_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int32, c_int32,
                                               c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

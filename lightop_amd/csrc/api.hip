@@ -3,7 +3,7 @@
 #include <cstdarg>
 #include <cstdio>
 
-#include "common.h"
+#include "gemm.h"
 
 namespace lo {
 
@@ -112,37 +112,56 @@ extern "C" int lo_version(void) { return 100; }
 
 extern "C" const char *lo_last_error(void) { return lo::g_err; }
 
-extern "C" int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
-                                 int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
+extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_local, int32_t num_experts,
+                                      int32_t top_k, int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
   using namespace lo;
-  (void)E_local;
+  LO_REQUIRE(form == LO_FORM_BLOCK || form == LO_FORM_CHANNEL || form == LO_FORM_W4, LO_EINVAL,
+             "moe_tile_query_form: unknown form %d", form);
   LO_REQUIRE(M >= 0 && num_experts >= 1 && top_k >= 1 && H > 0 && I > 0, LO_EINVAL,
-             "moe_tile_query: bad problem size");
-  const int32_t bm = pick_block_m(M, num_experts, top_k, H);
-  if (gemm1) *gemm1 = lo_moe_tile{bm, 1, 8, 256};
-  if (gemm2) *gemm2 = lo_moe_tile{bm, 0, 4, 64};
+             "moe_tile_query_form: bad problem size");
+  if (form == LO_FORM_W4) flags |= LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED;
+  const bool pre = (flags & LO_GEMM_W_PRESHUFFLED) != 0;
+  const int32_t bm = pick_block_m(M, num_experts, top_k, H, form, pre);
+  // the argument blocks the stage entry points would build for this problem
+  GemmArgs a{};
+  a.num_valid = M * top_k;
+  a.E = E_local > 0 ? E_local : num_experts;
+  a.experts_routed = num_experts;
+  a.top_k = top_k;
+  a.w_shuffled = pre ? 1 : 0;
+  a.w4 = form == LO_FORM_W4 ? 1 : 0;
+  a.per_channel = form == LO_FORM_CHANNEL ? 1 : 0;
+  if (gemm1) {
+    a.N = 2 * I; a.K = H; a.a_rows = M;
+    const bool fused = form != LO_FORM_CHANNEL; // the per-channel form quantises in a launch of its own
+    describe_gemm_kernel(pick_gemm_kernel(a, fused, bm, flags), fused, bm, gemm1);
+  }
+  if (gemm2) {
+    a.N = H; a.K = I; a.a_rows = M * top_k;
+    describe_gemm_kernel(pick_gemm_kernel(a, false, bm, flags), false, bm, gemm2);
+  }
   return LO_OK;
 }
 
-extern "C" int lo_moe_tile_query_form(int form, int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
-                                      int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
-  using namespace lo;
-  if (form == LO_FORM_BLOCK) return lo_moe_tile_query(M, E_local, num_experts, top_k, H, I, gemm1, gemm2);
-  LO_REQUIRE(form == LO_FORM_CHANNEL || form == LO_FORM_W4, LO_EINVAL, "moe_tile_query_form: unknown form %d", form);
-  LO_REQUIRE(M >= 0 && num_experts >= 1 && top_k >= 1 && H > 0 && I > 0, LO_EINVAL,
-             "moe_tile_query_form: bad problem size");
-  const int32_t bm = pick_block_m(M, num_experts, top_k, H, form);
-  if (gemm1) *gemm1 = lo_moe_tile{bm, bm >= 64 ? 2 : 0, bm >= 64 || form == LO_FORM_CHANNEL ? 4 : 8, bm >= 64 ? 256 : 64};
-  if (gemm2) *gemm2 = lo_moe_tile{bm, bm >= 64 ? 2 : 0, 4, bm >= 64 ? 256 : 64};
-  return LO_OK;
+extern "C" int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
+                                 int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
+  return lo_moe_tile_query_form(LO_FORM_BLOCK, LO_GEMM_W_PRESHUFFLED, M, E_local, num_experts, top_k, H, I, gemm1,
+                                gemm2);
 }
 
 extern "C" int64_t lo_fused_experts_workspace_bytes(int64_t M, int32_t top_k, int64_t H, int64_t I,
                                                     int32_t num_experts, int32_t block_size_m) {
   using namespace lo;
   if (M < 0 || top_k < 1 || H < kGroup || I < kGroup || num_experts < 1) return LO_EINVAL;
-  if (block_size_m == 0) block_size_m = 128; // the largest tile bounds every choice of the table
-  return ws_layout(M, top_k, H, I, num_experts, block_size_m).total + 256;
+  if (block_size_m != 0) return ws_layout(M, top_k, H, I, num_experts, block_size_m).total + 256;
+  // 0: whatever the table (or a later explicit choice) picks.  The sorted ids grow with the block
+  // size, the per-block expert ids shrink with it: take the largest layout of the four.
+  int64_t most = 0;
+  for (int32_t bs : {16, 32, 64, 128}) {
+    const int64_t t = ws_layout(M, top_k, H, I, num_experts, bs).total;
+    most = t > most ? t : most;
+  }
+  return most + 256;
 }
 
 extern "C" int64_t lo_fused_experts_workspace_offset(int which, int64_t M, int32_t top_k, int64_t H,
@@ -208,11 +227,11 @@ extern "C" int lo_fused_experts_block_int8(
   }
   if (rc) return rc;
   rc = lo_moe_gemm1_silu_quant_block_int8(a1q, a1s, w1, w1s, a2q, a2s, dtype, topk_w, sorted, eids,
-                                          ntpp, L.sorted_cap, S, M, E, I, H, top_k, block_size_m,
+                                          ntpp, L.sorted_cap, S, M, E, num_experts, I, H, top_k, block_size_m,
                                           apply_router_weight_on_input, flags, stream);
   if (rc) return rc;
   rc = lo_moe_gemm_block_int8(a2q, a2s, w2, w2s, cache3, dtype, topk_w, sorted, eids, ntpp,
-                              L.sorted_cap, S, S, E, H, I, 1, block_size_m,
+                              L.sorted_cap, S, S, E, num_experts, H, I, 1, block_size_m,
                               !apply_router_weight_on_input, flags | (mask ? LO_GEMM_SKIP_NONLOCAL : 0),
                               stream);
   if (rc) return rc;
@@ -272,12 +291,12 @@ extern "C" int lo_fused_experts_channel_int8(
   if (rc) return rc;
   // rows of experts on other ranks are zero-filled here: the activation kernel reads every row
   rc = lo_moe_gemm_w8a8(a1q, a1s, w1, w1s, cache13, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, M, E,
-                        2 * I, H, top_k, block_size_m, apply_router_weight_on_input, flags, stream);
+                        num_experts, 2 * I, H, top_k, block_size_m, apply_router_weight_on_input, flags, stream);
   if (rc) return rc;
   rc = lo_fuse_silu_mul_quant(cache13, dtype, S, I, a2q, a2s, nullptr, 1, stream);
   if (rc) return rc;
   rc = lo_moe_gemm_w8a8(a2q, a2s, w2, w2s, cache13, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, S, E,
-                        H, I, 1, block_size_m, !apply_router_weight_on_input,
+                        num_experts, H, I, 1, block_size_m, !apply_router_weight_on_input,
                         flags | (mask ? LO_GEMM_SKIP_NONLOCAL : 0), stream);
   if (rc) return rc;
   return lo_moe_sum(cache13, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor, nullptr,

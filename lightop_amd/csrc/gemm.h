@@ -2,6 +2,15 @@
 #pragma once
 #include "common.h"
 
+// Shape of the plain (not fused) weight-streaming workgroup: waves, and 16-row fragments per wave
+// at token blocks of 16 or 32 (gemm_ws.hip; the tile query reports the same numbers).
+#ifndef LO_WS_PLAIN_WAVES
+#define LO_WS_PLAIN_WAVES 4
+#endif
+#ifndef LO_WS_RPW
+#define LO_WS_RPW 4
+#endif
+
 namespace lo {
 
 struct GemmArgs {
@@ -31,6 +40,14 @@ struct GemmArgs {
   int32_t w4;            // W is packed int4 (load-time layout), Ws is [E, K/128, N]
   int32_t per_channel;   // As is [a_rows], Ws is [E, N]: scales applied once, after the whole-K int32 sum
 };
+
+// Order of the scale arithmetic per 128-wide K block.  Every kernel computes the canonical
+// acc = acc + (f32(d) * a_s) * b_s (three roundings, the order the CPU checker restates) unless the
+// caller asks for LO_GEMM_FUSED_SCALE: acc = fma(f32(d), a_s * b_s, acc), two vector instructions per
+// accumulator element instead of four, last-ulp differences in fp32.
+inline bool fused_scale_order(int flags) {
+  return (flags & LO_GEMM_FUSED_SCALE) != 0 && (flags & LO_GEMM_CANONICAL_ORDER) == 0;
+}
 
 __device__ __forceinline__ v4i ld16(const int8_t *p) { return *reinterpret_cast<const v4i *>(p); }
 
@@ -104,6 +121,10 @@ __device__ __forceinline__ void wave_store_32x64_bf16(int8_t *stg, const v4u16 (
   }
   __builtin_amdgcn_wave_barrier();
 }
+
+// Kernel a stage is served by, and its workgroup shape (gemm_api.hip).
+int pick_gemm_kernel(const GemmArgs &a, bool fused_act, int block_size_m, int flags);
+void describe_gemm_kernel(int kernel, bool fused_act, int block_size_m, lo_moe_tile *t);
 
 // Weight-streaming kernels (gemm_ws.hip): block_size_m in {16, 32, 64, 128}.
 int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,

@@ -12,14 +12,7 @@ static int64_t grid_m_blocks(int64_t sorted_cap, int64_t num_valid, int bs) {
   return blocks;
 }
 
-// The alignment buffers are sized S + E_global * (bs - 1): recover E_global from them.
-static int32_t routed_experts(int64_t sorted_cap, int64_t num_valid, int bs, int32_t E) {
-  if (bs > 1 && sorted_cap > num_valid) {
-    const int64_t eg = (sorted_cap - num_valid) / (bs - 1);
-    if (eg >= E && eg <= 4096) return static_cast<int32_t>(eg);
-  }
-  return E;
-}
+static bool valid_block_m(int bs) { return bs == 16 || bs == 32 || bs == 64 || bs == 128; }
 
 static int validate_common(const char *who, const void *A, const void *As, const void *W,
                            const void *Ws, const void *sorted, const void *eids, const void *ntpp,
@@ -36,25 +29,59 @@ static int validate_common(const char *who, const void *A, const void *As, const
   return LO_OK;
 }
 
-// Token blocks of 64 or 128 rows go to the LDS-tiled kernels (tokens per expert large enough
-// for operand reuse to matter); smaller ones stream weights.
+// Which kernel serves a stage.  Token blocks of 64 or 128 rows go to the LDS-tiled kernels (tokens
+// per expert large enough for operand reuse to matter); smaller ones stream weights.  The tile
+// query (lo_moe_tile_query_form) reports this very choice.
+int pick_gemm_kernel(const GemmArgs &a, bool fused_act, int bs, int flags) {
+  const bool tiled = !(flags & LO_GEMM_FORCE_STREAMING);
+  if (a.w4) { // int4 weights: 128- or 64-token LDS tiles, else streaming
+    if (tiled && gemm_t128_supports(a, fused_act, bs)) return LO_KERNEL_T128;
+    if (tiled && gemm_w4_tile_supports(a, fused_act, bs)) return LO_KERNEL_W4_TILE;
+    return LO_KERNEL_WS;
+  }
+  if (tiled) {
+    if (gemm_pc_supports(a, bs)) return LO_KERNEL_PC;
+    if (a.per_channel) return LO_KERNEL_WS;
+    if (gemm_as_supports(a, fused_act, bs)) return LO_KERNEL_AS;
+    if (gemm_t128_supports(a, fused_act, bs)) return LO_KERNEL_T128;
+    if (gemm_tile_supports(a, fused_act, bs)) return LO_KERNEL_TILE;
+  }
+  return LO_KERNEL_WS;
+}
+
+// Workgroup shape of that kernel: wavefronts and weight rows per workgroup.
+void describe_gemm_kernel(int kernel, bool fused_act, int bs, lo_moe_tile *t) {
+  t->block_size_m = bs;
+  t->kernel = kernel;
+  switch (kernel) {
+  case LO_KERNEL_WS: { // gemm_ws.hip: launch_ws
+    const int tm = bs / 16;
+    const int rpw = tm <= 2 ? LO_WS_RPW : (tm == 4 ? 2 : 1);
+    t->waves = fused_act ? 8 : LO_WS_PLAIN_WAVES;
+    t->block_n = fused_act ? 256 : 16 * LO_WS_PLAIN_WAVES * rpw;
+    break;
+  }
+  case LO_KERNEL_TILE:
+    t->waves = bs == 128 ? 8 : 4;
+    t->block_n = 256;
+    break;
+  default: // t128, activation-stationary, per-channel and int4 tiles: four waves x 64 rows
+    t->waves = 4;
+    t->block_n = 256;
+    break;
+  }
+}
+
 static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int64_t m_blocks,
                        hipStream_t s) {
-  if (a.w4) { // int4 weights: the LDS-tiled kernel at 64-token blocks, else streaming
-    if (!(flags & LO_GEMM_FORCE_STREAMING) && gemm_t128_supports(a, fused_act, bs))
-      return launch_gemm_t128(a, fused_act, flags, m_blocks, s);
-    if (!(flags & LO_GEMM_FORCE_STREAMING) && gemm_w4_tile_supports(a, fused_act, bs))
-      return launch_gemm_w4_tile(a, fused_act, flags, m_blocks, s);
-    return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
+  switch (pick_gemm_kernel(a, fused_act, bs, flags)) {
+  case LO_KERNEL_T128: return launch_gemm_t128(a, fused_act, flags, m_blocks, s);
+  case LO_KERNEL_W4_TILE: return launch_gemm_w4_tile(a, fused_act, flags, m_blocks, s);
+  case LO_KERNEL_PC: return launch_gemm_pc(a, bs, m_blocks, s);
+  case LO_KERNEL_AS: return launch_gemm_as(a, flags, bs, m_blocks, s);
+  case LO_KERNEL_TILE: return launch_gemm_tile(a, fused_act, bs, flags, m_blocks, s);
+  default: return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
   }
-  if (!(flags & LO_GEMM_FORCE_STREAMING)) {
-    if (gemm_pc_supports(a, bs)) return launch_gemm_pc(a, bs, m_blocks, s);
-    if (a.per_channel) return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
-    if (gemm_as_supports(a, fused_act, bs)) return launch_gemm_as(a, flags, bs, m_blocks, s);
-    if (gemm_t128_supports(a, fused_act, bs)) return launch_gemm_t128(a, fused_act, flags, m_blocks, s);
-    if (gemm_tile_supports(a, fused_act, bs)) return launch_gemm_tile(a, fused_act, bs, flags, m_blocks, s);
-  }
-  return launch_gemm_ws(a, fused_act, bs, flags, m_blocks, s);
 }
 
 } // namespace lo
@@ -63,13 +90,15 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
                                       const float *Ws, void *C, int c_dtype, const float *topk_w,
                                       const int32_t *sorted_ids, const int32_t *expert_ids,
                                       const int32_t *num_tokens_post_pad, int64_t sorted_cap,
-                                      int64_t num_valid, int64_t a_rows, int32_t E, int64_t N,
-                                      int64_t K, int32_t top_k, int32_t block_size_m,
+                                      int64_t num_valid, int64_t a_rows, int32_t E, int32_t num_experts,
+                                      int64_t N, int64_t K, int32_t top_k, int32_t block_size_m,
                                       int mul_routed, int flags, lo_stream_t stream) {
   using namespace lo;
   int rc = validate_common("moe_gemm", A, As, W, Ws, sorted_ids, expert_ids, num_tokens_post_pad, K,
                            top_k, E, a_rows);
   if (rc) return rc;
+  LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL, "moe_gemm: block_size_m %d is not one of 16, 32, 64, 128",
+             block_size_m);
   LO_REQUIRE(C, LO_EINVAL, "moe_gemm: null output");
   LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm: only bf16 output is built");
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm: N (%lld) must be a multiple of 16", (long long)N);
@@ -83,7 +112,7 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   GemmArgs a{};
   a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.C = static_cast<uint16_t *>(C);
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
-  a.E = E; a.experts_routed = routed_experts(sorted_cap, num_valid, block_size_m, E); a.a_rows = a_rows; a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.E = E; a.experts_routed = num_experts > E ? num_experts : E; a.a_rows = a_rows; a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
@@ -100,12 +129,14 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
     const int8_t *A, const float *As, const int8_t *W, const float *Ws, int8_t *A2q, float *A2s,
     int c_dtype, const float *topk_w, const int32_t *sorted_ids, const int32_t *expert_ids,
     const int32_t *num_tokens_post_pad, int64_t sorted_cap, int64_t num_valid, int64_t a_rows,
-    int32_t E, int64_t I, int64_t K, int32_t top_k, int32_t block_size_m, int mul_routed, int flags,
-    lo_stream_t stream) {
+    int32_t E, int32_t num_experts, int64_t I, int64_t K, int32_t top_k, int32_t block_size_m, int mul_routed,
+    int flags, lo_stream_t stream) {
   using namespace lo;
   int rc = validate_common("moe_gemm1_silu_quant", A, As, W, Ws, sorted_ids, expert_ids,
                            num_tokens_post_pad, K, top_k, E, a_rows);
   if (rc) return rc;
+  LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL,
+             "moe_gemm1_silu_quant: block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
   LO_REQUIRE(A2q && A2s, LO_EINVAL, "moe_gemm1_silu_quant: null output");
   LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm1_silu_quant: only bf16 rounding is built");
   LO_REQUIRE(I > 0 && I % kGroup == 0, LO_EINVAL,
@@ -121,7 +152,7 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
   GemmArgs a{};
   a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.A2q = A2q; a.A2s = A2s;
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
-  a.E = E; a.experts_routed = routed_experts(sorted_cap, num_valid, block_size_m, E); a.a_rows = a_rows; a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
+  a.E = E; a.experts_routed = num_experts > E ? num_experts : E; a.a_rows = a_rows; a.num_valid = num_valid; a.N = 2 * I; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
@@ -141,12 +172,14 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
                                 void *C, int c_dtype, const float *topk_w, const int32_t *sorted_ids,
                                 const int32_t *expert_ids, const int32_t *num_tokens_post_pad,
                                 int64_t sorted_cap, int64_t num_valid, int64_t a_rows, int32_t E,
-                                int64_t N, int64_t K, int32_t top_k, int32_t block_size_m,
-                                int mul_routed, int flags, lo_stream_t stream) {
+                                int32_t num_experts, int64_t N, int64_t K, int32_t top_k,
+                                int32_t block_size_m, int mul_routed, int flags, lo_stream_t stream) {
   using namespace lo;
   int rc = validate_common("moe_gemm_w8a8", A, As, W, Ws, sorted_ids, expert_ids, num_tokens_post_pad, K,
                            top_k, E, a_rows);
   if (rc) return rc;
+  LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL, "moe_gemm_w8a8: block_size_m %d is not one of 16, 32, 64, 128",
+             block_size_m);
   LO_REQUIRE(C, LO_EINVAL, "moe_gemm_w8a8: null output");
   LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm_w8a8: only bf16 output is built");
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm_w8a8: N (%lld) must be a multiple of 16", (long long)N);
@@ -163,7 +196,7 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   GemmArgs a{};
   a.A = A; a.As = As; a.W = W; a.Ws = Ws; a.C = static_cast<uint16_t *>(C);
   a.topk_w = topk_w; a.sorted = sorted_ids; a.expert_ids = expert_ids; a.ntpp = num_tokens_post_pad;
-  a.E = E; a.experts_routed = routed_experts(sorted_cap, num_valid, block_size_m, E); a.a_rows = a_rows;
+  a.E = E; a.experts_routed = num_experts > E ? num_experts : E; a.a_rows = a_rows;
   a.num_valid = num_valid; a.N = N; a.K = K; a.top_k = top_k; a.mul_routed = mul_routed ? 1 : 0;
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;

@@ -36,8 +36,11 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
   if (static_cast<int64_t>(mb) * kTileM >= a.ntpp[0]) return;
   // mb counts 64-token pieces; an alignment block of 128 tokens is two of them (sub_shift = 1), and
   // a piece that holds padding only is skipped
-  const int e = a.expert_ids[mb >> sub_shift];
-  if (e >= a.E) return;
+  // An expert_map entry outside the weight tensor is treated like an expert of another rank, but its
+  // rows are always zero-filled: the slot mask of the alignment counts such a slot as local.
+  const int e_raw = a.expert_ids[mb >> sub_shift];
+  const bool e_oob = e_raw >= a.E;
+  const int e = e_oob ? -1 : e_raw;
   const int tid = threadIdx.x, lane = tid & 63;
   if (sub_shift &&
       __builtin_amdgcn_ballot_w64(a.sorted[static_cast<int64_t>(mb) * kTileM + lane] < a.num_valid) == 0)
@@ -60,7 +63,7 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
   }
 
   if (e < 0) {
-    if (!a.skip_nonlocal) {
+    if ((!a.skip_nonlocal || e_oob)) {
       for (int nt = nt0; nt < nt_end; ++nt)
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb)
@@ -289,7 +292,7 @@ int launch_gemm_as(const GemmArgs &a0, int flags, int block_size_m, int64_t m_bl
   const int64_t chunks = (m_blocks + G - 1) / G;
   const int64_t grid = (chunks + 7) / 8 * (G * n_groups) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
-  const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
+  const bool fast = fused_scale_order(flags);
   const size_t lds = static_cast<size_t>(as_lds_bytes(a.K));
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), Gi = static_cast<int>(G);

@@ -31,8 +31,11 @@ __device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
   if (static_cast<int64_t>(mb) * kTileM >= a.ntpp[0]) return;
-  const int e = a.expert_ids[mb];
-  if (e >= a.E) return;
+  // An expert_map entry outside the weight tensor is treated like an expert of another rank, but its
+  // rows are always zero-filled: the slot mask of the alignment counts such a slot as local.
+  const int e_raw = a.expert_ids[mb];
+  const bool e_oob = e_raw >= a.E;
+  const int e = e_oob ? -1 : e_raw;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wr = __builtin_amdgcn_readfirstlane(tid >> 6); // which 64 weight rows of the tile
   const int r = lane & 31, c = lane >> 5;
@@ -52,7 +55,7 @@ __device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks
   const bool wave_active = nrow[0] < N; // N % 64 == 0 is checked on the host
 
   if (e < 0) { // expert of another rank: its rows are defined to be zero
-    if (wave_active && !a.skip_nonlocal) {
+    if (wave_active && (!a.skip_nonlocal || e_oob)) {
 #pragma unroll
       for (int tb = 0; tb < TB; ++tb)
         if (valid[tb])

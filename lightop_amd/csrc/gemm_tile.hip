@@ -43,8 +43,11 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
   if (static_cast<int64_t>(mb) * kTileM >= a.ntpp[0]) return;
-  const int e = a.expert_ids[mb];
-  if (e >= a.E) return;
+  // An expert_map entry outside the weight tensor is treated like an expert of another rank, but its
+  // rows are always zero-filled: the slot mask of the alignment counts such a slot as local.
+  const int e_raw = a.expert_ids[mb];
+  const bool e_oob = e_raw >= a.E;
+  const int e = e_oob ? -1 : e_raw;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: scalar address math
   const int wr = wave & 3;  // which 64 weight rows of the tile
@@ -76,7 +79,7 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
 
   if (e < 0) {
     if constexpr (!FUSED_ACT) {
-      if (wave_active && !a.skip_nonlocal) {
+      if (wave_active && (!a.skip_nonlocal || e_oob)) {
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb)
           if (valid[tb])
@@ -339,7 +342,7 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int block_size_m, int f
   const int64_t chunks = (m_blocks + G - 1) / G;
   const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
-  const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
+  const bool fast = fused_scale_order(flags);
   const int wt = block_size_m / 64;
   const dim3 g(static_cast<unsigned>(grid)), b(256 * wt);
   const int mbi = static_cast<int>(m_blocks);

@@ -38,8 +38,11 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
   if (static_cast<int64_t>(mb) * kTileM >= a.ntpp[0]) return;
-  const int e = a.expert_ids[mb];
-  if (e >= a.E) return;
+  // An expert_map entry outside the weight tensor is treated like an expert of another rank, but its
+  // rows are always zero-filled: the slot mask of the alignment counts such a slot as local.
+  const int e_raw = a.expert_ids[mb];
+  const bool e_oob = e_raw >= a.E;
+  const int e = e_oob ? -1 : e_raw;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wr = __builtin_amdgcn_readfirstlane(tid >> 6); // which 64 weight rows of the tile
   const int r = lane & 15, q = lane >> 4;
@@ -66,7 +69,7 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
 
   if (e < 0) {
     if constexpr (!FUSED_ACT) {
-      if (!a.skip_nonlocal) {
+      if ((!a.skip_nonlocal || e_oob)) {
 #pragma unroll
         for (int tf = 0; tf < 4; ++tf)
           if (valid[tf])
@@ -333,7 +336,7 @@ int launch_gemm_w4_tile(const GemmArgs &a0, bool fused_act, int flags, int64_t m
   const int64_t chunks = (m_blocks + G - 1) / G;
   const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm(w4): grid too large");
-  const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 || (flags & LO_GEMM_CANONICAL_ORDER) == 0;
+  const bool fast = fused_scale_order(flags);
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
   if (fused_act) {

@@ -26,12 +26,6 @@
 #ifndef LO_WS_PD_SMALL
 #define LO_WS_PD_SMALL 4
 #endif
-#ifndef LO_WS_PLAIN_WAVES
-#define LO_WS_PLAIN_WAVES 4
-#endif
-#ifndef LO_WS_RPW
-#define LO_WS_RPW 4
-#endif
 #ifndef LO_WS_PD_PLAIN
 #define LO_WS_PD_PLAIN 2
 #endif
@@ -65,8 +59,11 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   const int bid = blockIdx.x;
   const int mb = bid / a.n_tiles, nt = bid - mb * a.n_tiles;
   if (static_cast<int64_t>(mb) * BM >= a.ntpp[0]) return;
-  const int e = a.expert_ids[mb];
-  if (e >= a.E) return; // an expert_map entry outside the weight tensor: nothing to read
+  // An expert_map entry outside the weight tensor is treated like an expert of another rank, but its
+  // rows are always zero-filled: the slot mask of the alignment counts such a slot as local.
+  const int e_raw = a.expert_ids[mb];
+  const bool e_oob = e_raw >= a.E;
+  const int e = e_oob ? -1 : e_raw;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform: scalar address math
   const int r = lane & 15, c = lane >> 4;
@@ -92,7 +89,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
     const int64_t n0 = static_cast<int64_t>(nt) * (16 * NWAVES * RPW) + wave * (16 * RPW);
     if (n0 >= N) return;
     if (e < 0) { // expert not held by this rank: the rows are defined to be zero
-      if (a.skip_nonlocal) return;
+      if (a.skip_nonlocal && !e_oob) return;
 #pragma unroll
       for (int j = 0; j < TM; ++j)
         if (valid[j])
@@ -394,7 +391,7 @@ static void launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
 
 template <bool FUSED_ACT>
 static int dispatch_ws(const GemmArgs &a, int bs, int flags, int64_t m_blocks, hipStream_t s) {
-  const bool fast = (flags & LO_GEMM_FUSED_SCALE) != 0 && !a.per_channel;
+  const bool fast = fused_scale_order(flags) && !a.per_channel;
 #define LO_WS_CASE(TMV)                                               \
   case 16 * TMV:                                                      \
     if (fast) launch_ws<TMV, FUSED_ACT, true>(a, m_blocks, s);        \

@@ -16,6 +16,7 @@ _NATIVE_APIS = {
     "invoke_fused_moe_gemm1_silu_quant",
     "silu_and_mul",
     "fused_experts_workspace_bytes",
+    "fused_experts_workspace_views",
     "preshuffle_moe_weight",
     "moe_gemm_w8a8",
 }
@@ -33,6 +34,7 @@ __all__ = [
     "fused_experts_impl_int8",
     "fused_experts_impl_w4a8",
     "fused_experts_workspace_bytes",
+    "fused_experts_workspace_views",
     "get_moe_cache",
     "get_w8a8moe_json",
     "invoke_fused_moe_gemm1_silu_quant",

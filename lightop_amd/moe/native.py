@@ -2,6 +2,7 @@
 python/lightop/_lmslim_native/layers/fused_moe/int8.py:543-908)."""
 from __future__ import annotations
 
+import functools
 from typing import Any, Dict, List, Optional, Tuple
 
 import torch
@@ -12,29 +13,34 @@ from ..op import _act_dtype, _ids_dtype, _on_device, _require_cuda
 
 def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bool,
                      block_shape: Optional[List[int]], topk: int,
-                     global_num_experts: int = -1) -> Tuple[Dict[str, Any], Dict[str, Any]]:
+                     global_num_experts: int = -1, preshuffled: bool = True) -> Tuple[Dict[str, Any], Dict[str, Any]]:
     """Tile configuration of both GEMMs for ``m`` tokens (reference: get_w8a8moe_json,
     int8.py:220-256, backed there by per-device JSON files).  Here the table is compiled
     into the library; the dictionaries keep the reference's keys.  ``n1`` = 2*I, ``n2`` = H,
     ``k`` = I.  ``block_shape=None`` asks for the per-channel form (the reference consults
-    get_moe_cuda_config first there, int8.py:735-741), ``[1, 128]`` for W4A8 with K-group scales."""
+    get_moe_cuda_config first there, int8.py:735-741), ``[1, 128]`` for W4A8 with K-group scales.
+    ``preshuffled``: the weights are in the load-time layout of ``preshuffle_moe_weight`` (the table
+    differs for row-major weights).  ``kernel`` / ``num_warps`` / ``BLOCK_SIZE_N`` describe the kernel
+    the stage calls launch for that ``BLOCK_SIZE_M``."""
     del use_int8_w8a8
     t1, t2 = _lib.LoMoeTile(), _lib.LoMoeTile()
     Eg = E if global_num_experts in (-1, None) else global_num_experts
     form = _lib.LO_FORM_CHANNEL if block_shape is None else (
         _lib.LO_FORM_W4 if list(block_shape) == [1, 128] else _lib.LO_FORM_BLOCK)
-    _lib.check(_lib.lib().lo_moe_tile_query_form(form, m, E, Eg, topk, n2, k, t1, t2))
+    flags = _lib.LO_GEMM_W_PRESHUFFLED if preshuffled else 0
+    _lib.check(_lib.lib().lo_moe_tile_query_form(form, flags, m, E, Eg, topk, n2, k, t1, t2))
 
     def as_dict(t):
         return {"BLOCK_SIZE_M": t.block_size_m, "BLOCK_SIZE_N": t.block_n, "BLOCK_SIZE_K": 128,
-                "GROUP_SIZE_M": 1, "num_warps": t.waves, "num_stages": 0, "kernel": t.kernel}
+                "GROUP_SIZE_M": 1, "num_warps": t.waves, "num_stages": 0, "kernel": t.kernel,
+                "kernel_name": _lib.KERNEL_NAMES.get(t.kernel, "?")}
 
     return as_dict(t1), as_dict(t2)
 
 
 def _scale_flags(fused_scale: Optional[bool]) -> int:
-    """None: the library's choice per kernel; True: acc += d * (a_s * b_s) everywhere;
-    False: the canonical (d * a_s) * b_s + acc everywhere."""
+    """None or False: the canonical (d * a_s) * b_s + acc, which is the library's default;
+    True: acc = fma(d, a_s * b_s, acc) everywhere (last-ulp differences)."""
     if fused_scale is None:
         return 0
     return _lib.LO_GEMM_FUSED_SCALE if fused_scale else _lib.LO_GEMM_CANONICAL_ORDER
@@ -115,7 +121,7 @@ def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tens
                                  sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                                  num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
                                  top_k: int, config: Dict[str, Any], fused_scale: Optional[bool] = None,
-                                 flags: int = 0) -> None:
+                                 flags: int = 0, global_num_experts: int = 0) -> None:
     """One grouped block-INT8 GEMM stage: C[f] = bf16(sum_kb dot(A[f // top_k], B[e])_kb *
     A_scale * B_scale) (* topk_weights[f]) for every routed slot f (reference:
     invoke_fused_moe_kernel_int8, int8.py:543-626).  ``C`` is [M, topk, N] or [S, N].
@@ -135,7 +141,8 @@ def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tens
         _lib.check(_lib.lib().lo_moe_gemm_block_int8(
             _lib.ptr(A), _lib.ptr(A_scale), _lib.ptr(B), _lib.ptr(B_scale), _lib.ptr(C), _act_dtype(C),
             _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(expert_ids),
-            _lib.ptr(num_tokens_post_padded), sorted_token_ids.numel(), num_valid, A.shape[0], E, N, K,
+            _lib.ptr(num_tokens_post_padded), sorted_token_ids.numel(), num_valid, A.shape[0], E,
+            int(global_num_experts or 0), N, K,
             int(top_k), int(config["BLOCK_SIZE_M"]), 1 if mul_routed_weight else 0,
             _scale_flags(fused_scale) | flags | (_lib.LO_GEMM_W_PRESHUFFLED if _is_preshuffled(B) else 0),
             _lib.stream_of(A)))
@@ -146,7 +153,8 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
                                       sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor,
                                       num_tokens_post_padded: torch.Tensor, mul_routed_weight: bool,
                                       top_k: int, num_valid: int, config: Dict[str, Any],
-                                      fused_scale: Optional[bool] = None, flags: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+                                      fused_scale: Optional[bool] = None, flags: int = 0,
+                                      global_num_experts: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
     """First GEMM with SiLU-and-mul and the 1x128 re-quantisation in its epilogue: the
     sequence int8.py:784-823 in one kernel.  Returns (A2q [num_valid, I] int8,
     A2s [num_valid, I/128] f32); rows of slots routed to non-local experts are not written."""
@@ -165,7 +173,8 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
         _lib.check(_lib.lib().lo_moe_gemm1_silu_quant_block_int8(
             _lib.ptr(A), _lib.ptr(A_scale), _lib.ptr(B), _lib.ptr(B_scale), _lib.ptr(a2q), _lib.ptr(a2s),
             _lib.LO_BF16, _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(expert_ids),
-            _lib.ptr(num_tokens_post_padded), sorted_token_ids.numel(), num_valid, A.shape[0], E, I, K,
+            _lib.ptr(num_tokens_post_padded), sorted_token_ids.numel(), num_valid, A.shape[0], E,
+            int(global_num_experts or 0), I, K,
             int(top_k), int(config["BLOCK_SIZE_M"]), 1 if mul_routed_weight else 0,
             _scale_flags(fused_scale) | flags | (_lib.LO_GEMM_W_PRESHUFFLED if _is_preshuffled(B) else 0),
             _lib.stream_of(A)))
@@ -175,7 +184,7 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
 def moe_gemm_w8a8(input: torch.Tensor, b_qweight: torch.Tensor, output: torch.Tensor, a_scale: torch.Tensor,
                   b_scale: torch.Tensor, topk_weights: Optional[torch.Tensor], sorted_token_ids: torch.Tensor,
                   experts_ids: torch.Tensor, num_tokens_post_pad: torch.Tensor, top_k: int,
-                  config: Dict[str, Any], flags: int = 0) -> torch.Tensor:
+                  config: Dict[str, Any], flags: int = 0, global_num_experts: int = 0) -> torch.Tensor:
     """One grouped GEMM stage in the per-channel form (reference: moe_gemm_w8a8, gemmopt.py:437-457):
     output[f] = T((sum_k input[f // top_k] * b_qweight[e]) * ts * b_scale[e]) with
     ts = a_scale[f // top_k], times topk_weights[f] when they are given (the second stage).
@@ -199,7 +208,8 @@ def moe_gemm_w8a8(input: torch.Tensor, b_qweight: torch.Tensor, output: torch.Te
         _lib.check(_lib.lib().lo_moe_gemm_w8a8(
             _lib.ptr(input), _lib.ptr(a_scale), _lib.ptr(b_qweight), _lib.ptr(b_scale), _lib.ptr(output),
             _act_dtype(output), _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(experts_ids),
-            _lib.ptr(num_tokens_post_pad), sorted_token_ids.numel(), num_valid, input.shape[0], E, N, K, int(top_k),
+            _lib.ptr(num_tokens_post_pad), sorted_token_ids.numel(), num_valid, input.shape[0], E,
+            int(global_num_experts or 0), N, K, int(top_k),
             int(config["BLOCK_SIZE_M"]), 1 if tw is not None else 0,
             flags | (_lib.LO_GEMM_W_PRESHUFFLED if _is_preshuffled(b_qweight) else 0), _lib.stream_of(input)))
     return output
@@ -216,11 +226,40 @@ def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
                                               _lib.stream_of(x)))
 
 
+@functools.lru_cache(maxsize=256)
 def fused_experts_workspace_bytes(M: int, top_k: int, H: int, I: int, num_experts: int,
                                   block_size_m: int = 0) -> int:
+    """Bytes of scratch one whole-path call needs (0: enough for every block size)."""
     n = _lib.lib().lo_fused_experts_workspace_bytes(M, top_k, H, I, num_experts, block_size_m)
     _lib.check(n)
     return int(n)
+
+
+def fused_experts_workspace_views(workspace: torch.Tensor, M: int, top_k: int, H: int, I: int, num_experts: int,
+                                  block_size_m: int) -> Dict[str, torch.Tensor]:
+    """The intermediates a whole-path call left in ``workspace`` (the uint8 tensor given to it as
+    ``lightop_amd_workspace``), as tensors: a1q, a1s, sorted_ids, expert_ids, num_tokens_post_pad,
+    a2q, a2s, slot_mask.  ``block_size_m`` must be the block size the call used."""
+    lib = _lib.lib()
+    base = (workspace.data_ptr() + 255) // 256 * 256 - workspace.data_ptr()
+    S = M * top_k
+    cap = S + num_experts * (block_size_m - 1)
+    if S < num_experts:
+        cap = min(cap, S * block_size_m)
+    spec = [("a1q", torch.int8, (M, H)), ("a1s", torch.float32, (M, H // 128)), ("sorted_ids", torch.int32, (cap,)),
+            ("expert_ids", torch.int32, ((cap + block_size_m - 1) // block_size_m,)),
+            ("num_tokens_post_pad", torch.int32, (1,)), ("a2q", torch.int8, (S, I)),
+            ("a2s", torch.float32, (S, I // 128)), ("slot_mask", torch.uint8, (S,))]
+    views = {}
+    for which, (name, dt, shape) in enumerate(spec):
+        off = lib.lo_fused_experts_workspace_offset(which, M, top_k, H, I, num_experts, block_size_m)
+        _lib.check(off)
+        n = 1
+        for d in shape:
+            n *= d
+        nbytes = n * torch.empty((), dtype=dt).element_size()
+        views[name] = workspace[base + off: base + off + nbytes].view(dt).view(shape)
+    return views
 
 
 def fused_experts_impl_int8(hidden_states: torch.Tensor,
@@ -264,7 +303,7 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     performed: ``out = routed_scaling_factor * sum_k(...) (+ shared_output)``.
     Unknown keyword arguments are ignored, as in the reference.
     """
-    extra = _  # private tuning knobs: lightop_amd_flags, lightop_amd_block_size_m
+    extra = _  # private knobs: lightop_amd_flags, lightop_amd_block_size_m, lightop_amd_workspace
     # Check constraints (int8.py:658-667).
     assert use_int8_w8a8 or use_fp8_w8a8
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
@@ -314,7 +353,8 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
                               apply_router_weight_on_input, global_num_experts, expert_map, w1_scale, w2_scale,
                               routed_scaling_factor, shared_output, I, flags,
-                              int(extra.get("lightop_amd_block_size_m", 0)), channel=channel)
+                              int(extra.get("lightop_amd_block_size_m", 0)), channel=channel,
+                              workspace=extra.get("lightop_amd_workspace"))
 
 
 def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
@@ -397,12 +437,12 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
                               apply_router_weight_on_input, global_num_experts, expert_map, w1_scale, w2_scale,
                               routed_scaling_factor, shared_output, I, flags,
-                              int(extra.get("lightop_amd_block_size_m", 0)))
+                              int(extra.get("lightop_amd_block_size_m", 0)), workspace=extra.get("lightop_amd_workspace"))
 
 
 def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace, apply_router_weight_on_input,
                        global_num_experts, expert_map, w1_scale, w2_scale, routed_scaling_factor, shared_output,
-                       I, flags, block_size_m, channel=False):
+                       I, flags, block_size_m, channel=False, workspace=None):
     """Chunk loop shared by the block-INT8, per-channel and W4A8 entry points (int8.py:703-888)."""
     num_tokens, H = hidden_states.shape
     E = w1.shape[0]
@@ -429,7 +469,12 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
 
     lib = _lib.lib()
     ws_bytes = fused_experts_workspace_bytes(M, top_k_num, H, I, global_num_experts, 0)
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=hidden_states.device)
+    if workspace is None:
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=hidden_states.device)
+    else:  # the caller's own scratch (tests read the intermediates out of it afterwards)
+        assert workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.numel() >= ws_bytes
+        assert workspace.device == hidden_states.device
+        ws_bytes = workspace.numel()
     ws_ptr = (workspace.data_ptr() + 255) // 256 * 256
     ws_avail = ws_bytes - (ws_ptr - workspace.data_ptr())
     assert _is_preshuffled(w1) == _is_preshuffled(w2), "preshuffle both w1 and w2 or neither"
@@ -464,4 +509,5 @@ def ctypes_void(addr: int):
 
 __all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "preshuffle_moe_weight",
            "preshuffle_moe_weight_int4", "preshuffle_moe_scale_int4", "invoke_fused_moe_kernel_int8",
-           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes", "moe_gemm_w8a8"]
+           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes",
+           "fused_experts_workspace_views", "moe_gemm_w8a8"]

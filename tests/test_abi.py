@@ -77,13 +77,49 @@ def test_version_and_tile_table(lib):
         assert lib.lo_moe_tile_query(M, 128, 128, 8, 2048, 768, t1, t2) == 0 and t1.block_size_m == want
     # per-channel form: same small tiles, 128 tokens once an expert sees that many
     for M, want in ((1, 16), (64, 16), (1024, 64), (2048, 128), (8192, 128)):
-        assert lib.lo_moe_tile_query_form(_lib.LO_FORM_CHANNEL, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
+        assert lib.lo_moe_tile_query_form(_lib.LO_FORM_CHANNEL, 0, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
         assert t1.block_size_m == want and t2.block_size_m == want
     # W4A8: streaming for a handful of slots per expert, the 64-token LDS tile from 8 on, 128 tokens from 48 on
     for M, want in ((1, 16), (128, 16), (256, 16), (512, 64), (1024, 64), (2048, 128), (8192, 128)):
-        assert lib.lo_moe_tile_query_form(_lib.LO_FORM_W4, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
+        assert lib.lo_moe_tile_query_form(_lib.LO_FORM_W4, 0, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
         assert t1.block_size_m == want
-    assert lib.lo_moe_tile_query_form(7, 1, 32, 256, 8, 7168, 2048, t1, t2) < 0
+    assert lib.lo_moe_tile_query_form(7, 0, 1, 32, 256, 8, 7168, 2048, t1, t2) < 0
+
+
+def test_tile_query_names_the_kernel_that_is_launched(lib):
+    """kernel / waves / block_n are those of the kernel the stage entry points pick for the block size,
+    for both weight layouts (they share one selection function with the launcher)."""
+    from lightop_amd import _lib
+
+    t1, t2 = _lib.LoMoeTile(), _lib.LoMoeTile()
+    pre = _lib.LO_GEMM_W_PRESHUFFLED
+    q = lambda form, flags, M, *shape: lib.lo_moe_tile_query_form(form, flags, M, *shape, t1, t2)
+    qwen, dsv3 = (128, 128, 8, 2048, 768), (32, 256, 8, 7168, 2048)
+    # decode sizes: weight streaming, eight waves own one 128-column activation group in the fused GEMM
+    assert q(_lib.LO_FORM_BLOCK, pre, 16, *dsv3) == 0
+    assert (t1.block_size_m, t1.kernel, t1.waves, t1.block_n) == (16, _lib.LO_KERNEL_WS, 8, 256)
+    assert (t2.kernel, t2.waves, t2.block_n) == (_lib.LO_KERNEL_WS, 4, 256)
+    # prefill, load-time layout: 128-token direct-to-LDS kernel for GEMM1, activation-stationary GEMM2 on a short K
+    assert q(_lib.LO_FORM_BLOCK, pre, 8192, *qwen) == 0
+    assert (t1.block_size_m, t1.kernel, t1.waves, t1.block_n) == (128, _lib.LO_KERNEL_T128, 4, 256)
+    assert t2.kernel == _lib.LO_KERNEL_AS
+    assert q(_lib.LO_FORM_BLOCK, pre, 4096, *dsv3) == 0
+    assert t1.kernel == _lib.LO_KERNEL_T128 and t2.kernel == _lib.LO_KERNEL_T128  # K = 2048: too long to stay in LDS
+    # row-major weights: 64-token register-fed tiles, and a different block size than the load-time layout
+    assert q(_lib.LO_FORM_BLOCK, 0, 8192, *qwen) == 0
+    assert (t1.block_size_m, t1.kernel, t1.waves) == (64, _lib.LO_KERNEL_TILE, 4)
+    assert q(_lib.LO_FORM_BLOCK, 0, 256, *qwen) == 0 and t1.block_size_m == 32 and t1.kernel == _lib.LO_KERNEL_WS
+    assert q(_lib.LO_FORM_BLOCK, pre, 256, *qwen) == 0 and t1.block_size_m == 128
+    # forced streaming is honoured
+    assert q(_lib.LO_FORM_BLOCK, pre | _lib.LO_GEMM_FORCE_STREAMING, 8192, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_WS
+    # per-channel and int4 forms
+    assert q(_lib.LO_FORM_CHANNEL, pre, 8192, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_PC == t2.kernel
+    assert q(_lib.LO_FORM_W4, 0, 512, *dsv3) == 0 and t1.kernel == _lib.LO_KERNEL_W4_TILE
+    assert q(_lib.LO_FORM_W4, 0, 8192, *dsv3) == 0 and t1.kernel == _lib.LO_KERNEL_T128
+    # the convenience query is the block form with the load-time layout
+    t3 = _lib.LoMoeTile()
+    assert lib.lo_moe_tile_query(8192, *qwen, t3, None) == 0 and q(_lib.LO_FORM_BLOCK, pre, 8192, *qwen) == 0
+    assert (t1.block_size_m, t1.kernel, t1.waves, t1.block_n) == (t3.block_size_m, t3.kernel, t3.waves, t3.block_n)
 
 
 def test_workspace_sizing(lib):
@@ -96,6 +132,13 @@ def test_workspace_sizing(lib):
     offs = [lib.lo_fused_experts_workspace_offset(i, 64, 8, 7168, 2048, 256, 16) for i in range(8)]
     assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
     assert lib.lo_fused_experts_workspace_offset(8, 64, 8, 7168, 2048, 256, 16) < 0
+    # block_size_m = 0 must cover every block size the call may end up with: few experts and many
+    # tokens make the per-block expert ids of small blocks the larger segment
+    for (M, k, H, I, E) in ((16384, 2, 1024, 512, 2), (16384, 2, 1024, 512, 8), (64, 8, 7168, 2048, 256),
+                            (1, 8, 2048, 768, 128), (8192, 8, 2048, 768, 128)):
+        n0 = lib.lo_fused_experts_workspace_bytes(M, k, H, I, E, 0)
+        for bs in (16, 32, 64, 128):
+            assert n0 >= lib.lo_fused_experts_workspace_bytes(M, k, H, I, E, bs), (M, E, bs)
 
 
 def test_validation_happens_before_any_launch(lib):
@@ -112,3 +155,19 @@ def test_validation_happens_before_any_launch(lib):
     assert lib.lo_per_token_group_quant_int8(p, 1, 1, 128, 1e-10, p, p, null) == -4              # fp16 not built
     assert lib.lo_moe_sum(p, p, null, null, 0, 1, 8, 100, 1.0, null, null) == -1                       # H % 8
     assert lib.lo_preshuffle_weight_int8(p, p, 1, 16, 128, null) == -1                           # src == dst
+
+
+def test_stage_entry_points_reject_a_bad_block_size(lib):
+    """block_size_m divides the sorted-id extent: 0 (the whole-path call's "ask the table") and sizes
+    that are not 16 / 32 / 64 / 128 are an error here, not a division by zero."""
+    null = ctypes.c_void_p(0)
+    buf = (ctypes.c_int32 * 1024)()
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 15) // 16 * 16)
+    for bad in (0, 48, -16, 256):
+        rc = lib.lo_moe_gemm_block_int8(p, p, p, p, p, 0, null, p, p, p, 128, 8, 8, 1, 1, 16, 128, 1, bad, 0, 0, null)
+        assert rc == -1 and b"block_size_m" in lib.lo_last_error(), bad
+        rc = lib.lo_moe_gemm1_silu_quant_block_int8(p, p, p, p, p, p, 0, null, p, p, p, 128, 8, 8, 1, 1, 128, 128,
+                                                    1, bad, 0, 0, null)
+        assert rc == -1 and b"block_size_m" in lib.lo_last_error(), bad
+        rc = lib.lo_moe_gemm_w8a8(p, p, p, p, p, 0, null, p, p, p, 128, 8, 8, 1, 1, 16, 128, 1, bad, 0, 0, null)
+        assert rc == -1 and b"block_size_m" in lib.lo_last_error(), bad

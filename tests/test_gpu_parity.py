@@ -491,7 +491,7 @@ def test_preshuffle_layout(dev):
 
 # ---------------------------------------------------------------- whole path ---
 
-def run_fused(dev, layer, M, seed, bs=0, flags=4, shared=False, on_input=False, inplace=False, preshuffle=False):
+def run_fused(dev, layer, M, seed, bs=0, flags=0, shared=False, on_input=False, inplace=False, preshuffle=False):
     from lightop_amd import workloads as wl
     from lightop_amd.moe import fused_experts_impl_int8, preshuffle_moe_weight
 
@@ -547,13 +547,45 @@ def test_fused_experts_ep_share_bit_exact(dev, oracle, M, variant):
 
 
 def test_fused_experts_default_tile_and_fused_scale(dev, oracle):
+    """Block size from the tile table: the default arithmetic is bit-exact, the optional fused-scale
+    order within the tolerance."""
     from lightop_amd import _lib, workloads as wl
 
     say("fused default tile + fused-scale tolerance")
     layer = wl.MoeLayer("q", E=16, E_global=16, top_k=4, H=512, I=256, routing="softmax")
-    (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, layer, 200, 1, flags=_lib.LO_GEMM_FUSED_SCALE)
-    ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 64)
-    assert within_tolerance(out, ref)
+    for pre in (False, True):
+        (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, layer, 200, 1, preshuffle=pre)
+        ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 64)
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"default order, preshuffle={pre}"
+        _, out_f = run_fused(dev, layer, 200, 1, flags=_lib.LO_GEMM_FUSED_SCALE, preshuffle=pre)
+        assert within_tolerance(out_f, ref)
+
+
+@pytest.mark.parametrize("bs", BS_ALL)
+def test_expert_map_entry_outside_the_weights_gives_zero_rows(dev, oracle, bs):
+    """A malformed expert_map (a local id >= the number of experts held) must not read past the
+    weights nor leave garbage in the sum: such slots contribute zero, exactly as if the entry were -1."""
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import fused_experts_impl_int8, preshuffle_moe_weight
+
+    say(f"expert_map entry >= E, bs={bs}")
+    layer = wl.MoeLayer("oob", E=4, E_global=8, top_k=2, H=256, I=128, routing="softmax")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=2)
+    M = 150
+    x, tw, ids = wl.make_inputs(layer, M, seed=2)
+    bad = torch.tensor([0, 1, 2, 3, 4, 9, -1, 1000], dtype=torch.int32)     # 4, 9, 1000: outside w1 / w2
+    good = torch.tensor([0, 1, 2, 3, -1, -1, -1, -1], dtype=torch.int32)
+    ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, bs, global_num_experts=8, expert_map=good)
+    for pre in (False, True):
+        w1d, w2d = w1.to(dev), w2.to(dev)
+        if pre:
+            w1d, w2d = preshuffle_moe_weight(w1d), preshuffle_moe_weight(w2d)
+        cache13 = torch.full((M * 2 * 256,), float("nan"), dtype=torch.bfloat16, device=dev)
+        out = fused_experts_impl_int8(x.to(dev), w1d, w2d, tw.to(dev), ids.to(dev), cache13, use_int8_w8a8=True,
+                                      global_num_experts=8, expert_map=bad.to(dev), w1_scale=w1s.to(dev),
+                                      w2_scale=w2s.to(dev), block_shape=[128, 128], lightop_amd_block_size_m=bs)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16)), f"preshuffle={pre}"
 
 
 def test_fused_experts_rejects_unsupported(dev):

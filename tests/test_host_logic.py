@@ -272,3 +272,27 @@ def test_torch_restatement_agrees_with_oracle_on_config1(oracle):
     err = (out - ref).abs()
     assert err.max() <= 1e-2 * ref.abs().max()
     assert err.sum() / ref.abs().sum() <= 2e-3 * 3
+
+
+def test_moe_cache_is_keyed_and_grows(monkeypatch):
+    """get_moe_cache hands out one buffer per (device, dtype), large enough for the call at hand:
+    a later call with another dtype or a larger layer must not receive the first call's tensor
+    (the reference's singleton does, fused_moe_cache.py:19-24)."""
+    import torch
+
+    from lightop_amd.moe import cache
+
+    monkeypatch.setenv("LMSLIM_FUSED_MOE_CHUNK_SIZE", "4")
+    cache.release_moe_cache()
+    a = cache.get_moe_cache(2, 256, 128, "cpu", torch.bfloat16)
+    assert a.dtype == torch.bfloat16 and a.dim() == 1 and a.numel() == 4 * 2 * 256
+    assert cache.get_moe_cache(2, 128, 256, "cpu", torch.bfloat16) is a          # same need: shared
+    assert cache.get_moe_cache(1, 64, 64, "cpu", torch.bfloat16) is a            # smaller need: shared
+    b = cache.get_moe_cache(2, 256, 128, "cpu", torch.float16)
+    assert b.dtype == torch.float16 and b is not a                               # another dtype: its own buffer
+    c = cache.get_moe_cache(8, 512, 128, "cpu", torch.bfloat16)
+    assert c.numel() == 4 * 8 * 512 and c is not a                               # larger need: grows
+    assert cache.get_moe_cache(2, 256, 128, "cpu", torch.bfloat16) is c
+    assert cache.moe_cache_singleton is c
+    cache.release_moe_cache()
+    assert cache.moe_cache_singleton is None

@@ -260,11 +260,22 @@ def test_moe_sum_cases(oracle):
     x = torch.randn(9, 1, 64, generator=g).to(torch.bfloat16)
     assert torch.equal(oracle.moe_sum(x), x[:, 0])                      # k = 1, factor 1: identity
     x = torch.randn(9, 8, 64, generator=g).to(torch.bfloat16)
-    assert torch.equal(oracle.moe_sum(x), x.float().sum(dim=1).to(torch.bfloat16)) or \
-        torch.allclose(oracle.moe_sum(x).float(), x.float().sum(dim=1), rtol=2 ** -8)
-    # sequential fp32 order, one rounding: hand-worked
-    v = bf16([[[1.0], [2.0 ** -9], [2.0 ** -9]]])                       # 1 + 2^-9 + 2^-9 = 1 + 2^-8
-    assert oracle.moe_sum(v).float().item() == 1.0 + 2.0 ** -7 or oracle.moe_sum(v).float().item() == 1.0
+    seq = torch.zeros(9, 64)
+    for j in range(8):                                                  # IEEE fp32 adds in slot order,
+        seq = seq + x[:, j].float()
+    assert torch.equal(oracle.moe_sum(x), seq.to(torch.bfloat16))       # one rounding at the end
+    # the order matters: ((2^24 + 1) - 2^24) + 1 = 1 in fp32 slot order; a pairwise or reversed sum gives 0 or 2
+    v = bf16([[[2.0 ** 24], [1.0], [-(2.0 ** 24)], [1.0]]])
+    assert oracle.moe_sum(v).float().item() == 1.0
+    # the accumulator is fp32, not bf16: 1 + 2^-8 + 2^-8 = 1 + 2^-7 exactly (a bf16 accumulator stays at 1)
+    v = bf16([[[1.0], [2.0 ** -8], [2.0 ** -8]]])
+    assert oracle.moe_sum(v).float().item() == 1.0 + 2.0 ** -7
+    # one rounding, to nearest even: 1 + 2^-9 + 2^-9 = 1 + 2^-8 lies halfway between 1 and 1 + 2^-7 -> 1
+    v = bf16([[[1.0], [2.0 ** -9], [2.0 ** -9]]])
+    assert oracle.moe_sum(v).float().item() == 1.0
+    # ... and 1 + 2^-7 + 2^-8 lies halfway between 1 + 2^-7 (odd) and 1 + 2^-6 (even) -> up
+    assert oracle.moe_sum(bf16([[[1.0 + 2.0 ** -7], [2.0 ** -8]]])).float().item() == 1.0 + 2.0 ** -6
+    v = bf16([[[1.0], [2.0 ** -9], [2.0 ** -9]]])
     f = np.float32
     acc = (f(0) + f(1.0)) + f(2.0 ** -9) + f(2.0 ** -9)
     assert oracle.moe_sum(v, factor=2.5).float().item() == torch.tensor(float(acc * f(2.5))).to(torch.bfloat16).item()
