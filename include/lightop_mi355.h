@@ -71,7 +71,8 @@ const char *lo_last_error(void);
 
 /*
  * Optional one-time set-up for the current device: builds the 128 KB bf16 SiLU table
- * that the fused GEMM epilogue looks activations up in.  The first fused-GEMM call on a
+ * that the fused GEMM epilogue looks activations up in and looks up the address of the
+ * built-in scratch of lo_fused_experts_block_int8_noalloc.  The first fused-GEMM call on a
  * device does this by itself (and synchronises the stream once); call lo_init() first
  * when that first call would fall inside a HIP graph capture.  No counterpart in the
  * reference.
@@ -310,6 +311,28 @@ int lo_fused_experts_block_int8(const void *x, int dtype, int64_t M, int64_t H, 
                                 float routed_scaling_factor, const void *shared_output,
                                 void *cache3, void *out, void *workspace, int64_t workspace_bytes,
                                 int32_t block_size_m, int flags, lo_stream_t stream);
+
+/*
+ * The same call for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no workspace argument, the scratch is a
+ * device array inside the library, LO_NOALLOC_SCRATCH_BYTES (32 MiB) per GPU, held until the
+ * process ends.  No counterpart in the reference, whose path allocates four
+ * tensors per call (int8.py:685-701, moe_align_block_size.py:87-95).  Problems whose scratch
+ * (lo_fused_experts_workspace_bytes(..., block_size_m)) exceeds that size are refused with
+ * LO_ENOSPC.  The function calls no allocator; lo_init() looks the array's address up
+ * beforehand (otherwise the first call on a device does), and must have run before a graph
+ * capture, as for every fused call.  All calls on one GPU share that GPU's array: calls that
+ * overlap there (two streams, two threads) race; serialise them or use the workspace form.
+ */
+#define LO_NOALLOC_SCRATCH_BYTES (32ll << 20)
+int lo_fused_experts_block_int8_noalloc(const void *x, int dtype, int64_t M, int64_t H, int64_t I,
+                                        int32_t E, int32_t num_experts, int32_t top_k,
+                                        const int8_t *w1, const float *w1s, const int8_t *w2,
+                                        const float *w2s, const float *topk_w, const void *topk_ids,
+                                        int ids_dtype, const int32_t *expert_map,
+                                        int apply_router_weight_on_input, float routed_scaling_factor,
+                                        const void *shared_output, void *cache3, void *out,
+                                        int32_t block_size_m, int flags, lo_stream_t stream);
 
 /*
  * Views into the workspace of the last layout computed for the same arguments, so

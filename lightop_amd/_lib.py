@@ -15,6 +15,7 @@ LO_GEMM_W_PRESHUFFLED = 8
 LO_GEMM_SKIP_NONLOCAL = 16
 LO_GEMM_W4 = 32
 LO_FORM_BLOCK, LO_FORM_CHANNEL, LO_FORM_W4 = 0, 1, 2
+LO_NOALLOC_SCRATCH_BYTES = 32 << 20
 LO_KERNEL_WS, LO_KERNEL_TILE, LO_KERNEL_PC, LO_KERNEL_AS, LO_KERNEL_T128, LO_KERNEL_W4_TILE = 0, 1, 2, 3, 4, 5
 KERNEL_NAMES = {LO_KERNEL_WS: "moe_gemm_ws_kernel", LO_KERNEL_TILE: "moe_gemm_tile_kernel",
                 LO_KERNEL_PC: "moe_gemm_pc_kernel", LO_KERNEL_AS: "moe_gemm_as_kernel",
@@ -79,6 +80,10 @@ SIGNATURES = {
                                             c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_int64, c_int32, c_int, c_void_p]),
+    "lo_fused_experts_block_int8_noalloc": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int32, c_int32,
+                                                    c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                    c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,
+                                                    c_void_p, c_int32, c_int, c_void_p]),
 }
 
 _lib = None

@@ -2,6 +2,7 @@
 // entry point that chains the stage kernels on one stream.
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 #include "gemm.h"
 
@@ -301,4 +302,77 @@ extern "C" int lo_fused_experts_channel_int8(
   if (rc) return rc;
   return lo_moe_sum(cache13, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor, nullptr,
                     stream);
+}
+
+// ---- whole path for callers that cannot allocate -------------------------------------------
+// The scratch of the whole-path call (quantised activations, alignment buffers, slot mask) in a
+// device array that is part of the library's image instead of a caller workspace.  Every GPU the
+// library runs on holds its own copy at its own address for the life of the process; the address
+// is looked up once per device and only that pointer is ever handed to kernels.
+namespace lo {
+
+constexpr int64_t kScratchBytes = LO_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[64] = {};
+
+// Device address of `scratch` on the current device.
+static int static_scratch(void **out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    set_error("static scratch: no current HIP device");
+    return LO_ELAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      set_error("static scratch: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+      return LO_ELAUNCH;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return LO_OK;
+}
+
+} // namespace lo
+
+extern "C" int lo_init(lo_stream_t stream) {
+  const uint16_t *t = nullptr;
+  int rc = lo::silu_table(static_cast<hipStream_t>(stream), &t);
+  if (rc) return rc;
+  void *p = nullptr;
+  return lo::static_scratch(&p);
+}
+
+extern "C" int lo_fused_experts_block_int8_noalloc(
+    const void *x, int dtype, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts,
+    int32_t top_k, const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s,
+    const float *topk_w, const void *topk_ids, int ids_dtype, const int32_t *expert_map,
+    int apply_router_weight_on_input, float routed_scaling_factor, const void *shared_output,
+    void *cache3, void *out, int32_t block_size_m, int flags, lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(M >= 0 && top_k >= 1 && H >= kGroup && I >= kGroup && num_experts >= 1, LO_EINVAL,
+             "fused_experts(noalloc): bad problem size");
+  if (block_size_m == 0)
+    block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
+                                (flags & LO_GEMM_W_PRESHUFFLED) != 0);
+  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
+             LO_EINVAL, "fused_experts(noalloc): block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
+  const int64_t need = ws_layout(M, top_k, H, I, num_experts, block_size_m).total;
+  LO_REQUIRE(need <= kScratchBytes, LO_ENOSPC,
+             "fused_experts(noalloc): this problem needs %lld bytes of scratch, the built-in scratch holds %lld; "
+             "use lo_fused_experts_block_int8 with a caller workspace",
+             (long long)need, (long long)kScratchBytes);
+  void *ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc) return rc;
+  // Nothing in the scratch has to start at zero: every segment is written before it is read
+  // (padding values, expert ids past the last block and the alignment's counters included).
+  return lo_fused_experts_block_int8(x, dtype, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w, topk_ids,
+                                     ids_dtype, expert_map, apply_router_weight_on_input, routed_scaling_factor,
+                                     shared_output, cache3, out, ws, kScratchBytes, block_size_m, flags, stream);
 }

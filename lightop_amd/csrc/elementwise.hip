@@ -346,11 +346,6 @@ int silu_table(hipStream_t stream, const uint16_t **out) {
 
 } // namespace lo
 
-extern "C" int lo_init(lo_stream_t stream) {
-  const uint16_t *t = nullptr;
-  return lo::silu_table(static_cast<hipStream_t>(stream), &t);
-}
-
 extern "C" int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t rows,
                                              int64_t cols, float eps, int8_t *q, float *s,
                                              lo_stream_t stream) {
