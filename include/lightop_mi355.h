@@ -63,7 +63,14 @@ enum {
    * scales per token and per channel in the epilogue instead; its nibble order (even k in
    * the high nibble, :341, :375-377) is the one lo_preshuffle_weight_int4 reads.  Served by
    * an LDS-tiled kernel at block_size_m 64 and by the weight-streaming kernels otherwise. */
-  LO_GEMM_W4 = 32
+  LO_GEMM_W4 = 32,
+  /* whole-path calls only.  With block_size_m = 0 and weights in the load-time layout the block
+   * form serves small batches (few routed slots per expert) with a two-launch path that needs no
+   * alignment, no quantised copy of x and no per-slot output rows; same results bit for bit.
+   * NO_DECODE_PATH: never take it.  FORCE_DECODE_PATH: take it whenever it can serve the problem
+   * (at most 512 routed slots), whatever the size heuristic says. */
+  LO_FUSED_NO_DECODE_PATH = 64,
+  LO_FUSED_FORCE_DECODE_PATH = 128
 };
 
 int lo_version(void);
@@ -270,7 +277,12 @@ enum {
   LO_KERNEL_PC = 2,      /* per-channel LDS-tiled */
   LO_KERNEL_AS = 3,      /* activation-stationary second GEMM (short K) */
   LO_KERNEL_T128 = 4,    /* 128 tokens, both operands copied global -> LDS (pre-shuffled weights) */
-  LO_KERNEL_W4_TILE = 5  /* packed-int4 LDS-tiled, 64 tokens */
+  LO_KERNEL_W4_TILE = 5, /* packed-int4 LDS-tiled, 64 tokens */
+  LO_KERNEL_DEC = 6      /* the whole-path call's two-launch path for a few tokens (weights in the load-time
+                          * layout, block_size_m = 0): 16 weight rows per workgroup, the waves of the first
+                          * kernel split K, those of the second take one routed slot each.  The stage entry
+                          * points have no such kernel: given the reported block_size_m they launch
+                          * LO_KERNEL_WS. */
 };
 
 /* Block form with weights in the load-time layout (flags = LO_GEMM_W_PRESHUFFLED). */

@@ -14,12 +14,15 @@ LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE, LO_GEMM_FORCE_STREAMING, LO_GEMM_CANONICAL
 LO_GEMM_W_PRESHUFFLED = 8
 LO_GEMM_SKIP_NONLOCAL = 16
 LO_GEMM_W4 = 32
+LO_FUSED_NO_DECODE_PATH = 64
+LO_FUSED_FORCE_DECODE_PATH = 128
 LO_FORM_BLOCK, LO_FORM_CHANNEL, LO_FORM_W4 = 0, 1, 2
 LO_NOALLOC_SCRATCH_BYTES = 32 << 20
-LO_KERNEL_WS, LO_KERNEL_TILE, LO_KERNEL_PC, LO_KERNEL_AS, LO_KERNEL_T128, LO_KERNEL_W4_TILE = 0, 1, 2, 3, 4, 5
+LO_KERNEL_WS, LO_KERNEL_TILE, LO_KERNEL_PC, LO_KERNEL_AS, LO_KERNEL_T128, LO_KERNEL_W4_TILE, LO_KERNEL_DEC = 0, 1, 2, 3, 4, 5, 6
 KERNEL_NAMES = {LO_KERNEL_WS: "moe_gemm_ws_kernel", LO_KERNEL_TILE: "moe_gemm_tile_kernel",
                 LO_KERNEL_PC: "moe_gemm_pc_kernel", LO_KERNEL_AS: "moe_gemm_as_kernel",
-                LO_KERNEL_T128: "moe_gemm_t128_kernel", LO_KERNEL_W4_TILE: "moe_gemm_w4_tile_kernel"}
+                LO_KERNEL_T128: "moe_gemm_t128_kernel", LO_KERNEL_W4_TILE: "moe_gemm_w4_tile_kernel",
+                LO_KERNEL_DEC: "dec_gemm1_kernel / dec_gemm2_kernel"}
 
 
 class LoMoeTile(ctypes.Structure):

@@ -141,6 +141,14 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
     a.N = H; a.K = I; a.a_rows = M * top_k;
     describe_gemm_kernel(pick_gemm_kernel(a, false, bm, flags), false, bm, gemm2);
   }
+  // a few tokens: the whole-path call serves the block form with its two-launch path
+  if (form == LO_FORM_BLOCK && pre && !(flags & LO_FUSED_NO_DECODE_PATH) && M > 0 &&
+      decode_path_applies(M, top_k, H, I, num_experts, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0)) {
+    int w1 = 0, w2 = 0;
+    decode_path_waves(top_k, H, &w1, &w2);
+    if (gemm1) { gemm1->kernel = LO_KERNEL_DEC; gemm1->waves = w1; gemm1->block_n = 16; }
+    if (gemm2) { gemm2->kernel = LO_KERNEL_DEC; gemm2->waves = w2; gemm2->block_n = 16; }
+  }
   return LO_OK;
 }
 
@@ -194,6 +202,7 @@ extern "C" int lo_fused_experts_block_int8(
   LO_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, LO_EINVAL,
              "fused_experts: workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
+  const bool block_size_m_auto = block_size_m == 0;
   if (block_size_m == 0)
     block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
                                 (flags & LO_GEMM_W_PRESHUFFLED) != 0);
@@ -214,6 +223,15 @@ extern "C" int lo_fused_experts_block_int8(
   // neither zero-filled by the second GEMM nor read by the reduction.
   uint8_t *mask = expert_map ? reinterpret_cast<uint8_t *>(ws + L.off[7]) : nullptr;
   const int64_t S = M * top_k;
+
+  // Decode sizes: routing, quantisation, both GEMMs and the reduction in two launches.
+  if (block_size_m_auto && (flags & LO_GEMM_W_PRESHUFFLED) && !(flags & (LO_GEMM_W4 | LO_FUSED_NO_DECODE_PATH))) {
+    // (cache3 is the front of the caller's cache13: the path keeps its bf16 activations [S, I] there)
+    const int rc2 = launch_decode_path(x, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w, topk_ids, ids_dtype,
+                                       expert_map, apply_router_weight_on_input, routed_scaling_factor, shared_output,
+                                       cache3, out, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0, static_cast<hipStream_t>(stream));
+    if (rc2 != LO_ENOTSUP) return rc2;
+  }
 
   // the quantisation rides in the alignment's launch
   int rc = launch_quant_align(x, M, H, 1e-10f, a1q, a1s, topk_ids, ids_dtype, S, num_experts, block_size_m,
@@ -357,6 +375,7 @@ extern "C" int lo_fused_experts_block_int8_noalloc(
   using namespace lo;
   LO_REQUIRE(M >= 0 && top_k >= 1 && H >= kGroup && I >= kGroup && num_experts >= 1, LO_EINVAL,
              "fused_experts(noalloc): bad problem size");
+  const int32_t block_size_m_arg = block_size_m;
   if (block_size_m == 0)
     block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
                                 (flags & LO_GEMM_W_PRESHUFFLED) != 0);
@@ -374,5 +393,5 @@ extern "C" int lo_fused_experts_block_int8_noalloc(
   // (padding values, expert ids past the last block and the alignment's counters included).
   return lo_fused_experts_block_int8(x, dtype, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w, topk_ids,
                                      ids_dtype, expert_map, apply_router_weight_on_input, routed_scaling_factor,
-                                     shared_output, cache3, out, ws, kScratchBytes, block_size_m, flags, stream);
+                                     shared_output, cache3, out, ws, kScratchBytes, block_size_m_arg, flags, stream);
 }
