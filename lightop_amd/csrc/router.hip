@@ -246,9 +246,218 @@ __global__ __launch_bounds__(256) void moe_fused_gate_kernel(const void *__restr
   }
 }
 
+// ---- sixteen lanes per token row ------------------------------------------------------------------
+// With thousands of rows the kernels above are bound by instruction issue: a wavefront spends the
+// same few hundred instructions on one row whether the row fills its lanes or not.  Up to 256
+// experts a row fits 16 lanes (one DPP row: the arg-max needs no scalar step across rows), so a
+// wavefront serves four token rows at once.  Lane l of a row holds experts l, l + 16, ...; every
+// result is bit for bit the one of the 64-lane kernels (the full-row softmax sum keeps their order:
+// four partial sums per lane, one per 64-lane row that the expert would have sat in).
+__device__ __forceinline__ void row_argmax(float &v, int &idx) {
+  argmax_step<kXor1>(v, idx);
+  argmax_step<kXor2>(v, idx);
+  argmax_step<kMirror8>(v, idx);
+  argmax_step<kMirror16>(v, idx);
+}
+__device__ __forceinline__ float row_max(float v) {
+  v = fmaxf(v, dpp_f<kXor1>(v));
+  v = fmaxf(v, dpp_f<kXor2>(v));
+  v = fmaxf(v, dpp_f<kMirror8>(v));
+  return fmaxf(v, dpp_f<kMirror16>(v));
+}
+__device__ __forceinline__ float row_sum_tree(float v) {
+  v = v + dpp_f<kXor1>(v);
+  v = v + dpp_f<kXor2>(v);
+  v = v + dpp_f<kMirror8>(v);
+  return v + dpp_f<kMirror16>(v);
+}
+template <int VPT> __device__ __forceinline__ void pick_best16(float (&v)[VPT], int sub, float &best, int &bidx) {
+  best = kNeg;
+  bidx = sub;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j)
+    if (v[j] > best) {
+      best = v[j];
+      bidx = sub + 16 * j;
+    }
+  row_argmax(best, bidx);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j)
+    if (bidx == sub + 16 * j) v[j] = kNeg;
+}
+
+template <int VPT, int DT, typename IdxT>
+__global__ __launch_bounds__(256) void topk_softmax16_kernel(const void *__restrict__ gating, int64_t T, int E, int k,
+                                                             int renormalize, float *__restrict__ weights,
+                                                             IdxT *__restrict__ indices, int32_t *__restrict__ source_rows) {
+  const int sub = threadIdx.x & 15;
+  const int64_t t_raw = static_cast<int64_t>(blockIdx.x) * 16 + (threadIdx.x >> 4);
+  const bool active = t_raw < T;
+  const int64_t t = active ? t_raw : T - 1; // rows past the end compute the last row again and store nothing
+  float x[VPT], v[VPT];
+  float mx = kNeg;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int e = sub + 16 * j;
+    x[j] = e < E ? load_as_f32<DT>(gating, t * E + e) : kNeg;
+    mx = fmaxf(mx, x[j]);
+  }
+  mx = row_max(mx);
+  float scale = 0.0f;
+  if (renormalize) {
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) v[j] = x[j];
+  } else {
+    float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // expert e sat in 64-lane row (e / 16) % 4
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+      const bool in = sub + 16 * j < E;
+      const float p = in ? det_expf(x[j] - mx) : 0.0f;
+      v[j] = in ? p : kNeg;
+      s4[j & 3] = s4[j & 3] + p;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s4[r] = row_sum_tree(s4[r]);
+    scale = 1.0f / (((s4[0] + s4[1]) + (s4[2] + s4[3])) + 1e-6f);
+  }
+  float mine = 0.0f;
+  int mine_idx = 0;
+  for (int j = 0; j < k; ++j) { // k <= 16 (host check): lane j of the row keeps winner j
+    float best;
+    int bidx;
+    pick_best16<VPT>(v, sub, best, bidx);
+    if (sub == j) {
+      mine = best;
+      mine_idx = bidx;
+    }
+  }
+  // one exponential per winner, in the lane that keeps it; then the sum in selection order
+  if (renormalize) mine = det_expf(mine - mx);
+  float sum = 0.0f;
+  const int row_base = threadIdx.x & 48;
+  for (int j = 0; j < k; ++j) sum = sum + __shfl(mine, row_base | j);
+  if (renormalize) scale = 1.0f / (sum + 1e-6f);
+  if (active && sub < k) {
+    weights[t * k + sub] = mine * scale;
+    indices[t * k + sub] = static_cast<IdxT>(mine_idx);
+    if (source_rows) source_rows[t * k + sub] = static_cast<int32_t>(sub * T + t);
+  }
+}
+
+template <int VPT, int DT, int BT, typename IdxT>
+__global__ __launch_bounds__(256) void moe_fused_gate16_kernel(const void *__restrict__ input, const void *__restrict__ bias,
+                                                               int64_t T, int E, int G, int topk_group, int topk,
+                                                               int n_share, float rsf, float route_scale,
+                                                               float *__restrict__ weights, IdxT *__restrict__ indices) {
+  __shared__ float sC[16][16 * VPT]; // biased scores of the row, for the group ranking
+  __shared__ float sS[16][16 * VPT]; // its sigmoids, for the winners
+  const int lane = threadIdx.x & 63, sub = threadIdx.x & 15, row = threadIdx.x >> 4;
+  const int64_t t_raw = static_cast<int64_t>(blockIdx.x) * 16 + row;
+  const bool active = t_raw < T;
+  const int64_t t = active ? t_raw : T - 1;
+  const int gs = E / G, kr = topk - n_share;
+  float s[VPT], c[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int e = sub + 16 * j;
+    if (e < E) {
+      const float xv = load_as_f32<DT>(input, t * E + e);
+      s[j] = 1.0f / (1.0f + det_expf(-xv));
+      c[j] = load_as_f32<BT>(bias, e) + s[j];
+      if (G > 1) sC[row][e] = c[j];
+      sS[row][e] = s[j];
+    } else {
+      s[j] = 0.0f;
+      c[j] = kNeg;
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  uint32_t keep = ~0u;
+  if (G > 1) { // G <= 16 (host check)
+    int lpg = 16;
+    while (lpg * G > 16) lpg >>= 1;
+    const int g = sub / lpg, lsub = sub % lpg;
+    float t1 = kNeg, t2 = kNeg;
+    if (g < G)
+      for (int i = g * gs + lsub; i < (g + 1) * gs; i += lpg) {
+        const float cv = sC[row][i];
+        if (cv > t1) {
+          t2 = t1;
+          t1 = cv;
+        } else if (cv > t2) {
+          t2 = cv;
+        }
+      }
+#define LO_TOP2_MERGE(CTRL)                                  \
+  do {                                                       \
+    const float o1 = dpp_f<CTRL>(t1), o2 = dpp_f<CTRL>(t2);  \
+    const float n1 = fmaxf(t1, o1);                          \
+    t2 = fmaxf(fminf(t1, o1), fmaxf(t2, o2));                \
+    t1 = n1;                                                 \
+  } while (0)
+    if (lpg > 1) LO_TOP2_MERGE(kXor1);
+    if (lpg > 2) LO_TOP2_MERGE(kXor2);
+    if (lpg > 4) LO_TOP2_MERGE(kMirror8);
+    if (lpg > 8) LO_TOP2_MERGE(kMirror16);
+#undef LO_TOP2_MERGE
+    float gscore = (g < G && lsub == 0) ? t1 + t2 : kNeg;
+    keep = 0;
+    for (int r = 0; r < topk_group; ++r) {
+      float bv = gscore;
+      int bi = g;
+      row_argmax(bv, bi);
+      keep |= 1u << bi;
+      if (g == bi) gscore = kNeg;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int e = sub + 16 * j;
+    if (e < E && !((keep >> (e / gs)) & 1)) c[j] = kNeg;
+  }
+  float mine = 0.0f;
+  int mine_idx = 0;
+  for (int j = 0; j < kr; ++j) {
+    float best;
+    int bidx;
+    pick_best16<VPT>(c, sub, best, bidx);
+    if (sub == j) mine_idx = bidx;
+  }
+  // the winners' sigmoids (without the bias), then their sum in selection order
+  if (sub < kr) mine = sS[row][mine_idx];
+  float sum = 0.0f;
+  for (int j = 0; j < kr; ++j) sum = sum + __shfl(mine, (lane & 48) | j);
+  if (sub >= kr && sub < topk) {
+    mine = sum / (rsf > 0.0f ? rsf : 1.0f);
+    mine_idx = E + (sub - kr);
+  }
+  if (active && sub < topk) {
+    weights[t * topk + sub] = (mine / sum) * route_scale;
+    indices[t * topk + sub] = static_cast<IdxT>(mine_idx);
+  }
+}
+
+// Rows from which the 16-lane kernels are used: below, a row per wavefront finishes sooner (a
+// quarter of the per-lane work) and there are compute units to spare.
+constexpr int64_t kRows16From = 65;
+
 template <int VPT, int DT> static void launch_topk_softmax(const void *g, int64_t T, int E, int k, int renorm,
                                                            float *w, void *idx, int idx_dtype, int32_t *src,
                                                            hipStream_t s) {
+  if constexpr (VPT <= 4) { // up to 256 experts
+    if (T >= kRows16From && k <= 16) {
+      const dim3 grid16(static_cast<unsigned>((T + 15) / 16)), block16(256);
+      if (idx_dtype == LO_I64)
+        hipLaunchKernelGGL((topk_softmax16_kernel<4 * VPT, DT, int64_t>), grid16, block16, 0, s, g, T, E, k, renorm, w,
+                           static_cast<int64_t *>(idx), src);
+      else
+        hipLaunchKernelGGL((topk_softmax16_kernel<4 * VPT, DT, int32_t>), grid16, block16, 0, s, g, T, E, k, renorm, w,
+                           static_cast<int32_t *>(idx), src);
+      return;
+    }
+  }
   const dim3 grid(static_cast<unsigned>((T + 3) / 4)), block(256);
   if (idx_dtype == LO_I64)
     hipLaunchKernelGGL((topk_softmax_kernel<VPT, DT, int64_t>), grid, block, 0, s, g, T, E, k, renorm, w,
@@ -261,6 +470,19 @@ template <int VPT, int DT> static void launch_topk_softmax(const void *g, int64_
 template <int VPT, int DT, int BT>
 static void launch_gate(const void *x, const void *b, int64_t T, int E, int G, int tg, int topk, int ns, float rsf,
                         float scale, float *w, void *idx, int idx_dtype, hipStream_t s) {
+  if constexpr (VPT <= 4) { // up to 256 experts
+    // (256 experts: 16 scores per lane make every selection round longer than the 64-lane kernel's)
+    if (T >= kRows16From && topk <= 16 && G <= 16 && VPT <= 2) {
+      const dim3 grid16(static_cast<unsigned>((T + 15) / 16)), block16(256);
+      if (idx_dtype == LO_I64)
+        hipLaunchKernelGGL((moe_fused_gate16_kernel<4 * VPT, DT, BT, int64_t>), grid16, block16, 0, s, x, b, T, E, G, tg,
+                           topk, ns, rsf, scale, w, static_cast<int64_t *>(idx));
+      else
+        hipLaunchKernelGGL((moe_fused_gate16_kernel<4 * VPT, DT, BT, int32_t>), grid16, block16, 0, s, x, b, T, E, G, tg,
+                           topk, ns, rsf, scale, w, static_cast<int32_t *>(idx));
+      return;
+    }
+  }
   const dim3 grid(static_cast<unsigned>((T + 3) / 4)), block(256);
   if (idx_dtype == LO_I64)
     hipLaunchKernelGGL((moe_fused_gate_kernel<VPT, DT, BT, int64_t>), grid, block, 0, s, x, b, T, E, G, tg, topk, ns,
