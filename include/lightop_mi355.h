@@ -380,6 +380,13 @@ int lo_per_token_quant_int8(const void *x, int x_dtype, int64_t rows, int64_t co
  */
 int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, int64_t I, int8_t *q, float *s,
                            const int32_t *num_local_tokens, int32_t top_k, lo_stream_t stream);
+/* The same with the reference's expert_ids argument (fuse_silu_mul_quant.py:45-62, kernel
+ * act_and_mul_quant_kernel_opt1_new, fuse_silu_mul_quant.cu:269-283, dispatch :649-705):
+ * row_expert_ids [rows] int32 or NULL; a row whose entry is -1 (its expert is held by another
+ * rank) is skipped, q and s of that row are left untouched. */
+int lo_fuse_silu_mul_quant_ids(const void *c1, int dtype, int64_t rows, int64_t I, int8_t *q, float *s,
+                               const int32_t *num_local_tokens, int32_t top_k,
+                               const int32_t *row_expert_ids, lo_stream_t stream);
 
 /*
  * One grouped-GEMM stage in the per-channel form.  Replaces

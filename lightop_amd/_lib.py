@@ -72,6 +72,8 @@ SIGNATURES = {
     "lo_per_token_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),
     "lo_fuse_silu_mul_quant": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32,
                                        c_void_p]),
+    "lo_fuse_silu_mul_quant_ids": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32,
+                                           c_void_p, c_void_p]),
     "lo_moe_gemm_w8a8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32,
                                  c_int64, c_int64, c_int32, c_int32, c_int, c_int, c_void_p]),

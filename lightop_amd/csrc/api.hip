@@ -26,6 +26,23 @@ int check_launch(const char *what) {
   return LO_OK;
 }
 
+int reserve_lds_once(const void *kernel, int bytes, unsigned long long *done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    set_error("no current HIP device");
+    return LO_ELAUNCH;
+  }
+  const unsigned long long bit = 1ull << dev;
+  if (__atomic_load_n(done, __ATOMIC_ACQUIRE) & bit) return LO_OK;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    set_error("cannot reserve %d bytes of LDS for a kernel", bytes);
+    return LO_ELAUNCH;
+  }
+  __atomic_fetch_or(done, bit, __ATOMIC_RELEASE);
+  return LO_OK;
+}
+
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 // Extents of the alignment buffers (moe_align_block_size.py:80-93 of the reference).

@@ -39,6 +39,10 @@ int check_launch(const char *what);
 // bf16(silu(g)) for all 65536 bf16 patterns g, built on first use (per device).
 int silu_table(hipStream_t stream, const uint16_t **table);
 
+// Raises a kernel's dynamic-LDS limit once per device instead of on every launch (kernels that use
+// more than the default 64 KB).  `done` is the call site's own static flag set, one bit per device.
+int reserve_lds_once(const void *kernel, int bytes, unsigned long long *done);
+
 #define LO_REQUIRE(cond, code, ...)  \
   do {                               \
     if (!(cond)) {                   \

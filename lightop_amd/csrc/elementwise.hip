@@ -56,7 +56,8 @@ template <bool SILU, int CH>
 __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restrict__ x, int64_t rows, int64_t C,
                                                         const uint16_t *__restrict__ silu, int8_t *__restrict__ q,
                                                         float *__restrict__ s,
-                                                        const int32_t *__restrict__ num_local_tokens, int32_t top_k) {
+                                                        const int32_t *__restrict__ num_local_tokens, int32_t top_k,
+                                                        const int32_t *__restrict__ row_ids) {
   __shared__ float sRed[4];
   __shared__ uint16_t sSilu[SILU ? 2 * kSiluBandN : 2];
   const int tid = threadIdx.x;
@@ -74,6 +75,7 @@ __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restri
   const int64_t in_stride = SILU ? 2 * C : C; // C = output columns
   const int pieces = static_cast<int>(C / 8);
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    if (row_ids && row_ids[row] == -1) continue; // a row of an expert held elsewhere: left untouched
     const uint16_t *xr = x + row * in_stride;
     auto piece = [&](int p, float (&v)[8]) {
       const v8u16 a = *reinterpret_cast<const v8u16 *>(xr + p * 8);
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
                                                              const uint16_t *__restrict__ silu,
                                                              int8_t *__restrict__ q, float *__restrict__ s,
                                                              const int32_t *__restrict__ num_local_tokens,
-                                                             int32_t top_k) {
+                                                             int32_t top_k, const int32_t *__restrict__ row_ids) {
   __shared__ uint16_t sSilu[SILU ? 2 * kSiluBandN : 2];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   if (num_local_tokens) {
@@ -160,6 +162,7 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
   const int64_t in_stride = SILU ? 2 * C : C;
   const int pieces = static_cast<int>(C / 8);
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + wave; row < rows; row += static_cast<int64_t>(gridDim.x) * 4) {
+    if (row_ids && row_ids[row] == -1) continue; // a row of an expert held elsewhere: left untouched
     const uint16_t *xr = x + row * in_stride;
     v8u16 ga[CH], up[CH];
 #pragma unroll
@@ -205,20 +208,20 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
 
 template <bool SILU>
 static void launch_row_quant(const uint16_t *x, int64_t rows, int64_t C, const uint16_t *silu, int8_t *q, float *s,
-                             const int32_t *nlt, int32_t top_k, hipStream_t st) {
+                             const int32_t *nlt, int32_t top_k, const int32_t *row_ids, hipStream_t st) {
   const int pieces = static_cast<int>(C / 8);
   if (pieces <= 256 && rows >= 4) {
     int64_t grid = (rows + 3) / 4;
     if (grid > 256 * 32) grid = 256 * 32;
     const dim3 g(static_cast<unsigned>(grid)), b(256);
-    if (pieces <= 64) hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 1>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k);
-    else if (pieces <= 128) hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 2>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k);
-    else hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 4>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k);
+    if (pieces <= 64) hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 1>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
+    else if (pieces <= 128) hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 2>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
+    else hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 4>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
     return;
   }
   const unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
   hipLaunchKernelGGL((row_quant_kernel<SILU, SILU ? 2 : 4>), dim3(grid), dim3(256), 0, st, x, rows, C, silu, q, s, nlt,
-                     top_k);
+                     top_k, row_ids);
 }
 
 // ---- moe_sum -------------------------------------------------------------------
@@ -427,13 +430,14 @@ extern "C" int lo_per_token_quant_int8(const void *x, int x_dtype, int64_t rows,
   LO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0,
              LO_EINVAL, "per_token_quant_int8: x must be 16-byte and q 8-byte aligned");
   if (rows == 0) return LO_OK;
-  launch_row_quant<false>(static_cast<const uint16_t *>(x), rows, cols, nullptr, q, s, nullptr, 1,
+  launch_row_quant<false>(static_cast<const uint16_t *>(x), rows, cols, nullptr, q, s, nullptr, 1, nullptr,
                           static_cast<hipStream_t>(stream));
   return check_launch("per_token_quant_int8");
 }
 
-extern "C" int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, int64_t I, int8_t *q, float *s,
-                                      const int32_t *num_local_tokens, int32_t top_k, lo_stream_t stream) {
+extern "C" int lo_fuse_silu_mul_quant_ids(const void *c1, int dtype, int64_t rows, int64_t I, int8_t *q, float *s,
+                                          const int32_t *num_local_tokens, int32_t top_k, const int32_t *row_expert_ids,
+                                          lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(c1 && q && s, LO_EINVAL, "fuse_silu_mul_quant: null pointer");
   LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "fuse_silu_mul_quant: only bf16 input is built");
@@ -446,6 +450,11 @@ extern "C" int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, i
   int rc = silu_table(static_cast<hipStream_t>(stream), &table);
   if (rc) return rc;
   launch_row_quant<true>(static_cast<const uint16_t *>(c1), rows, I, table, q, s, num_local_tokens, top_k,
-                         static_cast<hipStream_t>(stream));
+                         row_expert_ids, static_cast<hipStream_t>(stream));
   return check_launch("fuse_silu_mul_quant");
+}
+
+extern "C" int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, int64_t I, int8_t *q, float *s,
+                                      const int32_t *num_local_tokens, int32_t top_k, lo_stream_t stream) {
+  return lo_fuse_silu_mul_quant_ids(c1, dtype, rows, I, q, s, num_local_tokens, top_k, nullptr, stream);
 }

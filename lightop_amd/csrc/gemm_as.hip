@@ -299,12 +299,9 @@ int launch_gemm_as(const GemmArgs &a0, int flags, int block_size_m, int64_t m_bl
 #define LO_AS_LAUNCH(FS, SH)                                                                          \
   do {                                                                                                \
     auto kern = moe_gemm_as_kernel<FS, SH>;                                                           \
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            80 * 1024) != hipSuccess) {                                               \
-      (void)hipGetLastError();                                                                        \
-      set_error("moe_gemm: cannot reserve %zu bytes of LDS", lds);                                    \
-      return LO_ELAUNCH;                                                                              \
-    }                                                                                                 \
+    static unsigned long long lds_done = 0; /* per instantiation: one bit per device */               \
+    const int rc_lds = reserve_lds_once(reinterpret_cast<const void *>(kern), 80 * 1024, &lds_done);  \
+    if (rc_lds) return rc_lds;                                                                        \
     hipLaunchKernelGGL(kern, g, b, lds, s, a, mbi, Gi, n_groups, n_cnt, sub_shift);                   \
   } while (0)
   if (fast) {

@@ -617,11 +617,10 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
 #define LO_T128_LAUNCH(FA, FS, ST, W)                                                                           \
   do {                                                                                                          \
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_gemm_t128_kernel<FA, FS, ST, W>),               \
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kTLds) != hipSuccess) {                 \
-      set_error("moe_gemm(t128): cannot reserve %d bytes of LDS", kTLds);                                       \
-      return LO_ELAUNCH;                                                                                        \
-    }                                                                                                           \
+    static unsigned long long lds_done = 0; /* per instantiation: one bit per device */                         \
+    const int rc_lds = reserve_lds_once(reinterpret_cast<const void *>(&moe_gemm_t128_kernel<FA, FS, ST, W>),    \
+                                        kTLds, &lds_done);                                                      \
+    if (rc_lds) return rc_lds;                                                                                  \
     hipLaunchKernelGGL((moe_gemm_t128_kernel<FA, FS, ST, W>), g, b, kTLds, s, a, mbi, gi);                      \
   } while (0)
 #define LO_T128_PICK(FA, FS)                                                                                    \

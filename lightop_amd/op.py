@@ -136,11 +136,11 @@ def fuse_silu_mul_quant(input: torch.Tensor, output: torch.Tensor, scales: torch
                         expert_ids: Optional[torch.Tensor] = None) -> None:
     """``op.fuse_silu_mul_quant`` (export.cpp:1532; fuse_silu_mul_quant.cu:90-199): SiLU(gate) * up of
     ``input`` [rows, 2d], then one int8 scale per row: ``output`` [rows, d] int8, ``scales`` [rows(, 1)] f32.
-    With ``num_local_tokens_tensor`` (device int32[1]) only the first ``n * topk`` rows are processed."""
+    With ``num_local_tokens_tensor`` (device int32[1]) only the first ``n * topk`` rows are processed; with
+    ``expert_ids`` (int32 [rows]; fuse_silu_mul_quant.cu:269-283) rows whose entry is -1 are skipped and their
+    ``output`` / ``scales`` left untouched."""
     del expect_m
-    if expert_ids is not None:
-        raise NotImplementedError("lightop_amd.op.fuse_silu_mul_quant: the expert_ids variant is not built")
-    _require_cuda(input, output, scales, num_local_tokens_tensor)
+    _require_cuda(input, output, scales, num_local_tokens_tensor, expert_ids)
     if input.dim() != 2 or not input.is_contiguous() or input.shape[1] % 16:
         raise RuntimeError("lightop_amd.op.fuse_silu_mul_quant: input must be a contiguous [rows, 2*d] tensor, d % 8 == 0")
     rows, d = input.shape[0], input.shape[1] // 2
@@ -151,10 +151,14 @@ def fuse_silu_mul_quant(input: torch.Tensor, output: torch.Tensor, scales: torch
     if num_local_tokens_tensor is not None and (num_local_tokens_tensor.dtype != torch.int32
                                                 or num_local_tokens_tensor.numel() < 1):
         raise RuntimeError("lightop_amd.op.fuse_silu_mul_quant: num_local_tokens_tensor must be int32 with one element")
+    if expert_ids is not None and (expert_ids.dtype != torch.int32 or not expert_ids.is_contiguous()
+                                   or expert_ids.numel() < rows):
+        raise RuntimeError("lightop_amd.op.fuse_silu_mul_quant: expert_ids must be a contiguous int32 tensor with one "
+                           "entry per row")
     with _on_device(input):
-        _lib.check(_lib.lib().lo_fuse_silu_mul_quant(_lib.ptr(input), _act_dtype(input), rows, d, _lib.ptr(output),
-                                                     _lib.ptr(scales), _lib.ptr(num_local_tokens_tensor), int(topk),
-                                                     _lib.stream_of(input)))
+        _lib.check(_lib.lib().lo_fuse_silu_mul_quant_ids(_lib.ptr(input), _act_dtype(input), rows, d, _lib.ptr(output),
+                                                         _lib.ptr(scales), _lib.ptr(num_local_tokens_tensor), int(topk),
+                                                         _lib.ptr(expert_ids), _lib.stream_of(input)))
 
 
 def _float_dtype(t: torch.Tensor, what: str) -> int:

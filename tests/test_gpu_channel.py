@@ -71,6 +71,27 @@ def test_fuse_silu_mul_quant_bit_exact(dev, oracle, rows, I):
         assert torch.equal(out.cpu()[:2], rq[:2]) and (out.cpu()[2:] == 77).all() and (sc.cpu()[2:] == -1).all()
 
 
+def test_fuse_silu_mul_quant_skips_rows_of_other_ranks(dev, oracle):
+    """expert_ids (fuse_silu_mul_quant.cu:269-283): rows marked -1 keep whatever output and scales held."""
+    from lightop_amd import fuse_silu_mul_quant
+
+    for rows, I in ((37, 768), (9, 4096)):  # one wavefront per row, one workgroup per row
+        say(f"fuse_silu_mul_quant expert_ids rows={rows} I={I}")
+        g = torch.Generator().manual_seed(rows)
+        c1 = torch.randn(rows, 2 * I, generator=g).to(torch.bfloat16)
+        eids = torch.randint(-1, 3, (rows,), generator=g, dtype=torch.int32)
+        eids[1], eids[rows - 1], eids[0] = -1, -1, 2
+        rq, rs = oracle.fuse_silu_mul_quant(c1)
+        out = torch.full((rows, I), 77, dtype=torch.int8, device=dev)
+        sc = torch.full((rows, 1), -5.0, dtype=torch.float32, device=dev)
+        fuse_silu_mul_quant(c1.to(dev), None, 1, -1, out, sc, eids.to(dev))
+        torch.cuda.synchronize()
+        keep = eids != -1
+        assert keep.any() and (~keep).any()
+        assert torch.equal(out.cpu()[keep], rq[keep]) and torch.equal(sc.cpu()[keep].view(torch.int32), rs[keep].view(torch.int32).reshape(-1, 1))
+        assert (out.cpu()[~keep] == 77).all() and (sc.cpu()[~keep] == -5.0).all()
+
+
 def gemm_case(seed, M, k, E, Eg, N, K):
     g = torch.Generator().manual_seed(seed)
     Aq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8)
