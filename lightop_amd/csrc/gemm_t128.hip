@@ -245,16 +245,17 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[h][tb][rf][i] = 0.0f;
 
-  // W4: every product carries the factor 16 of the unpacked nibbles; the canonical order takes it out
-  // of the exact int32 sum with a shift, the fused order puts 1/16 into the row scale (a power of
-  // two: the same value unless the scale is denormal).  One scale per weight row: bs4[i] for row 4q + i.
+  // W4: every product carries the factor 16 of the unpacked nibbles; it is taken out through the row
+  // scale, which read_w() multiplies by 1/16 once per K block (a power of two: (f32(d) * a_s) * (b_s / 16)
+  // is bit for bit (f32(d / 16) * a_s) * b_s unless b_s lies below 2^-122 or the product above 2^124).
+  // One scale per weight row: bs4[i] for row 4q + i.
   auto fold4 = [&](const v4i &d, float as, const v4f &bs4, float *dst) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if constexpr (FAST_SCALE) {
         dst[i] = __builtin_fmaf(static_cast<float>(d[i]), as * bs4[i], dst[i]); // bs4 already holds scale / 16
       } else {
-        float t = static_cast<float>(d[i] >> 4) * as;
+        float t = static_cast<float>(d[i]) * as;
         t = t * bs4[i];
         dst[i] = dst[i] + t;
       }
@@ -299,7 +300,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
           // rows of fragment (h, rf) among the wave's 64: fused 32*rf + 16*h, plain 32*h + 16*rf
           const int row0 = (FUSED_ACT ? 32 * rf + 16 * h : 32 * h + 16 * rf) + 4 * q;
           wsc[h][rf] = *reinterpret_cast<const v4f *>(sWw + 4096 + row0 * 4);
-          if constexpr (FAST_SCALE) wsc[h][rf] = wsc[h][rf] * 0.0625f;
+          wsc[h][rf] = wsc[h][rf] * 0.0625f;
         }
     } else {
 #pragma unroll

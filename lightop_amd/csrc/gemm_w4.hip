@@ -148,9 +148,9 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
       bsreg[b][rf] = __builtin_bit_cast(v4f, bld16(rWs, wsoff[rf], kc * static_cast<int>(N) * 4));
   };
   auto fold = [&](const v4i (&d)[4], const v4f &bs, const float (&as)[4], v4f (&dst)[4]) {
-    // every product carries the factor 16 of the unpacked nibbles: the canonical order takes it
-    // out of the exact int32 sum with a shift, the fused order puts 1/16 into the row scale
-    // (a power of two: the same value unless the scale is denormal)
+    // every product carries the factor 16 of the unpacked nibbles: 1/16 goes into the row scale (a
+    // power of two: (f32(d) * a_s) * (b_s / 16) is bit for bit (f32(d / 16) * a_s) * b_s unless b_s
+    // lies below 2^-122 or the product above 2^124)
     v4f bs16;
 #pragma unroll
     for (int i = 0; i < 4; ++i) bs16[i] = bs[i] * 0.0625f;
@@ -161,8 +161,8 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
         if constexpr (FAST_SCALE) {
           dst[tf][i] = __builtin_fmaf(static_cast<float>(d[tf][i]), as[tf] * bs16[i], dst[tf][i]);
         } else {
-          float t = static_cast<float>(d[tf][i] >> 4) * as[tf];
-          t = t * bs[i];
+          float t = static_cast<float>(d[tf][i]) * as[tf];
+          t = t * bs16[i];
           dst[tf][i] = dst[tf][i] + t;
         }
       }

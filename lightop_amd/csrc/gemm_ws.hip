@@ -231,10 +231,6 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
 #pragma unroll
           for (int ks = 0; ks < 2; ++ks)
             d[g][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop[ks], abuf[p][j][ks], d[g][j], 0, 0, 0);
-          if constexpr (W4) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) d[g][j][i] >>= 4; // exact: every product carries the factor 16
-          }
         }
       }
       float bs[NW][NS], as[TM];
@@ -247,6 +243,11 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
             bs[g][NS > 1 ? 1 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0x55, 0xf, 0xf, false));
             bs[g][NS > 2 ? 2 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0xaa, 0xf, 0xf, false));
             bs[g][NS > 3 ? 3 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0xff, 0xf, 0xf, false));
+            // every product carries the factor 16 of the unpacked nibbles: 1/16 goes into the row scales (a
+            // power of two: (f32(d) * a_s) * (b_s / 16) is bit for bit (f32(d / 16) * a_s) * b_s unless b_s
+            // lies below 2^-122 or the product above 2^124)
+#pragma unroll
+            for (int i = 0; i < NS; ++i) bs[g][i] = bs[g][i] * 0.0625f;
           } else {
             bs[g][0] = bsbuf[p][g][0];
           }
