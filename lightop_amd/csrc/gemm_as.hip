@@ -17,7 +17,12 @@ namespace lo {
 
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-template <bool FAST_SCALE, bool SHUF>
+// KBT: K / 128 as a compile-time constant (a multiple of three, so that a tile starts on ring buffer 0),
+// or 0 for any K.  With it a tile's steps and its stores are straight-line code: the compiler then
+// knows how many memory operations follow each weight load and waits for exactly those; in the
+// general form the stores sit in a branch, the wait counts assume they did not happen, and after
+// every tile the wave waits for loads it has only just issued.
+template <bool FAST_SCALE, bool SHUF, int KBT = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
                                                           int n_groups, int n_cnt, int sub_shift) {
@@ -257,10 +262,32 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
   }
   __syncthreads(); // the only barrier: the token block is complete
   zero_acc();
-  for (int s = 0; s < total; s += 3) {
-    step(B0{}, B2{});
-    step(B1{}, B0{});
-    step(B2{}, B1{});
+  if constexpr (KBT > 0) {
+    static_assert(KBT % 3 == 0, "a tile must start on ring buffer 0");
+    for (int nt = nt0; nt < nt_end; ++nt) {
+#pragma unroll
+      for (int kb = 0; kb < KBT; ++kb) {
+        // the step two ahead: this tile's, or the next tile's first two (the last tile re-reads its end)
+        const bool wrap = kb + 2 >= KBT;
+        const bool past = wrap && nt + 1 >= nt_end;
+        const int lnt = past ? nt : (wrap ? nt + 1 : nt), lkb = past ? KBT - 1 : (wrap ? kb + 2 - KBT : kb + 2);
+        if (kb % 3 == 0) load_w(B2{}, lnt, lkb);
+        else if (kb % 3 == 1) load_w(B0{}, lnt, lkb);
+        else load_w(B1{}, lnt, lkb);
+        __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMAs
+        if (kb % 3 == 0) compute(B0{}, kb, true);
+        else if (kb % 3 == 1) compute(B1{}, kb, true);
+        else compute(B2{}, kb, true);
+      }
+      store_tile(nt);
+      zero_acc();
+    }
+  } else {
+    for (int s = 0; s < total; s += 3) {
+      step(B0{}, B2{});
+      step(B1{}, B0{});
+      step(B2{}, B1{});
+    }
   }
 }
 
@@ -298,7 +325,12 @@ int launch_gemm_as(const GemmArgs &a0, int flags, int block_size_m, int64_t m_bl
   const int mbi = static_cast<int>(m_blocks), Gi = static_cast<int>(G);
 #define LO_AS_LAUNCH(FS, SH)                                                                          \
   do {                                                                                                \
-    auto kern = moe_gemm_as_kernel<FS, SH>;                                                           \
+    if (a.K == 6 * kGroup) LO_AS_LAUNCH_K(FS, SH, 6);                                                 \
+    else LO_AS_LAUNCH_K(FS, SH, 0);                                                                   \
+  } while (0)
+#define LO_AS_LAUNCH_K(FS, SH, KBT)                                                                   \
+  do {                                                                                                \
+    auto kern = moe_gemm_as_kernel<FS, SH, KBT>;                                                      \
     static unsigned long long lds_done = 0; /* per instantiation: one bit per device */               \
     const int rc_lds = reserve_lds_once(reinterpret_cast<const void *>(kern), 80 * 1024, &lds_done);  \
     if (rc_lds) return rc_lds;                                                                        \
@@ -312,6 +344,7 @@ int launch_gemm_as(const GemmArgs &a0, int flags, int block_size_m, int64_t m_bl
     else LO_AS_LAUNCH(false, false);
   }
 #undef LO_AS_LAUNCH
+#undef LO_AS_LAUNCH_K
   return check_launch("moe_gemm(activation-stationary)");
 }
 
