@@ -36,7 +36,6 @@ namespace lo {
 
 constexpr int kDecTP = 4;     // token rows the first kernel multiplies per pass
 constexpr int kDecMaxKBw = 7; // K blocks per wave of the first kernel (all held in registers)
-constexpr int kDecPD = 8;     // weight K blocks in flight per wave of the second kernel
 constexpr int kDecMaxSlots = 512;
 constexpr int kDecMaxKB2 = 32;  // K blocks of the second kernel (I <= 4096): its activation row is held in registers
 
@@ -90,7 +89,8 @@ __device__ __forceinline__ float lane_value(float v, int l) {
 // long as the streaming itself at these sizes, so everything whose address does not depend on the
 // routing is requested before the routing is looked at, and everything that depends on the expert
 // only is requested the moment the expert is known.
-__global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
+template <int KBW> // K blocks a wave holds in registers at most: 4, or kDecMaxKBw
+__device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -105,8 +105,8 @@ __global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
   int32_t *const sSlots = reinterpret_cast<int32_t *>(smem);                    // [S rounded up to 4]
   int32_t *const sMeta = sSlots + ((a.S + 3) & ~3);                             // [4]
   float *const sT = reinterpret_cast<float *>(sMeta + 4);                       // [KB][8 values][4 c][TP tokens]
-  float *const sAs = sT + KB * 128 + wave * (kDecTP * kDecMaxKBw);              // [TP][KBw] of this wave
-  int8_t *const sA = reinterpret_cast<int8_t *>(sT + KB * 128 + W * (kDecTP * kDecMaxKBw)) + wave * (kDecTP * pitch);
+  float *const sAs = sT + KB * 128 + wave * (kDecTP * KBW);              // [TP][KBw] of this wave
+  int8_t *const sA = reinterpret_cast<int8_t *>(sT + KB * 128 + W * (kDecTP * KBW)) + wave * (kDecTP * pitch);
 
   // ---- requests that do not wait for the routing: the slot's own token row ----------------------
   const int sub = lane & 15, gq = lane >> 4;
@@ -120,18 +120,18 @@ __global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
       if (g < KBw) raw_own[q] = *reinterpret_cast<const v8u16 *>(a.x + t * a.H + (kb0 + g) * kGroup + sub * 8);
     }
   }
-  // (wave 0) every slot's expert id, for the search below
-  int32_t gid[kDecMaxSlots / 64]; // (expert ids fit 32 bits: anything else is no expert at all)
+  // (wave 0) the expert ids of the first 128 slots, for the search below (further slots, which only a
+  // forced call has, are fetched when the search gets there)
+  auto slot_gid = [&](int i) __attribute__((always_inline)) -> int32_t {
+    // (expert ids fit 32 bits: anything else is no expert at all)
+    if (i >= a.S) return -1;
+    const int64_t g = a.ids64 ? static_cast<const int64_t *>(a.ids)[i] : static_cast<const int32_t *>(a.ids)[i];
+    return g >= 0 && g < a.Eg ? static_cast<int32_t>(g) : -1;
+  };
+  int32_t gid[2] = {-1, -1};
   if (wave == 0) {
-#pragma unroll
-    for (int b = 0; b < kDecMaxSlots / 64; ++b) {
-      const int i = b * 64 + lane;
-      gid[b] = -1;
-      if (i < a.S) {
-        const int64_t g = a.ids64 ? static_cast<const int64_t *>(a.ids)[i] : static_cast<const int32_t *>(a.ids)[i];
-        gid[b] = g >= 0 && g < a.Eg ? static_cast<int32_t>(g) : -1;
-      }
-    }
+    gid[0] = slot_gid(lane);
+    gid[1] = slot_gid(64 + lane);
   }
 
   int64_t g0;
@@ -146,10 +146,10 @@ __global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
   int woff[2];
   woff[0] = rb * shuf_nb_stride(KB) + lane * 16;
   woff[1] = (I / 16 + rb) * shuf_nb_stride(KB) + lane * 16;
-  v4i wbuf[kDecMaxKBw][2][2];
+  v4i wbuf[KBW][2][2];
   auto issue_all = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int p = 0; p < kDecMaxKBw; ++p)
+    for (int p = 0; p < KBW; ++p)
       if (p < KBw) {
 #pragma unroll
         for (int g = 0; g < 2; ++g)
@@ -167,14 +167,12 @@ __global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
   // ---- slots routed to the same expert, ascending; the workgroup of the first one serves them ---
   if (wave == 0) {
     int cnt = 0;
-#pragma unroll
-    for (int b = 0; b < kDecMaxSlots / 64; ++b) {
-      if (b * 64 < a.S) {
-        const bool mine = gid[b] == static_cast<int32_t>(g0); // (slots past S hold -1, 0 <= g0 < Eg)
-        const uint64_t bal = __builtin_amdgcn_ballot_w64(mine);
-        if (mine) sSlots[cnt + __builtin_popcountll(bal & ((1ull << lane) - 1))] = b * 64 + lane;
-        cnt += __builtin_popcountll(bal);
-      }
+    for (int b = 0; b * 64 < a.S; ++b) {
+      const int32_t gb = b == 0 ? gid[0] : (b == 1 ? gid[1] : slot_gid(b * 64 + lane));
+      const bool mine = gb == static_cast<int32_t>(g0); // (slots past S hold -1, 0 <= g0 < Eg)
+      const uint64_t bal = __builtin_amdgcn_ballot_w64(mine);
+      if (mine) sSlots[cnt + __builtin_popcountll(bal & ((1ull << lane) - 1))] = b * 64 + lane;
+      cnt += __builtin_popcountll(bal);
     }
     if (lane == 0) sMeta[0] = cnt;
   }
@@ -205,7 +203,7 @@ __global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
         float sc;
         const v2i packed = dec_quant8(raw, sc);
         *reinterpret_cast<v2i *>(sA + tokl * pitch + kbl * kGroup + sub * 8) = packed;
-        if (sub == 0) sAs[tokl * kDecMaxKBw + kbl] = sc;
+        if (sub == 0) sAs[tokl * KBW + kbl] = sc;
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -213,14 +211,14 @@ __global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
     // ---- one term per K block: weights from registers, tokens from LDS; the terms of the pass's
     //      tokens go to LDS, K block by K block -----------------------------------------------------
 #pragma unroll
-    for (int p = 0; p < kDecMaxKBw; ++p) {
+    for (int p = 0; p < KBW; ++p) {
       if (p < KBw) {
         v4i b0 = v4i{0, 0, 0, 0}, b1 = v4i{0, 0, 0, 0};
         float as = 0.0f;
         if (n < nc) {
           b0 = *reinterpret_cast<const v4i *>(sA + n * pitch + p * kGroup + c * 16);
           b1 = *reinterpret_cast<const v4i *>(sA + n * pitch + p * kGroup + 64 + c * 16);
-          as = sAs[n * kDecMaxKBw + p];
+          as = sAs[n * KBW + p];
         }
         const float bs[2] = {lane_value(bs_l, p), lane_value(bs_l, 8 + p)};
 #pragma unroll
@@ -245,15 +243,15 @@ __global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
     if (wave == W - 1) {
       float accg = 0.0f, accu = 0.0f;
       int kb = 0;
-      for (; kb + 8 <= KB; kb += 8) {
-        float tg[8], tu[8];
+      for (; kb + 4 <= KB; kb += 4) {
+        float tg[4], tu[4];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < 4; ++j) {
           tg[j] = sT[(kb + j) * 128 + lane];
           tu[j] = sT[(kb + j) * 128 + 64 + lane];
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < 4; ++j) {
           accg = accg + tg[j];
           accu = accu + tu[j];
         }
@@ -277,6 +275,14 @@ __global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) {
   }
 }
 
+// Up to four K blocks per wave: half the registers, so four waves per SIMD (twice the workgroups in
+// flight per compute unit) instead of two.
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void dec_gemm1_small_kernel(const DecArgs a) {
+  dec_gemm1_body<4>(a);
+}
+__global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) { dec_gemm1_body<kDecMaxKBw>(a); }
+
+template <int PD, int RAWN> // weight K blocks in flight per wave; 16-byte pieces of the activation row per lane
 __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -296,9 +302,9 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
   for (int j = wave; j < k; j += W) {
     const int s = t * k + j;
     // the slot's activation row and routed weight do not wait for the routing
-    v8u16 raw[kDecMaxKB2 / 4];
+    v8u16 raw[RAWN];
 #pragma unroll
-    for (int q = 0; q < kDecMaxKB2 / 4; ++q) {
+    for (int q = 0; q < RAWN; ++q) {
       raw[q] = v8u16{0, 0, 0, 0, 0, 0, 0, 0};
       if (gq + 4 * q < KB)
         raw[q] = *reinterpret_cast<const v8u16 *>(a.act + static_cast<int64_t>(s) * I + (gq + 4 * q) * kGroup + sub * 8);
@@ -312,9 +318,9 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
     const brsrc rW = make_rsrc(a.w2 + static_cast<int64_t>(e) * H * I, static_cast<uint32_t>(static_cast<int64_t>(H) * I));
     const int wkstride = shuf_kb_stride(H / 16);
     const int woff = rb * shuf_nb_stride(KB) + lane * 16;
-    v4i wbuf[kDecPD][2];
+    v4i wbuf[PD][2];
 #pragma unroll
-    for (int p = 0; p < kDecPD; ++p)
+    for (int p = 0; p < PD; ++p)
       if (p < KB) {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) wbuf[p][ks] = bld16<kCacheStream>(rW, woff, p * wkstride + ks * 1024);
@@ -324,7 +330,7 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
 
     // the activation row, re-quantised in 1x128 groups, into the wave's LDS row
 #pragma unroll
-    for (int q = 0; q < kDecMaxKB2 / 4; ++q) {
+    for (int q = 0; q < RAWN; ++q) {
       const int gi = gq + 4 * q;
       if (gi < KB) {
         float sc;
@@ -336,9 +342,9 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
     __builtin_amdgcn_wave_barrier();
 
     v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
-    for (int kb0 = 0; kb0 < KB; kb0 += kDecPD) {
+    for (int kb0 = 0; kb0 < KB; kb0 += PD) {
 #pragma unroll
-      for (int p = 0; p < kDecPD; ++p) {
+      for (int p = 0; p < PD; ++p) {
         const int kb = kb0 + p;
         if (kb < KB) {
           // every column of the token operand is the same row: all lanes end up with valid sums
@@ -346,10 +352,10 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
           const v4i b1 = *reinterpret_cast<const v4i *>(sA + kb * kGroup + 64 + c * 16);
           v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[p][0], b0, v4i{0, 0, 0, 0}, 0, 0, 0);
           d = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[p][1], b1, d, 0, 0, 0);
-          if (kb + kDecPD < KB) {
+          if (kb + PD < KB) {
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
-              wbuf[p][ks] = bld16<kCacheStream>(rW, woff, (kb + kDecPD) * wkstride + ks * 1024);
+              wbuf[p][ks] = bld16<kCacheStream>(rW, woff, (kb + PD) * wkstride + ks * 1024);
           }
           const float as = sAs[kb], bs = lane_value(bs_l, kb);
 #pragma unroll
@@ -426,10 +432,13 @@ bool decode_path_applies(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_t
   const int forced = decode_max_slots();
   if (forced >= 0) return S <= forced;
   // measured on both benchmark layers (top-8 routing): well ahead of the five-stage path at one and
-  // two tokens, level with it or just ahead at four, behind from eight on (its workgroups hold their
-  // whole share of the weights in registers and live too briefly to overlap one another)
+  // two tokens, ahead at four; at eight only where a wave holds at most four K blocks (the first
+  // kernel then fits four waves per SIMD: Qwen3 layer 62 against 67 us, DeepSeek share 114 against
+  // 78 us); behind from sixteen on: its workgroups hold their whole share of the weights in
+  // registers and live too briefly to overlap one another
   (void)num_experts;
-  return S <= 32;
+  const int KB = static_cast<int>(H / kGroup);
+  return S <= 32 || (S <= 64 && KB / pick_waves(KB) <= 4);
 }
 
 void decode_path_waves(int32_t top_k, int64_t H, int *gemm1_waves, int *gemm2_waves) {
@@ -467,10 +476,15 @@ int launch_decode_path(const void *x, int64_t M, int64_t H, int64_t I, int32_t E
                     static_cast<size_t>(W2) * I;
   if (l1 > 64 * 1024 || l2 > 64 * 1024) return LO_ENOTSUP;
   const dim3 g1(static_cast<unsigned>(I / 16), static_cast<unsigned>(S)), g2(static_cast<unsigned>(H / 16), static_cast<unsigned>(M));
-  hipLaunchKernelGGL(dec_gemm1_kernel, g1, dim3(64 * W1), l1, stream, a);
+  // fewer registers where the shape allows it: more workgroups in flight per compute unit
+  if (a.kbw <= 4) hipLaunchKernelGGL(dec_gemm1_small_kernel, g1, dim3(64 * W1), l1, stream, a);
+  else hipLaunchKernelGGL(dec_gemm1_kernel, g1, dim3(64 * W1), l1, stream, a);
   const int rc = check_launch("fused_experts(decode, gemm1)");
   if (rc) return rc;
-  hipLaunchKernelGGL(dec_gemm2_kernel, g2, dim3(64 * W2), l2, stream, a);
+  if (KB2 <= 6) hipLaunchKernelGGL((dec_gemm2_kernel<6, 2>), g2, dim3(64 * W2), l2, stream, a);
+  else if (KB2 <= 8) hipLaunchKernelGGL((dec_gemm2_kernel<8, 2>), g2, dim3(64 * W2), l2, stream, a);
+  else if (KB2 <= 16) hipLaunchKernelGGL((dec_gemm2_kernel<8, 4>), g2, dim3(64 * W2), l2, stream, a);
+  else hipLaunchKernelGGL((dec_gemm2_kernel<8, 8>), g2, dim3(64 * W2), l2, stream, a);
   return check_launch("fused_experts(decode, gemm2)");
 }
 

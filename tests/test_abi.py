@@ -106,8 +106,10 @@ def test_tile_query_names_the_kernel_that_is_launched(lib):
     assert q(_lib.LO_FORM_BLOCK, pre, 4, *dsv3) == 0 and (t1.kernel, t1.waves) == (_lib.LO_KERNEL_DEC, 8)
     assert q(_lib.LO_FORM_BLOCK, pre | _lib.LO_FUSED_NO_DECODE_PATH, 1, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_WS
     assert q(_lib.LO_FORM_BLOCK, 0, 1, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_WS  # row-major weights
-    assert q(_lib.LO_FORM_BLOCK, pre, 8, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_WS
-    assert q(_lib.LO_FORM_BLOCK, pre | _lib.LO_FUSED_FORCE_DECODE_PATH, 8, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_DEC
+    assert q(_lib.LO_FORM_BLOCK, pre, 8, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_DEC  # four K blocks per wave
+    assert q(_lib.LO_FORM_BLOCK, pre, 8, *dsv3) == 0 and t1.kernel == _lib.LO_KERNEL_WS   # seven: up to four tokens
+    assert q(_lib.LO_FORM_BLOCK, pre, 16, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_WS
+    assert q(_lib.LO_FORM_BLOCK, pre | _lib.LO_FUSED_FORCE_DECODE_PATH, 16, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_DEC
     # prefill, load-time layout: 128-token direct-to-LDS kernel for GEMM1, activation-stationary GEMM2 on a short K
     assert q(_lib.LO_FORM_BLOCK, pre, 8192, *qwen) == 0
     assert (t1.block_size_m, t1.kernel, t1.waves, t1.block_n) == (128, _lib.LO_KERNEL_T128, 4, 256)
