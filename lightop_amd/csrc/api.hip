@@ -159,8 +159,8 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
     describe_gemm_kernel(pick_gemm_kernel(a, false, bm, flags), false, bm, gemm2);
   }
   // a few tokens: the whole-path call serves the block form with its two-launch path
-  if (form == LO_FORM_BLOCK && pre && !(flags & LO_FUSED_NO_DECODE_PATH) && M > 0 &&
-      decode_path_applies(M, top_k, H, I, num_experts, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0)) {
+  if ((form == LO_FORM_BLOCK || form == LO_FORM_W4) && pre && !(flags & LO_FUSED_NO_DECODE_PATH) && M > 0 &&
+      decode_path_applies(M, top_k, H, I, num_experts, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0, form == LO_FORM_W4)) {
     int w1 = 0, w2 = 0;
     decode_path_waves(top_k, H, &w1, &w2);
     if (gemm1) { gemm1->kernel = LO_KERNEL_DEC; gemm1->waves = w1; gemm1->block_n = 16; }
@@ -242,11 +242,12 @@ extern "C" int lo_fused_experts_block_int8(
   const int64_t S = M * top_k;
 
   // Decode sizes: routing, quantisation, both GEMMs and the reduction in two launches.
-  if (block_size_m_auto && (flags & LO_GEMM_W_PRESHUFFLED) && !(flags & (LO_GEMM_W4 | LO_FUSED_NO_DECODE_PATH))) {
+  if (block_size_m_auto && (flags & (LO_GEMM_W_PRESHUFFLED | LO_GEMM_W4)) && !(flags & LO_FUSED_NO_DECODE_PATH)) {
     // (cache3 is the front of the caller's cache13: the path keeps its bf16 activations [S, I] there)
     const int rc2 = launch_decode_path(x, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w, topk_ids, ids_dtype,
                                        expert_map, apply_router_weight_on_input, routed_scaling_factor, shared_output,
-                                       cache3, out, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0, static_cast<hipStream_t>(stream));
+                                       cache3, out, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0, (flags & LO_GEMM_W4) != 0,
+                                       static_cast<hipStream_t>(stream));
     if (rc2 != LO_ENOTSUP) return rc2;
   }
 

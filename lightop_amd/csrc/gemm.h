@@ -127,13 +127,13 @@ int pick_gemm_kernel(const GemmArgs &a, bool fused_act, int block_size_m, int fl
 void describe_gemm_kernel(int kernel, bool fused_act, int block_size_m, lo_moe_tile *t);
 
 // Decode-size whole path in two launches (gemm_dec.hip): LO_ENOTSUP when it does not apply.
-// act: room for [M * top_k, I] bf16.
-bool decode_path_applies(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_t num_experts, bool force);
+// act: room for [M * top_k, I] bf16.  w4: packed int4 weights with K-group scales [E, K/128, N].
+bool decode_path_applies(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_t num_experts, bool force, bool w4);
 void decode_path_waves(int32_t top_k, int64_t H, int *gemm1_waves, int *gemm2_waves);
 int launch_decode_path(const void *x, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts, int32_t top_k,
                        const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s, const float *topk_w,
                        const void *topk_ids, int ids_dtype, const int32_t *expert_map, int apply_router_weight_on_input,
-                       float factor, const void *shared_output, void *act, void *out, bool force, hipStream_t stream);
+                       float factor, const void *shared_output, void *act, void *out, bool force, bool w4, hipStream_t stream);
 
 // Weight-streaming kernels (gemm_ws.hip): block_size_m in {16, 32, 64, 128}.
 int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,

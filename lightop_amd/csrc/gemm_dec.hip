@@ -81,6 +81,19 @@ __device__ __forceinline__ v2i dec_quant8(const v8u16 raw, float &scale) {
   return packed;
 }
 
+// The two MFMA operands (k-steps) of a K block from a lane's 16 bytes of packed int4 in the load-time
+// layout: int8 values 16 times too large (reference nibble order: layers/fused_moe/w4a8.py:341, :375-377).
+__device__ __forceinline__ void unpack_int4(const v4i pk, v4i &w0, v4i &w1) {
+#pragma unroll
+  for (int x = 0; x < 2; ++x) {
+    const uint32_t a0 = static_cast<uint32_t>(pk[x]), a1 = static_cast<uint32_t>(pk[2 + x]);
+    w0[2 * x] = static_cast<int>((a0 << 4) & 0xf0f0f0f0u);
+    w0[2 * x + 1] = static_cast<int>(a0 & 0xf0f0f0f0u);
+    w1[2 * x] = static_cast<int>((a1 << 4) & 0xf0f0f0f0u);
+    w1[2 * x + 1] = static_cast<int>(a1 & 0xf0f0f0f0u);
+  }
+}
+
 __device__ __forceinline__ float lane_value(float v, int l) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
 }
@@ -89,7 +102,10 @@ __device__ __forceinline__ float lane_value(float v, int l) {
 // long as the streaming itself at these sizes, so everything whose address does not depend on the
 // routing is requested before the routing is looked at, and everything that depends on the expert
 // only is requested the moment the expert is known.
-template <int KBW> // K blocks a wave holds in registers at most: 4, or kDecMaxKBw
+// KBW: K blocks a wave holds in registers at most (4, or kDecMaxKBw).  W4: packed int4 weights in their
+// load-time layout (one 16-byte piece per lane holds both k-steps of a K block) with one scale per weight
+// row and K block, [E, K/128, N]; the factor 16 of the unpacked nibbles leaves through the scales.
+template <int KBW, bool W4>
 __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -141,28 +157,42 @@ __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
   // ---- the wave's weights: its K blocks of 16 gate rows and of the matching 16 up rows.  Requested
   //      before it is known whether this workgroup is the one that serves the expert: the path is
   //      meant for batches in which two slots rarely meet on an expert. -----------------------------
-  const brsrc rW = make_rsrc(a.w1 + static_cast<int64_t>(e) * N * a.H, static_cast<uint32_t>(static_cast<int64_t>(N) * a.H));
-  const int wkstride = shuf_kb_stride(N / 16);
-  int woff[2];
-  woff[0] = rb * shuf_nb_stride(KB) + lane * 16;
-  woff[1] = (I / 16 + rb) * shuf_nb_stride(KB) + lane * 16;
-  v4i wbuf[KBW][2][2];
+  const int64_t wbytes = W4 ? static_cast<int64_t>(N) * a.H / 2 : static_cast<int64_t>(N) * a.H;
+  const brsrc rW = make_rsrc(a.w1 + static_cast<int64_t>(e) * wbytes, static_cast<uint32_t>(wbytes));
+  const brsrc rWs = make_rsrc(a.w1s + static_cast<int64_t>(e) * KB * N, static_cast<uint32_t>(W4 ? static_cast<int64_t>(KB) * N * 4 : 0));
+  const int wkstride = W4 ? shuf_kb_stride(N / 16) / 2 : shuf_kb_stride(N / 16);
+  const int wnstride = W4 ? shuf_nb_stride(KB) / 2 : shuf_nb_stride(KB);
+  int woff[2], wsoff[2];
+  woff[0] = rb * wnstride + lane * 16;
+  woff[1] = (I / 16 + rb) * wnstride + lane * 16;
+  wsoff[0] = (rb * 16 + 4 * c) * 4; // W4: the scales of the lane's four gate rows, then of its four up rows
+  wsoff[1] = (I + rb * 16 + 4 * c) * 4;
+  v4i wbuf[KBW][2][W4 ? 1 : 2];
+  v4f wsc[W4 ? KBW : 1][2];
   auto issue_all = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int p = 0; p < KBW; ++p)
       if (p < KBw) {
 #pragma unroll
-        for (int g = 0; g < 2; ++g)
+        for (int g = 0; g < 2; ++g) {
+          if constexpr (W4) {
+            wbuf[p][g][0] = bld16<kCacheStream>(rW, woff[g], (kb0 + p) * wkstride);
+            wsc[p][g] = __builtin_bit_cast(v4f, bld16(rWs, wsoff[g], (kb0 + p) * N * 4));
+          } else {
 #pragma unroll
-          for (int ks = 0; ks < 2; ++ks)
-            wbuf[p][g][ks] = bld16<kCacheStream>(rW, woff[g], (kb0 + p) * wkstride + ks * 1024);
+            for (int ks = 0; ks < 2; ++ks)
+              wbuf[p][g][ks] = bld16<kCacheStream>(rW, woff[g], (kb0 + p) * wkstride + ks * 1024);
+          }
+        }
       }
   };
   issue_all();
   // block scales of the wave's K range: lanes 0..7 the gate rows', lanes 8..15 the up rows'
   float bs_l = 0.0f;
-  if (lane < 16 && (lane & 7) < KBw)
-    bs_l = a.w1s[(static_cast<int64_t>(e) * (N / kGroup) + (lane >> 3) * (I / kGroup) + rb / 8) * KB + kb0 + (lane & 7)];
+  if constexpr (!W4) {
+    if (lane < 16 && (lane & 7) < KBw)
+      bs_l = a.w1s[(static_cast<int64_t>(e) * (N / kGroup) + (lane >> 3) * (I / kGroup) + rb / 8) * KB + kb0 + (lane & 7)];
+  }
 
   // ---- slots routed to the same expert, ascending; the workgroup of the first one serves them ---
   if (wave == 0) {
@@ -223,13 +253,20 @@ __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
         const float bs[2] = {lane_value(bs_l, p), lane_value(bs_l, 8 + p)};
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-          v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[p][g][0], b0, v4i{0, 0, 0, 0}, 0, 0, 0);
-          d = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[p][g][1], b1, d, 0, 0, 0);
+          v4i w0, w1;
+          if constexpr (W4) {
+            unpack_int4(wbuf[p][g][0], w0, w1);
+          } else {
+            w0 = wbuf[p][g][0];
+            w1 = wbuf[p][g][W4 ? 0 : 1];
+          }
+          v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, b0, v4i{0, 0, 0, 0}, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, b1, d, 0, 0, 0);
           if (n < nc) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const float t = static_cast<float>(d[i]) * as;
-              sT[((kb0 + p) * 8 + g * 4 + i) * 16 + c * kDecTP + n] = t * bs[g];
+              sT[((kb0 + p) * 8 + g * 4 + i) * 16 + c * kDecTP + n] = t * (W4 ? wsc[W4 ? p : 0][g][i] * 0.0625f : bs[g]);
             }
           }
         }
@@ -277,12 +314,14 @@ __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
 
 // Up to four K blocks per wave: half the registers, so four waves per SIMD (twice the workgroups in
 // flight per compute unit) instead of two.
+template <bool W4>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void dec_gemm1_small_kernel(const DecArgs a) {
-  dec_gemm1_body<4>(a);
+  dec_gemm1_body<4, W4>(a);
 }
-__global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) { dec_gemm1_body<kDecMaxKBw>(a); }
+template <bool W4>
+__global__ __launch_bounds__(512) void dec_gemm1_kernel(const DecArgs a) { dec_gemm1_body<kDecMaxKBw, W4>(a); }
 
-template <int PD, int RAWN> // weight K blocks in flight per wave; 16-byte pieces of the activation row per lane
+template <int PD, int RAWN, bool W4> // weight K blocks in flight per wave; 16-byte pieces of the activation row per lane
 __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -315,18 +354,30 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
     if (lane == 0) sLoc[j] = e >= 0 ? 1 : 0;
     if (e < 0) continue; // (its activation row was never written: nothing of it is used)
 
-    const brsrc rW = make_rsrc(a.w2 + static_cast<int64_t>(e) * H * I, static_cast<uint32_t>(static_cast<int64_t>(H) * I));
-    const int wkstride = shuf_kb_stride(H / 16);
-    const int woff = rb * shuf_nb_stride(KB) + lane * 16;
-    v4i wbuf[PD][2];
+    const int64_t wbytes = W4 ? static_cast<int64_t>(H) * I / 2 : static_cast<int64_t>(H) * I;
+    const brsrc rW = make_rsrc(a.w2 + static_cast<int64_t>(e) * wbytes, static_cast<uint32_t>(wbytes));
+    const brsrc rWs = make_rsrc(a.w2s + static_cast<int64_t>(e) * KB * H, static_cast<uint32_t>(W4 ? static_cast<int64_t>(KB) * H * 4 : 0));
+    const int wkstride = W4 ? shuf_kb_stride(H / 16) / 2 : shuf_kb_stride(H / 16);
+    const int woff = rb * (W4 ? shuf_nb_stride(KB) / 2 : shuf_nb_stride(KB)) + lane * 16;
+    const int wsoff = (rb * 16 + 4 * c) * 4; // W4: the scales of the lane's four rows
+    v4i wbuf[PD][W4 ? 1 : 2];
+    v4f wsc[W4 ? PD : 1];
+    auto issue = [&](int p, int kb) __attribute__((always_inline)) {
+      if constexpr (W4) {
+        wbuf[p][0] = bld16<kCacheStream>(rW, woff, kb * wkstride);
+        wsc[p] = __builtin_bit_cast(v4f, bld16(rWs, wsoff, kb * H * 4));
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) wbuf[p][ks] = bld16<kCacheStream>(rW, woff, kb * wkstride + ks * 1024);
+      }
+    };
 #pragma unroll
     for (int p = 0; p < PD; ++p)
-      if (p < KB) {
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) wbuf[p][ks] = bld16<kCacheStream>(rW, woff, p * wkstride + ks * 1024);
-      }
+      if (p < KB) issue(p, p);
     float bs_l = 0.0f; // lane l: the block scale of K block l
-    if (lane < KB) bs_l = a.w2s[(static_cast<int64_t>(e) * (H / kGroup) + rb / 8) * KB + lane];
+    if constexpr (!W4) {
+      if (lane < KB) bs_l = a.w2s[(static_cast<int64_t>(e) * (H / kGroup) + rb / 8) * KB + lane];
+    }
 
     // the activation row, re-quantised in 1x128 groups, into the wave's LDS row
 #pragma unroll
@@ -350,18 +401,23 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
           // every column of the token operand is the same row: all lanes end up with valid sums
           const v4i b0 = *reinterpret_cast<const v4i *>(sA + kb * kGroup + c * 16);
           const v4i b1 = *reinterpret_cast<const v4i *>(sA + kb * kGroup + 64 + c * 16);
-          v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[p][0], b0, v4i{0, 0, 0, 0}, 0, 0, 0);
-          d = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[p][1], b1, d, 0, 0, 0);
-          if (kb + PD < KB) {
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-              wbuf[p][ks] = bld16<kCacheStream>(rW, woff, (kb + PD) * wkstride + ks * 1024);
+          v4i w0, w1;
+          v4f bs4 = v4f{0.f, 0.f, 0.f, 0.f};
+          if constexpr (W4) {
+            unpack_int4(wbuf[p][0], w0, w1);
+            bs4 = wsc[W4 ? p : 0] * 0.0625f;
+          } else {
+            w0 = wbuf[p][0];
+            w1 = wbuf[p][W4 ? 0 : 1];
           }
+          v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, b0, v4i{0, 0, 0, 0}, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, b1, d, 0, 0, 0);
+          if (kb + PD < KB) issue(p, kb + PD);
           const float as = sAs[kb], bs = lane_value(bs_l, kb);
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             float tt = static_cast<float>(d[i]) * as;
-            tt = tt * bs;
+            tt = tt * (W4 ? bs4[i] : bs);
             acc[i] = acc[i] + tt;
           }
         }
@@ -422,7 +478,7 @@ static int decode_max_slots() {
   return v;
 }
 
-bool decode_path_applies(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_t num_experts, bool force) {
+bool decode_path_applies(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_t num_experts, bool force, bool w4) {
   const int64_t S = M * top_k;
   if (S > kDecMaxSlots || top_k > 64) return false;
   if (H % kGroup || I % kGroup || 2 * I * H >= (1ll << 31)) return false;
@@ -438,6 +494,8 @@ bool decode_path_applies(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_t
   // registers and live too briefly to overlap one another
   (void)num_experts;
   const int KB = static_cast<int>(H / kGroup);
+  // packed int4 (Qwen3-235B-A22B-shaped layer): 33 against 41 us at one token, level at two, behind at four
+  if (w4) return S <= 16;
   return S <= 32 || (S <= 64 && KB / pick_waves(KB) <= 4);
 }
 
@@ -451,8 +509,8 @@ void decode_path_waves(int32_t top_k, int64_t H, int *gemm1_waves, int *gemm2_wa
 int launch_decode_path(const void *x, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts, int32_t top_k,
                        const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s, const float *topk_w,
                        const void *topk_ids, int ids_dtype, const int32_t *expert_map, int apply_router_weight_on_input,
-                       float factor, const void *shared_output, void *act, void *out, bool force, hipStream_t stream) {
-  if (!decode_path_applies(M, top_k, H, I, num_experts, force)) return LO_ENOTSUP;
+                       float factor, const void *shared_output, void *act, void *out, bool force, bool w4, hipStream_t stream) {
+  if (!decode_path_applies(M, top_k, H, I, num_experts, force, w4)) return LO_ENOTSUP;
   const int64_t S = M * top_k;
   const int KB1 = static_cast<int>(H / kGroup), KB2 = static_cast<int>(I / kGroup);
   int W1, W2;
@@ -477,14 +535,20 @@ int launch_decode_path(const void *x, int64_t M, int64_t H, int64_t I, int32_t E
   if (l1 > 64 * 1024 || l2 > 64 * 1024) return LO_ENOTSUP;
   const dim3 g1(static_cast<unsigned>(I / 16), static_cast<unsigned>(S)), g2(static_cast<unsigned>(H / 16), static_cast<unsigned>(M));
   // fewer registers where the shape allows it: more workgroups in flight per compute unit
-  if (a.kbw <= 4) hipLaunchKernelGGL(dec_gemm1_small_kernel, g1, dim3(64 * W1), l1, stream, a);
-  else hipLaunchKernelGGL(dec_gemm1_kernel, g1, dim3(64 * W1), l1, stream, a);
-  const int rc = check_launch("fused_experts(decode, gemm1)");
-  if (rc) return rc;
-  if (KB2 <= 6) hipLaunchKernelGGL((dec_gemm2_kernel<6, 2>), g2, dim3(64 * W2), l2, stream, a);
-  else if (KB2 <= 8) hipLaunchKernelGGL((dec_gemm2_kernel<8, 2>), g2, dim3(64 * W2), l2, stream, a);
-  else if (KB2 <= 16) hipLaunchKernelGGL((dec_gemm2_kernel<8, 4>), g2, dim3(64 * W2), l2, stream, a);
-  else hipLaunchKernelGGL((dec_gemm2_kernel<8, 8>), g2, dim3(64 * W2), l2, stream, a);
+#define LO_DEC_LAUNCH(W4)                                                                                        \
+  do {                                                                                                           \
+    if (a.kbw <= 4) hipLaunchKernelGGL(dec_gemm1_small_kernel<W4>, g1, dim3(64 * W1), l1, stream, a);            \
+    else hipLaunchKernelGGL(dec_gemm1_kernel<W4>, g1, dim3(64 * W1), l1, stream, a);                             \
+    const int rc = check_launch("fused_experts(decode, gemm1)");                                                 \
+    if (rc) return rc;                                                                                           \
+    if (KB2 <= 6) hipLaunchKernelGGL((dec_gemm2_kernel<6, 2, W4>), g2, dim3(64 * W2), l2, stream, a);            \
+    else if (KB2 <= 8) hipLaunchKernelGGL((dec_gemm2_kernel<8, 2, W4>), g2, dim3(64 * W2), l2, stream, a);       \
+    else if (KB2 <= 16) hipLaunchKernelGGL((dec_gemm2_kernel<8, 4, W4>), g2, dim3(64 * W2), l2, stream, a);      \
+    else hipLaunchKernelGGL((dec_gemm2_kernel<8, 8, W4>), g2, dim3(64 * W2), l2, stream, a);                     \
+  } while (0)
+  if (w4) LO_DEC_LAUNCH(true);
+  else LO_DEC_LAUNCH(false);
+#undef LO_DEC_LAUNCH
   return check_launch("fused_experts(decode, gemm2)");
 }
 

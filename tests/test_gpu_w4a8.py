@@ -123,6 +123,32 @@ def test_whole_path_tiny_bit_exact(dev, oracle, bs, with_map):
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
+@pytest.mark.parametrize("M", [1, 5, 40, 200])
+@pytest.mark.parametrize("with_map", [False, True])
+def test_two_launch_path_w4a8_bit_exact(dev, oracle, M, with_map):
+    """The two-launch path for a few tokens on packed int4 weights (forced beyond its default size)."""
+    from lightop_amd import _lib, workloads as wl
+    from lightop_amd.moe import preshuffle_moe_weight_int4
+
+    layer = wl.TINY_W4
+    say(f"w4a8 two-launch path M={M} map={with_map}")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=1)
+    x, tw, ids = wl.make_inputs(layer, M, seed=M)
+    emap, n = None, layer.E
+    if with_map:
+        n = 5
+        emap = torch.full((layer.E,), -1, dtype=torch.int32)
+        emap[:n] = torch.arange(n, dtype=torch.int32)
+    wd = (preshuffle_moe_weight_int4(w1[:n].contiguous().to(dev)), preshuffle_moe_weight_int4(w2[:n].contiguous().to(dev)),
+          w1s[:n].contiguous().to(dev), w2s[:n].contiguous().to(dev))
+    ref = oracle.fused_experts_w4a8(x, w1[:n], w2[:n], w1s[:n], w2s[:n], tw, ids, 16, global_num_experts=layer.E,
+                                    expert_map=emap)
+    for _ in range(2):
+        out = run_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None if emap is None else emap.to(dev), dev, 0,
+                       _lib.LO_FUSED_FORCE_DECODE_PATH)
+        assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
 def test_w4a8_rejects_what_is_not_built(dev):
     from lightop_amd import workloads as wl
     from lightop_amd.moe import fused_experts_impl_w4a8, preshuffle_moe_weight_int4
