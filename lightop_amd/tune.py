@@ -118,7 +118,8 @@ def main(argv=None):
         os.makedirs(args.out, exist_ok=True)
         props = torch.cuda.get_device_properties(dev)
         devname = f"{props.gcnArchName.split(':')[0]}_{props.multi_processor_count}cu"
-        kind = "W4A8[1,128]" if layer.weight_bits == 4 else ("CHANNELINT8" if block_shape is None else "BLOCKINT8[128,128]")
+        # file names as the reference's reader builds them (w8a8_get_cache_json.py:133-149)
+        kind = "W4A8INT8[1,128]" if layer.weight_bits == 4 else ("W8A8INT8" if block_shape is None else "BLOCKINT8[128,128]")
         name = (f"MOE_{kind}_E={layer.E}_N1={2 * layer.I}_N2={layer.H}_K={layer.I}_"
                 f"TOPK{layer.top_k}_{devname}.json")
         with open(os.path.join(args.out, name), "w") as f:
