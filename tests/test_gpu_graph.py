@@ -9,21 +9,23 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("M", [1, 16, 64])
-@pytest.mark.parametrize("form", ["block", "channel", "w4"])
+@pytest.mark.parametrize("form", ["block", "block_preshuffled", "channel", "w4"])
 def test_graph_replays_match_eager(M, form):
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     from lightop_amd import _lib, workloads as wl
     from lightop_amd.moe import (fused_experts_impl_int8, fused_experts_impl_w4a8, preshuffle_moe_scale_int4,
-                                 preshuffle_moe_weight_int4)
+                                 preshuffle_moe_weight, preshuffle_moe_weight_int4)
 
     _lib.lib()
     dev = torch.device("cuda:0")
-    layer = {"block": wl.TINY, "channel": wl.TINY_PC, "w4": wl.TINY_W4}[form]
+    layer = {"block": wl.TINY, "block_preshuffled": wl.TINY, "channel": wl.TINY_PC, "w4": wl.TINY_W4}[form]
     w1, w2, w1s, w2s = wl.make_weights(layer, seed=0, device=dev)
     if form == "w4":
         w1, w2 = preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2)
         w1s, w2s = preshuffle_moe_scale_int4(w1s), preshuffle_moe_scale_int4(w2s)
+    if form == "block_preshuffled":  # load-time layout: the two-launch path at 1 and 16 tokens
+        w1, w2 = preshuffle_moe_weight(w1), preshuffle_moe_weight(w2)
     x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, M, seed=5))
     cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
 
