@@ -397,9 +397,15 @@ int lo_fuse_silu_mul_quant_ids(const void *c1, int dtype, int64_t rows, int64_t 
  *   As [a_rows] f32, Ws [E, N] f32 (16-byte aligned, like C); everything else as lo_moe_gemm_block_int8.
  *   C[f, n] = T((f32(sum_k A*W) * ts) * Ws[e, n]),  ts = As[f / top_k], or
  *   topk_w[f] * As[f / top_k] with mul_routed;  rows of expert -1 are zero.
- *   flags: LO_GEMM_W_PRESHUFFLED, LO_GEMM_SKIP_NONLOCAL, LO_GEMM_FORCE_STREAMING.
+ *   flags: LO_GEMM_W_PRESHUFFLED, LO_GEMM_SKIP_NONLOCAL, LO_GEMM_FORCE_STREAMING, LO_GEMM_W4.
  * The reference picks a kernel by `mode`/`delta` from its tuning tables; here block_size_m
  * selects it.
+ *
+ * With LO_GEMM_W4 (and LO_GEMM_W_PRESHUFFLED) the stage is the reference's own int4 kernel,
+ * fused_moe_kernel_int4_w4a8 (python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341-395):
+ * W is the load-time layout of lo_preshuffle_weight_int4, K counts unpacked elements, every
+ * nibble enters the sum as int8(nibble << 4), i.e. 16 times the signed int4, and
+ *   C[f, n] = T(((f32(sum_k A*w16) [* topk_w[f]]) * As[f / top_k]) * Ws[e, n]).
  */
 int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *W, const float *Ws, void *C,
                      int c_dtype, const float *topk_w, const int32_t *sorted_ids,
@@ -416,6 +422,9 @@ int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *W, const fl
  *   cache13 [M*top_k, max(2I, H)] act dtype: holds the first GEMM's output, then the second's
  *   (the reference shares the buffer the same way, int8.py:681-682).
  * The workspace is the one of lo_fused_experts_workspace_bytes.
+ * flags LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED: both stages are the int4 kernel described at
+ * lo_moe_gemm_w8a8, which makes the call the reference's fused_experts_impl_w4a8 (w4a8.py:480-658)
+ * with w1 [E, 2I, H/2] and w2 [E, H, I/2] in the layout of lo_preshuffle_weight_int4.
  */
 int lo_fused_experts_channel_int8(const void *x, int dtype, int64_t M, int64_t H, int64_t I,
                                   int32_t E, int32_t num_experts, int32_t top_k, const int8_t *w1,

@@ -147,7 +147,7 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
   a.experts_routed = num_experts;
   a.top_k = top_k;
   a.w_shuffled = pre ? 1 : 0;
-  a.w4 = form == LO_FORM_W4 ? 1 : 0;
+  a.w4 = (form == LO_FORM_W4 || (form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4))) ? 1 : 0;
   a.per_channel = form == LO_FORM_CHANNEL ? 1 : 0;
   if (gemm1) {
     a.N = 2 * I; a.K = H; a.a_rows = M;

@@ -34,6 +34,7 @@ static int validate_common(const char *who, const void *A, const void *As, const
 // query (lo_moe_tile_query_form) reports this very choice.
 int pick_gemm_kernel(const GemmArgs &a, bool fused_act, int bs, int flags) {
   const bool tiled = !(flags & LO_GEMM_FORCE_STREAMING);
+  if (a.w4 && a.per_channel) return LO_KERNEL_WS; // the reference's own int4 form: streaming kernel only
   if (a.w4) { // int4 weights: 128- or 64-token LDS tiles, else streaming
     if (tiled && gemm_t128_supports(a, fused_act, bs)) return LO_KERNEL_T128;
     if (tiled && gemm_w4_tile_supports(a, fused_act, bs)) return LO_KERNEL_W4_TILE;
@@ -186,7 +187,8 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   LO_REQUIRE(N * K < (1ll << 31), LO_ENOTSUP, "moe_gemm_w8a8: one expert's weights exceed 2 GiB");
   LO_REQUIRE(K <= 131072, LO_ENOTSUP, "moe_gemm_w8a8: K (%lld) could overflow the int32 sum", (long long)K);
   LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm_w8a8: mul_routed needs topk_weights");
-  LO_REQUIRE(!(flags & LO_GEMM_W4), LO_ENOTSUP, "moe_gemm_w8a8: int4 weights are not built for the per-channel form");
+  LO_REQUIRE(!(flags & LO_GEMM_W4) || (flags & LO_GEMM_W_PRESHUFFLED), LO_ENOTSUP,
+             "moe_gemm_w8a8: int4 weights exist in the load-time layout only (lo_preshuffle_weight_int4)");
   LO_REQUIRE((reinterpret_cast<uintptr_t>(C) & 15) == 0 && (reinterpret_cast<uintptr_t>(Ws) & 15) == 0, LO_EINVAL,
              "moe_gemm_w8a8: C and the weight scales must be 16-byte aligned");
   LO_REQUIRE((num_valid + top_k - 1) / top_k <= a_rows, LO_EINVAL,
@@ -201,6 +203,7 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.per_channel = 1;
+  a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 30), LO_EINVAL, "moe_gemm_w8a8: grid too large");

@@ -35,20 +35,25 @@ namespace lo {
 //
 // W4: the weights are packed signed int4 in the load-time layout of preshuffle_int4_kernel
 // (one 16-byte load per lane holds both k-steps of a 128-wide K block; two vector
-// instructions per 8 elements turn them into int8 values 16 times too large, which an
-// arithmetic shift of the exact int32 sum takes out again) and every weight row has its
-// own scale per K block, stored K-group-major, Ws [E, K/128, N], so that the four rows a
-// lane accumulates are one 16-byte load.
+// instructions per 8 elements turn them into int8 values 16 times too large, which the
+// row scales take out again as a factor 1/16) and every weight row has its own scale per K
+// block, stored K-group-major, Ws [E, K/128, N], so that the four rows a lane accumulates
+// are one 16-byte load.
 //
 // PC (per-channel W8A8, reference csrc/moe_gemm/w8a8/moe_w8a8.cu:156-166, :445-470): one scale
 // per token row, As [a_rows], and one per weight row, Ws [E, N]; the int32 sum runs over the
 // whole K inside the MFMA accumulator and the scales are applied once, in the epilogue:
 // C = bf16((f32(d) * ts) * Ws[e, n]) with ts = As[row], or topk_w[f] * As[row].
+//
+// W4 and PC together are the reference's own int4 form (fused_moe_kernel_int4_w4a8,
+// python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341-395): the nibbles enter the sum as
+// int8(nibble << 4), the factor 16 stays in it, and C = bf16(((f32(d) [* topk_w[f]]) * As[row])
+// * Ws[e, n]).
 template <int TM, bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int NWAVES, int PD, int RPW, bool W4 = false,
           bool PC = false>
 __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs a) {
   static_assert(!W4 || SHUF, "int4 weights exist in the load-time layout only");
-  static_assert(!PC || (!W4 && !FUSED_ACT), "the per-channel form is a plain int8 GEMM");
+  static_assert(!PC || !FUSED_ACT, "the per-channel form is a plain GEMM");
   constexpr int BM = 16 * TM;
   constexpr int NS = W4 ? 4 : 1; // weight scales per 16-row fragment and lane
   // 16-row weight fragments per wave: (gate, up) when fused, else RPW consecutive ones
@@ -289,15 +294,26 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
       if (!valid[j]) continue;
-      float ts = bld_f32(rAs, asoff[j], 0);
-      if (a.mul_routed) ts = a.topk_w[f[j]] * ts;
+      const float as = bld_f32(rAs, asoff[j], 0);
+      const float w = a.mul_routed ? a.topk_w[f[j]] : 1.0f;
+      const float ts = a.mul_routed ? w * as : as;
 #pragma unroll
       for (int g = 0; g < NW; ++g) {
         if (nrow[g] >= N) continue;
         v4u16 o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float t = static_cast<float>(acci[g][j][i]) * ts;
+          float t;
+          if constexpr (W4) {
+            // the reference's int4 kernel keeps the factor 16 of its unpacked nibbles in the sum
+            // (a multiple of 16 below 2^28, exact in fp32) and scales left to right: routed
+            // weight, token scale, channel scale (w4a8.py:386-395)
+            t = static_cast<float>(acci[g][j][i]);
+            if (a.mul_routed) t = t * w;
+            t = t * as;
+          } else {
+            t = static_cast<float>(acci[g][j][i]) * ts;
+          }
           o[i] = f32_to_bf16(t * bs4[g][i]);
         }
         *reinterpret_cast<v4u16 *>(a.C + f[j] * N + nrow[g] + 4 * c) = o;
@@ -375,7 +391,9 @@ static void launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
   const dim3 grid(static_cast<unsigned>(m_blocks * a.n_tiles)), block(NWAVES * 64);
   if constexpr (!FUSED_ACT && !FAST_SCALE) {
     if (a.per_channel) {
-      if (a.w_shuffled)
+      if (a.w4)
+        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, true, NWAVES, PD, RPW, true, true>), grid, block, 0, s, a);
+      else if (a.w_shuffled)
         hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, true, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
       else
         hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, false, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);

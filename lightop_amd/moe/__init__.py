@@ -13,6 +13,7 @@ _NATIVE_APIS = {
     "preshuffle_moe_scale_int4",
     "get_w8a8moe_json",
     "invoke_fused_moe_kernel_int8",
+    "invoke_fused_moe_kernel_w4a8",
     "invoke_fused_moe_gemm1_silu_quant",
     "silu_and_mul",
     "fused_experts_workspace_bytes",
@@ -39,6 +40,7 @@ __all__ = [
     "get_w8a8moe_json",
     "invoke_fused_moe_gemm1_silu_quant",
     "invoke_fused_moe_kernel_int8",
+    "invoke_fused_moe_kernel_w4a8",
     "moe_align_block_size",
     "moe_align_block_size_out",
     "moe_fused_gate",

@@ -215,6 +215,47 @@ def moe_gemm_w8a8(input: torch.Tensor, b_qweight: torch.Tensor, output: torch.Te
     return output
 
 
+def invoke_fused_moe_kernel_w4a8(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, A_scale: torch.Tensor,
+                                 B_scale: torch.Tensor, B_zp: Optional[torch.Tensor],
+                                 topk_weights: Optional[torch.Tensor], sorted_token_ids: torch.Tensor,
+                                 expert_ids: torch.Tensor, num_tokens_post_padded: torch.Tensor,
+                                 mul_routed_weight: bool, top_k: int, config: Dict[str, Any],
+                                 compute_type=None, block_shape: Optional[List[int]] = None,
+                                 global_num_experts: int = 0) -> None:
+    """One grouped GEMM stage of the reference's own int4 form (invoke_fused_moe_kernel_w4a8,
+    w4a8.py:405-478; kernel :202-401): ``A`` int8 [rows, K], ``B`` packed int4 [E, N, K/2] from
+    ``preshuffle_moe_weight_int4``, ``A_scale`` one per row, ``B_scale`` one per weight row.
+    C[f] = T(((sum_k A[f // top_k] * w16[e]) [* topk_weights[f]]) * A_scale[f // top_k] * B_scale[e]),
+    w16 = int8(nibble << 4).  ``config`` needs ``BLOCK_SIZE_M``."""
+    assert B_zp is None, "lightop_amd: W4A8 zero points are not built (symmetric int4 only)"
+    assert block_shape is None, "the K-group form goes through fused_experts_impl_w4a8(block_shape=[1, 128])"
+    del compute_type
+    _require_cuda(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded)
+    assert A.dtype == torch.int8 and B.dtype in (torch.int8, torch.uint8)
+    assert A.is_contiguous() and B.is_contiguous() and C.is_contiguous()
+    if not getattr(B, "lo_int4", False):
+        raise RuntimeError("lightop_amd: pass the weights through preshuffle_moe_weight_int4 once at load time")
+    E, N, K2 = B.shape
+    K = 2 * K2
+    assert A.shape[1] == K and C.shape[-1] == N
+    assert A_scale.dtype == torch.float32 and A_scale.is_contiguous() and A_scale.numel() == A.shape[0]
+    assert B_scale.dtype == torch.float32 and B_scale.is_contiguous() and B_scale.numel() == E * N
+    assert sorted_token_ids.dtype == torch.int32 and expert_ids.dtype == torch.int32
+    assert topk_weights is not None or not mul_routed_weight
+    num_valid = C.numel() // N
+    tw = None
+    if mul_routed_weight:
+        tw = topk_weights if topk_weights.dtype == torch.float32 and topk_weights.is_contiguous() \
+            else topk_weights.to(torch.float32).contiguous()
+    with _on_device(A):
+        _lib.check(_lib.lib().lo_moe_gemm_w8a8(
+            _lib.ptr(A), _lib.ptr(A_scale), _lib.ptr(B), _lib.ptr(B_scale), _lib.ptr(C), _act_dtype(C),
+            _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(expert_ids), _lib.ptr(num_tokens_post_padded),
+            sorted_token_ids.numel(), num_valid, A.shape[0], E, int(global_num_experts or 0), N, K, int(top_k),
+            int(config["BLOCK_SIZE_M"]), 1 if mul_routed_weight else 0,
+            _lib.LO_GEMM_W4 | _lib.LO_GEMM_W_PRESHUFFLED, _lib.stream_of(A)))
+
+
 def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
     """out[:, i] = T(T(silu(x[:, i])) * x[:, d + i])  (the op called at int8.py:811)."""
     _require_cuda(out, x)
@@ -381,14 +422,19 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     """Fused MoE experts with packed int4 weights and int8 activations (signature of the
     reference's fused_experts_impl_w4a8, w4a8.py:480-501).
 
-    This build implements the K-group form: ``block_shape=[1, 128]``, ``w1`` [E, 2I, H/2] and
-    ``w2`` [E, H, I/2] packed two int4 per byte along K (even k in the high nibble, the
-    reference's order) and passed through ``preshuffle_moe_weight_int4``, one fp32 scale per
-    output row and 128-wide K group (``w1_scale`` [E, 2I, H/128], ``w2_scale`` [E, H, I/128], or
-    their load-time form from ``preshuffle_moe_scale_int4``),
-    activations quantised per 1x128 group on the fly, SiLU.  The reference's own form (scales
-    per token and per channel in the epilogue, ``block_shape=None``, w4a8.py:395) is not
-    built and raises.  The reduce is always performed.
+    ``w1`` [E, 2I, H/2] and ``w2`` [E, H, I/2] hold two int4 per byte along K (even k in the high
+    nibble, the reference's order) and have been passed through ``preshuffle_moe_weight_int4``.
+
+    ``block_shape=None`` is the reference's own form (w4a8.py:480-658): activations quantised per
+    token, ``w1_scale`` [E, 2I(, 1)] and ``w2_scale`` [E, H(, 1)] one fp32 scale per weight row,
+    both applied in the epilogue of each stage to a sum that keeps the factor 16 of the nibbles
+    (w4a8.py:375-395).
+
+    ``block_shape=[1, 128]`` is the K-group form: one fp32 scale per weight row and 128-wide K
+    group (``w1_scale`` [E, 2I, H/128], ``w2_scale`` [E, H, I/128], or their load-time form from
+    ``preshuffle_moe_scale_int4``), activations quantised per 1x128 group on the fly.
+
+    SiLU only; the reduce is always performed.
     """
     extra = _
     assert hidden_states.shape[1] == w1.shape[2] * 2, "Hidden size mismatch"  # w4a8.py:503
@@ -397,8 +443,10 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     assert w1.stride(-1) == 1, "Stride of last dimension must be 1"
     assert w2.stride(-1) == 1, "Stride of last dimension must be 1"
     assert hidden_states.dtype in [torch.float32, torch.float16, torch.bfloat16]
-    if block_shape is None or list(block_shape) != [1, 128]:
-        raise NotImplementedError("lightop_amd: W4A8 is built for K-group scales, block_shape=[1, 128]")
+    channel = block_shape is None
+    if not channel and list(block_shape) != [1, 128]:
+        raise NotImplementedError("lightop_amd: W4A8 is built for block_shape=None (per token x per channel) "
+                                  "and for K-group scales, block_shape=[1, 128]")
     if activation != "silu":
         if activation == "gelu":
             raise NotImplementedError("lightop_amd: the gelu activation is not built")
@@ -419,6 +467,19 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     assert w1.dtype in (torch.int8, torch.uint8) and w2.dtype == w1.dtype
     if not (getattr(w1, "lo_int4", False) and getattr(w2, "lo_int4", False)):
         raise RuntimeError("lightop_amd: pass w1 and w2 through preshuffle_moe_weight_int4 once at load time")
+    if global_num_experts == -1:
+        global_num_experts = E
+    if channel:
+        assert w1_scale.numel() == E * N and w2_scale.numel() == E * H, "scales must be [E, 2I] and [E, H]"
+        M = min(num_tokens, envs.LMSLIM_FUSED_MOE_CHUNK_SIZE)
+        assert cache13.dtype == hidden_states.dtype and cache13.is_contiguous()
+        assert cache13.numel() >= M * topk_ids.shape[1] * max(N, H), "cache13 is too small"
+        flags = int(extra.get("lightop_amd_flags", 0)) | _lib.LO_GEMM_W4
+        return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
+                                  apply_router_weight_on_input, global_num_experts, expert_map,
+                                  w1_scale.reshape(E, N), w2_scale.reshape(E, H), routed_scaling_factor,
+                                  shared_output, I, flags, int(extra.get("lightop_amd_block_size_m", 0)),
+                                  channel=True, workspace=extra.get("lightop_amd_workspace"))
     # scales: [E, N, K/128] as a checkpoint holds them (transposed here, on every call) or, better,
     # already K-group-major from preshuffle_moe_scale_int4
     if not getattr(w1_scale, "lo_kmajor", False):
@@ -428,8 +489,6 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
         assert w2_scale.shape == (E, H, I // 128), "w2_scale must be [E, H, I/128]"
         w2_scale = preshuffle_moe_scale_int4(w2_scale)
     assert w1_scale.shape == (E, H // 128, N) and w2_scale.shape == (E, I // 128, H)
-    if global_num_experts == -1:
-        global_num_experts = E
     M = min(num_tokens, envs.LMSLIM_FUSED_MOE_CHUNK_SIZE)
     assert cache13.dtype == hidden_states.dtype and cache13.is_contiguous()
     assert cache13.numel() >= M * topk_ids.shape[1] * max(N, H), "cache13 is too small"
@@ -509,5 +568,6 @@ def ctypes_void(addr: int):
 
 __all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "preshuffle_moe_weight",
            "preshuffle_moe_weight_int4", "preshuffle_moe_scale_int4", "invoke_fused_moe_kernel_int8",
+           "invoke_fused_moe_kernel_w4a8",
            "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes",
            "fused_experts_workspace_views", "moe_gemm_w8a8"]

@@ -48,21 +48,28 @@ TINY_W4 = MoeLayer("tiny-e8-w4a8", E=8, E_global=8, top_k=2, H=1024, I=512, rout
 QWEN3_235B_W4 = MoeLayer("qwen3-235b-a22b-w4a8", E=128, E_global=128, top_k=8, H=4096, I=1536, routing="softmax",
                          weight_bits=4)
 
+# the reference's own int4 form: scales per token and per weight row, both in the epilogue
+TINY_W4_PC = MoeLayer("tiny-e8-w4a8-channel", E=8, E_global=8, top_k=2, H=1024, I=512, routing="softmax",
+                      weight_bits=4, quant="channel")
+QWEN3_235B_W4_PC = MoeLayer("qwen3-235b-a22b-w4a8-channel", E=128, E_global=128, top_k=8, H=4096, I=1536,
+                            routing="softmax", weight_bits=4, quant="channel")
+
 TINY_PC = MoeLayer("tiny-e8-channel", E=8, E_global=8, top_k=2, H=1024, I=512, routing="softmax", quant="channel")
 QWEN3_30B_PC = MoeLayer("qwen3-30b-a3b-channel", E=128, E_global=128, top_k=8, H=2048, I=768, routing="softmax",
                         quant="channel")
 DSV3_EP_PC = MoeLayer("deepseek-v3-ep8-share-channel", E=32, E_global=256, top_k=8, H=7168, I=2048,
                       routing="grouped_sigmoid", n_group=8, topk_group=4, routed_scaling=2.5, quant="channel")
 
-LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL, TINY_W4, QWEN3_235B_W4, TINY_PC, QWEN3_30B_PC,
-                              DSV3_EP_PC)}
+LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL, TINY_W4, QWEN3_235B_W4, TINY_W4_PC,
+                              QWEN3_235B_W4_PC, TINY_PC, QWEN3_30B_PC, DSV3_EP_PC)}
 
 
 def make_weights(layer: MoeLayer, seed: int = 0, device="cpu", gen_device: Optional[str] = None):
     """(w1 [E,2I,H] int8, w2 [E,H,I] int8, w1_scale [E,2I/128,H/128], w2_scale [E,H/128,I/128]); for a
     per-channel layer the scales are [E,2I,1] and [E,H,1]; for a
     4-bit layer (w1 [E,2I,H/2], w2 [E,H,I/2] uint8: int4 uniform in [-8, 7], two per byte along K, even k
-    in the high nibble; w1_scale [E,2I,H/128], w2_scale [E,H,I/128])."""
+    in the high nibble; w1_scale [E,2I,H/128], w2_scale [E,H,I/128], or [E,2I,1] and [E,H,1] in the
+    per-channel form, whose sums carry the factor 16 of the nibbles)."""
     gen_device = gen_device or "cpu"
     g = torch.Generator(device=gen_device).manual_seed(seed)
     E, H, I = layer.E, layer.H, layer.I
@@ -74,6 +81,9 @@ def make_weights(layer: MoeLayer, seed: int = 0, device="cpu", gen_device: Optio
             return torch.exp(torch.randn(shape, generator=g, dtype=torch.float32, device=gen_device) * 0.3
                              + math.log(1e-2))
 
+        if layer.quant == "channel":
+            return tuple(t.to(device) for t in (w4((E, 2 * I, H // 2)), w4((E, H, I // 2)),
+                                                s4((E, 2 * I, 1)) / 16, s4((E, H, 1)) / 16))
         return tuple(t.to(device) for t in (w4((E, 2 * I, H // 2)), w4((E, H, I // 2)),
                                             s4((E, 2 * I, H // 128)), s4((E, H, I // 128))))
 

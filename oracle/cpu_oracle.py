@@ -174,6 +174,23 @@ def moe_gemm_w4a8(A, As, W4, Ws, *args, **kwargs):
     return moe_gemm_block_int8(A, As, unpack_int4(W4), Ws, *args, _fn="orc_moe_gemm_rowscale_int8", **kwargs)
 
 
+def moe_gemm_w4a8_channel(A, As, W4, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_routed, top_k, num_valid,
+                          block_size, dump_acc=False, out=None):
+    """The reference's own int4 stage (w4a8.py:341-395): W4 [E, N, K/2] packed bytes, As one scale
+    per row of A, Ws [E, N(, 1)].  Returns C [num_valid, N] bf16 (and the int32 sums, factor 16
+    of the nibbles included, when dump_acc)."""
+    E, N, K2 = W4.shape
+    C = torch.zeros(num_valid, N, dtype=torch.bfloat16) if out is None else out
+    acc = torch.zeros(num_valid, N, dtype=torch.int32) if dump_acc else None
+    tw = None if topk_w is None else topk_w.reshape(-1).to(torch.float32).contiguous()
+    lib().orc_moe_gemm_w4a8_channel(
+        _p(A.contiguous()), _p(As.reshape(-1).contiguous()), _p(W4.contiguous().view(torch.uint8)),
+        _p(Ws.reshape(E, N).contiguous()), _p(sorted_ids), _p(expert_ids), _p(ntpp), _p(tw),
+        ctypes.c_int(1 if mul_routed else 0), _i32(top_k), _i64(num_valid), _i64(N), _i64(2 * K2),
+        _i32(block_size), _p(C), _p(acc))
+    return (C, acc) if dump_acc else C
+
+
 def moe_gemm_block_int8(A, As, W, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_routed,
                         top_k, num_valid, block_size, dump_acc=False, out=None, _fn="orc_moe_gemm_block_int8"):
     """One grouped-GEMM stage.  Returns C[num_valid, N] bf16 (and the int32
@@ -247,6 +264,16 @@ def fused_experts_w4a8(x, w1_packed, w2_packed, w1_scale, w2_scale, *args, **kwa
                                     *args, _fn="orc_fused_experts_w4a8", **kwargs)
 
 
+def fused_experts_w4a8_channel(x, w1_packed, w2_packed, w1_scale, w2_scale, *args, **kwargs):
+    """Whole path in the reference's own int4 form (w4a8.py:480-658): packed weights
+    [E, 2I, H/2] and [E, H, I/2], w1_scale [E, 2I(, 1)], w2_scale [E, H(, 1)]; a1s and a2s hold one
+    scale per row.  Other arguments as fused_experts_block_int8."""
+    E = w1_packed.shape[0]
+    return fused_experts_block_int8(x, w1_packed.contiguous().view(torch.uint8), w2_packed.contiguous().view(torch.uint8),
+                                    w1_scale.reshape(E, -1), w2_scale.reshape(E, -1), *args,
+                                    _fn="orc_fused_experts_w4a8_channel", **kwargs)
+
+
 def fused_experts_channel_int8(x, w1, w2, w1_scale, w2_scale, *args, **kwargs):
     """Whole path in the per-channel form: w1_scale [E, 2I(, 1)], w2_scale [E, H(, 1)]; the
     intermediates a1s and a2s hold one scale per row.  Other arguments as fused_experts_block_int8."""
@@ -293,7 +320,7 @@ def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_i
     if rc != 0:
         raise RuntimeError("oracle fused_experts: alignment failed")
     if return_intermediates:
-        if _fn == "orc_fused_experts_channel_int8":  # one scale per row, written densely at the front
+        if _fn in ("orc_fused_experts_channel_int8", "orc_fused_experts_w4a8_channel"):  # one scale per row, written densely at the front
             inter["a1s"] = inter["a1s"].reshape(-1)[:M].reshape(M, 1).clone()
             inter["a2s"] = inter["a2s"].reshape(-1)[:S].reshape(S, 1).clone()
         inter.update(sorted_ids=sorted_ids, expert_ids=expert_ids, num_tokens_post_pad=ntpp, out=out)

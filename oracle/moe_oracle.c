@@ -584,6 +584,114 @@ int orc_fused_experts_channel_int8(
 }
 
 /* ------------------------------------------------------------------------- *
+ * The reference's own W4A8 form: packed int4 weights, one scale per token row
+ * and one per weight row, both applied in the epilogue.
+ *
+ * Reference: python/lightop/_lmslim_native/layers/fused_moe/w4a8.py
+ *   kernel fused_moe_kernel_int4_w4a8 :202-401
+ *     weight of element k of row n: byte k/2, shifted left by 4*(k%2) and masked with 0xF0
+ *     (:341, :375-377), read as int8: the HIGH nibble for even k, the LOW one for odd k, each
+ *     16 times the signed int4 it encodes
+ *     accumulator (fp32) += dot(a, b) per K tile (:381)
+ *     accumulator *= moe_weight when MUL_ROUTED_WEIGHT (:386-388)
+ *     C = compute_type(accumulator * a_scale * b_scale), left to right (:395)
+ *     expert -1: zeros (:326-333)
+ *   host chain fused_experts_impl_w4a8 :480-658: per_token_quant_int8 -> align -> kernel ->
+ *     fuse_silu_mul_quant -> kernel (routed weight, top_k = 1) -> moe_sum
+ *
+ * Every product is a multiple of 16 and so is every partial sum; below 2^28 in magnitude such
+ * a number is exact in fp32, so while K * 128 * 127 < 2^28 (K <= 16512) the reference's fp32
+ * running sum equals the exact integer sum whatever its K tile is.  The restatement sums in
+ * int32 and converts once; beyond that K the reference's result depends on its tile choice and
+ * this one is the exact sum.
+ *
+ * Parity pins (tests/test_oracle_w4a8.py): the nibble order and the factor 16 on hand-worked
+ * bytes; the left-to-right scale order on operands chosen so that every other association
+ * rounds differently; the whole stage against an independent numpy restatement that
+ * dequantises first (exact in float64) and against orc_moe_gemm_w8a8 on weights pre-multiplied
+ * to int8 (identical sums, a different scale order only where the routed weight enters).
+ * ------------------------------------------------------------------------- */
+
+/* Wp [E, N, K/2] bytes as the checkpoint packs them.  acc_dump (optional, [num_valid, N] int32)
+ * receives the integer sums, factor 16 included. */
+void orc_moe_gemm_w4a8_channel(const int8_t *A, const float *As, const uint8_t *Wp, const float *Ws,
+                               const int32_t *sorted, const int32_t *expert_ids,
+                               const int32_t *num_tokens_post_pad, const float *topk_w,
+                               int mul_routed, int32_t top_k, int64_t num_valid, int64_t N,
+                               int64_t K, int32_t bs, uint16_t *C, int32_t *acc_dump) {
+  int64_t P = num_tokens_post_pad[0];
+  int64_t nblk = P / bs;
+#pragma omp parallel for schedule(dynamic, 1) collapse(2)
+  for (int64_t b = 0; b < nblk; ++b) {
+    for (int32_t i = 0; i < bs; ++i) {
+      int64_t f = sorted[b * bs + i];
+      if (f >= num_valid) continue;
+      int32_t e = expert_ids[b];
+      uint16_t *c = C + f * N;
+      if (e < 0) {
+        for (int64_t n = 0; n < N; ++n) c[n] = 0;
+        continue;
+      }
+      int64_t row = f / top_k;
+      const int8_t *a = A + row * K;
+      for (int64_t n = 0; n < N; ++n) {
+        const uint8_t *wn = Wp + ((int64_t)e * N + n) * (K / 2);
+        int32_t d = 0;
+        for (int64_t k = 0; k < K; ++k) {
+          const int8_t w = (int8_t)(uint8_t)((wn[k >> 1] << (4 * (k & 1))) & 0xF0);
+          d += (int32_t)a[k] * (int32_t)w;
+        }
+        if (acc_dump) acc_dump[f * N + n] = d;
+        float t = (float)d;
+        if (mul_routed) t = t * topk_w[f];
+        t = t * As[row];
+        c[n] = f32_to_bf16(t * Ws[(int64_t)e * N + n]);
+      }
+    }
+  }
+}
+
+/* Chain of w4a8.py:480-658 with the reduce always performed; buffers as in
+ * orc_fused_experts_channel_int8, w1 [E, 2I, H/2] and w2 [E, H, I/2] packed bytes. */
+int orc_fused_experts_w4a8_channel(
+    const uint16_t *x, int64_t M, int64_t H, int64_t I, int32_t E_local,
+    int32_t num_experts_global, int32_t top_k, const uint8_t *w1, const float *w1s,
+    const uint8_t *w2, const float *w2s, const float *topk_w, const int32_t *topk_ids,
+    const int32_t *expert_map, int32_t bs, int apply_router_weight_on_input,
+    float routed_scaling_factor, const uint16_t *shared_output, uint16_t *out,
+    int32_t *sorted, int64_t sorted_cap, int32_t *expert_ids, int64_t expert_ids_cap,
+    int32_t *ntpp, int8_t *a1q, float *a1s, uint16_t *c1, uint16_t *act, int8_t *a2q,
+    float *a2s, uint16_t *c3) {
+  (void)E_local;
+  int64_t S = M * top_k;
+  int own_a1q = !a1q, own_a1s = !a1s, own_c1 = !c1, own_a2q = !a2q, own_a2s = !a2s, own_c3 = !c3;
+  if (own_a1q) a1q = (int8_t *)malloc((size_t)(M * H));
+  if (own_a1s) a1s = (float *)malloc(sizeof(float) * (size_t)M);
+  if (own_c1) c1 = (uint16_t *)calloc((size_t)(S * 2 * I), 2);
+  if (own_a2q) a2q = (int8_t *)malloc((size_t)(S * I));
+  if (own_a2s) a2s = (float *)malloc(sizeof(float) * (size_t)S);
+  if (own_c3) c3 = (uint16_t *)calloc((size_t)(S * H), 2);
+  orc_per_token_quant_int8(x, M, H, a1q, a1s);
+  int rc = orc_moe_align_block_size(topk_ids, S, num_experts_global, bs, expert_map, 0,
+                                    sorted, sorted_cap, expert_ids, expert_ids_cap, ntpp);
+  if (rc == 0) {
+    orc_moe_gemm_w4a8_channel(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
+                              apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL);
+    orc_fuse_silu_mul_quant(c1, S, I, a2q, a2s, act);
+    orc_moe_gemm_w4a8_channel(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
+                              !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL);
+    orc_moe_sum(c3, M, top_k, H, shared_output, routed_scaling_factor, out);
+  }
+  if (own_a1q) free(a1q);
+  if (own_a1s) free(a1s);
+  if (own_c1) free(c1);
+  if (own_a2q) free(a2q);
+  if (own_a2s) free(a2s);
+  if (own_c3) free(c3);
+  return rc;
+}
+
+/* ------------------------------------------------------------------------- *
  * Routers upstream of the path (they produce topk_ids / topk_weights).
  *
  * Reference: csrc/kernels/softmax/topk_softmax_kernels.cu:1381-1582 (generic

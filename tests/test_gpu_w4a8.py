@@ -160,8 +160,11 @@ def test_w4a8_rejects_what_is_not_built(dev):
     with pytest.raises(RuntimeError):  # weights not in the load-time layout
         fused_experts_impl_w4a8(x, w1, w2, tw, ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=[1, 128])
     w1p, w2p = preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2)
-    with pytest.raises(NotImplementedError):  # the reference's per-channel form
-        fused_experts_impl_w4a8(x, w1p, w2p, tw, ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=None)
+    with pytest.raises(NotImplementedError):  # neither the reference's per-channel form nor K groups of 128
+        fused_experts_impl_w4a8(x, w1p, w2p, tw, ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=[128, 128])
+    with pytest.raises(NotImplementedError):
+        fused_experts_impl_w4a8(x, w1p, w2p, tw, ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=[1, 128],
+                                w1_zp=torch.zeros(1, device=dev))
 
 
 @pytest.mark.parametrize("M", [1, 32, 256, 2048])
@@ -194,3 +197,152 @@ def test_baseline_int4_layer_sampled_tokens(dev, oracle, M):
     out2 = run_path(layer, (w1p, w2p, w1sp, w2sp), x, tw, ids, None, dev, 0, 0)  # library default order
     err = (out2.float() - out.float()).abs()
     assert err.max() <= 1e-2 * out.float().abs().max() and err.sum() <= 2e-3 * out.float().abs().sum()
+
+
+# ---- the reference's own form: block_shape=None, scales per token and per weight row ---------
+
+def channel_gemm_case(seed, M, k, E, Eg, N, K):
+    g = torch.Generator().manual_seed(seed)
+    Aq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8)
+    As = torch.rand(M, 1, generator=g) * 0.05 + 0.005
+    W4 = torch.randint(0, 256, (E, N, K // 2), generator=g, dtype=torch.int16).to(torch.uint8)
+    Ws = torch.randn(E, N, 1, generator=g) * 1e-3
+    ids = torch.stack([torch.randperm(Eg, generator=g)[:k] for _ in range(M)]).to(torch.int32)
+    tw = torch.rand(M, k, generator=g) + 0.1
+    emap = None
+    if Eg != E:
+        emap = torch.full((Eg,), -1, dtype=torch.int32)
+        emap[:E] = torch.arange(E, dtype=torch.int32)
+    return Aq, As, W4, Ws, ids, tw, emap
+
+
+@pytest.mark.parametrize("M,k,E,Eg,N,K", [(1, 2, 4, 4, 64, 128), (5, 2, 4, 4, 256, 512), (40, 4, 8, 8, 320, 1152),
+                                          (100, 8, 4, 16, 512, 768), (300, 2, 3, 3, 128, 2048), (70, 2, 2, 2, 48, 384)])
+@pytest.mark.parametrize("bs", [16, 32, 64, 128])
+def test_channel_form_gemm_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
+    from lightop_amd.moe import invoke_fused_moe_kernel_w4a8, moe_align_block_size, preshuffle_moe_weight_int4
+
+    say(f"w4a8 channel gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs}")
+    Aq, As, W4, Ws, ids, tw, emap = channel_gemm_case(M + N + bs, M, k, E, Eg, N, K)
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
+    s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
+    Wd = preshuffle_moe_weight_int4(W4.to(dev))
+    for mul in (False, True):
+        ref = oracle.moe_gemm_w4a8_channel(Aq, As, W4, Ws, rs, re, rp, tw, mul, k, M * k, bs)
+        C = torch.full((M, k, N), 9.0, dtype=torch.bfloat16, device=dev)
+        invoke_fused_moe_kernel_w4a8(Aq.to(dev), Wd, C, As.to(dev), Ws.to(dev), None, tw.to(dev), s, e, p, mul, k,
+                                     {"BLOCK_SIZE_M": bs}, global_num_experts=Eg)
+        torch.cuda.synchronize()
+        assert torch.equal(C.cpu().view(M * k, N).view(torch.int16), ref.view(torch.int16)), f"mul_routed={mul}"
+
+
+def test_channel_form_extreme_sums(dev, oracle):
+    """Every product at its extreme: |sum| = K * 128 * 128 is a multiple of 16 below 2^28, exact in fp32."""
+    from lightop_amd.moe import invoke_fused_moe_kernel_w4a8, moe_align_block_size, preshuffle_moe_weight_int4
+
+    say("w4a8 channel gemm extreme sums")
+    M, E, N, K = 20, 1, 64, 7168
+    Aq = torch.full((M, K), -128, dtype=torch.int8)
+    W4 = torch.full((E, N, K // 2), 0x88, dtype=torch.uint8)  # every weight -8
+    W4[0, 1::2] = 0x77                                        # odd rows: every weight 7
+    As, Ws = torch.ones(M, 1), torch.ones(E, N, 1)
+    ids = torch.zeros(M, 1, dtype=torch.int32)
+    rs, re, rp = oracle.moe_align_block_size(ids, 16, E)
+    ref, acc = oracle.moe_gemm_w4a8_channel(Aq, As, W4, Ws, rs, re, rp, None, False, 1, M, 16, dump_acc=True)
+    assert int(acc[0, 0]) == K * 16384 and int(acc[0, 1]) == -K * 128 * 112
+    s, e, p = moe_align_block_size(ids.to(dev), 16, E)
+    C = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    invoke_fused_moe_kernel_w4a8(Aq.to(dev), preshuffle_moe_weight_int4(W4.to(dev)), C, As.to(dev), Ws.to(dev), None,
+                                 None, s, e, p, False, 1, {"BLOCK_SIZE_M": 16})
+    torch.cuda.synchronize()
+    assert torch.equal(C.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+def run_channel_path(layer, weights_dev, x, tw, ids, emap, dev, bs, **kw):
+    from lightop_amd.moe import fused_experts_impl_w4a8
+
+    w1, w2, w1s, w2s = weights_dev
+    M = x.shape[0]
+    cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
+    out = fused_experts_impl_w4a8(x, w1, w2, tw, ids, cache13, global_num_experts=layer.E_global, expert_map=emap,
+                                  w1_scale=w1s, w2_scale=w2s, block_shape=None, lightop_amd_block_size_m=bs, **kw)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("bs", [0, 16, 32, 64, 128])
+@pytest.mark.parametrize("with_map", [False, True])
+def test_channel_form_whole_path_tiny_bit_exact(dev, oracle, bs, with_map):
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import preshuffle_moe_weight_int4
+
+    layer = wl.TINY_W4_PC
+    say(f"w4a8 channel whole path tiny bs={bs} map={with_map}")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
+    x, tw, ids = wl.make_inputs(layer, 96, seed=4)
+    emap = None
+    if with_map:
+        emap = torch.full((layer.E,), -1, dtype=torch.int32)
+        emap[:5] = torch.arange(5, dtype=torch.int32)
+        w1, w2, w1s, w2s = (t[:5].contiguous() for t in (w1, w2, w1s, w2s))
+    wd = (preshuffle_moe_weight_int4(w1.to(dev)), preshuffle_moe_weight_int4(w2.to(dev)), w1s.to(dev), w2s.to(dev))
+    shared = (torch.randn(96, layer.H, generator=torch.Generator().manual_seed(9)) * 0.1).to(torch.bfloat16)
+    for so, rsf in ((None, 1.0), (shared, 2.5)):
+        out = run_channel_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None if emap is None else emap.to(dev),
+                               dev, bs, shared_output=None if so is None else so.to(dev), routed_scaling_factor=rsf)
+        ref = oracle.fused_experts_w4a8_channel(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=layer.E,
+                                                expert_map=emap, shared_output=so, routed_scaling_factor=rsf)
+        assert ref.float().abs().max() > 0.05
+        assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 77])
+@pytest.mark.parametrize("variant", ["plain", "on_input", "inplace"])
+def test_channel_form_ep_share_variants_bit_exact(dev, oracle, M, variant):
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import fused_experts_impl_w4a8, preshuffle_moe_weight_int4
+
+    say(f"w4a8 channel ep-share M={M} {variant}")
+    layer = wl.MoeLayer("ep-w4pc", E=4, E_global=32, top_k=8, H=512, I=256, routing="grouped_sigmoid", n_group=8,
+                        topk_group=4, routed_scaling=2.5, weight_bits=4, quant="channel")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=3)
+    x, tw, ids = wl.make_inputs(layer, M, seed=3)
+    emap = wl.expert_map_for(layer)
+    cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
+    xd = x.to(dev)
+    out = fused_experts_impl_w4a8(
+        xd, preshuffle_moe_weight_int4(w1.to(dev)), preshuffle_moe_weight_int4(w2.to(dev)), tw.to(dev), ids.to(dev),
+        cache13, inplace=variant == "inplace", apply_router_weight_on_input=variant == "on_input",
+        global_num_experts=32, expert_map=emap.to(dev), w1_scale=w1s.to(dev), w2_scale=w2s.to(dev), block_shape=None)
+    torch.cuda.synchronize()
+    if variant == "inplace":
+        assert out.data_ptr() == xd.data_ptr()
+    ref = oracle.fused_experts_w4a8_channel(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=32, expert_map=emap,
+                                            apply_router_weight_on_input=variant == "on_input")
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("M", [1, 32, 512])
+def test_channel_form_int4_layer_sampled_tokens(dev, oracle, M):
+    """Qwen3-235B-A22B-shaped layer in the reference's own int4 form, sampled tokens against the oracle."""
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import preshuffle_moe_weight_int4
+
+    layer = wl.QWEN3_235B_W4_PC
+    say(f"w4a8 channel {layer.name} M={M}")
+    me = test_channel_form_int4_layer_sampled_tokens
+    if not hasattr(me, "w"):
+        w1, w2, w1s, w2s = wl.make_weights(layer, seed=0, device=dev, gen_device="cuda")
+        me.w = (w1, w2, w1s, w2s, preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2))
+    w1, w2, w1s, w2s, w1p, w2p = me.w
+    x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, M, seed=3))
+    tokens = torch.randperm(M, generator=torch.Generator().manual_seed(M))[: min(M, 4)].sort().values.to(dev)
+    sub_ids = ids[tokens].cpu().long()
+    used = torch.unique(sub_ids)
+    remap = torch.full((layer.E,), -1, dtype=torch.int64)
+    remap[used] = torch.arange(used.numel())
+    sel = used.to(dev)
+    ref = oracle.fused_experts_w4a8_channel(x[tokens].cpu(), w1[sel].cpu(), w2[sel].cpu(), w1s[sel].cpu(),
+                                            w2s[sel].cpu(), tw[tokens].cpu(), remap[sub_ids].to(torch.int32), 16)
+    out = run_channel_path(layer, (w1p, w2p, w1s, w2s), x, tw, ids, None, dev, 0)
+    assert torch.equal(out[tokens].cpu().view(torch.int16), ref.view(torch.int16))
