@@ -136,8 +136,8 @@ class Point:
         if L.weight_bits == 4:
             return fused_experts_impl_w4a8(
                 x, self.w1, self.w2, tw, ids, self.cache13, global_num_experts=L.E_global, expert_map=self.emap,
-                w1_scale=self.w1s, w2_scale=self.w2s, block_shape=[1, 128], lightop_amd_block_size_m=bs,
-                lightop_amd_flags=flags)
+                w1_scale=self.w1s, w2_scale=self.w2s, block_shape=None if L.quant == "channel" else [1, 128],
+                lightop_amd_block_size_m=bs, lightop_amd_flags=flags)
         if L.quant == "channel":
             return fused_experts_impl_int8(
                 x, self.w1, self.w2, tw, ids, self.cache13, use_int8_w8a8=True, per_channel_quant=True,
@@ -156,8 +156,9 @@ class Point:
         L = self.layer
         wflag = _lib_flags_w4(L)
         if bs == 0:
-            shape = [1, 128] if L.weight_bits == 4 else (None if L.quant == "channel" else [128, 128])
-            bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, shape, L.top_k, L.E_global)[0]["BLOCK_SIZE_M"]
+            shape = None if L.quant == "channel" else ([1, 128] if L.weight_bits == 4 else [128, 128])
+            bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, shape, L.top_k, L.E_global,
+                                      int4=L.weight_bits == 4)[0]["BLOCK_SIZE_M"]
         cfg = {"BLOCK_SIZE_M": bs}
         S = self.M * L.top_k
         c3 = self.cache13[: S * L.H].view(self.M, L.top_k, L.H)
@@ -222,12 +223,21 @@ class Point:
             ev[1].record()
             s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
             ev[2].record()
-            moe.moe_gemm_w8a8(a1q, self.w1, c1, a1s, self.w1s, None, s, e, p, L.top_k, cfg,
-                              global_num_experts=L.E_global)
+            if L.weight_bits == 4:
+                moe.invoke_fused_moe_kernel_w4a8(a1q, self.w1, c1, a1s, self.w1s, None, None, s, e, p, False, L.top_k,
+                                                 cfg, global_num_experts=L.E_global)
+            else:
+                moe.moe_gemm_w8a8(a1q, self.w1, c1, a1s, self.w1s, None, s, e, p, L.top_k, cfg,
+                                  global_num_experts=L.E_global)
             ev[3].record()
             a2q, a2s = fuse_silu_mul_quant(c1)
             ev[4].record()
-            moe.moe_gemm_w8a8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, 1, cfg, global_num_experts=L.E_global)
+            if L.weight_bits == 4:
+                moe.invoke_fused_moe_kernel_w4a8(a2q, self.w2, c3, a2s, self.w2s, None, tw, s, e, p, True, 1, cfg,
+                                                 global_num_experts=L.E_global)
+            else:
+                moe.moe_gemm_w8a8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, 1, cfg,
+                                  global_num_experts=L.E_global)
             ev[5].record()
             moe.moe_sum(c3, out)
             ev[6].record()
@@ -398,6 +408,8 @@ def cpu_baseline(layer, weights, M_sample, seed=0):
     w1, w2, w1s, w2s = weights
     x, tw, ids = wl.make_inputs(layer, M_sample, seed=seed)
     emap = wl.expert_map_for(layer)
+    if layer.weight_bits == 4 and layer.quant == "channel":
+        return None  # no torch restatement of this form is kept: the C oracle checks it in the tests
     ref = torch_ref.torch_w4a8_group_moe if layer.weight_bits == 4 else (
         torch_ref.torch_w8a8_per_column_moe if layer.quant == "channel" else torch_ref.torch_w8a8_block_int8_moe)
     runs = []
@@ -441,7 +453,8 @@ def main():
             cpu_weights.extend(t.cpu() for t in (w1, w2, w1s, w2s))
         if lay.weight_bits == 4:
             w1, w2 = preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2)
-            w1s, w2s = preshuffle_moe_scale_int4(w1s), preshuffle_moe_scale_int4(w2s)
+            if lay.quant != "channel":
+                w1s, w2s = preshuffle_moe_scale_int4(w1s), preshuffle_moe_scale_int4(w2s)
         elif not args.row_major_weights:
             w1, w2 = preshuffle_moe_weight(w1), preshuffle_moe_weight(w2)
         return w1, w2, w1s, w2s
@@ -456,10 +469,11 @@ def main():
         other = time_steps(lambda: pt.step(args.block_size_m, flags_other), args.steps, args.warmup, flush)
     stages, bs_used = pt.stage_times(args.steps, args.warmup, flush, args.block_size_m,
                                      fused_scale=args.fused_scale == 1)
-    shape = [1, 128] if layer.weight_bits == 4 else (None if layer.quant == "channel" else [128, 128])
+    shape = None if layer.quant == "channel" else ([1, 128] if layer.weight_bits == 4 else [128, 128])
     from lightop_amd import moe as _moe
     tile1, tile2 = _moe.get_w8a8moe_json(args.tokens, layer.E, 2 * layer.I, layer.H, layer.I, True, shape, layer.top_k,
-                                         layer.E_global, preshuffled=not args.row_major_weights)
+                                         layer.E_global, preshuffled=not args.row_major_weights,
+                                         int4=layer.weight_bits == 4)
 
     # dominant kernel: the first grouped GEMM with its fused SiLU*mul + re-quantisation
     L = layer
@@ -470,7 +484,7 @@ def main():
         else (2 * L.I * L.H + 4 * (2 * L.I // 128) * (L.H // 128))
     g1_bytes = pt.E_act * g1_w + args.tokens * (L.H + 4 * L.H // 128) + pt.S_loc * (L.I + 4 * L.I // 128)
     if L.quant == "channel":  # whole-row scales; bf16 [S, 2I] out instead of int8 [S, I]
-        g1_w = 2 * L.I * L.H + 4 * 2 * L.I
+        g1_w = 2 * L.I * L.H * L.weight_bits // 8 + 4 * 2 * L.I
         g1_bytes = pt.E_act * g1_w + args.tokens * (L.H + 4) + pt.S_loc * 2 * L.I * 2
     g1_name = "gemm1" if L.quant == "channel" else "gemm1_silu_quant"
     g1_t = stages[g1_name] * 1e-3

@@ -89,8 +89,14 @@ static WsLayout ws_layout(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_
 // of slots per expert: small tiles waste no MFMA columns on padding while the layer
 // is weight-streaming bound, larger ones amortise each pass over an expert's weights.
 static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64_t H, int form = LO_FORM_BLOCK,
-                            bool preshuffled = true) {
+                            bool preshuffled = true, bool int4_channel = false) {
   const double per_expert = static_cast<double>(M) * top_k / (num_experts > 0 ? num_experts : 1);
+  // Packed int4 weights with per-channel scales: the 128-token kernel has no scale arithmetic in
+  // its K loop and skips the padded part of a block, so it takes over as soon as an expert sees more
+  // than a dozen tokens (measured on the Qwen3-235B-A22B-shaped layer, whole path in us, 16 / 32 /
+  // 64 / 128: at 128 tokens 247 / 254 / 401 / 267, at 256: 365 / 294 / 433 / 285, at 1024: 953 / 727 /
+  // 842 / 382, at 2048: 1610 / 1224 / 1455 / 596).
+  if (form == LO_FORM_CHANNEL && int4_channel) return per_expert <= 12.0 ? 16 : 128;
   // W4A8: the streaming kernel re-reads the token rows per wave, which outweighs the half-size
   // weights early; the LDS-tiled kernel (64 tokens) wins above about 8 slots per expert.
   // From 48 slots per expert on the 128-token kernel takes over (measured, 64 / 128: 475 / 394 us at
@@ -139,7 +145,8 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
              "moe_tile_query_form: bad problem size");
   if (form == LO_FORM_W4) flags |= LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED;
   const bool pre = (flags & LO_GEMM_W_PRESHUFFLED) != 0;
-  const int32_t bm = pick_block_m(M, num_experts, top_k, H, form, pre);
+  const int32_t bm = pick_block_m(M, num_experts, top_k, H, form, pre,
+                                  form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4));
   // the argument blocks the stage entry points would build for this problem
   GemmArgs a{};
   a.num_valid = M * top_k;
@@ -301,7 +308,8 @@ extern "C" int lo_fused_experts_channel_int8(
   LO_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, LO_EINVAL,
              "fused_experts(channel): workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
-  if (block_size_m == 0) block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_CHANNEL);
+  if (block_size_m == 0)
+    block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_CHANNEL, true, (flags & LO_GEMM_W4) != 0);
   LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
              LO_EINVAL, "fused_experts(channel): block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
   // the block layout is roomy enough: its scale segments hold one float per 128 values

@@ -34,7 +34,8 @@ static int validate_common(const char *who, const void *A, const void *As, const
 // query (lo_moe_tile_query_form) reports this very choice.
 int pick_gemm_kernel(const GemmArgs &a, bool fused_act, int bs, int flags) {
   const bool tiled = !(flags & LO_GEMM_FORCE_STREAMING);
-  if (a.w4 && a.per_channel) return LO_KERNEL_WS; // the reference's own int4 form: streaming kernel only
+  if (a.w4 && a.per_channel) // the reference's own int4 form: 128-token LDS tiles, else streaming
+    return tiled && gemm_t128_supports(a, fused_act, bs) ? LO_KERNEL_T128 : LO_KERNEL_WS;
   if (a.w4) { // int4 weights: 128- or 64-token LDS tiles, else streaming
     if (tiled && gemm_t128_supports(a, fused_act, bs)) return LO_KERNEL_T128;
     if (tiled && gemm_w4_tile_supports(a, fused_act, bs)) return LO_KERNEL_W4_TILE;

@@ -57,9 +57,15 @@ __device__ __forceinline__ void wait_copies_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM, bool W4>
+//
+// PC (with W4): the reference's own int4 form (fused_moe_kernel_int4_w4a8,
+// python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341-395): one scale per token row and one
+// per weight row, both applied in the epilogue, so the int32 sums run over the whole K inside the
+// MFMA accumulators and the K loop has no scale arithmetic at all.
+template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM, bool W4, bool PC = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
+  static_assert(!PC || (W4 && !FUSED_ACT && !FAST_SCALE), "per-channel scales: plain int4 GEMM only");
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   int8_t *const sA = smem + kTW;
   float *const sS = reinterpret_cast<float *>(smem + kTW + kTA);
@@ -114,9 +120,9 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   // k-steps in one 16-byte piece) and one scale per weight row and K block, [E, K/128, N]
   const int64_t wbytes = W4 ? N * K / 2 : N * K; // one expert
   const brsrc rW = make_rsrc(a.W + static_cast<int64_t>(e) * wbytes, static_cast<uint32_t>(wbytes));
-  const brsrc rWs = make_rsrc(a.Ws + static_cast<int64_t>(e) * N * KB, static_cast<uint32_t>(N * KB * 4));
+  const brsrc rWs = make_rsrc(a.Ws + static_cast<int64_t>(e) * N * (PC ? 1 : KB), static_cast<uint32_t>(N * (PC ? 1 : KB) * 4));
   const brsrc rA = make_rsrc(a.A, static_cast<uint32_t>(a.a_rows * K));
-  const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * KB * 4));
+  const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * (PC ? 1 : KB) * 4));
   const int wkstride = W4 ? shuf_kb_stride(NBLK) / 2 : shuf_kb_stride(NBLK);
   int wvoff[2][2]; // [step half][fragment]: the 2 KB block of 16 rows x 128 K, in lane order
 #pragma unroll
@@ -150,7 +156,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
     for (int p = 0; p < 4; ++p)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 1][p & 1], 0, 0, kWAux);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rWs, sWw + 4096, 4, wsvoff, 0, 0, 0);
+    if constexpr (!PC) __builtin_amdgcn_raw_ptr_buffer_load_lds(rWs, sWw + 4096, 4, wsvoff, 0, 0, 0);
   } else {
 #pragma unroll
     for (int p = 0; p < 8; ++p)
@@ -181,7 +187,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   {
     const int64_t lf = sorted[tid & (kT - 1)];
     const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
-    asoff = static_cast<int>(lrow * KB * 4);
+    asoff = static_cast<int>(lrow * (PC ? 1 : KB) * 4);
     // The epilogues take the ids from LDS: a global load in each of their exec-masked blocks is a
     // full memory round trip that nothing overlaps.
     if (tid < kT) sIds[tid] = static_cast<int32_t>(lf);
@@ -207,7 +213,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
         if (p < 4)
           __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 1][p & 1],
                                                    __builtin_amdgcn_readfirstlane(kc * wkstride), 0, kWAux);
-        else if (p == 4)
+        else if (p == 4 && !PC)
           __builtin_amdgcn_raw_ptr_buffer_load_lds(rWs, sWw + 4096, 4, wsvoff,
                                                    __builtin_amdgcn_readfirstlane(kc) * static_cast<int>(N) * 4, 0, 0);
       } else {
@@ -226,6 +232,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     for (int p = 8; p < 12; ++p) copy_piece(p, kb);
   };
   auto load_scale = [&](int kb) __attribute__((always_inline)) {
+    if constexpr (PC) return 0.0f; // one scale per token, read by the epilogue
     return bld_f32(rAs, asoff, (kb < KB ? kb : KB - 1) * 4);
   };
 
@@ -244,6 +251,13 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
       for (int rf = 0; rf < 2; ++rf)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[h][tb][rf][i] = 0.0f;
+  v4i acci[2][8][2]; // PC: the whole-K int32 sums
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int tb = 0; tb < 8; ++tb)
+#pragma unroll
+      for (int rf = 0; rf < 2; ++rf) acci[h][tb][rf] = v4i{0, 0, 0, 0};
 
   // W4: every product carries the factor 16 of the unpacked nibbles; it is taken out through the row
   // scale, which read_w() multiplies by 1/16 once per K block (a power of two: (f32(d) * a_s) * (b_s / 16)
@@ -298,9 +312,11 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
               w[h][rf][ks][2 * x + 1] = static_cast<int>(word & 0xf0f0f0f0u);
             }
           // rows of fragment (h, rf) among the wave's 64: fused 32*rf + 16*h, plain 32*h + 16*rf
-          const int row0 = (FUSED_ACT ? 32 * rf + 16 * h : 32 * h + 16 * rf) + 4 * q;
-          wsc[h][rf] = *reinterpret_cast<const v4f *>(sWw + 4096 + row0 * 4);
-          wsc[h][rf] = wsc[h][rf] * 0.0625f;
+          if constexpr (!PC) {
+            const int row0 = (FUSED_ACT ? 32 * rf + 16 * h : 32 * h + 16 * rf) + 4 * q;
+            wsc[h][rf] = *reinterpret_cast<const v4f *>(sWw + 4096 + row0 * 4);
+            wsc[h][rf] = wsc[h][rf] * 0.0625f;
+          }
         }
     } else {
 #pragma unroll
@@ -348,6 +364,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     float sc0 = 0.0f, sc1 = 0.0f; // scale products of the token fragment being folded (both row halves)
     auto fold_stage = [&](int st) __attribute__((always_inline)) { // fold the fragments of stage st
       const int tb = st >> 1, h = st & 1;
+      if constexpr (PC) return;
       if constexpr (W4) {
         fold4(dprev[0], as_p, wsc[h][0], acc[h][tb][0]);
         fold4(dprev[1], as_p, wsc[h][1], acc[h][tb][1]);
@@ -391,10 +408,14 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
         v4i d[2];
 #pragma unroll
         for (int rf = 0; rf < 2; ++rf)
-          d[rf] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[h][rf][0], bf[cur][0], cinit, 0, 0, 0);
+          d[rf] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[h][rf][0], bf[cur][0], PC ? acci[h][tb][rf] : cinit, 0, 0, 0);
 #pragma unroll
         for (int rf = 0; rf < 2; ++rf)
           d[rf] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[h][rf][1], bf[cur][1], d[rf], 0, 0, 0);
+        if constexpr (PC) {
+          acci[h][tb][0] = d[0];
+          acci[h][tb][1] = d[1];
+        }
         if (kEarly && st >= 14) { // the next K block's operands of this half, over the ones just used
 #pragma unroll
           for (int rf = 0; rf < 2; ++rf)
@@ -480,6 +501,21 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     // A lane holds 4 consecutive columns of one token per fragment.  Each wave turns a 16-token x
     // 64-column piece around in its own (now idle) weight ring and stores 128-byte row segments.
     int8_t *stg = sWw;
+    // PC: the scales of the lane's rows and of its eight tokens, fetched in one batch up front
+    v4f pbs[2][2];
+    float pas[8];
+    if constexpr (PC) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int rf = 0; rf < 2; ++rf)
+          pbs[h][rf] = __builtin_bit_cast(v4f, bld16(rWs, static_cast<int>((nrow0 + h * 32 + rf * 16 + 4 * q) * 4), 0));
+#pragma unroll
+      for (int tb = 0; tb < 8; ++tb) {
+        const int64_t ft = sIds[tb * 16 + r];
+        pas[tb] = bld_f32(rAs, static_cast<int>((ft < a.num_valid ? ft / a.top_k : 0) * 4), 0);
+      }
+    }
 #pragma unroll
     for (int tb = 0; tb < 8; ++tb) {
       if (2 * tb >= nst) continue;
@@ -494,8 +530,16 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
           v4u16 o;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            float v = acc[h][tb][rf][i];
-            if (a.mul_routed) v = v * wgt;
+            float v;
+            if constexpr (PC) { // left to right: routed weight, token scale, channel scale (w4a8.py:386-395)
+              v = static_cast<float>(acci[h][tb][rf][i]);
+              if (a.mul_routed) v = v * wgt;
+              v = v * pas[tb];
+              v = v * pbs[h][rf][i];
+            } else {
+              v = acc[h][tb][rf][i];
+              if (a.mul_routed) v = v * wgt;
+            }
             o[i] = f32_to_bf16(v);
           }
           *reinterpret_cast<v4u16 *>(stg + r * kTPitch + (h * 32 + rf * 16 + 4 * q) * 2) = o;
@@ -600,7 +644,8 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 }
 
 bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
-  if (block_size_m != 128 || !a.w_shuffled || a.per_channel) return false;
+  if (block_size_m != 128 || !a.w_shuffled) return false;
+  if (a.per_channel && (!a.w4 || fused_act)) return false; // int8 per-channel weights have gemm_pc.hip
   if (!fused_act && a.N % 64 != 0) return false;
   return a.K / kGroup <= kTMaxKB;
 }
@@ -624,6 +669,14 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
     if (rc_lds) return rc_lds;                                                                                  \
     hipLaunchKernelGGL((moe_gemm_t128_kernel<FA, FS, ST, W>), g, b, kTLds, s, a, mbi, gi);                      \
   } while (0)
+#define LO_T128_LAUNCH_PC(ST)                                                                                   \
+  do {                                                                                                          \
+    static unsigned long long lds_done = 0;                                                                     \
+    const int rc_lds = reserve_lds_once(                                                                        \
+        reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, false, ST, true, true>), kTLds, &lds_done); \
+    if (rc_lds) return rc_lds;                                                                                  \
+    hipLaunchKernelGGL((moe_gemm_t128_kernel<false, false, ST, true, true>), g, b, kTLds, s, a, mbi, gi);       \
+  } while (0)
 #define LO_T128_PICK(FA, FS)                                                                                    \
   do {                                                                                                          \
     if (a.w4) {                                                                                                 \
@@ -636,7 +689,10 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
   } while (0)
   // one token block per expert, by and large: the slots spread over the routed experts fill half a block
   const bool stream = a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * (kT / 2);
-  if (fused_act) {
+  if (a.per_channel) {
+    if (stream) LO_T128_LAUNCH_PC(true);
+    else LO_T128_LAUNCH_PC(false);
+  } else if (fused_act) {
     if (fast) LO_T128_PICK(true, true);
     else LO_T128_PICK(true, false);
   } else {
@@ -644,6 +700,7 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
     else LO_T128_PICK(false, false);
   }
 #undef LO_T128_PICK
+#undef LO_T128_LAUNCH_PC
 #undef LO_T128_LAUNCH
   return check_launch(fused_act ? "moe_gemm1_silu_quant(t128)" : "moe_gemm(t128)");
 }

@@ -13,12 +13,15 @@ from ..op import _act_dtype, _ids_dtype, _on_device, _require_cuda
 
 def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bool,
                      block_shape: Optional[List[int]], topk: int,
-                     global_num_experts: int = -1, preshuffled: bool = True) -> Tuple[Dict[str, Any], Dict[str, Any]]:
+                     global_num_experts: int = -1, preshuffled: bool = True,
+                     int4: bool = False) -> Tuple[Dict[str, Any], Dict[str, Any]]:
     """Tile configuration of both GEMMs for ``m`` tokens (reference: get_w8a8moe_json,
     int8.py:220-256, backed there by per-device JSON files).  Here the table is compiled
     into the library; the dictionaries keep the reference's keys.  ``n1`` = 2*I, ``n2`` = H,
     ``k`` = I.  ``block_shape=None`` asks for the per-channel form (the reference consults
     get_moe_cuda_config first there, int8.py:735-741), ``[1, 128]`` for W4A8 with K-group scales.
+    ``int4`` with ``block_shape=None``: the reference's own W4A8 form (w4a8.py:587, which passes only
+    the first five arguments).
     ``preshuffled``: the weights are in the load-time layout of ``preshuffle_moe_weight`` (the table
     differs for row-major weights).  ``kernel`` / ``num_warps`` / ``BLOCK_SIZE_N`` describe the kernel
     the stage calls launch for that ``BLOCK_SIZE_M``."""
@@ -28,6 +31,8 @@ def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bo
     form = _lib.LO_FORM_CHANNEL if block_shape is None else (
         _lib.LO_FORM_W4 if list(block_shape) == [1, 128] else _lib.LO_FORM_BLOCK)
     flags = _lib.LO_GEMM_W_PRESHUFFLED if preshuffled else 0
+    if int4 and block_shape is None:
+        flags |= _lib.LO_GEMM_W4 | _lib.LO_GEMM_W_PRESHUFFLED
     _lib.check(_lib.lib().lo_moe_tile_query_form(form, flags, m, E, Eg, topk, n2, k, t1, t2))
 
     def as_dict(t):

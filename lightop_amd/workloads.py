@@ -161,7 +161,9 @@ def algorithmic_work(layer: MoeLayer, topk_ids: torch.Tensor, expert_map: Option
     E_act = int(torch.unique(local).numel())
     H, I = layer.H, layer.I
     M = topk_ids.shape[0]
-    if layer.weight_bits == 4:  # half a byte per weight, one scale per row and K group
+    if layer.weight_bits == 4 and layer.quant == "channel":  # half a byte per weight, one scale per row
+        per_expert = 3 * I * H // 2 + 4 * (2 * I + H)
+    elif layer.weight_bits == 4:  # half a byte per weight, one scale per row and K group
         per_expert = 3 * I * H // 2 + 4 * (2 * I * (H // 128) + H * (I // 128))
     elif layer.quant == "channel":
         per_expert = 3 * I * H + 4 * (2 * I + H)

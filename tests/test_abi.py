@@ -125,9 +125,10 @@ def test_tile_query_names_the_kernel_that_is_launched(lib):
     assert q(_lib.LO_FORM_BLOCK, pre | _lib.LO_GEMM_FORCE_STREAMING, 8192, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_WS
     # per-channel and int4 forms
     assert q(_lib.LO_FORM_CHANNEL, pre, 8192, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_PC == t2.kernel
-    # the reference's own int4 form (per-channel scales on packed int4 weights): the streaming kernel only
+    # the reference's own int4 form (per-channel scales on packed int4 weights): 128-token tiles or streaming
     assert q(_lib.LO_FORM_CHANNEL, pre | _lib.LO_GEMM_W4, 8192, *qwen) == 0
-    assert t1.kernel == _lib.LO_KERNEL_WS == t2.kernel and t1.block_size_m == 128
+    assert t1.kernel == _lib.LO_KERNEL_T128 == t2.kernel and t1.block_size_m == 128
+    assert q(_lib.LO_FORM_CHANNEL, pre | _lib.LO_GEMM_W4, 16, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_WS == t2.kernel
     assert q(_lib.LO_FORM_W4, 0, 2, *dsv3) == 0 and t1.kernel == _lib.LO_KERNEL_DEC  # int4: up to 16 slots
     assert q(_lib.LO_FORM_W4, 0, 4, *dsv3) == 0 and t1.kernel == _lib.LO_KERNEL_WS
     assert q(_lib.LO_FORM_W4, 0, 512, *dsv3) == 0 and t1.kernel == _lib.LO_KERNEL_W4_TILE
