@@ -70,7 +70,11 @@ enum {
    * NO_DECODE_PATH: never take it.  FORCE_DECODE_PATH: take it whenever it can serve the problem
    * (at most 512 routed slots), whatever the size heuristic says. */
   LO_FUSED_NO_DECODE_PATH = 64,
-  LO_FUSED_FORCE_DECODE_PATH = 128
+  LO_FUSED_FORCE_DECODE_PATH = 128,
+  /* whole-path calls only: activation="gelu" (int8.py:825-838, w4a8.py:602-605) instead of SiLU.
+   * No fused epilogue exists for it: the first GEMM writes bf16 [S, 2I], one launch applies
+   * GELU-and-mul and quantises, so cache3 / cache13 must hold S * max(2I, H) elements. */
+  LO_FUSED_ACT_GELU = 256
 };
 
 int lo_version(void);
@@ -221,6 +225,18 @@ int lo_moe_gemm1_silu_quant_block_int8(const int8_t *A, const float *As, const i
  */
 int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *act,
                     lo_stream_t stream);
+
+/*
+ * GELU-and-mul, erf form: act[f, i] = T( T(gelu(c1[f, i])) * c1[f, I + i] ),
+ * gelu(x) = (x * 0.5f) * (1.0f + erf(x * float(M_SQRT1_2))) in fp32 with erf correctly rounded.
+ * Replaces torch.ops._C.gelu_and_mul at int8.py:826 (in-repo twin: gelu_and_mul_opt,
+ * csrc/kernels/activation_kernels_opt.cu:234-242, :159-161, :319-323).
+ */
+int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *act,
+                    lo_stream_t stream);
+/* The 65536 bf16 values bf16(gelu(g)), indexed by the bit pattern of g, that the GELU kernels look
+ * up, copied to table_out (device memory, 128 KB).  For tests; no counterpart in the reference. */
+int lo_gelu_bf16_table(void *table_out, lo_stream_t stream);
 
 /*
  * Top-k reduction back to token order: out[t, :] = factor * sum_j in[t, j, :] (+ bias[t, :]).

@@ -249,7 +249,9 @@ extern "C" int lo_fused_experts_block_int8(
   const int64_t S = M * top_k;
 
   // Decode sizes: routing, quantisation, both GEMMs and the reduction in two launches.
-  if (block_size_m_auto && (flags & (LO_GEMM_W_PRESHUFFLED | LO_GEMM_W4)) && !(flags & LO_FUSED_NO_DECODE_PATH)) {
+  const bool gelu = (flags & LO_FUSED_ACT_GELU) != 0;
+  if (block_size_m_auto && (flags & (LO_GEMM_W_PRESHUFFLED | LO_GEMM_W4)) &&
+      !(flags & (LO_FUSED_NO_DECODE_PATH | LO_FUSED_ACT_GELU))) {
     // (cache3 is the front of the caller's cache13: the path keeps its bf16 activations [S, I] there)
     const int rc2 = launch_decode_path(x, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w, topk_ids, ids_dtype,
                                        expert_map, apply_router_weight_on_input, routed_scaling_factor, shared_output,
@@ -270,14 +272,23 @@ extern "C" int lo_fused_experts_block_int8(
                                     L.align_scratch, stream);
   }
   if (rc) return rc;
-  rc = lo_moe_gemm1_silu_quant_block_int8(a1q, a1s, w1, w1s, a2q, a2s, dtype, topk_w, sorted, eids,
-                                          ntpp, L.sorted_cap, S, M, E, num_experts, I, H, top_k, block_size_m,
-                                          apply_router_weight_on_input, flags, stream);
+  if (gelu) {
+    // rows of experts on other ranks are zero-filled by the first GEMM: the activation launch reads every row
+    rc = lo_moe_gemm_block_int8(a1q, a1s, w1, w1s, cache3, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, M, E,
+                                num_experts, 2 * I, H, top_k, block_size_m, apply_router_weight_on_input,
+                                flags & ~LO_FUSED_ACT_GELU, stream);
+    if (rc) return rc;
+    rc = launch_gelu_mul_group_quant(cache3, S, I, a2q, a2s, static_cast<hipStream_t>(stream));
+  } else {
+    rc = lo_moe_gemm1_silu_quant_block_int8(a1q, a1s, w1, w1s, a2q, a2s, dtype, topk_w, sorted, eids,
+                                            ntpp, L.sorted_cap, S, M, E, num_experts, I, H, top_k, block_size_m,
+                                            apply_router_weight_on_input, flags, stream);
+  }
   if (rc) return rc;
   rc = lo_moe_gemm_block_int8(a2q, a2s, w2, w2s, cache3, dtype, topk_w, sorted, eids, ntpp,
                               L.sorted_cap, S, S, E, num_experts, H, I, 1, block_size_m,
-                              !apply_router_weight_on_input, flags | (mask ? LO_GEMM_SKIP_NONLOCAL : 0),
-                              stream);
+                              !apply_router_weight_on_input,
+                              (flags & ~LO_FUSED_ACT_GELU) | (mask ? LO_GEMM_SKIP_NONLOCAL : 0), stream);
   if (rc) return rc;
   return lo_moe_sum(cache3, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor,
                     nullptr, stream);
@@ -335,14 +346,18 @@ extern "C" int lo_fused_experts_channel_int8(
                                   L.align_scratch, stream);
   if (rc) return rc;
   // rows of experts on other ranks are zero-filled here: the activation kernel reads every row
+  const int gflags = flags & ~LO_FUSED_ACT_GELU;
   rc = lo_moe_gemm_w8a8(a1q, a1s, w1, w1s, cache13, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, M, E,
-                        num_experts, 2 * I, H, top_k, block_size_m, apply_router_weight_on_input, flags, stream);
+                        num_experts, 2 * I, H, top_k, block_size_m, apply_router_weight_on_input, gflags, stream);
   if (rc) return rc;
-  rc = lo_fuse_silu_mul_quant(cache13, dtype, S, I, a2q, a2s, nullptr, 1, stream);
+  if (flags & LO_FUSED_ACT_GELU) // gelu_and_mul, then per_token_quant_int8 with its floor (int8.py:826-838)
+    rc = launch_gelu_mul_row_quant(cache13, S, I, a2q, a2s, static_cast<hipStream_t>(stream));
+  else
+    rc = lo_fuse_silu_mul_quant(cache13, dtype, S, I, a2q, a2s, nullptr, 1, stream);
   if (rc) return rc;
   rc = lo_moe_gemm_w8a8(a2q, a2s, w2, w2s, cache13, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, S, E,
                         num_experts, H, I, 1, block_size_m, !apply_router_weight_on_input,
-                        flags | (mask ? LO_GEMM_SKIP_NONLOCAL : 0), stream);
+                        gflags | (mask ? LO_GEMM_SKIP_NONLOCAL : 0), stream);
   if (rc) return rc;
   return lo_moe_sum(cache13, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor, nullptr,
                     stream);

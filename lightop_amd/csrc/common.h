@@ -38,6 +38,12 @@ void set_error(const char *fmt, ...);
 int check_launch(const char *what);
 // bf16(silu(g)) for all 65536 bf16 patterns g, built on first use (per device).
 int silu_table(hipStream_t stream, const uint16_t **table);
+// bf16(gelu(g)), erf form, the same way.
+int gelu_table(hipStream_t stream, const uint16_t **table);
+// GELU-and-mul of c1 [rows, 2I] followed by the 1x128 group quantisation (q [rows, I], s [rows, I/128])
+// or by the per-token quantisation (s [rows]), one launch each.
+int launch_gelu_mul_group_quant(const void *c1, int64_t rows, int64_t I, int8_t *q, float *s, hipStream_t stream);
+int launch_gelu_mul_row_quant(const void *c1, int64_t rows, int64_t I, int8_t *q, float *s, hipStream_t stream);
 
 // Raises a kernel's dynamic-LDS limit once per device instead of on every launch (kernels that use
 // more than the default 64 KB).  `done` is the call site's own static flag set, one bit per device.

@@ -40,6 +40,61 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
   }
 }
 
+// ---- gelu_and_mul ----------------------------------------------------------------
+// Reference: torch.ops._C.gelu_and_mul as called at int8.py:826; in-repo twin gelu_and_mul_opt,
+// csrc/kernels/activation_kernels_opt.cu:234-242 (erf form) and :159-161 (product in the tensor's
+// type): act = T(T(gelu(g)) * u).  bf16(gelu(g)) comes from a 64K-entry table (gelu_table below).
+__global__ __launch_bounds__(256) void gelu_mul_kernel(const uint16_t *__restrict__ c1, int64_t rows, int64_t I,
+                                                       const uint16_t *__restrict__ table,
+                                                       uint16_t *__restrict__ act) {
+  const int64_t vec_per_row = I / 8;
+  const int64_t total = rows * vec_per_row;
+  for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < total;
+       v += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t r = v / vec_per_row, c = (v % vec_per_row) * 8;
+    const v8u16 g = *reinterpret_cast<const v8u16 *>(c1 + r * 2 * I + c);
+    const v8u16 u = *reinterpret_cast<const v8u16 *>(c1 + r * 2 * I + I + c);
+    v8u16 o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = silu_mul_tab(table, g[i], u[i]);
+    *reinterpret_cast<v8u16 *>(act + r * I + c) = o;
+  }
+}
+
+// The same followed by the 1x128 group quantisation of per_token_group_quant_int8 (the pair of
+// calls at int8.py:826-838 on the block-shape branch) in one pass: c1 [rows, 2I] -> q [rows, I],
+// s [rows, I/128].  16 lanes own one group, as in group_quant_body.
+__global__ __launch_bounds__(256) void gelu_mul_group_quant_kernel(const uint16_t *__restrict__ c1, int64_t rows,
+                                                                   int64_t I, const uint16_t *__restrict__ table,
+                                                                   float eps, int8_t *__restrict__ q,
+                                                                   float *__restrict__ s) {
+  const int64_t gpr = I / kGroup, groups = rows * gpr;
+  const int sub = threadIdx.x & 15;
+  for (int64_t g = static_cast<int64_t>(blockIdx.x) * 16 + (threadIdx.x >> 4); g < groups;
+       g += static_cast<int64_t>(gridDim.x) * 16) {
+    const int64_t r = g / gpr, c = (g % gpr) * kGroup + sub * 8;
+    const v8u16 ga = *reinterpret_cast<const v8u16 *>(c1 + r * 2 * I + c);
+    const v8u16 up = *reinterpret_cast<const v8u16 *>(c1 + r * 2 * I + I + c);
+    float v[8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      v[i] = bf16_to_f32(silu_mul_tab(table, ga[i], up[i]));
+      amax = fmaxf(amax, fabsf(v[i]));
+    }
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+    amax = fmaxf(amax, eps);
+    const float sc = amax / 127.0f;
+    const float rsc = 1.0f / sc;
+    v2i packed;
+    packed[0] = static_cast<int>(quant4(&v[0], sc, rsc));
+    packed[1] = static_cast<int>(quant4(&v[4], sc, rsc));
+    *reinterpret_cast<v2i *>(q + r * I + c) = packed;
+    if (sub == 0) s[g] = sc;
+  }
+}
+
 // ---- per-token int8 quantisation, plain and behind SiLU-and-mul ----------------------
 // Reference: per_token_quant_int8, python/lightop/_lmslim_native/layers/gemm/int8_utils.py:20-44
 // (amax floored at 1e-10, s = amax / 127, q = rne(x * (127 / amax))) and fuse_silu_mul_quant,
@@ -47,17 +102,21 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
 // no floor: a zero row gets scale 0 and multiplier 0).  One workgroup per row; a thread keeps
 // up to CH 8-value pieces of the row in registers between the amax pass and the rounding pass,
 // longer rows are read a second time.
+// ACT: 0 plain rows; 1 SiLU-and-mul first (the fused kernel above: no floor); 2 GELU-and-mul first,
+// then per_token_quant_int8 with its floor (the two calls at int8.py:826-838 on the per-channel
+// branch), `silu` being the GELU table then.
 __device__ __forceinline__ int rne_i8(float v) {
   v = fminf(fmaxf(v, -128.0f), 127.0f);
   return static_cast<int>(__builtin_rintf(v)); // v_rndne_f32: ties to even
 }
 
-template <bool SILU, int CH>
+template <int ACT, int CH>
 __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restrict__ x, int64_t rows, int64_t C,
                                                         const uint16_t *__restrict__ silu, int8_t *__restrict__ q,
                                                         float *__restrict__ s,
                                                         const int32_t *__restrict__ num_local_tokens, int32_t top_k,
                                                         const int32_t *__restrict__ row_ids) {
+  constexpr bool SILU = ACT == 1, GATED = ACT != 0;
   __shared__ float sRed[4];
   __shared__ uint16_t sSilu[SILU ? 2 * kSiluBandN : 2];
   const int tid = threadIdx.x;
@@ -72,17 +131,18 @@ __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restri
     silu_band_store(sSilu, band_regs, tid);
     __syncthreads();
   }
-  const int64_t in_stride = SILU ? 2 * C : C; // C = output columns
+  const int64_t in_stride = GATED ? 2 * C : C; // C = output columns
   const int pieces = static_cast<int>(C / 8);
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     if (row_ids && row_ids[row] == -1) continue; // a row of an expert held elsewhere: left untouched
     const uint16_t *xr = x + row * in_stride;
     auto piece = [&](int p, float (&v)[8]) {
       const v8u16 a = *reinterpret_cast<const v8u16 *>(xr + p * 8);
-      if constexpr (SILU) {
+      if constexpr (GATED) {
         const v8u16 u = *reinterpret_cast<const v8u16 *>(xr + C + p * 8);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = bf16_to_f32(silu_mul_band(sSilu, silu, a[i], u[i]));
+        for (int i = 0; i < 8; ++i)
+          v[i] = bf16_to_f32(SILU ? silu_mul_band(sSilu, silu, a[i], u[i]) : silu_mul_tab(silu, a[i], u[i]));
       } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = bf16_to_f32(a[i]);
@@ -140,12 +200,13 @@ __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restri
 
 // The same for rows of at most 512 * CH values: one wavefront per row, four rows per workgroup,
 // the row stays in registers and the reduction needs no barrier.
-template <bool SILU, int CH>
+template <int ACT, int CH>
 __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__restrict__ x, int64_t rows, int64_t C,
                                                              const uint16_t *__restrict__ silu,
                                                              int8_t *__restrict__ q, float *__restrict__ s,
                                                              const int32_t *__restrict__ num_local_tokens,
                                                              int32_t top_k, const int32_t *__restrict__ row_ids) {
+  constexpr bool SILU = ACT == 1, GATED = ACT != 0;
   __shared__ uint16_t sSilu[SILU ? 2 * kSiluBandN : 2];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   if (num_local_tokens) {
@@ -159,7 +220,7 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
     silu_band_store(sSilu, band_regs, tid);
     __syncthreads();
   }
-  const int64_t in_stride = SILU ? 2 * C : C;
+  const int64_t in_stride = GATED ? 2 * C : C;
   const int pieces = static_cast<int>(C / 8);
   for (int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + wave; row < rows; row += static_cast<int64_t>(gridDim.x) * 4) {
     if (row_ids && row_ids[row] == -1) continue; // a row of an expert held elsewhere: left untouched
@@ -170,7 +231,7 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
       const int p = lane + 64 * j;
       const int pc = p < pieces ? p : 0; // lanes past the row re-read its start and are ignored
       ga[j] = *reinterpret_cast<const v8u16 *>(xr + pc * 8);
-      if constexpr (SILU) up[j] = *reinterpret_cast<const v8u16 *>(xr + C + pc * 8);
+      if constexpr (GATED) up[j] = *reinterpret_cast<const v8u16 *>(xr + C + pc * 8);
     }
     float v[CH][8];
     float amax = 0.0f;
@@ -180,6 +241,7 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if constexpr (SILU) v[j][i] = bf16_to_f32(silu_mul_band(sSilu, silu, ga[j][i], up[j][i]));
+        else if constexpr (GATED) v[j][i] = bf16_to_f32(silu_mul_tab(silu, ga[j][i], up[j][i]));
         else v[j][i] = bf16_to_f32(ga[j][i]);
         amax = fmaxf(amax, live ? fabsf(v[j][i]) : 0.0f);
       }
@@ -206,7 +268,7 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
   }
 }
 
-template <bool SILU>
+template <int ACT>
 static void launch_row_quant(const uint16_t *x, int64_t rows, int64_t C, const uint16_t *silu, int8_t *q, float *s,
                              const int32_t *nlt, int32_t top_k, const int32_t *row_ids, hipStream_t st) {
   const int pieces = static_cast<int>(C / 8);
@@ -214,13 +276,13 @@ static void launch_row_quant(const uint16_t *x, int64_t rows, int64_t C, const u
     int64_t grid = (rows + 3) / 4;
     if (grid > 256 * 32) grid = 256 * 32;
     const dim3 g(static_cast<unsigned>(grid)), b(256);
-    if (pieces <= 64) hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 1>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
-    else if (pieces <= 128) hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 2>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
-    else hipLaunchKernelGGL((row_quant_wave_kernel<SILU, 4>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
+    if (pieces <= 64) hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 1>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
+    else if (pieces <= 128) hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 2>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
+    else hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 4>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
     return;
   }
   const unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
-  hipLaunchKernelGGL((row_quant_kernel<SILU, SILU ? 2 : 4>), dim3(grid), dim3(256), 0, st, x, rows, C, silu, q, s, nlt,
+  hipLaunchKernelGGL((row_quant_kernel<ACT, ACT ? 2 : 4>), dim3(grid), dim3(256), 0, st, x, rows, C, silu, q, s, nlt,
                      top_k, row_ids);
 }
 
@@ -304,6 +366,19 @@ __global__ __launch_bounds__(256) void silu_table_init_kernel(uint16_t *table) {
   table[i] = f32_to_bf16(g / (1.0f + det_expf(-g)));
 }
 
+// bf16(gelu(g)) for every bf16 pattern g: (f * 0.5f) * (1.0f + erf(f * ALPHA)) in fp32 with erf
+// correctly rounded to fp32 (taken in double precision and rounded once more), the form of
+// csrc/kernels/activation_kernels_opt.cu:234-242.  Built once per device.
+__device__ uint16_t g_gelu_bf16_table[65536];
+
+__global__ __launch_bounds__(256) void gelu_table_init_kernel(uint16_t *table) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  const float f = bf16_to_f32(static_cast<uint16_t>(i));
+  const float alpha = 0.70710678118654752440f;
+  const float e = static_cast<float>(erf(static_cast<double>(f * alpha)));
+  table[i] = f32_to_bf16((f * 0.5f) * (1.0f + e));
+}
+
 static int grid_for(int64_t work_items, int per_block) {
   int64_t b = (work_items + per_block - 1) / per_block;
   if (b < 1) b = 1;
@@ -313,6 +388,60 @@ static int grid_for(int64_t work_items, int per_block) {
 
 static std::mutex g_table_mutex;
 static const uint16_t *g_table_ptr[64] = {};
+static const uint16_t *g_gelu_ptr[64] = {};
+
+int gelu_table(hipStream_t stream, const uint16_t **out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    set_error("gelu table: no current HIP device");
+    return LO_ELAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_table_mutex);
+  if (!g_gelu_ptr[dev]) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) {
+      set_error("the first GELU call on a device builds its table and must not be captured: "
+                "run the op once before capturing a graph");
+      return LO_EINVAL;
+    }
+    uint16_t *p = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(g_gelu_bf16_table)) != hipSuccess || !p) {
+      set_error("gelu table: hipGetSymbolAddress failed");
+      return LO_ELAUNCH;
+    }
+    hipLaunchKernelGGL(gelu_table_init_kernel, dim3(256), dim3(256), 0, stream, p);
+    int rc = check_launch("gelu_table_init");
+    if (rc) return rc;
+    if (hipStreamSynchronize(stream) != hipSuccess) {
+      set_error("gelu table: synchronisation failed");
+      return LO_ELAUNCH;
+    }
+    g_gelu_ptr[dev] = p;
+  }
+  *out = g_gelu_ptr[dev];
+  return LO_OK;
+}
+
+// The two launches between the GEMMs when the activation is GELU (no fused epilogue exists for it).
+int launch_gelu_mul_group_quant(const void *c1, int64_t rows, int64_t I, int8_t *q, float *s, hipStream_t stream) {
+  const uint16_t *table = nullptr;
+  int rc = gelu_table(stream, &table);
+  if (rc) return rc;
+  const int64_t groups = rows * (I / kGroup);
+  if (groups == 0) return LO_OK;
+  hipLaunchKernelGGL(gelu_mul_group_quant_kernel, dim3(grid_for(groups, 16)), dim3(256), 0, stream,
+                     static_cast<const uint16_t *>(c1), rows, I, table, 1e-10f, q, s);
+  return check_launch("gelu_mul_group_quant");
+}
+
+int launch_gelu_mul_row_quant(const void *c1, int64_t rows, int64_t I, int8_t *q, float *s, hipStream_t stream) {
+  const uint16_t *table = nullptr;
+  int rc = gelu_table(stream, &table);
+  if (rc) return rc;
+  if (rows == 0) return LO_OK;
+  launch_row_quant<2>(static_cast<const uint16_t *>(c1), rows, I, table, q, s, nullptr, 1, nullptr, stream);
+  return check_launch("gelu_mul_row_quant");
+}
 
 int silu_table(hipStream_t stream, const uint16_t **out) {
   int dev = 0;
@@ -384,6 +513,38 @@ extern "C" int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
   return check_launch("silu_and_mul");
 }
 
+extern "C" int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *act,
+                               lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(c1 && act, LO_EINVAL, "gelu_and_mul: null pointer");
+  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "gelu_and_mul: only bf16 is built");
+  LO_REQUIRE(rows >= 0 && I > 0 && I % 8 == 0, LO_EINVAL, "gelu_and_mul: I (%lld) must be a multiple of 8",
+             (long long)I);
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(act) & 15) == 0,
+             LO_EINVAL, "gelu_and_mul: pointers must be 16-byte aligned");
+  const uint16_t *table = nullptr;
+  int rc = gelu_table(static_cast<hipStream_t>(stream), &table);
+  if (rc) return rc;
+  if (rows == 0) return LO_OK;
+  hipLaunchKernelGGL(gelu_mul_kernel, dim3(grid_for(rows * (I / 8), 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I, table,
+                     static_cast<uint16_t *>(act));
+  return check_launch("gelu_and_mul");
+}
+
+extern "C" int lo_gelu_bf16_table(void *table_out, lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(table_out, LO_EINVAL, "gelu_bf16_table: null pointer");
+  const uint16_t *table = nullptr;
+  int rc = gelu_table(static_cast<hipStream_t>(stream), &table);
+  if (rc) return rc;
+  if (hipMemcpyAsync(table_out, table, 65536 * 2, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)) != hipSuccess) {
+    set_error("gelu_bf16_table: copy failed");
+    return LO_ELAUNCH;
+  }
+  return LO_OK;
+}
+
 extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uint8_t *expert_mask,
                           int dtype, int64_t M, int32_t topk, int64_t H, float factor,
                           const int32_t *num_local_tokens, lo_stream_t stream) {
@@ -430,7 +591,7 @@ extern "C" int lo_per_token_quant_int8(const void *x, int x_dtype, int64_t rows,
   LO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0,
              LO_EINVAL, "per_token_quant_int8: x must be 16-byte and q 8-byte aligned");
   if (rows == 0) return LO_OK;
-  launch_row_quant<false>(static_cast<const uint16_t *>(x), rows, cols, nullptr, q, s, nullptr, 1, nullptr,
+  launch_row_quant<0>(static_cast<const uint16_t *>(x), rows, cols, nullptr, q, s, nullptr, 1, nullptr,
                           static_cast<hipStream_t>(stream));
   return check_launch("per_token_quant_int8");
 }
@@ -449,7 +610,7 @@ extern "C" int lo_fuse_silu_mul_quant_ids(const void *c1, int dtype, int64_t row
   const uint16_t *table = nullptr;
   int rc = silu_table(static_cast<hipStream_t>(stream), &table);
   if (rc) return rc;
-  launch_row_quant<true>(static_cast<const uint16_t *>(c1), rows, I, table, q, s, num_local_tokens, top_k,
+  launch_row_quant<1>(static_cast<const uint16_t *>(c1), rows, I, table, q, s, num_local_tokens, top_k,
                          row_expert_ids, static_cast<hipStream_t>(stream));
   return check_launch("fuse_silu_mul_quant");
 }

@@ -16,6 +16,7 @@ _NATIVE_APIS = {
     "invoke_fused_moe_kernel_w4a8",
     "invoke_fused_moe_gemm1_silu_quant",
     "silu_and_mul",
+    "gelu_and_mul",
     "fused_experts_workspace_bytes",
     "fused_experts_workspace_views",
     "preshuffle_moe_weight",
@@ -37,6 +38,7 @@ __all__ = [
     "fused_experts_workspace_bytes",
     "fused_experts_workspace_views",
     "get_moe_cache",
+    "gelu_and_mul",
     "get_w8a8moe_json",
     "invoke_fused_moe_gemm1_silu_quant",
     "invoke_fused_moe_kernel_int8",

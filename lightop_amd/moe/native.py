@@ -272,6 +272,18 @@ def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
                                               _lib.stream_of(x)))
 
 
+def gelu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
+    """out[:, i] = T(T(gelu(x[:, i])) * x[:, d + i]), gelu in its erf form (the op called at int8.py:826;
+    in-repo twin gelu_and_mul_opt, csrc/kernels/activation_kernels_opt.cu:234-242)."""
+    _require_cuda(out, x)
+    assert x.is_contiguous() and out.is_contiguous() and x.shape[-1] == 2 * out.shape[-1]
+    I = out.shape[-1]
+    rows = out.numel() // I
+    with _on_device(x):
+        _lib.check(_lib.lib().lo_gelu_and_mul(_lib.ptr(x), _act_dtype(x), rows, I, _lib.ptr(out),
+                                              _lib.stream_of(x)))
+
+
 @functools.lru_cache(maxsize=256)
 def fused_experts_workspace_bytes(M: int, top_k: int, H: int, I: int, num_experts: int,
                                   block_size_m: int = 0) -> int:
@@ -342,7 +354,8 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     Same signature as the reference (int8.py:628-656).  This build implements the branches
     ``use_int8_w8a8=True, block_shape=[128, 128]`` and ``use_int8_w8a8=True,
     per_channel_quant=True, block_shape=None`` (one scale per token and per weight row,
-    ``w1_scale`` [E, 2I, 1], ``w2_scale`` [E, H, 1]) with ``activation="silu"``; every other
+    ``w1_scale`` [E, 2I, 1], ``w2_scale`` [E, H, 1]) with ``activation="silu"`` or ``"gelu"`` (the
+    latter without the fused epilogue: one more launch and a bf16 round trip of [S, 2I]); every other
     combination raises.  ``cache13`` is the caller's workspace (dtype of ``hidden_states``,
     at least ``min(M, CHUNK) * topk * max(2I, H)`` elements); its first ``M*topk*H``
     elements receive the second GEMM's per-slot output.  The top-k reduction is always
@@ -363,9 +376,7 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     channel = bool(per_channel_quant) and block_shape is None  # int8.py:285-295: per-token x per-channel
     if not channel and (per_channel_quant or block_shape is None or list(block_shape) != [128, 128]):
         raise NotImplementedError("lightop_amd: block_shape must be [128, 128], or None with per_channel_quant=True")
-    if activation != "silu":
-        if activation == "gelu":
-            raise NotImplementedError("lightop_amd: the gelu activation is not built")
+    if activation not in ("silu", "gelu"):
         raise ValueError(f"Unsupported FusedMoe activation: {activation}")
     if hidden_states.dtype != torch.bfloat16:
         raise NotImplementedError("lightop_amd: hidden_states must be bfloat16")
@@ -393,7 +404,7 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     assert cache13.dtype == hidden_states.dtype and cache13.is_contiguous()
     assert cache13.numel() >= M * top_k_num * max(N, H), "cache13 is too small"
 
-    flags = int(extra.get("lightop_amd_flags", 0))
+    flags = int(extra.get("lightop_amd_flags", 0)) | (_lib.LO_FUSED_ACT_GELU if activation == "gelu" else 0)
     if extra.get("lightop_amd_weights_preshuffled", False):
         flags |= _lib.LO_GEMM_W_PRESHUFFLED
     return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
@@ -439,7 +450,7 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     group (``w1_scale`` [E, 2I, H/128], ``w2_scale`` [E, H, I/128], or their load-time form from
     ``preshuffle_moe_scale_int4``), activations quantised per 1x128 group on the fly.
 
-    SiLU only; the reduce is always performed.
+    ``activation``: "silu" or "gelu"; the reduce is always performed.
     """
     extra = _
     assert hidden_states.shape[1] == w1.shape[2] * 2, "Hidden size mismatch"  # w4a8.py:503
@@ -452,9 +463,7 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     if not channel and list(block_shape) != [1, 128]:
         raise NotImplementedError("lightop_amd: W4A8 is built for block_shape=None (per token x per channel) "
                                   "and for K-group scales, block_shape=[1, 128]")
-    if activation != "silu":
-        if activation == "gelu":
-            raise NotImplementedError("lightop_amd: the gelu activation is not built")
+    if activation not in ("silu", "gelu"):
         raise ValueError(f"Unsupported FusedMoe activation: {activation}")
     if hidden_states.dtype != torch.bfloat16:
         raise NotImplementedError("lightop_amd: hidden_states must be bfloat16")
@@ -479,7 +488,8 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
         M = min(num_tokens, envs.LMSLIM_FUSED_MOE_CHUNK_SIZE)
         assert cache13.dtype == hidden_states.dtype and cache13.is_contiguous()
         assert cache13.numel() >= M * topk_ids.shape[1] * max(N, H), "cache13 is too small"
-        flags = int(extra.get("lightop_amd_flags", 0)) | _lib.LO_GEMM_W4
+        flags = int(extra.get("lightop_amd_flags", 0)) | _lib.LO_GEMM_W4 | (
+        _lib.LO_FUSED_ACT_GELU if activation == "gelu" else 0)
         return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
                                   apply_router_weight_on_input, global_num_experts, expert_map,
                                   w1_scale.reshape(E, N), w2_scale.reshape(E, H), routed_scaling_factor,
@@ -497,7 +507,8 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
     M = min(num_tokens, envs.LMSLIM_FUSED_MOE_CHUNK_SIZE)
     assert cache13.dtype == hidden_states.dtype and cache13.is_contiguous()
     assert cache13.numel() >= M * topk_ids.shape[1] * max(N, H), "cache13 is too small"
-    flags = int(extra.get("lightop_amd_flags", 0)) | _lib.LO_GEMM_W4
+    flags = int(extra.get("lightop_amd_flags", 0)) | _lib.LO_GEMM_W4 | (
+        _lib.LO_FUSED_ACT_GELU if activation == "gelu" else 0)
     return _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace,
                               apply_router_weight_on_input, global_num_experts, expert_map, w1_scale, w2_scale,
                               routed_scaling_factor, shared_output, I, flags,
@@ -574,5 +585,5 @@ def ctypes_void(addr: int):
 __all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "preshuffle_moe_weight",
            "preshuffle_moe_weight_int4", "preshuffle_moe_scale_int4", "invoke_fused_moe_kernel_int8",
            "invoke_fused_moe_kernel_w4a8",
-           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "fused_experts_workspace_bytes",
+           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "gelu_and_mul", "fused_experts_workspace_bytes",
            "fused_experts_workspace_views", "moe_gemm_w8a8"]

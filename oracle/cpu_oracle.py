@@ -213,6 +213,22 @@ def silu_and_mul(c1):
     return act
 
 
+def gelu_and_mul(c1):
+    """act = bf16(bf16(gelu(g)) * u), gelu with erf (activation_kernels_opt.cu:234-242)."""
+    S, N = c1.shape
+    act = torch.empty(S, N // 2, dtype=torch.bfloat16)
+    lib().orc_gelu_and_mul(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(act))
+    return act
+
+
+def gelu_bf16_table():
+    """bf16(gelu(g)) for every bf16 pattern g, as int16 [65536]."""
+    fn = lib().orc_gelu_bf16
+    fn.restype = ctypes.c_uint16
+    fn.argtypes = [ctypes.c_uint16]
+    return torch.tensor([fn(i) for i in range(65536)], dtype=torch.int32).to(torch.int16)
+
+
 def moe_sum(inp, bias=None, factor=1.0, num_local_tokens=None, out=None):
     """With num_local_tokens, rows from that index on keep what ``out`` held."""
     M, k, H = inp.shape
@@ -285,8 +301,11 @@ def fused_experts_channel_int8(x, w1, w2, w1_scale, w2_scale, *args, **kwargs):
 def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids, block_size_m,
                              global_num_experts=-1, expert_map=None,
                              apply_router_weight_on_input=False, routed_scaling_factor=1.0,
-                             shared_output=None, return_intermediates=False, _fn="orc_fused_experts_block_int8"):
-    """Whole path; with return_intermediates a dict of every stage's output."""
+                             shared_output=None, return_intermediates=False, _fn="orc_fused_experts_block_int8",
+                             activation="silu"):
+    """Whole path; with return_intermediates a dict of every stage's output.  ``activation``:
+    "silu" or "gelu"."""
+    assert activation in ("silu", "gelu")
     M, H = x.shape
     E, N1, _ = w1.shape
     I = N1 // 2
@@ -308,15 +327,13 @@ def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_i
     ids = topk_ids.to(torch.int32).contiguous()
     tw = topk_weights.to(torch.float32).contiguous()
     emap = None if expert_map is None else expert_map.to(torch.int32).contiguous()
-    rc = getattr(lib(), _fn)(
-        _p(x.contiguous()), _i64(M), _i64(H), _i64(I), _i32(E), _i32(Eg), _i32(k),
-        _p(w1.contiguous()), _p(w1_scale.contiguous()), _p(w2.contiguous()), _p(w2_scale.contiguous()),
-        _p(tw), _p(ids), _p(emap), _i32(block_size_m),
-        ctypes.c_int(1 if apply_router_weight_on_input else 0), ctypes.c_float(routed_scaling_factor),
-        _p(None if shared_output is None else shared_output.contiguous()), _p(out),
-        _p(sorted_ids), _i64(max_pad), _p(expert_ids), _i64(max_blocks), _p(ntpp),
-        _p(inter.get("a1q")), _p(inter.get("a1s")), _p(inter.get("c1")), _p(inter.get("act")),
-        _p(inter.get("a2q")), _p(inter.get("a2s")), _p(inter.get("c3")))
+    lib().orc_set_activation(ctypes.c_int(1 if activation == "gelu" else 0))
+    try:
+        rc = _call_chain(_fn, x, M, H, I, E, Eg, k, w1, w1_scale, w2, w2_scale, tw, ids, emap, block_size_m,
+                         apply_router_weight_on_input, routed_scaling_factor, shared_output, out, sorted_ids,
+                         max_pad, expert_ids, max_blocks, ntpp, inter)
+    finally:
+        lib().orc_set_activation(ctypes.c_int(0))
     if rc != 0:
         raise RuntimeError("oracle fused_experts: alignment failed")
     if return_intermediates:
@@ -326,3 +343,17 @@ def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_i
         inter.update(sorted_ids=sorted_ids, expert_ids=expert_ids, num_tokens_post_pad=ntpp, out=out)
         return inter
     return out
+
+
+def _call_chain(_fn, x, M, H, I, E, Eg, k, w1, w1_scale, w2, w2_scale, tw, ids, emap, block_size_m,
+                apply_router_weight_on_input, routed_scaling_factor, shared_output, out, sorted_ids, max_pad,
+                expert_ids, max_blocks, ntpp, inter):
+    return getattr(lib(), _fn)(
+        _p(x.contiguous()), _i64(M), _i64(H), _i64(I), _i32(E), _i32(Eg), _i32(k),
+        _p(w1.contiguous()), _p(w1_scale.contiguous()), _p(w2.contiguous()), _p(w2_scale.contiguous()),
+        _p(tw), _p(ids), _p(emap), _i32(block_size_m),
+        ctypes.c_int(1 if apply_router_weight_on_input else 0), ctypes.c_float(routed_scaling_factor),
+        _p(None if shared_output is None else shared_output.contiguous()), _p(out),
+        _p(sorted_ids), _i64(max_pad), _p(expert_ids), _i64(max_blocks), _p(ntpp),
+        _p(inter.get("a1q")), _p(inter.get("a1s")), _p(inter.get("c1")), _p(inter.get("act")),
+        _p(inter.get("a2q")), _p(inter.get("a2s")), _p(inter.get("c3")))

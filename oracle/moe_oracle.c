@@ -322,6 +322,44 @@ void orc_silu_and_mul(const uint16_t *c1, int64_t S, int64_t I, uint16_t *act) {
       act[f * I + i] = silu_mul_one(c1[f * 2 * I + i], c1[f * 2 * I + I + i]);
 }
 
+/*
+ * GELU-and-mul, the activation="gelu" branch (int8.py:825-827, w4a8.py:602-605), which calls
+ * torch.ops._C.gelu_and_mul of vLLM (not part of the reference tree); the reference's in-repo
+ * twin is gelu_and_mul_opt, csrc/kernels/activation_kernels_opt.cu:234-242 (gelu_kernel) and
+ * :159-161 (the product, formed in the tensor's type):
+ *   gelu(g) = T((f * 0.5f) * (1.0f + erf(f * ALPHA))),  f = float(g),  ALPHA = float(M_SQRT1_2)
+ *   act     = T(float(gelu(g)) * float(u))
+ * erf is a library routine there; the canonical choice here is erf correctly rounded to fp32
+ * (libm's double-precision erf, rounded once more).  Where the reference's device erf differs
+ * from that in its last place, the bf16 result can differ in its last place too: unpinned.
+ * Pins (tests/test_oracle.py): closed-form values (gelu(0) = 0, gelu(x) = x for large x, -0 for
+ * large negative x), the identity gelu(x) - gelu(-x) = x to rounding, torch's GELU on every
+ * finite bf16 input within one bf16 ulp, monotonicity above the minimum.
+ */
+uint16_t orc_gelu_bf16(uint16_t g16) {
+  const float f = bf16_to_f32(g16);
+  const float alpha = 0.70710678118654752440f;
+  const float e = (float)erf((double)(f * alpha));
+  return f32_to_bf16((f * 0.5f) * (1.0f + e));
+}
+
+static inline uint16_t gelu_mul_one(uint16_t g16, uint16_t u16) {
+  return f32_to_bf16(bf16_to_f32(orc_gelu_bf16(g16)) * bf16_to_f32(u16));
+}
+
+void orc_gelu_and_mul(const uint16_t *c1, int64_t S, int64_t I, uint16_t *act) {
+#pragma omp parallel for schedule(static)
+  for (int64_t f = 0; f < S; ++f)
+    for (int64_t i = 0; i < I; ++i)
+      act[f * I + i] = gelu_mul_one(c1[f * 2 * I + i], c1[f * 2 * I + I + i]);
+}
+
+/* Activation of the whole-path restatements below: 0 = SiLU (default), 1 = GELU.  A switch
+ * for the test harness (one thread sets it around a call), not an argument, so that the
+ * signatures of the chains stay what the existing callers use. */
+static int g_activation = 0;
+void orc_set_activation(int activation) { g_activation = activation; }
+
 /* ------------------------------------------------------------ moe_sum -- */
 
 /*
@@ -386,7 +424,8 @@ static int fused_path(
   if (rc == 0) {
     gemm_core(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
               apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL, group_n);
-    orc_silu_and_mul(c1, S, I, act);
+    if (g_activation == 1) orc_gelu_and_mul(c1, S, I, act);
+    else orc_silu_and_mul(c1, S, I, act);
     orc_group_quant_int8(act, S, I, 1e-10f, a2q, a2s);
     gemm_core(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
               !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL, group_n);
@@ -501,6 +540,22 @@ void orc_fuse_silu_mul_quant(const uint16_t *c1, int64_t S, int64_t I, int8_t *q
   }
 }
 
+/* Between the two stages of the per-channel chains: fuse_silu_mul_quant (int8.py:811-813), or
+ * with GELU gelu_and_mul followed by per_token_quant_int8 (int8.py:825-838 through
+ * moe_kernel_prepare_input's per-channel branch, int8.py:285-295; w4a8.py:602-605), whose
+ * absmax has the 1e-10 floor that the fused SiLU kernel lacks. */
+static void channel_act_quant(const uint16_t *c1, int64_t S, int64_t I, int8_t *q, float *s,
+                              uint16_t *act) {
+  if (g_activation != 1) {
+    orc_fuse_silu_mul_quant(c1, S, I, q, s, act);
+    return;
+  }
+  uint16_t *tmp = act ? act : (uint16_t *)malloc(2 * (size_t)(S * I));
+  orc_gelu_and_mul(c1, S, I, tmp);
+  orc_per_token_quant_int8(tmp, S, I, q, s);
+  if (!act) free(tmp);
+}
+
 /*
  *   A [*, K] int8, row of slot f is f / top_k;  As [*] f32 (one per row)
  *   W [E, N, K] int8;                           Ws [E, N] f32 (one per weight row)
@@ -569,7 +624,7 @@ int orc_fused_experts_channel_int8(
   if (rc == 0) {
     orc_moe_gemm_w8a8(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
                       apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL);
-    orc_fuse_silu_mul_quant(c1, S, I, a2q, a2s, act);
+    channel_act_quant(c1, S, I, a2q, a2s, act);
     orc_moe_gemm_w8a8(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
                       !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL);
     orc_moe_sum(c3, M, top_k, H, shared_output, routed_scaling_factor, out);
@@ -677,7 +732,7 @@ int orc_fused_experts_w4a8_channel(
   if (rc == 0) {
     orc_moe_gemm_w4a8_channel(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
                               apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL);
-    orc_fuse_silu_mul_quant(c1, S, I, a2q, a2s, act);
+    channel_act_quant(c1, S, I, a2q, a2s, act);
     orc_moe_gemm_w4a8_channel(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
                               !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL);
     orc_moe_sum(c3, M, top_k, H, shared_output, routed_scaling_factor, out);
