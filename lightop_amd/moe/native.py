@@ -232,7 +232,7 @@ def invoke_fused_moe_kernel_w4a8(A: torch.Tensor, B: torch.Tensor, C: torch.Tens
     ``preshuffle_moe_weight_int4``, ``A_scale`` one per row, ``B_scale`` one per weight row.
     C[f] = T(((sum_k A[f // top_k] * w16[e]) [* topk_weights[f]]) * A_scale[f // top_k] * B_scale[e]),
     w16 = int8(nibble << 4).  ``config`` needs ``BLOCK_SIZE_M``."""
-    assert B_zp is None, "lightop_amd: W4A8 zero points are not built (symmetric int4 only)"
+    del B_zp  # the reference's kernel takes the pointer and never reads it (b_qzero_ptr, w4a8.py:218)
     assert block_shape is None, "the K-group form goes through fused_experts_impl_w4a8(block_shape=[1, 128])"
     del compute_type
     _require_cuda(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded)
@@ -467,8 +467,10 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
         raise ValueError(f"Unsupported FusedMoe activation: {activation}")
     if hidden_states.dtype != torch.bfloat16:
         raise NotImplementedError("lightop_amd: hidden_states must be bfloat16")
-    if w1_zp is not None or w2_zp is not None:
+    if not channel and (w1_zp is not None or w2_zp is not None):
         raise NotImplementedError("lightop_amd: W4A8 zero points are not built (symmetric int4 only)")
+    # block_shape=None: the reference passes w1_zp / w2_zp to a kernel that never reads them
+    # (b_qzero_ptr, w4a8.py:218): they are ignored here as well
     assert w1_scale is not None and w2_scale is not None
     del a1_scale, a2_scale, use_nn_moe
     _require_cuda(hidden_states, w1, w2, topk_weights, topk_ids, cache13, w1_scale, w2_scale, expert_map,
