@@ -28,8 +28,12 @@ enum {
   LO_ENOTSUP = -4   /* valid request that this build has no kernel for */
 };
 
-/* activation element types (LO_F32: router inputs only) */
+/* activation element types (LO_F32: router inputs only).  fp16 rows go the same way as bf16 ones except
+ * that no kernel fuses the gated activation for them: the first GEMM writes [S, 2I] in fp16 and one launch
+ * applies the activation and quantises (as with LO_FUSED_ACT_GELU), and the two-launch path is not taken. */
 enum { LO_BF16 = 0, LO_F16 = 1, LO_F32 = 2 };
+/* gated activations */
+enum { LO_ACT_SILU = 0, LO_ACT_GELU = 1 };
 /* index element types of topk_ids */
 enum { LO_I32 = 0, LO_I64 = 1 };
 
@@ -234,9 +238,10 @@ int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *ac
  */
 int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *act,
                     lo_stream_t stream);
-/* The 65536 bf16 values bf16(gelu(g)), indexed by the bit pattern of g, that the GELU kernels look
- * up, copied to table_out (device memory, 128 KB).  For tests; no counterpart in the reference. */
-int lo_gelu_bf16_table(void *table_out, lo_stream_t stream);
+/* The 65536 values T(act(g)), indexed by the bit pattern of g, that the kernels look up for activation
+ * LO_ACT_SILU / LO_ACT_GELU and element type LO_BF16 / LO_F16, copied to table_out (device memory,
+ * 128 KB).  For tests; no counterpart in the reference. */
+int lo_activation_table(int activation, int dtype, void *table_out, lo_stream_t stream);
 
 /*
  * Top-k reduction back to token order: out[t, :] = factor * sum_j in[t, j, :] (+ bias[t, :]).
@@ -320,9 +325,12 @@ int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_local, int3
  * -> weighted top-k reduce.  Replaces the body of fused_experts_impl_int8
  * (int8.py:703-888); the reduce is always performed.
  *
- *   x [M, H] bf16;  w1 [E, 2I, H], w2 [E, H, I] int8;  w1s [E, 2I/128, H/128], w2s [E, H/128, I/128]
+ *   x [M, H] bf16 or fp16 (dtype; compute_type of int8.py:689-696: every value stored between the
+ *   stages, cache3 and out have that type);  w1 [E, 2I, H], w2 [E, H, I] int8;
+ *   w1s [E, 2I/128, H/128], w2s [E, H/128, I/128]
  *   topk_w [M, top_k] f32;  topk_ids [M, top_k] int32/int64;  expert_map [num_experts] or NULL
- *   cache3 [M*top_k, H] act dtype: the caller's cache13 workspace (second GEMM's output)
+ *   cache3 [M*top_k, H] act dtype: the caller's cache13 workspace (second GEMM's output); with fp16
+ *   rows or LO_FUSED_ACT_GELU it also receives the first GEMM's output: [M*top_k, max(2I, H)]
  *   shared_output [M, H] or NULL;  out [M, H]
  *   workspace: lo_fused_experts_workspace_bytes(...) bytes of device memory, 256-byte aligned
  *   block_size_m: 0 = take it from the tile table (lo_fused_experts_workspace_bytes(.., 0) is

@@ -17,6 +17,7 @@ LO_GEMM_W4 = 32
 LO_FUSED_NO_DECODE_PATH = 64
 LO_FUSED_FORCE_DECODE_PATH = 128
 LO_FUSED_ACT_GELU = 256
+LO_ACT_SILU, LO_ACT_GELU = 0, 1
 LO_FORM_BLOCK, LO_FORM_CHANNEL, LO_FORM_W4 = 0, 1, 2
 LO_NOALLOC_SCRATCH_BYTES = 32 << 20
 LO_KERNEL_WS, LO_KERNEL_TILE, LO_KERNEL_PC, LO_KERNEL_AS, LO_KERNEL_T128, LO_KERNEL_W4_TILE, LO_KERNEL_DEC = 0, 1, 2, 3, 4, 5, 6
@@ -59,7 +60,7 @@ SIGNATURES = {
     "lo_preshuffle_weight_int4": (c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p]),
     "lo_silu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "lo_gelu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
-    "lo_gelu_bf16_table": (c_int, [c_void_p, c_void_p]),
+    "lo_activation_table": (c_int, [c_int, c_int, c_void_p, c_void_p]),
     "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float,
                            c_void_p, c_void_p]),
     "lo_topk_softmax": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_int, c_void_p, c_void_p, c_int,

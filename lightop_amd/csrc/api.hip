@@ -215,7 +215,7 @@ extern "C" int lo_fused_experts_block_int8(
   using namespace lo;
   LO_REQUIRE(x && w1 && w1s && w2 && w2s && topk_w && topk_ids && cache3 && out && workspace,
              LO_EINVAL, "fused_experts: null pointer");
-  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "fused_experts: only bf16 activations are built");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "fused_experts: activations are bf16 or fp16");
   LO_REQUIRE(M >= 0 && H >= kGroup && H % kGroup == 0 && I >= kGroup && I % kGroup == 0, LO_EINVAL,
              "fused_experts: hidden (%lld) and intermediate (%lld) sizes must be multiples of 128",
              (long long)H, (long long)I);
@@ -250,8 +250,11 @@ extern "C" int lo_fused_experts_block_int8(
 
   // Decode sizes: routing, quantisation, both GEMMs and the reduction in two launches.
   const bool gelu = (flags & LO_FUSED_ACT_GELU) != 0;
-  if (block_size_m_auto && (flags & (LO_GEMM_W_PRESHUFFLED | LO_GEMM_W4)) &&
-      !(flags & (LO_FUSED_NO_DECODE_PATH | LO_FUSED_ACT_GELU))) {
+  // GELU and fp16 activations have no fused epilogue: the first GEMM writes [S, 2I] in the activation
+  // type, one launch applies the gated activation and quantises
+  const bool unfused = gelu || dtype != LO_BF16;
+  if (block_size_m_auto && (flags & (LO_GEMM_W_PRESHUFFLED | LO_GEMM_W4)) && !unfused &&
+      !(flags & LO_FUSED_NO_DECODE_PATH)) {
     // (cache3 is the front of the caller's cache13: the path keeps its bf16 activations [S, I] there)
     const int rc2 = launch_decode_path(x, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w, topk_ids, ids_dtype,
                                        expert_map, apply_router_weight_on_input, routed_scaling_factor, shared_output,
@@ -260,10 +263,12 @@ extern "C" int lo_fused_experts_block_int8(
     if (rc2 != LO_ENOTSUP) return rc2;
   }
 
-  // the quantisation rides in the alignment's launch
-  int rc = launch_quant_align(x, M, H, 1e-10f, a1q, a1s, topk_ids, ids_dtype, S, num_experts, block_size_m,
-                              expert_map, sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, mask, ws + L.off[8],
-                              L.align_scratch, static_cast<hipStream_t>(stream));
+  // the quantisation rides in the alignment's launch (bf16 rows)
+  int rc = dtype != LO_BF16 ? LO_ENOTSUP
+                            : launch_quant_align(x, M, H, 1e-10f, a1q, a1s, topk_ids, ids_dtype, S, num_experts,
+                                                 block_size_m, expert_map, sorted, L.sorted_cap, eids, L.blocks_cap,
+                                                 ntpp, mask, ws + L.off[8], L.align_scratch,
+                                                 static_cast<hipStream_t>(stream));
   if (rc == LO_ENOTSUP) {
     rc = lo_per_token_group_quant_int8(x, dtype, M, H, 1e-10f, a1q, a1s, stream);
     if (rc) return rc;
@@ -272,13 +277,14 @@ extern "C" int lo_fused_experts_block_int8(
                                     L.align_scratch, stream);
   }
   if (rc) return rc;
-  if (gelu) {
+  if (unfused) {
     // rows of experts on other ranks are zero-filled by the first GEMM: the activation launch reads every row
     rc = lo_moe_gemm_block_int8(a1q, a1s, w1, w1s, cache3, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, M, E,
                                 num_experts, 2 * I, H, top_k, block_size_m, apply_router_weight_on_input,
                                 flags & ~LO_FUSED_ACT_GELU, stream);
     if (rc) return rc;
-    rc = launch_gelu_mul_group_quant(cache3, S, I, a2q, a2s, static_cast<hipStream_t>(stream));
+    rc = launch_act_mul_group_quant(cache3, dtype, gelu ? LO_ACT_GELU : LO_ACT_SILU, S, I, a2q, a2s,
+                                    static_cast<hipStream_t>(stream));
   } else {
     rc = lo_moe_gemm1_silu_quant_block_int8(a1q, a1s, w1, w1s, a2q, a2s, dtype, topk_w, sorted, eids,
                                             ntpp, L.sorted_cap, S, M, E, num_experts, I, H, top_k, block_size_m,
@@ -308,7 +314,7 @@ extern "C" int lo_fused_experts_channel_int8(
   using namespace lo;
   LO_REQUIRE(x && w1 && w1s && w2 && w2s && topk_w && topk_ids && cache13 && out && workspace,
              LO_EINVAL, "fused_experts(channel): null pointer");
-  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "fused_experts(channel): only bf16 activations are built");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "fused_experts(channel): activations are bf16 or fp16");
   LO_REQUIRE(M >= 0 && H >= kGroup && H % kGroup == 0 && I >= kGroup && I % kGroup == 0, LO_EINVAL,
              "fused_experts(channel): hidden (%lld) and intermediate (%lld) sizes must be multiples of 128",
              (long long)H, (long long)I);
@@ -351,7 +357,8 @@ extern "C" int lo_fused_experts_channel_int8(
                         num_experts, 2 * I, H, top_k, block_size_m, apply_router_weight_on_input, gflags, stream);
   if (rc) return rc;
   if (flags & LO_FUSED_ACT_GELU) // gelu_and_mul, then per_token_quant_int8 with its floor (int8.py:826-838)
-    rc = launch_gelu_mul_row_quant(cache13, S, I, a2q, a2s, static_cast<hipStream_t>(stream));
+    rc = launch_act_mul_row_quant(cache13, dtype, LO_ACT_GELU, S, I, a2q, a2s, nullptr, 1, nullptr,
+                                  static_cast<hipStream_t>(stream));
   else
     rc = lo_fuse_silu_mul_quant(cache13, dtype, S, I, a2q, a2s, nullptr, 1, stream);
   if (rc) return rc;

@@ -38,12 +38,16 @@ void set_error(const char *fmt, ...);
 int check_launch(const char *what);
 // bf16(silu(g)) for all 65536 bf16 patterns g, built on first use (per device).
 int silu_table(hipStream_t stream, const uint16_t **table);
-// bf16(gelu(g)), erf form, the same way.
-int gelu_table(hipStream_t stream, const uint16_t **table);
-// GELU-and-mul of c1 [rows, 2I] followed by the 1x128 group quantisation (q [rows, I], s [rows, I/128])
-// or by the per-token quantisation (s [rows]), one launch each.
-int launch_gelu_mul_group_quant(const void *c1, int64_t rows, int64_t I, int8_t *q, float *s, hipStream_t stream);
-int launch_gelu_mul_row_quant(const void *c1, int64_t rows, int64_t I, int8_t *q, float *s, hipStream_t stream);
+// T(act(g)) for all 65536 patterns g of the 16-bit type T (LO_BF16 / LO_F16), act = LO_ACT_SILU / LO_ACT_GELU.
+int act_table(hipStream_t stream, int act, int dtype, const uint16_t **table);
+// The gated activation of c1 [rows, 2I] from its table, followed by the 1x128 group quantisation
+// (q [rows, I], s [rows, I/128]) or by the per-token quantisation (s [rows]; SiLU without a floor
+// under the row maximum, as fuse_silu_mul_quant, GELU with per_token_quant_int8's), one launch each.
+int launch_act_mul_group_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
+                               hipStream_t stream);
+int launch_act_mul_row_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
+                             const int32_t *num_local_tokens, int32_t top_k, const int32_t *row_ids,
+                             hipStream_t stream);
 
 // Raises a kernel's dynamic-LDS limit once per device instead of on every launch (kernels that use
 // more than the default 64 KB).  `done` is the call site's own static flag set, one bit per device.
@@ -70,8 +74,13 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
 __device__ __forceinline__ float f16_to_f32(uint16_t h) {
   return static_cast<float>(__builtin_bit_cast(_Float16, h));
 }
+// The conversion is kept opaque: written as a cast, the compiler folds a preceding fp32
+// multiplication into v_fma_mixlo_f16 (a * b + 0 rounded straight to half), which rounds once where
+// the definition rounds twice and turns a -0 product into +0.
 __device__ __forceinline__ uint16_t f32_to_f16(float f) {
-  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+  uint32_t r;
+  asm("v_cvt_f16_f32 %0, %1" : "=v"(r) : "v"(f));
+  return static_cast<uint16_t>(r);
 }
 
 template <int DT> __device__ __forceinline__ float to_f32(uint16_t h) {
@@ -121,6 +130,12 @@ template <int DT> __device__ __forceinline__ uint16_t silu_mul(uint16_t g16, uin
 __device__ __forceinline__ uint16_t silu_mul_tab(const uint16_t *__restrict__ table, uint16_t g16, uint16_t u16) {
   const float sg = bf16_to_f32(table[g16]);
   return f32_to_bf16(sg * bf16_to_f32(u16));
+}
+
+// Any gated activation whose T(act(g)) sits in a 64K-entry table: act = T(T(act(g)) * u).
+template <int DT>
+__device__ __forceinline__ uint16_t act_mul_tab(const uint16_t *__restrict__ table, uint16_t g16, uint16_t u16) {
+  return from_f32<DT>(to_f32<DT>(table[g16]) * to_f32<DT>(u16));
 }
 
 // bf16(silu(g)) has closed forms outside a narrow band of inputs: for |g| <= 0x3bb5 (about

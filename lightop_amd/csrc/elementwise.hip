@@ -43,10 +43,12 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
 // ---- gelu_and_mul ----------------------------------------------------------------
 // Reference: torch.ops._C.gelu_and_mul as called at int8.py:826; in-repo twin gelu_and_mul_opt,
 // csrc/kernels/activation_kernels_opt.cu:234-242 (erf form) and :159-161 (product in the tensor's
-// type): act = T(T(gelu(g)) * u).  bf16(gelu(g)) comes from a 64K-entry table (gelu_table below).
-__global__ __launch_bounds__(256) void gelu_mul_kernel(const uint16_t *__restrict__ c1, int64_t rows, int64_t I,
-                                                       const uint16_t *__restrict__ table,
-                                                       uint16_t *__restrict__ act) {
+// type): act = T(T(gelu(g)) * u).  T(gelu(g)) comes from a 64K-entry table (act_table below); the
+// kernel serves any gated activation that has one.
+template <int DT>
+__global__ __launch_bounds__(256) void act_mul_tab_kernel(const uint16_t *__restrict__ c1, int64_t rows, int64_t I,
+                                                          const uint16_t *__restrict__ table,
+                                                          uint16_t *__restrict__ act) {
   const int64_t vec_per_row = I / 8;
   const int64_t total = rows * vec_per_row;
   for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < total;
@@ -56,7 +58,7 @@ __global__ __launch_bounds__(256) void gelu_mul_kernel(const uint16_t *__restric
     const v8u16 u = *reinterpret_cast<const v8u16 *>(c1 + r * 2 * I + I + c);
     v8u16 o;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = silu_mul_tab(table, g[i], u[i]);
+    for (int i = 0; i < 8; ++i) o[i] = act_mul_tab<DT>(table, g[i], u[i]);
     *reinterpret_cast<v8u16 *>(act + r * I + c) = o;
   }
 }
@@ -64,10 +66,11 @@ __global__ __launch_bounds__(256) void gelu_mul_kernel(const uint16_t *__restric
 // The same followed by the 1x128 group quantisation of per_token_group_quant_int8 (the pair of
 // calls at int8.py:826-838 on the block-shape branch) in one pass: c1 [rows, 2I] -> q [rows, I],
 // s [rows, I/128].  16 lanes own one group, as in group_quant_body.
-__global__ __launch_bounds__(256) void gelu_mul_group_quant_kernel(const uint16_t *__restrict__ c1, int64_t rows,
-                                                                   int64_t I, const uint16_t *__restrict__ table,
-                                                                   float eps, int8_t *__restrict__ q,
-                                                                   float *__restrict__ s) {
+template <int DT>
+__global__ __launch_bounds__(256) void act_mul_group_quant_kernel(const uint16_t *__restrict__ c1, int64_t rows,
+                                                                  int64_t I, const uint16_t *__restrict__ table,
+                                                                  float eps, int8_t *__restrict__ q,
+                                                                  float *__restrict__ s) {
   const int64_t gpr = I / kGroup, groups = rows * gpr;
   const int sub = threadIdx.x & 15;
   for (int64_t g = static_cast<int64_t>(blockIdx.x) * 16 + (threadIdx.x >> 4); g < groups;
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(256) void gelu_mul_group_quant_kernel(const uint16_
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      v[i] = bf16_to_f32(silu_mul_tab(table, ga[i], up[i]));
+      v[i] = to_f32<DT>(act_mul_tab<DT>(table, ga[i], up[i]));
       amax = fmaxf(amax, fabsf(v[i]));
     }
 #pragma unroll
@@ -102,21 +105,23 @@ __global__ __launch_bounds__(256) void gelu_mul_group_quant_kernel(const uint16_
 // no floor: a zero row gets scale 0 and multiplier 0).  One workgroup per row; a thread keeps
 // up to CH 8-value pieces of the row in registers between the amax pass and the rounding pass,
 // longer rows are read a second time.
-// ACT: 0 plain rows; 1 SiLU-and-mul first (the fused kernel above: no floor); 2 GELU-and-mul first,
-// then per_token_quant_int8 with its floor (the two calls at int8.py:826-838 on the per-channel
-// branch), `silu` being the GELU table then.
+// ACT: 0 plain rows; 1 SiLU-and-mul first (the fused kernel above: no floor), bf16 only, through the
+// band of the SiLU table; 2 a gated activation from its full table first (`silu` being that table),
+// then per_token_quant_int8 with its floor (GELU: the two calls at int8.py:826-838 on the per-channel
+// branch); 3 as 2 without the floor (SiLU for fp16 rows, which have no band).
 __device__ __forceinline__ int rne_i8(float v) {
   v = fminf(fmaxf(v, -128.0f), 127.0f);
   return static_cast<int>(__builtin_rintf(v)); // v_rndne_f32: ties to even
 }
 
-template <int ACT, int CH>
+template <int ACT, int CH, int DT>
 __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restrict__ x, int64_t rows, int64_t C,
                                                         const uint16_t *__restrict__ silu, int8_t *__restrict__ q,
                                                         float *__restrict__ s,
                                                         const int32_t *__restrict__ num_local_tokens, int32_t top_k,
                                                         const int32_t *__restrict__ row_ids) {
-  constexpr bool SILU = ACT == 1, GATED = ACT != 0;
+  static_assert(ACT != 1 || DT == LO_BF16, "the SiLU band is a bf16 table");
+  constexpr bool SILU = ACT == 1, GATED = ACT != 0, FLOOR = ACT == 0 || ACT == 2;
   __shared__ float sRed[4];
   __shared__ uint16_t sSilu[SILU ? 2 * kSiluBandN : 2];
   const int tid = threadIdx.x;
@@ -141,11 +146,13 @@ __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restri
       if constexpr (GATED) {
         const v8u16 u = *reinterpret_cast<const v8u16 *>(xr + C + p * 8);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          v[i] = bf16_to_f32(SILU ? silu_mul_band(sSilu, silu, a[i], u[i]) : silu_mul_tab(silu, a[i], u[i]));
+        for (int i = 0; i < 8; ++i) {
+          if constexpr (SILU) v[i] = bf16_to_f32(silu_mul_band(sSilu, silu, a[i], u[i]));
+          else v[i] = to_f32<DT>(act_mul_tab<DT>(silu, a[i], u[i]));
+        }
       } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = bf16_to_f32(a[i]);
+        for (int i = 0; i < 8; ++i) v[i] = to_f32<DT>(a[i]);
       }
     };
     float keep[CH][8];
@@ -172,7 +179,7 @@ __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restri
     amax = fmaxf(fmaxf(sRed[0], sRed[1]), fmaxf(sRed[2], sRed[3]));
     __syncthreads(); // sRed is reused by the next row
     float inv;
-    if constexpr (SILU) {
+    if constexpr (!FLOOR) {
       inv = amax == 0.0f ? 0.0f : 127.0f / amax;
     } else {
       amax = fmaxf(amax, 1e-10f);
@@ -200,13 +207,14 @@ __global__ __launch_bounds__(256) void row_quant_kernel(const uint16_t *__restri
 
 // The same for rows of at most 512 * CH values: one wavefront per row, four rows per workgroup,
 // the row stays in registers and the reduction needs no barrier.
-template <int ACT, int CH>
+template <int ACT, int CH, int DT>
 __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__restrict__ x, int64_t rows, int64_t C,
                                                              const uint16_t *__restrict__ silu,
                                                              int8_t *__restrict__ q, float *__restrict__ s,
                                                              const int32_t *__restrict__ num_local_tokens,
                                                              int32_t top_k, const int32_t *__restrict__ row_ids) {
-  constexpr bool SILU = ACT == 1, GATED = ACT != 0;
+  static_assert(ACT != 1 || DT == LO_BF16, "the SiLU band is a bf16 table");
+  constexpr bool SILU = ACT == 1, GATED = ACT != 0, FLOOR = ACT == 0 || ACT == 2;
   __shared__ uint16_t sSilu[SILU ? 2 * kSiluBandN : 2];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   if (num_local_tokens) {
@@ -241,15 +249,15 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if constexpr (SILU) v[j][i] = bf16_to_f32(silu_mul_band(sSilu, silu, ga[j][i], up[j][i]));
-        else if constexpr (GATED) v[j][i] = bf16_to_f32(silu_mul_tab(silu, ga[j][i], up[j][i]));
-        else v[j][i] = bf16_to_f32(ga[j][i]);
+        else if constexpr (GATED) v[j][i] = to_f32<DT>(act_mul_tab<DT>(silu, ga[j][i], up[j][i]));
+        else v[j][i] = to_f32<DT>(ga[j][i]);
         amax = fmaxf(amax, live ? fabsf(v[j][i]) : 0.0f);
       }
     }
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
     float inv;
-    if constexpr (SILU) {
+    if constexpr (!FLOOR) {
       inv = amax == 0.0f ? 0.0f : 127.0f / amax;
     } else {
       amax = fmaxf(amax, 1e-10f);
@@ -268,7 +276,7 @@ __global__ __launch_bounds__(256) void row_quant_wave_kernel(const uint16_t *__r
   }
 }
 
-template <int ACT>
+template <int ACT, int DT = LO_BF16>
 static void launch_row_quant(const uint16_t *x, int64_t rows, int64_t C, const uint16_t *silu, int8_t *q, float *s,
                              const int32_t *nlt, int32_t top_k, const int32_t *row_ids, hipStream_t st) {
   const int pieces = static_cast<int>(C / 8);
@@ -276,13 +284,13 @@ static void launch_row_quant(const uint16_t *x, int64_t rows, int64_t C, const u
     int64_t grid = (rows + 3) / 4;
     if (grid > 256 * 32) grid = 256 * 32;
     const dim3 g(static_cast<unsigned>(grid)), b(256);
-    if (pieces <= 64) hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 1>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
-    else if (pieces <= 128) hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 2>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
-    else hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 4>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
+    if (pieces <= 64) hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 1, DT>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
+    else if (pieces <= 128) hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 2, DT>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
+    else hipLaunchKernelGGL((row_quant_wave_kernel<ACT, 4, DT>), g, b, 0, st, x, rows, C, silu, q, s, nlt, top_k, row_ids);
     return;
   }
   const unsigned grid = static_cast<unsigned>(rows < 65536 ? rows : 65536);
-  hipLaunchKernelGGL((row_quant_kernel<ACT, ACT ? 2 : 4>), dim3(grid), dim3(256), 0, st, x, rows, C, silu, q, s, nlt,
+  hipLaunchKernelGGL((row_quant_kernel<ACT, ACT ? 2 : 4, DT>), dim3(grid), dim3(256), 0, st, x, rows, C, silu, q, s, nlt,
                      top_k, row_ids);
 }
 
@@ -366,17 +374,24 @@ __global__ __launch_bounds__(256) void silu_table_init_kernel(uint16_t *table) {
   table[i] = f32_to_bf16(g / (1.0f + det_expf(-g)));
 }
 
-// bf16(gelu(g)) for every bf16 pattern g: (f * 0.5f) * (1.0f + erf(f * ALPHA)) in fp32 with erf
-// correctly rounded to fp32 (taken in double precision and rounded once more), the form of
-// csrc/kernels/activation_kernels_opt.cu:234-242.  Built once per device.
-__device__ uint16_t g_gelu_bf16_table[65536];
+// Tables of the other gated activations: T(act(g)) for every 16-bit pattern g of the activation type T.
+//   GELU: (f * 0.5f) * (1.0f + erf(f * ALPHA)) in fp32 with erf correctly rounded to fp32 (taken in
+//         double precision and rounded once more), the form of csrc/kernels/activation_kernels_opt.cu:234-242;
+//   SiLU for fp16 rows: f / (1 + exp(-f)) with det_expf, as in the bf16 table above.
+// Slot = 2 * (T is fp16) + (activation is GELU); slot 0 is g_silu_bf16_table.  Built once per device.
+__device__ uint16_t g_act_tables[3][65536];
 
-__global__ __launch_bounds__(256) void gelu_table_init_kernel(uint16_t *table) {
+template <int DT, int ACT>
+__global__ __launch_bounds__(256) void act_table_init_kernel(uint16_t *table) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  const float f = bf16_to_f32(static_cast<uint16_t>(i));
-  const float alpha = 0.70710678118654752440f;
-  const float e = static_cast<float>(erf(static_cast<double>(f * alpha)));
-  table[i] = f32_to_bf16((f * 0.5f) * (1.0f + e));
+  const float f = to_f32<DT>(static_cast<uint16_t>(i));
+  if constexpr (ACT == LO_ACT_GELU) {
+    const float alpha = 0.70710678118654752440f;
+    const float e = static_cast<float>(erf(static_cast<double>(f * alpha)));
+    table[i] = from_f32<DT>((f * 0.5f) * (1.0f + e));
+  } else {
+    table[i] = from_f32<DT>(f / (1.0f + det_expf(-f)));
+  }
 }
 
 static int grid_for(int64_t work_items, int per_block) {
@@ -388,59 +403,86 @@ static int grid_for(int64_t work_items, int per_block) {
 
 static std::mutex g_table_mutex;
 static const uint16_t *g_table_ptr[64] = {};
-static const uint16_t *g_gelu_ptr[64] = {};
+static const uint16_t *g_act_ptr[64][4] = {};
 
-int gelu_table(hipStream_t stream, const uint16_t **out) {
+int act_table(hipStream_t stream, int act, int dtype, const uint16_t **out) {
+  if (act == LO_ACT_SILU && dtype == LO_BF16) return silu_table(stream, out);
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
-    set_error("gelu table: no current HIP device");
+    set_error("activation table: no current HIP device");
     return LO_ELAUNCH;
   }
+  if ((act != LO_ACT_SILU && act != LO_ACT_GELU) || (dtype != LO_BF16 && dtype != LO_F16)) {
+    set_error("activation table: unknown activation %d or element type %d", act, dtype);
+    return LO_EINVAL;
+  }
+  const int slot = 2 * (dtype == LO_F16) + (act == LO_ACT_GELU);
   std::lock_guard<std::mutex> lock(g_table_mutex);
-  if (!g_gelu_ptr[dev]) {
+  if (!g_act_ptr[dev][slot]) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) {
-      set_error("the first GELU call on a device builds its table and must not be captured: "
-                "run the op once before capturing a graph");
+      set_error("the first call with this activation and element type on a device builds a table and must "
+                "not be captured: run the op once before capturing a graph");
       return LO_EINVAL;
     }
-    uint16_t *p = nullptr;
-    if (hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(g_gelu_bf16_table)) != hipSuccess || !p) {
-      set_error("gelu table: hipGetSymbolAddress failed");
+    uint16_t *base = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void **>(&base), HIP_SYMBOL(g_act_tables)) != hipSuccess || !base) {
+      set_error("activation table: hipGetSymbolAddress failed");
       return LO_ELAUNCH;
     }
-    hipLaunchKernelGGL(gelu_table_init_kernel, dim3(256), dim3(256), 0, stream, p);
-    int rc = check_launch("gelu_table_init");
+    uint16_t *p = base + static_cast<size_t>(slot - 1) * 65536;
+    if (slot == 1) hipLaunchKernelGGL((act_table_init_kernel<LO_BF16, LO_ACT_GELU>), dim3(256), dim3(256), 0, stream, p);
+    else if (slot == 2) hipLaunchKernelGGL((act_table_init_kernel<LO_F16, LO_ACT_SILU>), dim3(256), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((act_table_init_kernel<LO_F16, LO_ACT_GELU>), dim3(256), dim3(256), 0, stream, p);
+    int rc = check_launch("act_table_init");
     if (rc) return rc;
     if (hipStreamSynchronize(stream) != hipSuccess) {
-      set_error("gelu table: synchronisation failed");
+      set_error("activation table: synchronisation failed");
       return LO_ELAUNCH;
     }
-    g_gelu_ptr[dev] = p;
+    g_act_ptr[dev][slot] = p;
   }
-  *out = g_gelu_ptr[dev];
+  *out = g_act_ptr[dev][slot];
   return LO_OK;
 }
 
-// The two launches between the GEMMs when the activation is GELU (no fused epilogue exists for it).
-int launch_gelu_mul_group_quant(const void *c1, int64_t rows, int64_t I, int8_t *q, float *s, hipStream_t stream) {
+// The launch between the GEMMs where no fused epilogue exists (GELU; fp16 activations): the gated
+// activation from its table and the quantisation of the form in one pass over c1 [rows, 2I].
+int launch_act_mul_group_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
+                               hipStream_t stream) {
   const uint16_t *table = nullptr;
-  int rc = gelu_table(stream, &table);
+  int rc = act_table(stream, act, dtype, &table);
   if (rc) return rc;
   const int64_t groups = rows * (I / kGroup);
   if (groups == 0) return LO_OK;
-  hipLaunchKernelGGL(gelu_mul_group_quant_kernel, dim3(grid_for(groups, 16)), dim3(256), 0, stream,
-                     static_cast<const uint16_t *>(c1), rows, I, table, 1e-10f, q, s);
-  return check_launch("gelu_mul_group_quant");
+  const dim3 g(grid_for(groups, 16)), b(256);
+  if (dtype == LO_F16)
+    hipLaunchKernelGGL(act_mul_group_quant_kernel<LO_F16>, g, b, 0, stream, static_cast<const uint16_t *>(c1), rows, I,
+                       table, 1e-10f, q, s);
+  else
+    hipLaunchKernelGGL(act_mul_group_quant_kernel<LO_BF16>, g, b, 0, stream, static_cast<const uint16_t *>(c1), rows, I,
+                       table, 1e-10f, q, s);
+  return check_launch("act_mul_group_quant");
 }
 
-int launch_gelu_mul_row_quant(const void *c1, int64_t rows, int64_t I, int8_t *q, float *s, hipStream_t stream) {
+// SiLU: the semantics of fuse_silu_mul_quant (no floor under the row maximum); GELU: gelu_and_mul, then
+// per_token_quant_int8 with its floor.
+int launch_act_mul_row_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
+                             const int32_t *num_local_tokens, int32_t top_k, const int32_t *row_ids,
+                             hipStream_t stream) {
   const uint16_t *table = nullptr;
-  int rc = gelu_table(stream, &table);
+  int rc = act_table(stream, act, dtype, &table);
   if (rc) return rc;
   if (rows == 0) return LO_OK;
-  launch_row_quant<2>(static_cast<const uint16_t *>(c1), rows, I, table, q, s, nullptr, 1, nullptr, stream);
-  return check_launch("gelu_mul_row_quant");
+  const uint16_t *x = static_cast<const uint16_t *>(c1);
+  if (dtype == LO_F16) {
+    if (act == LO_ACT_GELU) launch_row_quant<2, LO_F16>(x, rows, I, table, q, s, num_local_tokens, top_k, row_ids, stream);
+    else launch_row_quant<3, LO_F16>(x, rows, I, table, q, s, num_local_tokens, top_k, row_ids, stream);
+  } else {
+    if (act == LO_ACT_GELU) launch_row_quant<2>(x, rows, I, table, q, s, num_local_tokens, top_k, row_ids, stream);
+    else launch_row_quant<1>(x, rows, I, table, q, s, num_local_tokens, top_k, row_ids, stream);
+  }
+  return check_launch("act_mul_row_quant");
 }
 
 int silu_table(hipStream_t stream, const uint16_t **out) {
@@ -483,7 +525,7 @@ extern "C" int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t
                                              lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(x && q && s, LO_EINVAL, "per_token_group_quant_int8: null pointer");
-  LO_REQUIRE(x_dtype == LO_BF16, LO_ENOTSUP, "per_token_group_quant_int8: only bf16 input is built");
+  LO_REQUIRE(x_dtype == LO_BF16 || x_dtype == LO_F16, LO_ENOTSUP, "per_token_group_quant_int8: the input is bf16 or fp16");
   LO_REQUIRE(rows >= 0 && cols > 0 && cols % kGroup == 0, LO_EINVAL,
              "per_token_group_quant_int8: the last dimension (%lld) must be a multiple of 128",
              (long long)cols);
@@ -491,9 +533,12 @@ extern "C" int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t
              LO_EINVAL, "per_token_group_quant_int8: x must be 16-byte and q 8-byte aligned");
   const int64_t groups = rows * (cols / kGroup);
   if (groups == 0) return LO_OK;
-  hipLaunchKernelGGL(group_quant_kernel<LO_BF16>, dim3(grid_for(groups, 16)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(x), groups, eps,
-                     q, s);
+  if (x_dtype == LO_F16)
+    hipLaunchKernelGGL(group_quant_kernel<LO_F16>, dim3(grid_for(groups, 16)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(x), groups, eps, q, s);
+  else
+    hipLaunchKernelGGL(group_quant_kernel<LO_BF16>, dim3(grid_for(groups, 16)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(x), groups, eps, q, s);
   return check_launch("per_token_group_quant_int8");
 }
 
@@ -501,15 +546,20 @@ extern "C" int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
                                lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(c1 && act, LO_EINVAL, "silu_and_mul: null pointer");
-  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "silu_and_mul: only bf16 is built");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "silu_and_mul: bf16 or fp16");
   LO_REQUIRE(rows >= 0 && I > 0 && I % 8 == 0, LO_EINVAL, "silu_and_mul: I (%lld) must be a multiple of 8",
              (long long)I);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(act) & 15) == 0,
              LO_EINVAL, "silu_and_mul: pointers must be 16-byte aligned");
   if (rows == 0) return LO_OK;
-  hipLaunchKernelGGL(silu_mul_kernel<LO_BF16>, dim3(grid_for(rows * (I / 8), 256)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I,
-                     static_cast<uint16_t *>(act));
+  if (dtype == LO_F16)
+    hipLaunchKernelGGL(silu_mul_kernel<LO_F16>, dim3(grid_for(rows * (I / 8), 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I,
+                       static_cast<uint16_t *>(act));
+  else
+    hipLaunchKernelGGL(silu_mul_kernel<LO_BF16>, dim3(grid_for(rows * (I / 8), 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I,
+                       static_cast<uint16_t *>(act));
   return check_launch("silu_and_mul");
 }
 
@@ -517,29 +567,34 @@ extern "C" int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
                                lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(c1 && act, LO_EINVAL, "gelu_and_mul: null pointer");
-  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "gelu_and_mul: only bf16 is built");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "gelu_and_mul: bf16 or fp16");
   LO_REQUIRE(rows >= 0 && I > 0 && I % 8 == 0, LO_EINVAL, "gelu_and_mul: I (%lld) must be a multiple of 8",
              (long long)I);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(act) & 15) == 0,
              LO_EINVAL, "gelu_and_mul: pointers must be 16-byte aligned");
   const uint16_t *table = nullptr;
-  int rc = gelu_table(static_cast<hipStream_t>(stream), &table);
+  int rc = act_table(static_cast<hipStream_t>(stream), LO_ACT_GELU, dtype, &table);
   if (rc) return rc;
   if (rows == 0) return LO_OK;
-  hipLaunchKernelGGL(gelu_mul_kernel, dim3(grid_for(rows * (I / 8), 256)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I, table,
-                     static_cast<uint16_t *>(act));
+  if (dtype == LO_F16)
+    hipLaunchKernelGGL(act_mul_tab_kernel<LO_F16>, dim3(grid_for(rows * (I / 8), 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I, table,
+                       static_cast<uint16_t *>(act));
+  else
+    hipLaunchKernelGGL(act_mul_tab_kernel<LO_BF16>, dim3(grid_for(rows * (I / 8), 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I, table,
+                       static_cast<uint16_t *>(act));
   return check_launch("gelu_and_mul");
 }
 
-extern "C" int lo_gelu_bf16_table(void *table_out, lo_stream_t stream) {
+extern "C" int lo_activation_table(int activation, int dtype, void *table_out, lo_stream_t stream) {
   using namespace lo;
-  LO_REQUIRE(table_out, LO_EINVAL, "gelu_bf16_table: null pointer");
+  LO_REQUIRE(table_out, LO_EINVAL, "activation_table: null pointer");
   const uint16_t *table = nullptr;
-  int rc = gelu_table(static_cast<hipStream_t>(stream), &table);
+  int rc = act_table(static_cast<hipStream_t>(stream), activation, dtype, &table);
   if (rc) return rc;
   if (hipMemcpyAsync(table_out, table, 65536 * 2, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)) != hipSuccess) {
-    set_error("gelu_bf16_table: copy failed");
+    set_error("activation_table: copy failed");
     return LO_ELAUNCH;
   }
   return LO_OK;
@@ -550,7 +605,7 @@ extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uin
                           const int32_t *num_local_tokens, lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(in && out, LO_EINVAL, "moe_sum: null pointer");
-  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "moe_sum: only bf16 is built");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "moe_sum: bf16 or fp16");
   LO_REQUIRE(M >= 0 && topk >= 1 && H > 0 && H % 8 == 0, LO_EINVAL,
              "moe_sum: hidden size (%lld) must be a multiple of 8, topk >= 1", (long long)H);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(in) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
@@ -559,14 +614,17 @@ extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uin
   if (M == 0) return LO_OK;
   const int grid = grid_for(M * (H / 8), 256);
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define LO_SUM_LAUNCH(HB, TK)                                                                        \
-  hipLaunchKernelGGL((moe_sum_kernel<LO_BF16, HB, TK>), dim3(grid), dim3(256), 0, s,                \
+#define LO_SUM_LAUNCH(DTV, HB, TK)                                                                   \
+  hipLaunchKernelGGL((moe_sum_kernel<DTV, HB, TK>), dim3(grid), dim3(256), 0, s,                    \
                      static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out),               \
                      static_cast<const uint16_t *>(bias), expert_mask, M, topk, H, factor, num_local_tokens)
 #define LO_SUM_PICK(TK)                                                                              \
   do {                                                                                               \
-    if (bias) LO_SUM_LAUNCH(true, TK);                                                               \
-    else LO_SUM_LAUNCH(false, TK);                                                                   \
+    if (dtype == LO_F16) { /* fp16 rows: the run-time slot loop serves every width */               \
+      if (bias) LO_SUM_LAUNCH(LO_F16, true, 0);                                                      \
+      else LO_SUM_LAUNCH(LO_F16, false, 0);                                                          \
+    } else if (bias) LO_SUM_LAUNCH(LO_BF16, true, TK);                                               \
+    else LO_SUM_LAUNCH(LO_BF16, false, TK);                                                          \
   } while (0)
   switch (topk) { // the usual router widths get the unrolled form
     case 1: LO_SUM_PICK(1); break;
@@ -585,14 +643,18 @@ extern "C" int lo_per_token_quant_int8(const void *x, int x_dtype, int64_t rows,
                                        float *s, lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(x && q && s, LO_EINVAL, "per_token_quant_int8: null pointer");
-  LO_REQUIRE(x_dtype == LO_BF16, LO_ENOTSUP, "per_token_quant_int8: only bf16 input is built");
+  LO_REQUIRE(x_dtype == LO_BF16 || x_dtype == LO_F16, LO_ENOTSUP, "per_token_quant_int8: the input is bf16 or fp16");
   LO_REQUIRE(rows >= 0 && cols > 0 && cols % 8 == 0, LO_EINVAL,
              "per_token_quant_int8: the last dimension (%lld) must be a multiple of 8", (long long)cols);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0,
              LO_EINVAL, "per_token_quant_int8: x must be 16-byte and q 8-byte aligned");
   if (rows == 0) return LO_OK;
-  launch_row_quant<0>(static_cast<const uint16_t *>(x), rows, cols, nullptr, q, s, nullptr, 1, nullptr,
-                          static_cast<hipStream_t>(stream));
+  if (x_dtype == LO_F16)
+    launch_row_quant<0, LO_F16>(static_cast<const uint16_t *>(x), rows, cols, nullptr, q, s, nullptr, 1, nullptr,
+                                static_cast<hipStream_t>(stream));
+  else
+    launch_row_quant<0>(static_cast<const uint16_t *>(x), rows, cols, nullptr, q, s, nullptr, 1, nullptr,
+                        static_cast<hipStream_t>(stream));
   return check_launch("per_token_quant_int8");
 }
 
@@ -601,18 +663,14 @@ extern "C" int lo_fuse_silu_mul_quant_ids(const void *c1, int dtype, int64_t row
                                           lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(c1 && q && s, LO_EINVAL, "fuse_silu_mul_quant: null pointer");
-  LO_REQUIRE(dtype == LO_BF16, LO_ENOTSUP, "fuse_silu_mul_quant: only bf16 input is built");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "fuse_silu_mul_quant: the input is bf16 or fp16");
   LO_REQUIRE(rows >= 0 && I > 0 && I % 8 == 0 && top_k >= 1, LO_EINVAL,
              "fuse_silu_mul_quant: the output width (%lld) must be a multiple of 8, top_k >= 1", (long long)I);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0,
              LO_EINVAL, "fuse_silu_mul_quant: input must be 16-byte and q 8-byte aligned");
   if (rows == 0) return LO_OK;
-  const uint16_t *table = nullptr;
-  int rc = silu_table(static_cast<hipStream_t>(stream), &table);
-  if (rc) return rc;
-  launch_row_quant<1>(static_cast<const uint16_t *>(c1), rows, I, table, q, s, num_local_tokens, top_k,
-                         row_expert_ids, static_cast<hipStream_t>(stream));
-  return check_launch("fuse_silu_mul_quant");
+  return launch_act_mul_row_quant(c1, dtype, LO_ACT_SILU, rows, I, q, s, num_local_tokens, top_k, row_expert_ids,
+                                  static_cast<hipStream_t>(stream));
 }
 
 extern "C" int lo_fuse_silu_mul_quant(const void *c1, int dtype, int64_t rows, int64_t I, int8_t *q, float *s,

@@ -39,7 +39,18 @@ struct GemmArgs {
   int32_t skip_nonlocal; // blocks of expert -1: leave the output rows untouched
   int32_t w4;            // W is packed int4 (load-time layout), Ws is [E, K/128, N]
   int32_t per_channel;   // As is [a_rows], Ws is [E, N]: scales applied once, after the whole-K int32 sum
+  int32_t out_f16;       // C holds IEEE half instead of bf16 (plain epilogues only)
 };
+
+// The 16-bit form a plain epilogue stores: bf16, or IEEE half when the caller's activations are fp16.
+// `body(cvt)` is run with the conversion of the output type; the choice is one wave-uniform branch
+// around the caller's loops, so the bf16 path pays nothing per value (a per-value select cost the
+// activation-stationary second GEMM 10 %).
+template <typename Body>
+__device__ __forceinline__ void with_out16(int f16, Body body) {
+  if (__builtin_expect(f16 != 0, 0)) body([](float v) { return f32_to_f16(v); });
+  else body([](float v) { return f32_to_bf16(v); });
+}
 
 // Order of the scale arithmetic per 128-wide K block.  Every kernel computes the canonical
 // acc = acc + (f32(d) * a_s) * b_s (three roundings, the order the CPU checker restates) unless the

@@ -102,7 +102,7 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL, "moe_gemm: block_size_m %d is not one of 16, 32, 64, 128",
              block_size_m);
   LO_REQUIRE(C, LO_EINVAL, "moe_gemm: null output");
-  LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm: only bf16 output is built");
+  LO_REQUIRE(c_dtype == LO_BF16 || c_dtype == LO_F16, LO_ENOTSUP, "moe_gemm: the output is bf16 or fp16");
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm: N (%lld) must be a multiple of 16", (long long)N);
   LO_REQUIRE(N * K < (1ll << 31), LO_ENOTSUP, "moe_gemm: one expert's weights exceed 2 GiB");
   LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm: mul_routed needs topk_weights");
@@ -118,6 +118,7 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
+  a.out_f16 = c_dtype == LO_F16 ? 1 : 0;
   LO_REQUIRE(!a.w4 || a.w_shuffled, LO_ENOTSUP,
              "moe_gemm: int4 weights must be in the layout of lo_preshuffle_weight_int4 (LO_GEMM_W_PRESHUFFLED)");
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
@@ -183,7 +184,7 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL, "moe_gemm_w8a8: block_size_m %d is not one of 16, 32, 64, 128",
              block_size_m);
   LO_REQUIRE(C, LO_EINVAL, "moe_gemm_w8a8: null output");
-  LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm_w8a8: only bf16 output is built");
+  LO_REQUIRE(c_dtype == LO_BF16 || c_dtype == LO_F16, LO_ENOTSUP, "moe_gemm_w8a8: the output is bf16 or fp16");
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm_w8a8: N (%lld) must be a multiple of 16", (long long)N);
   LO_REQUIRE(N * K < (1ll << 31), LO_ENOTSUP, "moe_gemm_w8a8: one expert's weights exceed 2 GiB");
   LO_REQUIRE(K <= 131072, LO_ENOTSUP, "moe_gemm_w8a8: K (%lld) could overflow the int32 sum", (long long)K);
@@ -204,6 +205,7 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   a.w_shuffled = (flags & LO_GEMM_W_PRESHUFFLED) ? 1 : 0;
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.per_channel = 1;
+  a.out_f16 = c_dtype == LO_F16 ? 1 : 0;
   a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);

@@ -181,15 +181,17 @@ __device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks
       if (a.mul_routed) ts = a.topk_w[f[tb]] * ts;
     }
     v4u16 o[2][4];
+    with_out16(a.out_f16, [&](auto cvt) __attribute__((always_inline)) {
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+      for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float t = static_cast<float>(acc[tb][rb][4 * q + i]) * ts;
-          o[rb][q][i] = f32_to_bf16(t * bs4[rb][q][i]);
-        }
+          for (int i = 0; i < 4; ++i) {
+            const float t = static_cast<float>(acc[tb][rb][4 * q + i]) * ts;
+            o[rb][q][i] = cvt(t * bs4[rb][q][i]);
+          }
+    });
     wave_store_32x64_bf16(stg, o, valid[tb] ? static_cast<int>(f[tb]) : -1, a.C, N, nrow[0], lane);
   }
 }

@@ -523,27 +523,29 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
       const bool valid = ft < a.num_valid;
       float wgt = 1.0f;
       if (a.mul_routed && valid) wgt = a.topk_w[ft];
+      with_out16(a.out_f16, [&](auto cvt) __attribute__((always_inline)) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int rf = 0; rf < 2; ++rf) {
-          v4u16 o;
+          for (int rf = 0; rf < 2; ++rf) {
+            v4u16 o;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            float v;
-            if constexpr (PC) { // left to right: routed weight, token scale, channel scale (w4a8.py:386-395)
-              v = static_cast<float>(acci[h][tb][rf][i]);
-              if (a.mul_routed) v = v * wgt;
-              v = v * pas[tb];
-              v = v * pbs[h][rf][i];
-            } else {
-              v = acc[h][tb][rf][i];
-              if (a.mul_routed) v = v * wgt;
+            for (int i = 0; i < 4; ++i) {
+              float v;
+              if constexpr (PC) { // left to right: routed weight, token scale, channel scale (w4a8.py:386-395)
+                v = static_cast<float>(acci[h][tb][rf][i]);
+                if (a.mul_routed) v = v * wgt;
+                v = v * pas[tb];
+                v = v * pbs[h][rf][i];
+              } else {
+                v = acc[h][tb][rf][i];
+                if (a.mul_routed) v = v * wgt;
+              }
+              o[i] = cvt(v);
             }
-            o[i] = f32_to_bf16(v);
+            *reinterpret_cast<v4u16 *>(stg + r * kTPitch + (h * 32 + rf * 16 + 4 * q) * 2) = o;
           }
-          *reinterpret_cast<v4u16 *>(stg + r * kTPitch + (h * 32 + rf * 16 + 4 * q) * 2) = o;
-        }
+      });
       __builtin_amdgcn_wave_barrier();
       const int slot = valid ? static_cast<int>(ft) : -1;
 #pragma unroll

@@ -261,16 +261,18 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
       float w = 1.0f;
       if (a.mul_routed && valid[tb]) w = a.topk_w[f[tb]];
       v4u16 o[2][4];
+      with_out16(a.out_f16, [&](auto cvt) __attribute__((always_inline)) {
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
+        for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+          for (int q = 0; q < 4; ++q)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            float v = acc[tb][rb][4 * q + i];
-            if (a.mul_routed) v = v * w;
-            o[rb][q][i] = f32_to_bf16(v);
-          }
+            for (int i = 0; i < 4; ++i) {
+              float v = acc[tb][rb][4 * q + i];
+              if (a.mul_routed) v = v * w;
+              o[rb][q][i] = cvt(v);
+            }
+      });
       wave_store_32x64_bf16(stg, o, valid[tb] ? static_cast<int>(f[tb]) : -1, a.C, N, nrow[0], lane);
     }
   } else {

@@ -246,17 +246,19 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     for (int tf = 0; tf < 4; ++tf) {
       float w = 1.0f;
       if (a.mul_routed && valid[tf]) w = a.topk_w[f[tf]];
+      with_out16(a.out_f16, [&](auto cvt) __attribute__((always_inline)) {
 #pragma unroll
-      for (int rf = 0; rf < 4; ++rf) {
-        v4u16 o;
+        for (int rf = 0; rf < 4; ++rf) {
+          v4u16 o;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float v = acc[rf][tf][i];
-          if (a.mul_routed) v = v * w;
-          o[i] = f32_to_bf16(v);
+          for (int i = 0; i < 4; ++i) {
+            float v = acc[rf][tf][i];
+            if (a.mul_routed) v = v * w;
+            o[i] = cvt(v);
+          }
+          *reinterpret_cast<v4u16 *>(stg + r * kW4Row + (rf * 16 + 4 * q) * 2) = o;
         }
-        *reinterpret_cast<v4u16 *>(stg + r * kW4Row + (rf * 16 + 4 * q) * 2) = o;
-      }
+      });
       __builtin_amdgcn_wave_barrier();
       const int slot = valid[tf] ? static_cast<int>(f[tf]) : -1;
 #pragma unroll

@@ -301,21 +301,23 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       for (int g = 0; g < NW; ++g) {
         if (nrow[g] >= N) continue;
         v4u16 o;
+        with_out16(a.out_f16, [&](auto cvt) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float t;
-          if constexpr (W4) {
-            // the reference's int4 kernel keeps the factor 16 of its unpacked nibbles in the sum
-            // (a multiple of 16 below 2^28, exact in fp32) and scales left to right: routed
-            // weight, token scale, channel scale (w4a8.py:386-395)
-            t = static_cast<float>(acci[g][j][i]);
-            if (a.mul_routed) t = t * w;
-            t = t * as;
-          } else {
-            t = static_cast<float>(acci[g][j][i]) * ts;
+          for (int i = 0; i < 4; ++i) {
+            float t;
+            if constexpr (W4) {
+              // the reference's int4 kernel keeps the factor 16 of its unpacked nibbles in the sum
+              // (a multiple of 16 below 2^28, exact in fp32) and scales left to right: routed
+              // weight, token scale, channel scale (w4a8.py:386-395)
+              t = static_cast<float>(acci[g][j][i]);
+              if (a.mul_routed) t = t * w;
+              t = t * as;
+            } else {
+              t = static_cast<float>(acci[g][j][i]) * ts;
+            }
+            o[i] = cvt(t * bs4[g][i]);
           }
-          o[i] = f32_to_bf16(t * bs4[g][i]);
-        }
+        });
         *reinterpret_cast<v4u16 *>(a.C + f[j] * N + nrow[g] + 4 * c) = o;
       }
     }
@@ -329,12 +331,14 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       for (int g = 0; g < NW; ++g) {
         if (nrow[g] >= N) continue;
         v4u16 o;
+        with_out16(a.out_f16, [&](auto cvt) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float v = acc[g][j][i];
-          if (a.mul_routed) v = v * w;
-          o[i] = f32_to_bf16(v);
-        }
+          for (int i = 0; i < 4; ++i) {
+            float v = acc[g][j][i];
+            if (a.mul_routed) v = v * w;
+            o[i] = cvt(v);
+          }
+        });
         *reinterpret_cast<v4u16 *>(a.C + f[j] * N + nrow[g] + 4 * c) = o;
       }
     }

@@ -7,6 +7,7 @@ as their raw 16-bit patterns.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 import subprocess
@@ -105,26 +106,39 @@ def align_slot_mask(topk_ids, expert_map=None, num_local_tokens=None):
     return mask
 
 
+@contextlib.contextmanager
+def _elements_of(t):
+    """The C oracle reads and writes 16-bit floats as bf16 unless told otherwise: switch it to IEEE half
+    around a call whose tensors are torch.float16."""
+    assert t.dtype in (torch.bfloat16, torch.float16)
+    lib().orc_set_dtype(ctypes.c_int(1 if t.dtype == torch.float16 else 0))
+    try:
+        yield t.dtype
+    finally:
+        lib().orc_set_dtype(ctypes.c_int(0))
+
+
 def per_token_group_quant_int8(x, group_size=128, eps=1e-10):
-    assert group_size == 128 and x.dtype == torch.bfloat16
+    assert group_size == 128
     x = x.contiguous()
     C = x.shape[-1]
     R = x.numel() // C
     q = torch.empty(x.shape, dtype=torch.int8)
     s = torch.empty(x.shape[:-1] + (C // 128,), dtype=torch.float32)
-    lib().orc_group_quant_int8(_p(x), _i64(R), _i64(C), ctypes.c_float(eps), _p(q), _p(s))
+    with _elements_of(x):
+        lib().orc_group_quant_int8(_p(x), _i64(R), _i64(C), ctypes.c_float(eps), _p(q), _p(s))
     return q, s
 
 
 def per_token_quant_int8(x):
     """One scale per row, round to nearest even (int8_utils.py:20-44): q [.., C] int8, s [.., 1] f32."""
-    assert x.dtype == torch.bfloat16
     x = x.contiguous()
     C = x.shape[-1]
     R = x.numel() // C
     q = torch.empty(x.shape, dtype=torch.int8)
     s = torch.empty(x.shape[:-1] + (1,), dtype=torch.float32)
-    lib().orc_per_token_quant_int8(_p(x), _i64(R), _i64(C), _p(q), _p(s))
+    with _elements_of(x):
+        lib().orc_per_token_quant_int8(_p(x), _i64(R), _i64(C), _p(q), _p(s))
     return q, s
 
 
@@ -133,8 +147,9 @@ def fuse_silu_mul_quant(c1, return_act=False):
     S, N = c1.shape
     q = torch.empty(S, N // 2, dtype=torch.int8)
     s = torch.empty(S, 1, dtype=torch.float32)
-    act = torch.empty(S, N // 2, dtype=torch.bfloat16) if return_act else None
-    lib().orc_fuse_silu_mul_quant(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(q), _p(s), _p(act))
+    act = torch.empty(S, N // 2, dtype=c1.dtype) if return_act else None
+    with _elements_of(c1):
+        lib().orc_fuse_silu_mul_quant(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(q), _p(s), _p(act))
     return (q, s, act) if return_act else (q, s)
 
 
@@ -208,33 +223,42 @@ def moe_gemm_block_int8(A, As, W, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_
 
 def silu_and_mul(c1):
     S, N = c1.shape
-    act = torch.empty(S, N // 2, dtype=torch.bfloat16)
-    lib().orc_silu_and_mul(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(act))
+    act = torch.empty(S, N // 2, dtype=c1.dtype)
+    with _elements_of(c1):
+        lib().orc_silu_and_mul(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(act))
     return act
 
 
 def gelu_and_mul(c1):
     """act = bf16(bf16(gelu(g)) * u), gelu with erf (activation_kernels_opt.cu:234-242)."""
     S, N = c1.shape
-    act = torch.empty(S, N // 2, dtype=torch.bfloat16)
-    lib().orc_gelu_and_mul(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(act))
+    act = torch.empty(S, N // 2, dtype=c1.dtype)
+    with _elements_of(c1):
+        lib().orc_gelu_and_mul(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(act))
     return act
+
+
+def activation_table(activation="gelu", dtype=torch.bfloat16):
+    """T(act(g)) for every 16-bit pattern g of the type T, as int16 [65536]."""
+    fn = lib().orc_gelu_bf16 if activation == "gelu" else lib().orc_silu_bf16
+    fn.restype = ctypes.c_uint16
+    fn.argtypes = [ctypes.c_uint16]
+    with _elements_of(torch.empty(0, dtype=dtype)):
+        return torch.tensor([fn(i) for i in range(65536)], dtype=torch.int32).to(torch.int16)
 
 
 def gelu_bf16_table():
     """bf16(gelu(g)) for every bf16 pattern g, as int16 [65536]."""
-    fn = lib().orc_gelu_bf16
-    fn.restype = ctypes.c_uint16
-    fn.argtypes = [ctypes.c_uint16]
-    return torch.tensor([fn(i) for i in range(65536)], dtype=torch.int32).to(torch.int16)
+    return activation_table("gelu", torch.bfloat16)
 
 
 def moe_sum(inp, bias=None, factor=1.0, num_local_tokens=None, out=None):
     """With num_local_tokens, rows from that index on keep what ``out`` held."""
     M, k, H = inp.shape
-    res = torch.empty(M, H, dtype=torch.bfloat16)
-    lib().orc_moe_sum(_p(inp.contiguous()), _i64(M), _i32(k), _i64(H),
-                      _p(None if bias is None else bias.contiguous()), ctypes.c_float(factor), _p(res))
+    res = torch.empty(M, H, dtype=inp.dtype)
+    with _elements_of(inp):
+        lib().orc_moe_sum(_p(inp.contiguous()), _i64(M), _i32(k), _i64(H),
+                          _p(None if bias is None else bias.contiguous()), ctypes.c_float(factor), _p(res))
     if num_local_tokens is not None:
         n = max(0, min(M, int(num_local_tokens)))
         res[n:] = out[n:]
@@ -313,7 +337,8 @@ def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_i
     S = M * k
     Eg = E if global_num_experts == -1 else global_num_experts
     max_pad, max_blocks = align_buffer_sizes(S, Eg, block_size_m)
-    out = torch.empty(M, H, dtype=torch.bfloat16)
+    dt = x.dtype
+    out = torch.empty(M, H, dtype=dt)
     sorted_ids = torch.empty(max_pad, dtype=torch.int32)
     expert_ids = torch.empty(max_blocks, dtype=torch.int32)
     ntpp = torch.zeros(1, dtype=torch.int32)
@@ -321,19 +346,22 @@ def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_i
     if return_intermediates:
         inter = dict(
             a1q=torch.empty(M, H, dtype=torch.int8), a1s=torch.empty(M, H // 128, dtype=torch.float32),
-            c1=torch.zeros(S, 2 * I, dtype=torch.bfloat16), act=torch.empty(S, I, dtype=torch.bfloat16),
+            c1=torch.zeros(S, 2 * I, dtype=dt), act=torch.empty(S, I, dtype=dt),
             a2q=torch.empty(S, I, dtype=torch.int8), a2s=torch.empty(S, I // 128, dtype=torch.float32),
-            c3=torch.zeros(S, H, dtype=torch.bfloat16))
+            c3=torch.zeros(S, H, dtype=dt))
     ids = topk_ids.to(torch.int32).contiguous()
     tw = topk_weights.to(torch.float32).contiguous()
     emap = None if expert_map is None else expert_map.to(torch.int32).contiguous()
+    assert shared_output is None or shared_output.dtype == dt
     lib().orc_set_activation(ctypes.c_int(1 if activation == "gelu" else 0))
+    lib().orc_set_dtype(ctypes.c_int(1 if dt == torch.float16 else 0))
     try:
         rc = _call_chain(_fn, x, M, H, I, E, Eg, k, w1, w1_scale, w2, w2_scale, tw, ids, emap, block_size_m,
                          apply_router_weight_on_input, routed_scaling_factor, shared_output, out, sorted_ids,
                          max_pad, expert_ids, max_blocks, ntpp, inter)
     finally:
         lib().orc_set_activation(ctypes.c_int(0))
+        lib().orc_set_dtype(ctypes.c_int(0))
     if rc != 0:
         raise RuntimeError("oracle fused_experts: alignment failed")
     if return_intermediates:

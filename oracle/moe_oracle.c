@@ -38,9 +38,15 @@
 
 #define ORC_GROUP 128
 
-/* ---------------------------------------------------------------- bf16 -- */
+/* ------------------------------------------------------- 16-bit floats -- */
 
-static inline float bf16_to_f32(uint16_t h) {
+/* Element type of the activations: 0 = bf16 (default), 1 = IEEE half (hidden_states.dtype ==
+ * torch.float16, int8.py:689-696: compute_type follows it, so every value the path stores between
+ * its stages is rounded to that type).  A switch for the test harness, like the activation's. */
+static int g_f16 = 0;
+void orc_set_dtype(int f16) { g_f16 = f16; }
+
+static inline float raw_bf16_to_f32(uint16_t h) {
   union { uint32_t u; float f; } v;
   v.u = (uint32_t)h << 16;
   return v.f;
@@ -49,7 +55,7 @@ static inline float bf16_to_f32(uint16_t h) {
 /* Round-to-nearest-even, the rule of moe_sum_from_float
  * (moe_align_sum_kernels.cu:577-589) and of torch's BFloat16 conversion;
  * NaN is kept quiet. */
-static inline uint16_t f32_to_bf16(float f) {
+static inline uint16_t raw_f32_to_bf16(float f) {
   union { uint32_t u; float f; } v;
   v.f = f;
   if ((v.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((v.u >> 16) | 0x0040u);
@@ -57,6 +63,58 @@ static inline uint16_t f32_to_bf16(float f) {
   return (uint16_t)(v.u >> 16);
 }
 
+/* IEEE binary16 <-> binary32, spelled out on the bit patterns: subnormals on both sides, round to
+ * nearest even, overflow to infinity, NaN kept quiet.  Pinned in tests/test_oracle.py against
+ * torch's conversions on all 65536 halves and on every float that lies next to a rounding boundary
+ * of each of them. */
+static inline float raw_f16_to_f32(uint16_t h) {
+  union { uint32_t u; float f; } v;
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+  if (e == 0x1fu) {
+    v.u = sign | 0x7f800000u | (m << 13);
+  } else if (e != 0) {
+    v.u = sign | ((e + 112u) << 23) | (m << 13);
+  } else if (m == 0) {
+    v.u = sign;
+  } else { /* subnormal half: normalise */
+    int sh = 0;
+    while (!(m & 0x400u)) { m <<= 1; ++sh; }
+    v.u = sign | ((uint32_t)(113 - sh) << 23) | ((m & 0x3ffu) << 13);
+  }
+  return v.f;
+}
+
+static inline uint16_t raw_f32_to_f16(float f) {
+  union { uint32_t u; float f; } v;
+  v.f = f;
+  const uint16_t sign = (uint16_t)((v.u >> 16) & 0x8000u);
+  const uint32_t a = v.u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x3ffu)); /* NaN, quiet */
+  if (a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);                       /* >= 65536: inf */
+  if (a >= 0x38800000u) {                                                        /* normal half */
+    uint32_t r = a - 0x38000000u;             /* rebias: exponent 113 -> 1 */
+    r += 0xfffu + ((r >> 13) & 1u);           /* round to nearest even on bit 13 */
+    return (uint16_t)(sign | (r >> 13));      /* a carry out of the mantissa bumps the exponent, up to inf */
+  }
+  if (a < 0x33000000u) return sign;           /* below half of the smallest subnormal (2^-25): zero */
+  /* subnormal half: value = m * 2^-24 with m = round(|f| * 2^24) */
+  {
+    const int e = (int)(a >> 23);             /* 102 .. 112 */
+    const uint32_t m = (a & 0x7fffffu) | 0x800000u;
+    const int shift = 126 - e;                /* m * 2^(e-150) * 2^24 = m >> (126 - e) */
+    uint32_t q = m >> shift;
+    const uint32_t rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) ++q;
+    return (uint16_t)(sign | q);
+  }
+}
+
+static inline float bf16_to_f32(uint16_t h) { return g_f16 ? raw_f16_to_f32(h) : raw_bf16_to_f32(h); }
+static inline uint16_t f32_to_bf16(float f) { return g_f16 ? raw_f32_to_f16(f) : raw_f32_to_bf16(f); }
+
+uint16_t orc_f32_to_f16(float f) { return raw_f32_to_f16(f); }
+float orc_f16_to_f32(uint16_t h) { return raw_f16_to_f32(h); }
 uint16_t orc_f32_to_bf16(float f) { return f32_to_bf16(f); }
 float orc_bf16_to_f32(uint16_t h) { return bf16_to_f32(h); }
 

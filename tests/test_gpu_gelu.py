@@ -27,7 +27,7 @@ def test_gelu_table_equals_the_oracles(dev, oracle):
     say("gelu table, all 65536 entries")
     tab = torch.empty(65536, dtype=torch.int16, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().lo_gelu_bf16_table(_lib.ptr(tab), _lib.stream_of(tab)))
+        _lib.check(_lib.lib().lo_activation_table(_lib.LO_ACT_GELU, _lib.LO_BF16, _lib.ptr(tab), _lib.stream_of(tab)))
     torch.cuda.synchronize()
     ref = oracle.gelu_bf16_table()
     got = tab.cpu()

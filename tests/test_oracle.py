@@ -349,6 +349,80 @@ def test_whole_path_gelu_vs_float64_restatement(oracle, form):
     assert err.max() <= 1e-2 * ref.abs().max() and err.sum() <= 6e-3 * ref.abs().sum()
 
 
+def test_half_conversions_vs_torch(oracle):
+    """The oracle's binary16 conversions (used when the activations are float16) against torch's: every
+    half pattern, and every float that is a half, lies next to one, or lies on or next to the midpoint of
+    two neighbouring halves (the rounding boundaries), plus the overflow and underflow edges."""
+    import ctypes
+
+    import numpy as np
+
+    lib = oracle.lib()
+    lib.orc_f16_to_f32.restype = ctypes.c_float
+    lib.orc_f16_to_f32.argtypes = [ctypes.c_uint16]
+    lib.orc_f32_to_f16.restype = ctypes.c_uint16
+    lib.orc_f32_to_f16.argtypes = [ctypes.c_float]
+    h = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    ref = h.float()
+    got = torch.tensor([lib.orc_f16_to_f32(i) for i in range(65536)])
+    assert ((got.view(torch.int32) == ref.view(torch.int32)) | (got.isnan() & ref.isnan())).all()
+    fin = ref[ref.isfinite()].sort().values
+    mids = ((fin.double()[:-1] + fin.double()[1:]) / 2).float()
+    cands = [(t.view(torch.int32) + d).view(torch.float32) for t in (fin, mids) for d in (-1, 0, 1)]
+    cands.append(torch.tensor([65504.0, 65519.996, 65520.0, 65536.0, 1e10, -1e10, float("inf"), -float("inf"),
+                               2.0 ** -25, 2.0 ** -25 * 1.0000001, 2.0 ** -24, 2.0 ** -26, 0.0, -0.0]))
+    c = torch.cat(cands)
+    c = c[~c.isnan()]
+    want = c.half().view(torch.int16).numpy().astype(np.uint16)
+    have = np.array([lib.orc_f32_to_f16(float(v)) for v in c.tolist()], dtype=np.uint16)
+    assert (have == want).all()
+    assert lib.orc_f32_to_f16(float("nan")) & 0x7C00 == 0x7C00 and lib.orc_f32_to_f16(float("nan")) & 0x3FF
+
+
+@pytest.mark.parametrize("form", ["block", "channel"])
+@pytest.mark.parametrize("activation", ["silu", "gelu"])
+def test_whole_path_float16_vs_float64_restatement(oracle, form, activation):
+    """float16 activations (int8.py:689-696): the same chains with every stored value rounded to half."""
+    from lightop_amd import workloads as wl
+
+    layer = wl.TINY if form == "block" else wl.TINY_PC
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
+    M = 12
+    x, tw, ids = wl.make_inputs(layer, M, seed=2)
+    xh = x.to(torch.float16)
+    fn = oracle.fused_experts_block_int8 if form == "block" else oracle.fused_experts_channel_int8
+    out = fn(xh, w1, w2, w1s, w2s, tw, ids, 16, activation=activation)
+    assert out.dtype == torch.float16
+    assert not torch.equal(out.float(), fn(xh.to(torch.bfloat16), w1, w2, w1s, w2s, tw, ids, 16, activation=activation).float())
+    if form == "block":
+        W1 = w1.double() * w1s.double().repeat_interleave(128, 1).repeat_interleave(128, 2)
+        W2 = w2.double() * w2s.double().repeat_interleave(128, 1).repeat_interleave(128, 2)
+        a1q, a1s = oracle.per_token_group_quant_int8(xh)
+        a1 = a1q.double() * a1s.double().repeat_interleave(128, dim=1)
+    else:
+        W1, W2 = w1.double() * w1s.double(), w2.double() * w2s.double()
+        a1q, a1s = oracle.per_token_quant_int8(xh)
+        a1 = a1q.double() * a1s.double()
+    actf = torch.nn.functional.silu if activation == "silu" else torch.nn.functional.gelu
+    ref = torch.zeros(M, layer.H, dtype=torch.float64)
+    for t in range(M):
+        for j in range(layer.top_k):
+            e = int(ids[t, j])
+            c1 = (W1[e] @ a1[t]).float().to(torch.float16)
+            act = (actf(c1[: layer.I].float()).to(torch.float16).float() * c1[layer.I:].float()).to(torch.float16)
+            if form == "block":
+                a2q, a2s = oracle.per_token_group_quant_int8(act.reshape(1, -1))
+                a2 = (a2q.double() * a2s.double().repeat_interleave(128, dim=1))[0]
+            else:
+                a2q, a2s = oracle.per_token_quant_int8(act.reshape(1, -1))
+                a2 = (a2q.double() * a2s.double())[0]
+            ref[t] += float(tw[t, j]) * (W2[e] @ a2).float().to(torch.float16).double()
+    err = (out.double() - ref).abs()
+    assert ref.abs().max() > 0.05
+    # half keeps three more mantissa bits than bf16: the tolerance of the path with room to spare
+    assert err.max() <= 1e-2 * ref.abs().max() and err.sum() <= 6e-3 * ref.abs().sum()
+
+
 # ------------------------------------------------------------------ moe_sum ----
 
 def test_moe_sum_cases(oracle):
