@@ -514,6 +514,7 @@ def main():
     if args.sweep != "none":
         plan = [(wl.QWEN3_30B, [1, 8, 32, 128, 512, 2048, 8192]), (wl.DSV3_EP, [1, 16, 64, 256, 1024, 4096])]
         plan.append((wl.QWEN3_235B_W4, [1, 32, 256, 2048]))
+        plan.append((wl.QWEN3_235B_W4_PC, [32, 2048, 8192]))  # the reference's own W4A8 form
         plan.append((wl.QWEN3_30B_PC, [32, 512, 8192]))
         plan.append((wl.DSV3_EP_PC, [64, 4096]))
         plan.append((wl.DSV3_FULL, [8192]))  # all 256 experts resident (11.3 GB), Zipf-skewed routing
