@@ -186,9 +186,15 @@ class Point:
                 mask = None
                 s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
             ev[2].record()
-            a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
-                                                             L.top_k, S, cfg, fused_scale=fused_scale, flags=wflag,
-                                                             global_num_experts=L.E_global)
+            if bs == 160:  # 160-token blocks: plain first GEMM, activation and quantisation in a launch of their own
+                c1 = self.cache13[: S * 2 * L.I].view(S, 2 * L.I)
+                moe.invoke_fused_moe_kernel_int8(a1q, self.w1, c1, a1s, self.w1s, tw, s, e, p, False, L.top_k, cfg,
+                                                 fused_scale=fused_scale, flags=wflag, global_num_experts=L.E_global)
+                a2q, a2s = moe.act_and_mul_group_quant(c1)
+            else:
+                a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
+                                                                 L.top_k, S, cfg, fused_scale=fused_scale,
+                                                                 flags=wflag, global_num_experts=L.E_global)
             ev[3].record()
             moe.invoke_fused_moe_kernel_int8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, True, 1, cfg,
                                              fused_scale=fused_scale, flags=g2flag, global_num_experts=L.E_global)

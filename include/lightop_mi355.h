@@ -238,6 +238,14 @@ int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *ac
  */
 int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *act,
                     lo_stream_t stream);
+/*
+ * The gated activation followed by the 1x128 group quantisation in one pass: c1 [rows, 2I] ->
+ * q [rows, I] int8, s [rows, I/128] f32.  Replaces the pair of calls between the two GEMMs where the
+ * first GEMM's epilogue does not do it: silu_and_mul + per_token_group_quant_int8 (int8.py:811-823) or
+ * gelu_and_mul + per_token_group_quant_int8 (int8.py:826-838).  activation: LO_ACT_SILU / LO_ACT_GELU.
+ */
+int lo_act_mul_group_quant(const void *c1, int dtype, int activation, int64_t rows, int64_t I, int8_t *q,
+                           float *s, lo_stream_t stream);
 /* The 65536 values T(act(g)), indexed by the bit pattern of g, that the kernels look up for activation
  * LO_ACT_SILU / LO_ACT_GELU and element type LO_BF16 / LO_F16, copied to table_out (device memory,
  * 128 KB).  For tests; no counterpart in the reference. */

@@ -85,11 +85,15 @@ static WsLayout ws_layout(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_
   return L;
 }
 
+// 160-token blocks: the first GEMM's bf16 output [S, 2I] has to fit the caller's [S, H] buffer, and both K
+// extents the kernel's scale table (128 K blocks).
+static bool blocks_of_160_fit(int64_t H, int64_t I) { return 2 * I <= H && H / kGroup <= 128 && I / kGroup <= 128; }
+
 // gfx950 tile table.  The token tile (= alignment block) follows the expected number
 // of slots per expert: small tiles waste no MFMA columns on padding while the layer
 // is weight-streaming bound, larger ones amortise each pass over an expert's weights.
 static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64_t H, int form = LO_FORM_BLOCK,
-                            bool preshuffled = true, bool int4_channel = false) {
+                            bool preshuffled = true, bool int4_channel = false, bool allow160 = false) {
   const double per_expert = static_cast<double>(M) * top_k / (num_experts > 0 ? num_experts : 1);
   // Packed int4 weights with per-channel scales: the 128-token kernel has no scale arithmetic in
   // its K loop and skips the padded part of a block, so it takes over as soon as an expert sees more
@@ -115,6 +119,17 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   // 191, at 2048: 878 / 690 / 267 / 285, at 8192: - / - / 682 / 645; DeepSeek-V3 share of 32
   // experts at 128 tokens 248 / 262 / 315 / 241, at 2048: 1034 / 810 / 427 / 336, at 8192:
   // - / - / 928 / 776.
+  // Around 128 slots per expert a 128-token block spills a few tokens into a second block on half of
+  // the experts, and that remainder block is a second pass over the expert's weights - the bytes the
+  // stage is bound by at that size.  160-token blocks (the same kernel with ten token fragments, plain
+  // epilogues, the activation in a launch of its own) hold such an expert in one block.  Measured,
+  // whole path in us, table before / 160: Qwen3-30B-A3B layer at 1280 tokens (80 slots per expert)
+  // 239 / 229, 1536: 264 / 230, 1792: 275 / 239, 2048: 302 / 265, 2304: 351 / 301, 2560: 348 / 355;
+  // DeepSeek-V3 share at 3072 (96 per expert): 435 / 451, 3584: 544 / 468, 4096: 581 / 495, 4352:
+  // 610 / 616, 4608: 620 / 660.
+  if (form == LO_FORM_BLOCK && preshuffled && allow160) {
+    if (H >= 4096 ? (per_expert >= 104.0 && per_expert < 134.0) : (per_expert >= 80.0 && per_expert < 152.0)) return 160;
+  }
   if (form == LO_FORM_BLOCK && preshuffled) {
     if (per_expert < (H >= 4096 ? 4.0 : 12.0)) return 16;
     if (H < 4096 && per_expert >= 96.0 && per_expert < 192.0) return 64;
@@ -146,7 +161,9 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
   if (form == LO_FORM_W4) flags |= LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED;
   const bool pre = (flags & LO_GEMM_W_PRESHUFFLED) != 0;
   const int32_t bm = pick_block_m(M, num_experts, top_k, H, form, pre,
-                                  form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4));
+                                  form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4),
+                                  form == LO_FORM_BLOCK && pre && blocks_of_160_fit(H, I) &&
+                                      !(flags & LO_FUSED_ACT_GELU));
   // the argument blocks the stage entry points would build for this problem
   GemmArgs a{};
   a.num_valid = M * top_k;
@@ -158,7 +175,8 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
   a.per_channel = form == LO_FORM_CHANNEL ? 1 : 0;
   if (gemm1) {
     a.N = 2 * I; a.K = H; a.a_rows = M;
-    const bool fused = form != LO_FORM_CHANNEL; // the per-channel form quantises in a launch of its own
+    // the per-channel form and 160-token blocks apply the activation and quantise in a launch of their own
+    const bool fused = form != LO_FORM_CHANNEL && bm != 160;
     describe_gemm_kernel(pick_gemm_kernel(a, fused, bm, flags), fused, bm, gemm1);
   }
   if (gemm2) {
@@ -190,7 +208,7 @@ extern "C" int64_t lo_fused_experts_workspace_bytes(int64_t M, int32_t top_k, in
   // 0: whatever the table (or a later explicit choice) picks.  The sorted ids grow with the block
   // size, the per-block expert ids shrink with it: take the largest layout of the four.
   int64_t most = 0;
-  for (int32_t bs : {16, 32, 64, 128}) {
+  for (int32_t bs : {16, 32, 64, 128, 160}) {
     const int64_t t = ws_layout(M, top_k, H, I, num_experts, bs).total;
     most = t > most ? t : most;
   }
@@ -229,9 +247,17 @@ extern "C" int lo_fused_experts_block_int8(
   const bool block_size_m_auto = block_size_m == 0;
   if (block_size_m == 0)
     block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
-                                (flags & LO_GEMM_W_PRESHUFFLED) != 0);
-  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
-             LO_EINVAL, "fused_experts: block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
+                                (flags & LO_GEMM_W_PRESHUFFLED) != 0, false,
+                                !(flags & LO_GEMM_W4) && dtype == LO_BF16 && !(flags & LO_FUSED_ACT_GELU) &&
+                                    blocks_of_160_fit(H, I));
+  // 160: the 160-token form of the direct-to-LDS kernel (int8 block form, load-time layout), both GEMMs
+  // with plain epilogues and the activation in a launch of its own
+  const bool bs160 = block_size_m == 160 && (flags & LO_GEMM_W_PRESHUFFLED) && !(flags & LO_GEMM_W4) &&
+                     blocks_of_160_fit(H, I);
+  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 || bs160,
+             LO_EINVAL,
+             "fused_experts: block_size_m %d is not one of 16, 32, 64, 128 (160: int8 weights in the load-time "
+             "layout and 2I <= H only)", block_size_m);
   const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
   LO_REQUIRE(workspace_bytes >= L.total, LO_ENOSPC, "fused_experts: workspace holds %lld bytes, needs %lld",
              (long long)workspace_bytes, (long long)L.total);
@@ -252,7 +278,7 @@ extern "C" int lo_fused_experts_block_int8(
   const bool gelu = (flags & LO_FUSED_ACT_GELU) != 0;
   // GELU and fp16 activations have no fused epilogue: the first GEMM writes [S, 2I] in the activation
   // type, one launch applies the gated activation and quantises
-  const bool unfused = gelu || dtype != LO_BF16;
+  const bool unfused = gelu || dtype != LO_BF16 || bs160;
   if (block_size_m_auto && (flags & (LO_GEMM_W_PRESHUFFLED | LO_GEMM_W4)) && !unfused &&
       !(flags & LO_FUSED_NO_DECODE_PATH)) {
     // (cache3 is the front of the caller's cache13: the path keeps its bf16 activations [S, I] there)
@@ -278,12 +304,13 @@ extern "C" int lo_fused_experts_block_int8(
   }
   if (rc) return rc;
   if (unfused) {
-    // rows of experts on other ranks are zero-filled by the first GEMM: the activation launch reads every row
+    // rows of slots whose expert another rank holds are neither written by the first GEMM nor read by
+    // the activation launch (the slot mask of the alignment says which)
     rc = lo_moe_gemm_block_int8(a1q, a1s, w1, w1s, cache3, dtype, topk_w, sorted, eids, ntpp, L.sorted_cap, S, M, E,
                                 num_experts, 2 * I, H, top_k, block_size_m, apply_router_weight_on_input,
-                                flags & ~LO_FUSED_ACT_GELU, stream);
+                                (flags & ~LO_FUSED_ACT_GELU) | (mask ? LO_GEMM_SKIP_NONLOCAL : 0), stream);
     if (rc) return rc;
-    rc = launch_act_mul_group_quant(cache3, dtype, gelu ? LO_ACT_GELU : LO_ACT_SILU, S, I, a2q, a2s,
+    rc = launch_act_mul_group_quant(cache3, dtype, gelu ? LO_ACT_GELU : LO_ACT_SILU, S, I, a2q, a2s, mask,
                                     static_cast<hipStream_t>(stream));
   } else {
     rc = lo_moe_gemm1_silu_quant_block_int8(a1q, a1s, w1, w1s, a2q, a2s, dtype, topk_w, sorted, eids,
@@ -426,9 +453,12 @@ extern "C" int lo_fused_experts_block_int8_noalloc(
   const int32_t block_size_m_arg = block_size_m;
   if (block_size_m == 0)
     block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
-                                (flags & LO_GEMM_W_PRESHUFFLED) != 0);
-  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
-             LO_EINVAL, "fused_experts(noalloc): block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
+                                (flags & LO_GEMM_W_PRESHUFFLED) != 0, false,
+                                !(flags & LO_GEMM_W4) && dtype == LO_BF16 && !(flags & LO_FUSED_ACT_GELU) &&
+                                    blocks_of_160_fit(H, I));
+  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 ||
+                 block_size_m == 160,
+             LO_EINVAL, "fused_experts(noalloc): block_size_m %d is not one of 16, 32, 64, 128, 160", block_size_m);
   const int64_t need = ws_layout(M, top_k, H, I, num_experts, block_size_m).total;
   LO_REQUIRE(need <= kScratchBytes, LO_ENOSPC,
              "fused_experts(noalloc): this problem needs %lld bytes of scratch, the built-in scratch holds %lld; "

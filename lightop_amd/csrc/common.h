@@ -43,8 +43,9 @@ int act_table(hipStream_t stream, int act, int dtype, const uint16_t **table);
 // The gated activation of c1 [rows, 2I] from its table, followed by the 1x128 group quantisation
 // (q [rows, I], s [rows, I/128]) or by the per-token quantisation (s [rows]; SiLU without a floor
 // under the row maximum, as fuse_silu_mul_quant, GELU with per_token_quant_int8's), one launch each.
+// row_mask (optional, [rows] bytes): rows whose byte is 0 are skipped.
 int launch_act_mul_group_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
-                               hipStream_t stream);
+                               const uint8_t *row_mask, hipStream_t stream);
 int launch_act_mul_row_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
                              const int32_t *num_local_tokens, int32_t top_k, const int32_t *row_ids,
                              hipStream_t stream);

@@ -70,12 +70,14 @@ template <int DT>
 __global__ __launch_bounds__(256) void act_mul_group_quant_kernel(const uint16_t *__restrict__ c1, int64_t rows,
                                                                   int64_t I, const uint16_t *__restrict__ table,
                                                                   float eps, int8_t *__restrict__ q,
-                                                                  float *__restrict__ s) {
+                                                                  float *__restrict__ s,
+                                                                  const uint8_t *__restrict__ row_mask) {
   const int64_t gpr = I / kGroup, groups = rows * gpr;
   const int sub = threadIdx.x & 15;
   for (int64_t g = static_cast<int64_t>(blockIdx.x) * 16 + (threadIdx.x >> 4); g < groups;
        g += static_cast<int64_t>(gridDim.x) * 16) {
     const int64_t r = g / gpr, c = (g % gpr) * kGroup + sub * 8;
+    if (row_mask && !row_mask[r]) continue; // a slot of an expert held elsewhere: nobody reads its row
     const v8u16 ga = *reinterpret_cast<const v8u16 *>(c1 + r * 2 * I + c);
     const v8u16 up = *reinterpret_cast<const v8u16 *>(c1 + r * 2 * I + I + c);
     float v[8];
@@ -449,7 +451,7 @@ int act_table(hipStream_t stream, int act, int dtype, const uint16_t **out) {
 // The launch between the GEMMs where no fused epilogue exists (GELU; fp16 activations): the gated
 // activation from its table and the quantisation of the form in one pass over c1 [rows, 2I].
 int launch_act_mul_group_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
-                               hipStream_t stream) {
+                               const uint8_t *row_mask, hipStream_t stream) {
   const uint16_t *table = nullptr;
   int rc = act_table(stream, act, dtype, &table);
   if (rc) return rc;
@@ -458,10 +460,10 @@ int launch_act_mul_group_quant(const void *c1, int dtype, int act, int64_t rows,
   const dim3 g(grid_for(groups, 16)), b(256);
   if (dtype == LO_F16)
     hipLaunchKernelGGL(act_mul_group_quant_kernel<LO_F16>, g, b, 0, stream, static_cast<const uint16_t *>(c1), rows, I,
-                       table, 1e-10f, q, s);
+                       table, 1e-10f, q, s, row_mask);
   else
     hipLaunchKernelGGL(act_mul_group_quant_kernel<LO_BF16>, g, b, 0, stream, static_cast<const uint16_t *>(c1), rows, I,
-                       table, 1e-10f, q, s);
+                       table, 1e-10f, q, s, row_mask);
   return check_launch("act_mul_group_quant");
 }
 
@@ -585,6 +587,20 @@ extern "C" int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
                        static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I, table,
                        static_cast<uint16_t *>(act));
   return check_launch("gelu_and_mul");
+}
+
+extern "C" int lo_act_mul_group_quant(const void *c1, int dtype, int activation, int64_t rows, int64_t I, int8_t *q,
+                                      float *s, lo_stream_t stream) {
+  using namespace lo;
+  LO_REQUIRE(c1 && q && s, LO_EINVAL, "act_mul_group_quant: null pointer");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "act_mul_group_quant: bf16 or fp16");
+  LO_REQUIRE(activation == LO_ACT_SILU || activation == LO_ACT_GELU, LO_EINVAL,
+             "act_mul_group_quant: unknown activation %d", activation);
+  LO_REQUIRE(rows >= 0 && I > 0 && I % kGroup == 0, LO_EINVAL,
+             "act_mul_group_quant: the output width (%lld) must be a multiple of 128", (long long)I);
+  LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0, LO_EINVAL,
+             "act_mul_group_quant: input must be 16-byte and q 8-byte aligned");
+  return launch_act_mul_group_quant(c1, dtype, activation, rows, I, q, s, nullptr, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int lo_activation_table(int activation, int dtype, void *table_out, lo_stream_t stream) {

@@ -158,7 +158,7 @@ int launch_gemm_as(const GemmArgs &a, int flags, int block_size_m, int64_t m_blo
 bool gemm_as_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 
 // 128-token kernel, two four-wave workgroups per compute unit (gemm_t128.hip): pre-shuffled int8 weights.
-int launch_gemm_t128(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);
+int launch_gemm_t128(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks, hipStream_t s);
 bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m);
 // W4A8 LDS-tiled kernel (gemm_w4.hip): block_size_m 64.
 int launch_gemm_w4_tile(const GemmArgs &a, bool fused_act, int flags, int64_t m_blocks, hipStream_t s);

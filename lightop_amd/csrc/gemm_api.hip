@@ -33,6 +33,7 @@ static int validate_common(const char *who, const void *A, const void *As, const
 // per expert large enough for operand reuse to matter); smaller ones stream weights.  The tile
 // query (lo_moe_tile_query_form) reports this very choice.
 int pick_gemm_kernel(const GemmArgs &a, bool fused_act, int bs, int flags) {
+  if (bs == 160) return LO_KERNEL_T128; // 160-token blocks exist for that kernel only (the entry point checks)
   const bool tiled = !(flags & LO_GEMM_FORCE_STREAMING);
   if (a.w4 && a.per_channel) // the reference's own int4 form: 128-token LDS tiles, else streaming
     return tiled && gemm_t128_supports(a, fused_act, bs) ? LO_KERNEL_T128 : LO_KERNEL_WS;
@@ -77,7 +78,7 @@ void describe_gemm_kernel(int kernel, bool fused_act, int bs, lo_moe_tile *t) {
 static int launch_gemm(const GemmArgs &a, bool fused_act, int bs, int flags, int64_t m_blocks,
                        hipStream_t s) {
   switch (pick_gemm_kernel(a, fused_act, bs, flags)) {
-  case LO_KERNEL_T128: return launch_gemm_t128(a, fused_act, flags, m_blocks, s);
+  case LO_KERNEL_T128: return launch_gemm_t128(a, fused_act, bs, flags, m_blocks, s);
   case LO_KERNEL_W4_TILE: return launch_gemm_w4_tile(a, fused_act, flags, m_blocks, s);
   case LO_KERNEL_PC: return launch_gemm_pc(a, bs, m_blocks, s);
   case LO_KERNEL_AS: return launch_gemm_as(a, flags, bs, m_blocks, s);
@@ -99,8 +100,8 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   int rc = validate_common("moe_gemm", A, As, W, Ws, sorted_ids, expert_ids, num_tokens_post_pad, K,
                            top_k, E, a_rows);
   if (rc) return rc;
-  LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL, "moe_gemm: block_size_m %d is not one of 16, 32, 64, 128",
-             block_size_m);
+  LO_REQUIRE(valid_block_m(block_size_m) || block_size_m == 160, LO_EINVAL,
+             "moe_gemm: block_size_m %d is not one of 16, 32, 64, 128 (or 160)", block_size_m);
   LO_REQUIRE(C, LO_EINVAL, "moe_gemm: null output");
   LO_REQUIRE(c_dtype == LO_BF16 || c_dtype == LO_F16, LO_ENOTSUP, "moe_gemm: the output is bf16 or fp16");
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm: N (%lld) must be a multiple of 16", (long long)N);
@@ -122,6 +123,9 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   LO_REQUIRE(!a.w4 || a.w_shuffled, LO_ENOTSUP,
              "moe_gemm: int4 weights must be in the layout of lo_preshuffle_weight_int4 (LO_GEMM_W_PRESHUFFLED)");
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
+  LO_REQUIRE(block_size_m != 160 || gemm_t128_supports(a, false, 160), LO_ENOTSUP,
+             "moe_gemm: 160-token blocks need int8 weights in the load-time layout (LO_GEMM_W_PRESHUFFLED), "
+             "N a multiple of 64 and K <= %d", kGroup * 128);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 30), LO_EINVAL, "moe_gemm: grid too large");
   if (mblocks == 0) return LO_OK;
@@ -139,7 +143,8 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
                            num_tokens_post_pad, K, top_k, E, a_rows);
   if (rc) return rc;
   LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL,
-             "moe_gemm1_silu_quant: block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
+             "moe_gemm1_silu_quant: block_size_m %d is not one of 16, 32, 64, 128 (160-token blocks have no fused "
+             "epilogue: lo_moe_gemm_block_int8, then lo_act_mul_group_quant)", block_size_m);
   LO_REQUIRE(A2q && A2s, LO_EINVAL, "moe_gemm1_silu_quant: null output");
   LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm1_silu_quant: only bf16 rounding is built");
   LO_REQUIRE(I > 0 && I % kGroup == 0, LO_EINVAL,

@@ -43,6 +43,11 @@ constexpr int kTMaxKB = 128;                  // K blocks whose weight-block sca
 constexpr int kTBs = 2 * kTMaxKB * 4;         // [fragment][K block] weight-block scales of the tile
 constexpr int kTIds = kT * 4;                  // the tile's sorted ids, for the epilogues
 constexpr int kTLds = kTW + kTA + kTS + kTRed + kTBs + kTIds + 2 * kSiluBandN * 2;
+// NTB = 10: 160 tokens per workgroup (plain epilogue only: no amax exchange, no SiLU band), for layers
+// whose experts see a few tokens more than 128: a remainder block is a second pass over the expert's
+// weights, and at that size the weights are what the stage streams.
+constexpr int kT160 = 160;
+constexpr int kTLds160 = kTW + 2 * kT160 * kGroup + 2 * kT160 * 4 + kTBs + kT160 * 4;
 constexpr int kTPitch = 144;                  // staging pitch of the epilogues: 128 + 16
 
 // Wait until all but the newest `N` vector-memory operations of this wave are complete and its
@@ -62,21 +67,26 @@ __device__ __forceinline__ void wait_copies_barrier() {
 // python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341-395): one scale per token row and one
 // per weight row, both applied in the epilogue, so the int32 sums run over the whole K inside the
 // MFMA accumulators and the K loop has no scale arithmetic at all.
-template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM, bool W4, bool PC = false>
+template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM, bool W4, bool PC = false, int NTB = 8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   static_assert(!PC || (W4 && !FUSED_ACT && !FAST_SCALE), "per-channel scales: plain int4 GEMM only");
+  static_assert(NTB == 8 || (NTB == 10 && !FUSED_ACT && !W4 && !PC), "160-token tiles: plain int8 block form only");
+  constexpr int T = 16 * NTB;        // tokens per workgroup
+  constexpr int AST = T * kGroup;    // token rows of one K block
+  constexpr int APW = NTB / 2;       // 1 KB pieces (eight token rows) of a token stage that a wave copies
+  constexpr int RED = NTB == 8 ? kTRed : 0;
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   int8_t *const sA = smem + kTW;
-  float *const sS = reinterpret_cast<float *>(smem + kTW + kTA);
-  float *const sRed = reinterpret_cast<float *>(smem + kTW + kTA + kTS);
-  float *const sBs = reinterpret_cast<float *>(smem + kTW + kTA + kTS + kTRed);
-  int32_t *const sIds = reinterpret_cast<int32_t *>(smem + kTW + kTA + kTS + kTRed + kTBs);
-  uint16_t *const sSilu = reinterpret_cast<uint16_t *>(smem + kTW + kTA + kTS + kTRed + kTBs + kTIds);
+  float *const sS = reinterpret_cast<float *>(smem + kTW + 2 * AST);
+  float *const sRed = reinterpret_cast<float *>(smem + kTW + 2 * AST + 2 * T * 4);
+  float *const sBs = reinterpret_cast<float *>(smem + kTW + 2 * AST + 2 * T * 4 + RED);
+  int32_t *const sIds = reinterpret_cast<int32_t *>(smem + kTW + 2 * AST + 2 * T * 4 + RED + kTBs);
+  uint16_t *const sSilu = reinterpret_cast<uint16_t *>(smem + kTW + 2 * AST + 2 * T * 4 + RED + kTBs + T * 4);
 
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
-  if (static_cast<int64_t>(mb) * kT >= a.ntpp[0]) return;
+  if (static_cast<int64_t>(mb) * T >= a.ntpp[0]) return;
   // An expert_map entry outside the weight tensor is treated like an expert of another rank, but its
   // rows are always zero-filled: the slot mask of the alignment counts such a slot as local.
   const int e_raw = a.expert_ids[mb];
@@ -88,7 +98,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   const int64_t K = a.K, N = a.N;
   const int KB = static_cast<int>(K / kGroup);
   const int64_t I = N / 2;
-  const int32_t *const sorted = a.sorted + static_cast<int64_t>(mb) * kT;
+  const int32_t *const sorted = a.sorted + static_cast<int64_t>(mb) * T;
 
   // first row of the wave's 64 (plain) or of its 32 gate rows (fused)
   const int64_t nrow0 = FUSED_ACT ? static_cast<int64_t>(nt) * kGroup + wave * 32
@@ -99,7 +109,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     if constexpr (!FUSED_ACT) {
       if (wave_active && (!a.skip_nonlocal || e_oob)) {
 #pragma unroll
-        for (int tb = 0; tb < 8; ++tb) {
+        for (int tb = 0; tb < NTB; ++tb) {
           const int64_t ft = sorted[tb * 16 + r];
           if (ft < a.num_valid)
 #pragma unroll
@@ -163,10 +173,10 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 2][(p >> 1) & 1], (p & 1) * 1024, 0,
                                                kWAux);
   }
-  int avoff[4]; // 1 KB pieces wave*4 + j of a token stage: eight token rows each
+  int avoff[5]; // 1 KB pieces wave*APW + j of a token stage, j < APW: eight token rows each
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int t = (wave * 4 + j) * 8 + (lane >> 3);
+  for (int j = 0; j < APW; ++j) {
+    const int t = (wave * APW + j) * 8 + (lane >> 3);
     const int64_t lf = sorted[t];
     const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
     const int piece = (lane & 7) ^ (t & 7); // slot lane & 7 of row t holds piece slot ^ (t & 7)
@@ -180,17 +190,21 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   {
     const uint64_t v0 = __builtin_amdgcn_ballot_w64(sorted[lane] < a.num_valid);
     const uint64_t v1 = __builtin_amdgcn_ballot_w64(sorted[lane + 64] < a.num_valid);
-    const int last = v1 ? 127 - __builtin_clzll(v1) : (v0 ? 63 - __builtin_clzll(v0) : 0);
-    nst = __builtin_amdgcn_readfirstlane(4 * ((last >> 5) + 1)); // the K loop comes in variants of 2, 4, 6, 8 fragments
+    int last = v1 ? 127 - __builtin_clzll(v1) : (v0 ? 63 - __builtin_clzll(v0) : 0);
+    if constexpr (NTB == 10) {
+      const uint64_t v2 = __builtin_amdgcn_ballot_w64(lane < 32 && sorted[128 + (lane & 31)] < a.num_valid);
+      if (v2) last = 191 - __builtin_clzll(v2);
+    }
+    nst = __builtin_amdgcn_readfirstlane(4 * ((last >> 5) + 1)); // the K loop comes in variants of 2, 4, 6, 8 (, 10) fragments
   }
-  int asoff; // thread t and thread t + 128 both carry the scale of token t
+  int asoff; // thread t and thread t + T both carry the scale of token t
   {
-    const int64_t lf = sorted[tid & (kT - 1)];
+    const int64_t lf = sorted[NTB == 8 ? (tid & (T - 1)) : (tid < T ? tid : tid - T)];
     const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
     asoff = static_cast<int>(lrow * (PC ? 1 : KB) * 4);
     // The epilogues take the ids from LDS: a global load in each of their exec-masked blocks is a
     // full memory round trip that nothing overlaps.
-    if (tid < kT) sIds[tid] = static_cast<int32_t>(lf);
+    if (tid < T) sIds[tid] = static_cast<int32_t>(lf);
   }
   // weight-block scales of the tile: table row 0 / 1 = gate / up block (fused), or the first / second
   // 128 rows of the tile (plain: waves 0, 1 / waves 2, 3).  Thread t fetches entry (t >> 7, t & 127).
@@ -205,7 +219,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   const float *const sBs0 = sBs + (FUSED_ACT ? 0 : (wave >> 1) * kTMaxKB);
   const float *const sBs1 = sBs + (FUSED_ACT ? kTMaxKB : (wave >> 1) * kTMaxKB);
 
-  // piece p of the 12 copies a wave issues per K block: 0..7 its weights, 8..11 token rows
+  // piece p of the 8 + APW copies a wave issues per K block: 0..7 its weights, then its token rows
   auto copy_piece = [&](int p, int kb) __attribute__((always_inline)) {
     const int kc = kb < KB ? kb : KB - 1;
     if (p < 8) {
@@ -223,13 +237,13 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
       }
     } else {
       const int j = p - 8;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rA, sA + (kb & 1) * kTAStage + wave * 4096 + j * 1024, 16, avoff[j],
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rA, sA + (kb & 1) * AST + (wave * APW + j) * 1024, 16, avoff[j],
                                                __builtin_amdgcn_readfirstlane(kc) * kGroup, 0, 0);
     }
   };
   auto copy_a = [&](int kb) __attribute__((always_inline)) {
 #pragma unroll
-    for (int p = 8; p < 12; ++p) copy_piece(p, kb);
+    for (int p = 8; p < 8 + APW; ++p) copy_piece(p, kb);
   };
   auto load_scale = [&](int kb) __attribute__((always_inline)) {
     if constexpr (PC) return 0.0f; // one scale per token, read by the epilogue
@@ -242,20 +256,20 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
   for (int kh = 0; kh < 2; ++kh) alds[kh] = r * kGroup + (((4 * kh + q) ^ (r & 7)) * 16);
 
-  float acc[2][8][2][4]; // [step half][token fragment][fragment of the half][element]
+  float acc[2][NTB][2][4]; // [step half][token fragment][fragment of the half][element]
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int tb = 0; tb < 8; ++tb)
+    for (int tb = 0; tb < NTB; ++tb)
 #pragma unroll
       for (int rf = 0; rf < 2; ++rf)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[h][tb][rf][i] = 0.0f;
-  v4i acci[2][8][2]; // PC: the whole-K int32 sums
+  v4i acci[2][NTB][2]; // PC: the whole-K int32 sums
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int tb = 0; tb < 8; ++tb)
+    for (int tb = 0; tb < NTB; ++tb)
 #pragma unroll
       for (int rf = 0; rf < 2; ++rf) acci[h][tb][rf] = v4i{0, 0, 0, 0};
 
@@ -336,10 +350,12 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   v4i bf_first[2];   // first token fragment of the next K block
   float as_first = 0.0f;
   auto kblock = [&](auto NST, int kb) __attribute__((always_inline)) {
-    constexpr int nst_c = decltype(NST)::value; // stages of this variant: 4, 8, 12 or 16
-    constexpr bool kEarly = nst_c == 16 && !W4;
-    const int8_t *ta = sA + (kb & 1) * kTAStage;
-    const float *ts = sS + (kb & 1) * kT;
+    constexpr int nst_c = decltype(NST)::value; // stages of this variant: 4, 8, 12, 16 (or 20)
+    constexpr int kFull = 2 * NTB;              // stages of a full tile
+    constexpr int kE0 = kFull - 2, kE1 = kFull - 1;
+    constexpr bool kEarly = nst_c == kFull && !W4;
+    const int8_t *ta = sA + (kb & 1) * AST;
+    const float *ts = sS + (kb & 1) * T;
     v4i bf[2][2];
     float as_t[2];
     if constexpr (kEarly) {
@@ -380,22 +396,23 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     // pipeline stage (tb, h): its MFMAs are issued, then the previous stage's fragments are folded
     // while the matrix pipe works; the operands of token fragment tb + 1 are requested in (tb, 0)
 #pragma unroll
-    for (int st = 0; st < 16; ++st) {
+    for (int st = 0; st < kFull; ++st) {
       const int tb = st >> 1, h = st & 1;
       const int cur = tb & 1, nxt = cur ^ 1;
       if (nst_c >= 8 && st < 6) {
         copy_piece(2 * st, kb + 1);
         copy_piece(2 * st + 1, kb + 1);
       }
+      if (NTB == 10 && nst_c >= 8 && st == 6) copy_piece(12, kb + 1); // the fifth token piece of a 160-token stage
       if (nst_c < 8 && st < 4) {
         copy_piece(3 * st, kb + 1);
         copy_piece(3 * st + 1, kb + 1);
         copy_piece(3 * st + 2, kb + 1);
       }
       if (st < nst_c) {
-        if (kEarly && st == 14) {
+        if (kEarly && st == kE0) {
           wait_copies_barrier<0>();
-          if (tid < kT) sS[(kb & 1) * kT + tid] = kb + 2 < KB ? s_pending : 0.0f;
+          if (tid < T) sS[(kb & 1) * T + tid] = kb + 2 < KB ? s_pending : 0.0f;
           s_pending = load_scale(kb + 3);
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -416,17 +433,17 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
           acci[h][tb][0] = d[0];
           acci[h][tb][1] = d[1];
         }
-        if (kEarly && st >= 14) { // the next K block's operands of this half, over the ones just used
+        if (kEarly && st >= kE0) { // the next K block's operands of this half, over the ones just used
 #pragma unroll
           for (int rf = 0; rf < 2; ++rf)
 #pragma unroll
             for (int kh = 0; kh < 2; ++kh)
               w[h][rf][kh] = *reinterpret_cast<const v4i *>(sWw + ((h * 2 + rf) * 2 + kh) * 1024 + lane * 16);
-          if (st == 14) {
-            const int8_t *tan = sA + ((kb + 1) & 1) * kTAStage;
+          if (st == kE0) {
+            const int8_t *tan = sA + ((kb + 1) & 1) * AST;
 #pragma unroll
             for (int kh = 0; kh < 2; ++kh) bf_first[kh] = *reinterpret_cast<const v4i *>(tan + alds[kh]);
-            as_first = sS[((kb + 1) & 1) * kT + r];
+            as_first = sS[((kb + 1) & 1) * T + r];
           }
         }
         if (st > 0) fold_stage(st - 1);
@@ -434,11 +451,12 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (nst_c >= 8 ? (g < 2 && st < 6) : (g < 3 && st < 4)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          if (nst_c >= 8 ? ((g < 2 && st < 6) || (NTB == 10 && g == 0 && st == 6)) : (g < 3 && st < 4))
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x002, W4 ? 7 : 5, 0);
         }
-        if (kEarly && st == 14) __builtin_amdgcn_sched_group_barrier(0x100, 7, 0);
-        if (kEarly && st == 15) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        if (kEarly && st == kE0) __builtin_amdgcn_sched_group_barrier(0x100, 7, 0);
+        if (kEarly && st == kE1) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
         __builtin_amdgcn_sched_barrier(0);
         dprev[0] = d[0];
         dprev[1] = d[1];
@@ -461,16 +479,16 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   __builtin_amdgcn_sched_barrier(0);
   copy_a(0);
   __builtin_amdgcn_sched_barrier(0);
-  if (tid < kT) sS[tid] = s_now;
+  if (tid < T) sS[tid] = s_now;
   sBs[tid] = bs_mine;
   if constexpr (FUSED_ACT) silu_band_store(sSilu, band_regs, tid);
   wait_copies<0>();
   read_w();
 
   auto k_loop = [&](auto NST) __attribute__((always_inline)) {
-    if constexpr (decltype(NST)::value == 16 && !W4) {
+    if constexpr (decltype(NST)::value == 2 * NTB && !W4) {
       wait_copies_barrier<0>(); // K block 0 is complete in LDS
-      if (tid < kT) sS[kT + tid] = 1 < KB ? s_pending : 0.0f;
+      if (tid < T) sS[T + tid] = 1 < KB ? s_pending : 0.0f;
       s_pending = load_scale(2);
 #pragma unroll
       for (int kh = 0; kh < 2; ++kh) bf_first[kh] = *reinterpret_cast<const v4i *>(sA + alds[kh]);
@@ -484,17 +502,26 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
       // else's token rows, and nobody still reads the token stage and the scales of K block kb-1,
       // which are refilled below
       wait_copies_barrier<0>();
-      if (tid < kT) sS[((kb + 1) & 1) * kT + tid] = kb + 1 < KB ? s_pending : 0.0f;
+      if (tid < T) sS[((kb + 1) & 1) * T + tid] = kb + 1 < KB ? s_pending : 0.0f;
       s_pending = load_scale(kb + 2);
       __builtin_amdgcn_sched_barrier(0);
       kblock(NST, kb);
     }
   };
   // one K loop per number of token fragments that hold valid tokens (wave-uniform choice)
-  if (nst > 12) k_loop(std::integral_constant<int, 16>{});
-  else if (nst > 8) k_loop(std::integral_constant<int, 12>{});
-  else if (nst > 4) k_loop(std::integral_constant<int, 8>{});
-  else k_loop(std::integral_constant<int, 4>{});
+  if constexpr (NTB == 10) {
+    // three variants only (a block this size is chosen where experts fill it; a fourth one made the
+    // kernel spill): a tile in between runs the next larger one, whose surplus fragments compute on
+    // padding rows and are not stored
+    if (nst > 16) k_loop(std::integral_constant<int, 20>{});
+    else if (nst > 8) k_loop(std::integral_constant<int, 16>{});
+    else k_loop(std::integral_constant<int, 8>{});
+  } else {
+    if (nst > 12) k_loop(std::integral_constant<int, 16>{});
+    else if (nst > 8) k_loop(std::integral_constant<int, 12>{});
+    else if (nst > 4) k_loop(std::integral_constant<int, 8>{});
+    else k_loop(std::integral_constant<int, 4>{});
+  }
   wait_copies<0>(); // no copy may still be writing LDS when the epilogue reuses it or the wave ends
   if constexpr (!FUSED_ACT) {
     if (!wave_active) return;
@@ -503,7 +530,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     int8_t *stg = sWw;
     // PC: the scales of the lane's rows and of its eight tokens, fetched in one batch up front
     v4f pbs[2][2];
-    float pas[8];
+    float pas[NTB];
     if constexpr (PC) {
 #pragma unroll
       for (int h = 0; h < 2; ++h)
@@ -511,13 +538,13 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
         for (int rf = 0; rf < 2; ++rf)
           pbs[h][rf] = __builtin_bit_cast(v4f, bld16(rWs, static_cast<int>((nrow0 + h * 32 + rf * 16 + 4 * q) * 4), 0));
 #pragma unroll
-      for (int tb = 0; tb < 8; ++tb) {
+      for (int tb = 0; tb < NTB; ++tb) {
         const int64_t ft = sIds[tb * 16 + r];
         pas[tb] = bld_f32(rAs, static_cast<int>((ft < a.num_valid ? ft / a.top_k : 0) * 4), 0);
       }
     }
 #pragma unroll
-    for (int tb = 0; tb < 8; ++tb) {
+    for (int tb = 0; tb < NTB; ++tb) {
       if (2 * tb >= nst) continue;
       const int64_t ft = sIds[tb * 16 + r];
       const bool valid = ft < a.num_valid;
@@ -646,16 +673,19 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 }
 
 bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
+  if (block_size_m == kT160) // 160-token tiles: the plain int8 block form only
+    return a.w_shuffled && !fused_act && !a.w4 && !a.per_channel && a.N % 64 == 0 && a.K / kGroup <= kTMaxKB;
   if (block_size_m != 128 || !a.w_shuffled) return false;
   if (a.per_channel && (!a.w4 || fused_act)) return false; // int8 per-channel weights have gemm_pc.hip
   if (!fused_act && a.N % 64 != 0) return false;
   return a.K / kGroup <= kTMaxKB;
 }
 
-int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_blocks, hipStream_t s) {
+int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int flags, int64_t m_blocks,
+                     hipStream_t s) {
   GemmArgs a = a0;
   a.n_tiles = fused_act ? static_cast<int32_t>(a.N / 2 / kGroup) : static_cast<int32_t>((a.N + 255) / 256);
-  int64_t G = a.num_valid / (static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * kT);
+  int64_t G = a.num_valid / (static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * block_size_m);
   G = G < 2 ? 2 : (G > 16 ? 16 : G);
   const int64_t chunks = (m_blocks + G - 1) / G;
   const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
@@ -689,6 +719,22 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int flags, int64_t m_bl
       else LO_T128_LAUNCH(FA, FS, false, false);                                                                \
     }                                                                                                           \
   } while (0)
+  if (block_size_m == kT160) {
+    // chosen where an expert's tokens fill one block, so a weight byte has one reader: streaming hint
+#define LO_T160_LAUNCH(FS)                                                                                      \
+  do {                                                                                                          \
+    static unsigned long long lds_done = 0;                                                                     \
+    const int rc_lds = reserve_lds_once(                                                                        \
+        reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, FS, true, false, false, 10>), kTLds160,     \
+        &lds_done);                                                                                             \
+    if (rc_lds) return rc_lds;                                                                                  \
+    hipLaunchKernelGGL((moe_gemm_t128_kernel<false, FS, true, false, false, 10>), g, b, kTLds160, s, a, mbi, gi); \
+  } while (0)
+    if (fast) LO_T160_LAUNCH(true);
+    else LO_T160_LAUNCH(false);
+#undef LO_T160_LAUNCH
+    return check_launch("moe_gemm(t160)");
+  }
   // one token block per expert, by and large: the slots spread over the routed experts fill half a block
   const bool stream = a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * (kT / 2);
   if (a.per_channel) {

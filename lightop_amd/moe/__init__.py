@@ -17,6 +17,7 @@ _NATIVE_APIS = {
     "invoke_fused_moe_gemm1_silu_quant",
     "silu_and_mul",
     "gelu_and_mul",
+    "act_and_mul_group_quant",
     "fused_experts_workspace_bytes",
     "fused_experts_workspace_views",
     "preshuffle_moe_weight",
@@ -33,6 +34,7 @@ def __getattr__(name):
 
 
 __all__ = [
+    "act_and_mul_group_quant",
     "fused_experts_impl_int8",
     "fused_experts_impl_w4a8",
     "fused_experts_workspace_bytes",

@@ -284,6 +284,23 @@ def gelu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
                                               _lib.stream_of(x)))
 
 
+def act_and_mul_group_quant(x: torch.Tensor, activation: str = "silu") -> Tuple[torch.Tensor, torch.Tensor]:
+    """The gated activation of ``x`` [rows, 2I] and the 1x128 group quantisation of the result in one
+    launch: (q [rows, I] int8, s [rows, I/128] f32).  The pair silu_and_mul / gelu_and_mul +
+    per_token_group_quant_int8 of int8.py:811-838."""
+    _require_cuda(x)
+    assert x.is_contiguous() and x.dim() == 2 and x.shape[1] % 256 == 0
+    assert activation in ("silu", "gelu")
+    rows, I = x.shape[0], x.shape[1] // 2
+    q = torch.empty(rows, I, dtype=torch.int8, device=x.device)
+    s = torch.empty(rows, I // 128, dtype=torch.float32, device=x.device)
+    with _on_device(x):
+        _lib.check(_lib.lib().lo_act_mul_group_quant(
+            _lib.ptr(x), _act_dtype(x), _lib.LO_ACT_GELU if activation == "gelu" else _lib.LO_ACT_SILU, rows, I,
+            _lib.ptr(q), _lib.ptr(s), _lib.stream_of(x)))
+    return q, s
+
+
 @functools.lru_cache(maxsize=256)
 def fused_experts_workspace_bytes(M: int, top_k: int, H: int, I: int, num_experts: int,
                                   block_size_m: int = 0) -> int:
@@ -589,5 +606,5 @@ def ctypes_void(addr: int):
 __all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "preshuffle_moe_weight",
            "preshuffle_moe_weight_int4", "preshuffle_moe_scale_int4", "invoke_fused_moe_kernel_int8",
            "invoke_fused_moe_kernel_w4a8",
-           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "gelu_and_mul", "fused_experts_workspace_bytes",
+           "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "gelu_and_mul", "act_and_mul_group_quant", "fused_experts_workspace_bytes",
            "fused_experts_workspace_views", "moe_gemm_w8a8"]

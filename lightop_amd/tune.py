@@ -95,12 +95,15 @@ def main(argv=None):
 
     rows, table = [], {}
     print(f"{layer.name}: E={layer.E}/{layer.E_global} top{layer.top_k} H={layer.H} I={layer.I}")
-    print(f"{'tokens':>7} {'slots/expert':>12} | " + " ".join(f"bs={b:<4}" for b in BLOCK_SIZES) + " | best  table  loss")
+    # 160-token blocks exist for the block form with int8 weights where the first GEMM's output fits [S, H]
+    sizes = BLOCK_SIZES + ((160,) if (layer.weight_bits == 8 and block_shape is not None and 2 * layer.I <= layer.H)
+                           else ())
+    print(f"{'tokens':>7} {'slots/expert':>12} | " + " ".join(f"bs={b:<4}" for b in sizes) + " | best  table  loss")
     for M in (int(v) for v in args.tokens.split(",")):
         x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, M, seed=1))
         cache13 = torch.empty(M * layer.top_k * max(2 * layer.I, layer.H), dtype=torch.bfloat16, device=dev)
         ms = {}
-        for bs in BLOCK_SIZES:
+        for bs in sizes:
             ms[bs] = time_ms(lambda: run(x, tw, ids, cache13, bs), args.steps, flush)
         best = min(ms, key=ms.get)
         c1, c2 = get_w8a8moe_json(M, layer.E, 2 * layer.I, layer.H, layer.I, True, block_shape, layer.top_k,
@@ -108,7 +111,7 @@ def main(argv=None):
         pick = c1["BLOCK_SIZE_M"]
         loss = ms[pick] / ms[best] - 1.0
         rows.append((M, best, pick, loss))
-        print(f"{M:>7} {M * layer.top_k / layer.E_global:>12.1f} | " + " ".join(f"{ms[b]*1e3:7.1f}" for b in BLOCK_SIZES)
+        print(f"{M:>7} {M * layer.top_k / layer.E_global:>12.1f} | " + " ".join(f"{ms[b]*1e3:7.1f}" for b in sizes)
               + f" | {best:>4}  {pick:>5}  {loss*100:4.1f}%   (us)", flush=True)
         tile = dict(c1, BLOCK_SIZE_M=best), dict(c2, BLOCK_SIZE_M=best)
         table[str(M)] = {"config1": tile[0], "config2": tile[1]}

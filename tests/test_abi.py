@@ -63,18 +63,26 @@ def test_version_and_tile_table(lib):
     sizes = {}
     for M in (1, 16, 64, 256, 1024, 4096, 8192):
         assert lib.lo_moe_tile_query(M, 32, 256, 8, 7168, 2048, t1, t2) == 0
-        assert t1.block_size_m == t2.block_size_m and t1.block_size_m in (16, 32, 64, 128)
+        assert t1.block_size_m == t2.block_size_m and t1.block_size_m in (16, 32, 64, 128, 160)
         sizes[M] = t1.block_size_m
-    assert sizes[1] == 16 and sizes[64] == 16
-    assert all(sizes[a] <= sizes[b] for a, b in zip(list(sizes)[:-1], list(sizes)[1:]))
+    assert sizes[1] == 16 and sizes[64] == 16 and sizes[4096] == 160 and sizes[8192] == 128
     assert lib.lo_moe_tile_query(-1, 32, 256, 8, 7168, 2048, t1, t2) < 0
     assert b"moe_tile_query" in lib.lo_last_error()
     # the block-form table as the tuning harness last derived it (pre-shuffled weights): 128-token
-    # blocks from a handful of slots per expert on, 64 around 128 slots per expert on a short K
-    for M, want in ((64, 16), (128, 128), (1024, 128), (4096, 128)):
+    # blocks from a handful of slots per expert on, 160-token blocks around 128 slots per expert (where a
+    # 128-token block would spill a few tokens into a second pass over the expert's weights)
+    for M, want in ((64, 16), (128, 128), (1024, 128), (3072, 128), (3584, 160), (4096, 160), (4352, 128)):
         assert lib.lo_moe_tile_query(M, 32, 256, 8, 7168, 2048, t1, t2) == 0 and t1.block_size_m == want
-    for M, want in ((128, 16), (192, 128), (1024, 128), (1536, 64), (2048, 64), (3072, 128), (8192, 128)):
+    for M, want in ((128, 16), (192, 128), (1024, 128), (1280, 160), (1536, 160), (2048, 160), (2304, 160),
+                    (2560, 64), (3072, 128), (8192, 128)):
         assert lib.lo_moe_tile_query(M, 128, 128, 8, 2048, 768, t1, t2) == 0 and t1.block_size_m == want
+    # 160-token blocks: the same direct-to-LDS kernel for both GEMMs, the first one without its fused epilogue
+    assert lib.lo_moe_tile_query(4096, 32, 256, 8, 7168, 2048, t1, t2) == 0
+    assert t1.kernel == _lib.LO_KERNEL_T128 == t2.kernel and (t1.waves, t1.block_n) == (4, 256)
+    # not with row-major weights, and not where the first GEMM's output would not fit the caller's [S, H] buffer
+    assert lib.lo_moe_tile_query_form(_lib.LO_FORM_BLOCK, 0, 2048, 128, 128, 8, 2048, 768, t1, t2) == 0
+    assert t1.block_size_m == 64
+    assert lib.lo_moe_tile_query(2048, 128, 128, 8, 2048, 1536, t1, t2) == 0 and t1.block_size_m == 64
     # per-channel form: same small tiles, 128 tokens once an expert sees that many
     for M, want in ((1, 16), (64, 16), (1024, 64), (2048, 128), (8192, 128)):
         assert lib.lo_moe_tile_query_form(_lib.LO_FORM_CHANNEL, 0, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
