@@ -190,7 +190,8 @@ int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t rows, int6
  *   C  [num_valid, N] c_dtype, row f;  rows of blocks whose expert id is -1 are zeroed
  *   topk_w [num_valid] f32, used when mul_routed != 0
  *   sorted_ids / expert_ids / num_tokens_post_pad as produced by lo_moe_align_block_size
- *   with block_size == block_size_m (16, 32, 64 or 128); sorted_cap is the extent of sorted_ids
+ *   with block_size == block_size_m (16, 32, 64 or 128; also 160 with int8 weights in the load-time
+ *   layout, N % 64 == 0 and K <= 16384); sorted_cap is the extent of sorted_ids
  *   (any extent >= the alignment's own works, e.g. one rounded up by the caller).
  *   E: experts held by W.  num_experts: experts the routing spreads the slots over (the
  *   num_experts given to the alignment; 0 = E).  It only steers scheduling choices (tile order,
@@ -293,7 +294,9 @@ int lo_preshuffle_weight_int8(const int8_t *src, int8_t *dst, int32_t E, int64_t
  * configs/w8a8/MOE_BLOCKINT8[128,128]_*.json.
  */
 typedef struct lo_moe_tile {
-  int32_t block_size_m; /* 16, 32, 64 or 128 */
+  int32_t block_size_m; /* 16, 32, 64, 128 or 160; with 160 the first GEMM is the plain stage
+                         * (lo_moe_gemm_block_int8) followed by lo_act_mul_group_quant: the fused first
+                         * stage has no 160-token form */
   int32_t kernel;       /* LO_KERNEL_*: the kernel the stage entry points launch for this problem */
   int32_t waves;        /* wavefronts per workgroup of that kernel */
   int32_t block_n;      /* weight rows per workgroup of that kernel */
@@ -342,7 +345,11 @@ int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_local, int3
  *   shared_output [M, H] or NULL;  out [M, H]
  *   workspace: lo_fused_experts_workspace_bytes(...) bytes of device memory, 256-byte aligned
  *   block_size_m: 0 = take it from the tile table (lo_fused_experts_workspace_bytes(.., 0) is
- *   large enough for whatever the table picks and for every explicit block size)
+ *   large enough for whatever the table picks and for every explicit block size); 16, 32, 64, 128,
+ *   or 160 (int8 weights in the load-time layout, 2I <= H: 160-token blocks of the direct-to-LDS
+ *   kernel with plain epilogues and lo_act_mul_group_quant between the GEMMs - what the table picks
+ *   around 128 slots per expert, where a 128-token block would spill into a second pass over the
+ *   expert's weights; cache3 then also receives the first GEMM's output [M*top_k, 2I])
  */
 int64_t lo_fused_experts_workspace_bytes(int64_t M, int32_t top_k, int64_t H, int64_t I,
                                          int32_t num_experts, int32_t block_size_m);
