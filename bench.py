@@ -507,6 +507,8 @@ def main():
                 "frac": round(ach / peak, 4), "traffic": None if prof is None else prof["traffic_bytes"],
                 "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
                 "kernel": kname + (" (GEMM1, per-channel scales in the epilogue)" if L.quant == "channel"
+                                   else " with 160-token blocks (plain GEMM1), then act_mul_group_quant_kernel "
+                                        "(SiLU*mul + 1x128 re-quant)" if bs_used == 160
                                    else "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)"),
                 "kernel_ms": round(stages[g1_name], 4),
                 "scale_order": "fused" if args.fused_scale == 1 else "canonical",
