@@ -66,22 +66,12 @@ __global__ __launch_bounds__(256) void act_mul_tab_kernel(const uint16_t *__rest
 // The same followed by the 1x128 group quantisation of per_token_group_quant_int8 (the pair of
 // calls at int8.py:826-838 on the block-shape branch) in one pass: c1 [rows, 2I] -> q [rows, I],
 // s [rows, I/128].  16 lanes own one group, as in group_quant_body.
-// BAND (bf16 SiLU): the lookup goes through the band of the SiLU table in LDS, as in the fused epilogues,
-// instead of eight dependent global gathers per lane.
-template <int DT, bool BAND>
+template <int DT>
 __global__ __launch_bounds__(256) void act_mul_group_quant_kernel(const uint16_t *__restrict__ c1, int64_t rows,
                                                                   int64_t I, const uint16_t *__restrict__ table,
                                                                   float eps, int8_t *__restrict__ q,
                                                                   float *__restrict__ s,
                                                                   const uint8_t *__restrict__ row_mask) {
-  static_assert(!BAND || DT == LO_BF16, "the SiLU band is a bf16 table");
-  __shared__ uint16_t sSilu[BAND ? 2 * kSiluBandN : 2];
-  if constexpr (BAND) {
-    uint16_t band_regs[kSiluBandPer];
-    silu_band_load(band_regs, table, threadIdx.x);
-    silu_band_store(sSilu, band_regs, threadIdx.x);
-    __syncthreads();
-  }
   const int64_t gpr = I / kGroup, groups = rows * gpr;
   const int sub = threadIdx.x & 15;
   for (int64_t g = static_cast<int64_t>(blockIdx.x) * 16 + (threadIdx.x >> 4); g < groups;
@@ -94,8 +84,7 @@ __global__ __launch_bounds__(256) void act_mul_group_quant_kernel(const uint16_t
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if constexpr (BAND) v[i] = bf16_to_f32(silu_mul_band(sSilu, table, ga[i], up[i]));
-      else v[i] = to_f32<DT>(act_mul_tab<DT>(table, ga[i], up[i]));
+      v[i] = to_f32<DT>(act_mul_tab<DT>(table, ga[i], up[i]));
       amax = fmaxf(amax, fabsf(v[i]));
     }
 #pragma unroll
@@ -468,19 +457,13 @@ int launch_act_mul_group_quant(const void *c1, int dtype, int act, int64_t rows,
   if (rc) return rc;
   const int64_t groups = rows * (I / kGroup);
   if (groups == 0) return LO_OK;
-  // one pass of 16 groups per workgroup where the grid allows it: with a slot mask most workgroups leave
-  // after one dependent load, and a workgroup that walks several passes pays that round trip per pass
-  const int64_t wgs = (groups + 15) / 16;
-  const dim3 g(static_cast<unsigned>(wgs < 65536 ? wgs : 65536)), b(256);
+  const dim3 g(grid_for(groups, 16)), b(256);
   if (dtype == LO_F16)
-    hipLaunchKernelGGL((act_mul_group_quant_kernel<LO_F16, false>), g, b, 0, stream, static_cast<const uint16_t *>(c1),
-                       rows, I, table, 1e-10f, q, s, row_mask);
-  else if (act == LO_ACT_SILU)
-    hipLaunchKernelGGL((act_mul_group_quant_kernel<LO_BF16, true>), g, b, 0, stream, static_cast<const uint16_t *>(c1),
-                       rows, I, table, 1e-10f, q, s, row_mask);
+    hipLaunchKernelGGL(act_mul_group_quant_kernel<LO_F16>, g, b, 0, stream, static_cast<const uint16_t *>(c1), rows, I,
+                       table, 1e-10f, q, s, row_mask);
   else
-    hipLaunchKernelGGL((act_mul_group_quant_kernel<LO_BF16, false>), g, b, 0, stream, static_cast<const uint16_t *>(c1),
-                       rows, I, table, 1e-10f, q, s, row_mask);
+    hipLaunchKernelGGL(act_mul_group_quant_kernel<LO_BF16>, g, b, 0, stream, static_cast<const uint16_t *>(c1), rows, I,
+                       table, 1e-10f, q, s, row_mask);
   return check_launch("act_mul_group_quant");
 }
 
