@@ -37,8 +37,12 @@ namespace lo {
 // (one 16-byte load per lane holds both k-steps of a 128-wide K block; two vector
 // instructions per 8 elements turn them into int8 values 16 times too large, which the
 // row scales take out again as a factor 1/16) and every weight row has its own scale per K
-// block, stored K-group-major, Ws [E, K/128, N], so that the four rows a lane accumulates
-// are one 16-byte load.
+// block, stored K-group-major, Ws [E, K/128, N].  The workgroup copies the scales of its rows for
+// every K block into LDS before the K loop (6 % of its weight bytes, requested together with
+// the first weight blocks), already divided by 16; a lane then reads the scales of its four rows
+// as one 16-byte LDS read per fragment and K block (fetched inside the loop, one 4-byte load per
+// lane, fragment and K block and the other three rows by DPP from the quad, they were as many
+// memory instructions as the weights themselves).
 //
 // PC (per-channel W8A8, reference csrc/moe_gemm/w8a8/moe_w8a8.cu:156-166, :445-470): one scale
 // per token row, As [a_rows], and one per weight row, Ws [E, N]; the int32 sum runs over the
@@ -90,9 +94,13 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   const brsrc rA = make_rsrc(a.A, static_cast<uint32_t>(a.a_rows * K));
   const brsrc rAs = make_rsrc(a.As, static_cast<uint32_t>(a.a_rows * (PC ? 1 : KB) * 4));
 
+  constexpr bool kScalesInLds = W4 && !PC;
+  constexpr int ROWS = FUSED_ACT ? 256 : 16 * NWAVES * RPW; // weight rows of the workgroup
+  bool wave_dead = false; // no rows left for this wave (it still helps with the scale copy)
   if constexpr (!FUSED_ACT) {
     const int64_t n0 = static_cast<int64_t>(nt) * (16 * NWAVES * RPW) + wave * (16 * RPW);
-    if (n0 >= N) return;
+    wave_dead = n0 >= N;
+    if (wave_dead && (!kScalesInLds || e < 0)) return;
     if (e < 0) { // expert not held by this rank: the rows are defined to be zero
       if (a.skip_nonlocal && !e_oob) return;
 #pragma unroll
@@ -125,7 +133,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
                        : make_rsrc(a.Ws + static_cast<int64_t>(e) * N * KB, static_cast<uint32_t>(W4 ? N * KB * 4 : 0));
   int woff[NW];
   const float *wsrow[NW];
-  int wsoff[NW]; // W4: byte offset of the lane's first scale row
+  int wsoff[NW]; // W4 with PC: byte offset of the lane's first scale row; W4: the same inside the LDS copy
   const int wkstride = W4 ? shuf_kb_stride(static_cast<int>(N / 16)) / 2 : shuf_kb_stride(static_cast<int>(N / 16));
 #pragma unroll
   for (int g = 0; g < NW; ++g) {
@@ -137,11 +145,11 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       woff[g] = static_cast<int>((nrow[g] + r) * K) + c * 16;
     const int64_t nclamp = nrow[g] < N ? nrow[g] : 0; // fragments past N: loads return 0, nothing is stored
     wsrow[g] = a.Ws + (static_cast<int64_t>(e) * NB + nclamp / kGroup) * KB;
-    // accumulator rows of this lane: 4c .. 4c+3.  Inside the K loop (W4) a lane fetches only the
-    // scale of row 4c + (lane & 3) - a 4-byte load costs the texture path a quarter of a 16-byte
-    // one, and these kernels issue as many scale loads as weight loads - and gets the other
-    // three from its quad neighbours when the scales are used.
-    wsoff[g] = static_cast<int>((nclamp + 4 * c + ((W4 && !PC) ? (lane & 3) : 0)) * 4);
+    // accumulator rows of this lane: 4c .. 4c+3
+    if constexpr (kScalesInLds)
+      wsoff[g] = ((FUSED_ACT ? g * 128 + wave * 16 : wave * (16 * RPW) + g * 16) + 4 * c) * 4;
+    else
+      wsoff[g] = static_cast<int>((nclamp + 4 * c) * 4);
   }
 
   v4f acc[NW][TM];
@@ -161,7 +169,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   v4i wbuf[PD][NW][W4 ? 1 : 2];
   v4i abuf[PD][TM][2];
   float asbuf[PD][TM];
-  float bsbuf[PD][NW][1]; // W4: the scale of row 4c + (lane & 3); the quad holds the lane's four
+  float bsbuf[PD][NW][1]; // (int4 weights: the row scales come from LDS)
   // The loop body is kept free of branches: a slot past the end of K re-reads the last
   // K block and gets a token scale of zero, so it adds exactly 0 to every accumulator.
   // (Branches around the loads make the compiler fall back to waiting for all of them.)
@@ -185,19 +193,67 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
     if constexpr (PC) return; // no scales inside the K loop
 #pragma unroll
     for (int g = 0; g < NW; ++g) {
-      if constexpr (W4) { // scales are stored [E][K/128][N]
-        bsbuf[slot][g][0] = bld_f32(rWs, wsoff[g], kc * static_cast<int>(N) * 4);
-      } else {
-        bsbuf[slot][g][0] = wsrow[g][kc];
-      }
+      if constexpr (!W4) bsbuf[slot][g][0] = wsrow[g][kc];
     }
 #pragma unroll
     for (int j = 0; j < TM; ++j) asbuf[slot][j] = bld_f32(rAs, asoff[j], kc * 4);
   };
+  extern __shared__ __attribute__((aligned(16))) float sRowScale[]; // [K block][ROWS], already / 16
+  // scales are stored [E][K/128][N]: per K block the workgroup's rows are one run of ROWS floats
+  // (plain) or two of 128 (gate rows, up rows).  Four pieces of four rows per thread and pass, so
+  // that a pass is one memory round trip; rows past N and pieces past the last K block read zeros
+  // (an offset outside the buffer) and belong to fragments that are never stored.
+  constexpr int kPieces = ROWS / 4, kThreads = NWAVES * 64;
+  const int sc_total = KB * kPieces;
+  auto scale_load = [&](int base, v4i (&raw)[4]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int p = base + u * kThreads + static_cast<int>(threadIdx.x);
+      const int kb = p / kPieces, w4 = p - kb * kPieces;
+      int64_t grow;
+      if constexpr (FUSED_ACT) grow = (w4 < 32 ? 0 : I - kGroup) + static_cast<int64_t>(nt) * kGroup + 4 * w4;
+      else grow = static_cast<int64_t>(nt) * ROWS + 4 * w4;
+      const bool in = p < sc_total && grow < N;
+      // with the weights' cache policy: next to streaming weight loads, scale loads with the default policy
+      // cost 15 % of the launch (measured at 32 tokens of a 4096 x 1536 layer: 162 -> 138 us)
+      raw[u] = bld16<WAUX>(rWs, in ? static_cast<int>((static_cast<int64_t>(kb) * N + grow) * 4) : 0x7ffffff0, 0);
+    }
+  };
+  auto scale_store = [&](int base, const v4i (&raw)[4]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int p = base + u * kThreads + static_cast<int>(threadIdx.x);
+      if (p < sc_total) {
+        v4f sc = __builtin_bit_cast(v4f, raw[u]);
+        // every product carries the factor 16 of the unpacked nibbles: 1/16 goes into the row scales (a
+        // power of two: (f32(d) * a_s) * (b_s / 16) is bit for bit (f32(d / 16) * a_s) * b_s unless b_s
+        // lies below 2^-122 or the product above 2^124)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sc[i] = sc[i] * 0.0625f;
+        *reinterpret_cast<v4f *>(sRowScale + static_cast<int64_t>(p) * 4) = sc;
+      }
+    }
+  };
+  // the first pass of scale loads goes out ahead of the weight ring and lands first (loads return in
+  // order), so that it is in LDS while the first weight blocks are still on their way
+  v4i sc_raw[4];
+  if constexpr (kScalesInLds) {
+    scale_load(0, sc_raw);
+    __builtin_amdgcn_sched_barrier(0);
+  }
 #pragma unroll
   for (int p = 0; p < PD; ++p) {
     issue(p, p);
     __builtin_amdgcn_sched_barrier(0); // keep the slots in issue order: the waits count on it
+  }
+  if constexpr (kScalesInLds) {
+    scale_store(0, sc_raw);
+    for (int base = 4 * kThreads; base < sc_total; base += 4 * kThreads) { // more than 32 K blocks
+      scale_load(base, sc_raw);
+      scale_store(base, sc_raw);
+    }
+    __syncthreads();
+    if (wave_dead) return;
   }
 
   for (int kb0 = 0; kb0 < KB; kb0 += PD) {
@@ -242,17 +298,11 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       if constexpr (!PC) {
 #pragma unroll
         for (int g = 0; g < NW; ++g) {
-          if constexpr (W4) { // quad broadcasts: lane i of the quad holds row 4c + i
-            const int raw = __builtin_bit_cast(int, bsbuf[p][g][0]);
-            bs[g][0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0x00, 0xf, 0xf, false));
-            bs[g][NS > 1 ? 1 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0x55, 0xf, 0xf, false));
-            bs[g][NS > 2 ? 2 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0xaa, 0xf, 0xf, false));
-            bs[g][NS > 3 ? 3 : 0] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, raw, 0xff, 0xf, 0xf, false));
-            // every product carries the factor 16 of the unpacked nibbles: 1/16 goes into the row scales (a
-            // power of two: (f32(d) * a_s) * (b_s / 16) is bit for bit (f32(d / 16) * a_s) * b_s unless b_s
-            // lies below 2^-122 or the product above 2^124)
+          if constexpr (W4) { // a dead slot reads the last K block's scales (finite: its token scale is zero)
+            const int kc = kb < KB ? kb : KB - 1;
+            const v4f sc = *reinterpret_cast<const v4f *>(reinterpret_cast<const char *>(sRowScale) + kc * (ROWS * 4) + wsoff[g]);
 #pragma unroll
-            for (int i = 0; i < NS; ++i) bs[g][i] = bs[g][i] * 0.0625f;
+            for (int i = 0; i < NS; ++i) bs[g][i] = sc[i];
           } else {
             bs[g][0] = bsbuf[p][g][0];
           }
@@ -383,7 +433,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
 }
 
 template <int TM, bool FUSED_ACT, bool FAST_SCALE>
-static void launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
+static int launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
   constexpr int NWAVES = FUSED_ACT ? 8 : LO_WS_PLAIN_WAVES;
   // A plain-GEMM wave takes RPW consecutive 16-row fragments so that it streams a few
   // hundred KB even when K is short; the ring depth shrinks as the fragments multiply.
@@ -401,24 +451,37 @@ static void launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
         hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, true, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
       else
         hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, false, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
-      return;
+      return LO_OK;
     }
   }
-  if (a.w4)
-    hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, true, NWAVES, PD, RPW, true>), grid, block, 0, s, a);
-  else if (a.w_shuffled)
+  if (a.w4) {
+    // the row scales of the workgroup's rows, every K block, sit in LDS
+    constexpr int ROWS = FUSED_ACT ? 256 : 16 * NWAVES * RPW;
+    const int64_t lds = a.K / kGroup * ROWS * 4;
+    LO_REQUIRE(lds <= 128 * 1024, LO_ENOTSUP, "moe_gemm(int4): K = %lld is more than this kernel's %d K groups",
+               static_cast<long long>(a.K), 128 * 1024 / (ROWS * 4));
+    const auto kern = &moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, true, NWAVES, PD, RPW, true>;
+    if (lds > 48 * 1024) {
+      static unsigned long long lds_done = 0; // per instantiation: one bit per device
+      const int rc_lds = reserve_lds_once(reinterpret_cast<const void *>(kern), 128 * 1024, &lds_done);
+      if (rc_lds) return rc_lds;
+    }
+    hipLaunchKernelGGL(kern, grid, block, static_cast<size_t>(lds), s, a);
+  } else if (a.w_shuffled)
     hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, true, NWAVES, PD, RPW>), grid, block, 0, s, a);
   else
     hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, false, NWAVES, PD, RPW>), grid, block, 0, s, a);
+  return LO_OK;
 }
 
 template <bool FUSED_ACT>
 static int dispatch_ws(const GemmArgs &a, int bs, int flags, int64_t m_blocks, hipStream_t s) {
   const bool fast = fused_scale_order(flags) && !a.per_channel;
+  int rc = LO_OK;
 #define LO_WS_CASE(TMV)                                               \
   case 16 * TMV:                                                      \
-    if (fast) launch_ws<TMV, FUSED_ACT, true>(a, m_blocks, s);        \
-    else launch_ws<TMV, FUSED_ACT, false>(a, m_blocks, s);            \
+    rc = fast ? launch_ws<TMV, FUSED_ACT, true>(a, m_blocks, s)       \
+              : launch_ws<TMV, FUSED_ACT, false>(a, m_blocks, s);     \
     break;
   switch (bs) {
     LO_WS_CASE(1)
@@ -430,6 +493,7 @@ static int dispatch_ws(const GemmArgs &a, int bs, int flags, int64_t m_blocks, h
     return LO_EINVAL;
   }
 #undef LO_WS_CASE
+  if (rc) return rc;
   return check_launch(FUSED_ACT ? "moe_gemm1_silu_quant" : "moe_gemm");
 }
 
