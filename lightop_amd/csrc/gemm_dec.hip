@@ -177,7 +177,7 @@ __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
         for (int g = 0; g < 2; ++g) {
           if constexpr (W4) {
             wbuf[p][g][0] = bld16<kCacheStream>(rW, woff[g], (kb0 + p) * wkstride);
-            wsc[p][g] = __builtin_bit_cast(v4f, bld16(rWs, wsoff[g], (kb0 + p) * N * 4));
+            wsc[p][g] = __builtin_bit_cast(v4f, bld16<kCacheStream>(rWs, wsoff[g], (kb0 + p) * N * 4)); // the weights' policy: mixed policies cost time
           } else {
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
     auto issue = [&](int p, int kb) __attribute__((always_inline)) {
       if constexpr (W4) {
         wbuf[p][0] = bld16<kCacheStream>(rW, woff, kb * wkstride);
-        wsc[p] = __builtin_bit_cast(v4f, bld16(rWs, wsoff, kb * H * 4));
+        wsc[p] = __builtin_bit_cast(v4f, bld16<kCacheStream>(rWs, wsoff, kb * H * 4));
       } else {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) wbuf[p][ks] = bld16<kCacheStream>(rW, woff, kb * wkstride + ks * 1024);

@@ -11,6 +11,10 @@
 // double buffered) against all 32*TB tokens (gathered through sorted_token_ids into a
 // double-buffered, row-padded LDS tile), i.e. 2*TB accumulators of v_mfma_i32_32x32x32_i8.
 // Two workgroups share a compute unit (three with 64-token tiles).
+//
+// STREAM: an expert's weights are read by one token block, by and large, and are loaded with the
+// streaming cache policy; with several token blocks per expert the blocks share them through L2
+// and the default policy is the faster one.
 #include <type_traits>
 
 #include "gemm.h"
@@ -21,8 +25,9 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kPcRow = 144; // LDS row pitch in bytes: 128 + 16 keeps ds_read_b128 conflict-free
 
-template <bool SHUF, int TB>
+template <bool SHUF, int TB, bool STREAM>
 __device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks, int group_m) {
+  constexpr int kWAux = STREAM ? kCacheStream : kCacheDefault;
   constexpr int kTileM = 32 * TB;       // tokens per workgroup
   constexpr int kThrPerTok = 256 / kTileM; // threads that gather one token row
   constexpr int kPieces = 8 / kThrPerTok;  // 16-byte pieces per thread and K block
@@ -121,8 +126,8 @@ __device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks)
-        wreg[b][rb][ks] = SHUF ? bld16(rW, woff[rb], kc * wkstride + ks * 512)
-                               : bld16(rW, woff[rb], kc * kGroup + ks * 16);
+        wreg[b][rb][ks] = SHUF ? bld16<kWAux>(rW, woff[rb], kc * wkstride + ks * 512)
+                               : bld16<kWAux>(rW, woff[rb], kc * kGroup + ks * 16);
   };
   auto compute = [&](auto BUF) {
     constexpr int b = decltype(BUF)::value;
@@ -198,15 +203,15 @@ __device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks
 
 // 128 tokens: 246 registers, two waves per SIMD.  64 tokens: 162 registers, so three workgroups
 // fit a compute unit and hide each other's barrier and memory waits better than two.
-template <bool SHUF>
+template <bool SHUF, bool STREAM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_pc_kernel_128(const GemmArgs a, int m_blocks, int group_m) {
-  moe_gemm_pc_body<SHUF, 4>(a, m_blocks, group_m);
+  moe_gemm_pc_body<SHUF, 4, STREAM>(a, m_blocks, group_m);
 }
-template <bool SHUF>
+template <bool SHUF, bool STREAM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void moe_gemm_pc_kernel_64(const GemmArgs a, int m_blocks, int group_m) {
-  moe_gemm_pc_body<SHUF, 2>(a, m_blocks, group_m);
+  moe_gemm_pc_body<SHUF, 2, STREAM>(a, m_blocks, group_m);
 }
 
 bool gemm_pc_supports(const GemmArgs &a, int block_size_m) {
@@ -224,13 +229,22 @@ int launch_gemm_pc(const GemmArgs &a0, int block_size_m, int64_t m_blocks, hipSt
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm_w8a8: grid too large");
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
-  if (block_size_m == 128) {
-    if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_pc_kernel_128<true>), g, b, 0, s, a, mbi, gi);
-    else hipLaunchKernelGGL((moe_gemm_pc_kernel_128<false>), g, b, 0, s, a, mbi, gi);
-  } else {
-    if (a.w_shuffled) hipLaunchKernelGGL((moe_gemm_pc_kernel_64<true>), g, b, 0, s, a, mbi, gi);
-    else hipLaunchKernelGGL((moe_gemm_pc_kernel_64<false>), g, b, 0, s, a, mbi, gi);
-  }
+  // one token block per expert, by and large: the slots spread over the routed experts fill half a block
+  const bool stream =
+      a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * (block_size_m / 2);
+#define LO_PC_LAUNCH(KERN)                                                                    \
+  do {                                                                                        \
+    if (a.w_shuffled) {                                                                       \
+      if (stream) hipLaunchKernelGGL((KERN<true, true>), g, b, 0, s, a, mbi, gi);             \
+      else hipLaunchKernelGGL((KERN<true, false>), g, b, 0, s, a, mbi, gi);                   \
+    } else {                                                                                  \
+      if (stream) hipLaunchKernelGGL((KERN<false, true>), g, b, 0, s, a, mbi, gi);            \
+      else hipLaunchKernelGGL((KERN<false, false>), g, b, 0, s, a, mbi, gi);                  \
+    }                                                                                         \
+  } while (0)
+  if (block_size_m == 128) LO_PC_LAUNCH(moe_gemm_pc_kernel_128);
+  else LO_PC_LAUNCH(moe_gemm_pc_kernel_64);
+#undef LO_PC_LAUNCH
   return check_launch("moe_gemm_w8a8(tile)");
 }
 

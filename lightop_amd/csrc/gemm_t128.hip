@@ -166,7 +166,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
     for (int p = 0; p < 4; ++p)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[p >> 1][p & 1], 0, 0, kWAux);
-    if constexpr (!PC) __builtin_amdgcn_raw_ptr_buffer_load_lds(rWs, sWw + 4096, 4, wsvoff, 0, 0, 0);
+    if constexpr (!PC) __builtin_amdgcn_raw_ptr_buffer_load_lds(rWs, sWw + 4096, 4, wsvoff, 0, 0, kWAux);
   } else {
 #pragma unroll
     for (int p = 0; p < 8; ++p)
@@ -229,7 +229,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
                                                    __builtin_amdgcn_readfirstlane(kc * wkstride), 0, kWAux);
         else if (p == 4 && !PC)
           __builtin_amdgcn_raw_ptr_buffer_load_lds(rWs, sWw + 4096, 4, wsvoff,
-                                                   __builtin_amdgcn_readfirstlane(kc) * static_cast<int>(N) * 4, 0, 0);
+                                                   __builtin_amdgcn_readfirstlane(kc) * static_cast<int>(N) * 4, 0, kWAux);
       } else {
         const int h = p >> 2, rf = (p >> 1) & 1, kh = p & 1;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rW, sWw + p * 1024, 16, wvoff[h][rf],

@@ -14,7 +14,9 @@
 // tokens those reads outweigh the (half-size) weights four to one.  Here a workgroup of four
 // waves gathers the 64 token rows of the current K block once into a double-buffered,
 // row-padded LDS tile (with their group scales) and every wave multiplies its 64 weight rows
-// (four 16-row fragments, global -> registers, double buffered together with their row scales)
+// (four 16-row fragments, global -> registers, double buffered; the row scales of the
+// workgroup's 256 rows for every K block are copied to LDS before the K loop, already divided by
+// 16, and read from there: fetched per K block they were as many 16-byte loads as the weights)
 // against all of them: 16 accumulators of 16x16 per wave.  With FUSED_ACT the four fragments
 // are 32 gate rows and the matching 32 up rows, and the epilogue is the SiLU(gate)*up +
 // 1x128 re-quantisation of the block-INT8 path.
@@ -26,14 +28,21 @@ namespace lo {
 
 constexpr int kW4Row = 144; // LDS row pitch in bytes: 128 + 16 keeps ds_read_b128 conflict-free
 
-template <bool FUSED_ACT, bool FAST_SCALE>
+//
+// STREAM: an expert's weights and row scales are read by one token block, by and large: they are
+// loaded with the streaming cache policy (first GEMM of a 4096 x 1536 layer with 16 or 32 slots per
+// expert: 227 -> 180 us).  With several token blocks per expert the blocks share the weights through
+// L2 and the default policy is the faster one.
+template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   constexpr int kTileM = 64;
+  constexpr int kWAux = STREAM ? kCacheStream : kCacheDefault;
   __shared__ __attribute__((aligned(16))) int8_t sA[2][kTileM * kW4Row];
   __shared__ float sS[2][kTileM];
   __shared__ float sRed[4][kTileM];
   __shared__ uint16_t sSilu[FUSED_ACT ? 2 * kSiluBandN : 2];
+  extern __shared__ __attribute__((aligned(16))) float sRowScale[]; // [K block][256 rows], already / 16
 
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
@@ -104,8 +113,42 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   for (int rf = 0; rf < 4; ++rf) {
     const int64_t nr = nrow[rf] < N ? nrow[rf] : 0; // fragments past N: computed on row 0, never stored
     woff[rf] = static_cast<int>(nr / 16) * (shuf_nb_stride(KB) / 2) + lane * 16; // 1 KB blocks, lane order
-    wsoff[rf] = static_cast<int>((nr + 4 * q) * 4);                              // the lane's rows 4q .. 4q+3
+    // the lane's rows 4q .. 4q+3 inside the LDS copy of the row scales
+    wsoff[rf] = ((FUSED_ACT ? (rf >= 2 ? 128 : 0) + wr * 32 + (rf & 1) * 16 : wr * 64 + rf * 16) + 4 * q) * 4;
   }
+  // scales are stored [E][K/128][N]: per K block the workgroup's rows are one run of 256 floats (plain)
+  // or two of 128 (gate rows, up rows), copied in pieces of four rows; rows past N
+  // read zeros (an offset outside the buffer) and belong to fragments that are never stored.  Eight
+  // pieces per thread and pass: 32 K blocks are one memory round trip.
+  auto copy_row_scales = [&]() {
+    const int sc_total = KB * 64;
+    for (int base = 0; base < sc_total; base += 8 * 256) {
+      v4i raw[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int p = base + u * 256 + tid;
+        const int kb = p >> 6, w4 = p & 63;
+        int64_t grow;
+        if constexpr (FUSED_ACT) grow = (w4 < 32 ? 0 : I - kGroup) + static_cast<int64_t>(nt) * kGroup + 4 * w4;
+        else grow = static_cast<int64_t>(nt) * 256 + 4 * w4;
+        const bool in = p < sc_total && grow < N;
+        raw[u] = bld16<kWAux>(rWs, in ? static_cast<int>((static_cast<int64_t>(kb) * N + grow) * 4) : 0x7ffffff0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int p = base + u * 256 + tid;
+        if (p < sc_total) {
+          v4f sc = __builtin_bit_cast(v4f, raw[u]);
+          // every product carries the factor 16 of the unpacked nibbles: 1/16 goes into the row scale (a
+          // power of two: (f32(d) * a_s) * (b_s / 16) is bit for bit (f32(d / 16) * a_s) * b_s unless b_s
+          // lies below 2^-122 or the product above 2^124)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sc[i] = sc[i] * 0.0625f;
+          *reinterpret_cast<v4f *>(sRowScale + static_cast<int64_t>(p) * 4) = sc;
+        }
+      }
+    }
+  };
 
   using B0 = std::integral_constant<int, 0>;
   using B1 = std::integral_constant<int, 1>;
@@ -116,7 +159,6 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     for (int tf = 0; tf < 4; ++tf) acc[rf][tf] = v4f{0.f, 0.f, 0.f, 0.f};
 
   v4i wreg[2][4]; // [buffer][row fragment]: both k-steps of a K block, packed
-  v4f bsreg[2][4]; // the row scales that go with them
   v4i areg[2][2];  // [set][16-byte piece]: token bytes in flight for two K blocks
   float sreg[2] = {0.0f, 0.0f};
 
@@ -142,18 +184,9 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     constexpr int b = decltype(BUF)::value;
     const int kc = kb < KB ? kb : KB - 1;
 #pragma unroll
-    for (int rf = 0; rf < 4; ++rf) wreg[b][rf] = bld16(rW, woff[rf], kc * wkstride);
-#pragma unroll
-    for (int rf = 0; rf < 4; ++rf)
-      bsreg[b][rf] = __builtin_bit_cast(v4f, bld16(rWs, wsoff[rf], kc * static_cast<int>(N) * 4));
+    for (int rf = 0; rf < 4; ++rf) wreg[b][rf] = bld16<kWAux>(rW, woff[rf], kc * wkstride);
   };
-  auto fold = [&](const v4i (&d)[4], const v4f &bs, const float (&as)[4], v4f (&dst)[4]) {
-    // every product carries the factor 16 of the unpacked nibbles: 1/16 goes into the row scale (a
-    // power of two: (f32(d) * a_s) * (b_s / 16) is bit for bit (f32(d / 16) * a_s) * b_s unless b_s
-    // lies below 2^-122 or the product above 2^124)
-    v4f bs16;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) bs16[i] = bs[i] * 0.0625f;
+  auto fold = [&](const v4i (&d)[4], const v4f &bs16, const float (&as)[4], v4f (&dst)[4]) {
 #pragma unroll
     for (int tf = 0; tf < 4; ++tf)
 #pragma unroll
@@ -171,11 +204,16 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(dst[tf][i])); // keep the fold here
   };
-  auto compute = [&](auto BUF) {
+  auto compute = [&](auto BUF, int kb) {
     constexpr int b = decltype(BUF)::value;
     const int8_t *tile = sA[b];
     v4i bf[4][2];
     float as[4];
+    // a step past the end of K reads the last K block's scales (finite: its token scales are zero)
+    const char *const srow = reinterpret_cast<const char *>(sRowScale) + (kb < KB ? kb : KB - 1) * 1024;
+    v4f bsv[4];
+#pragma unroll
+    for (int rf = 0; rf < 4; ++rf) bsv[rf] = *reinterpret_cast<const v4f *>(srow + wsoff[rf]);
 #pragma unroll
     for (int tf = 0; tf < 4; ++tf) {
       const int8_t *src = tile + (tf * 16 + r) * kW4Row + q * 16;
@@ -206,18 +244,20 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
         for (int ks = 0; ks < 2; ++ks)
           d[tf] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop[ks], bf[tf][ks], d[tf], 0, 0, 0);
       }
-      if (rf > 0) fold(dprev, bsreg[b][rf - 1], as, acc[rf - 1]);
+      if (rf > 0) fold(dprev, bsv[rf - 1], as, acc[rf - 1]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int tf = 0; tf < 4; ++tf) dprev[tf] = d[tf];
     }
-    fold(dprev, bsreg[b][3], as, acc[3]);
+    fold(dprev, bsv[3], as, acc[3]);
     __builtin_amdgcn_sched_barrier(0);
   };
 
   load_act(B0{}, 0);
   load_act(B1{}, 1);
   load_w(B0{}, 0);
+  __builtin_amdgcn_sched_barrier(0); // the first K block's requests go out ahead of the scales'
+  copy_row_scales();
   store_act(B0{}, true);
   if constexpr (FUSED_ACT) silu_band_store(sSilu, band_regs, tid);
   __syncthreads();
@@ -225,13 +265,13 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     load_act(B0{}, kb + 2);            // needed in two iterations
     load_w(B1{}, kb + 1);              // needed in the next iteration
     __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMAs
-    compute(B0{});
+    compute(B0{}, kb);
     store_act(B1{}, kb + 1 < KB);      // requested one iteration ago
     __syncthreads();
     load_act(B1{}, kb + 3);
     load_w(B0{}, kb + 2);
     __builtin_amdgcn_sched_barrier(0);
-    compute(B1{});
+    compute(B1{}, kb + 1);
     store_act(B0{}, kb + 2 < KB);
     __syncthreads();
   }
@@ -341,13 +381,36 @@ int launch_gemm_w4_tile(const GemmArgs &a0, bool fused_act, int flags, int64_t m
   const bool fast = fused_scale_order(flags);
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
+  // the row scales of the workgroup's 256 rows, every K block, sit in LDS next to 28 KB of static arrays
+  const int64_t lds = a.K / kGroup * 1024;
+  LO_REQUIRE(lds <= 128 * 1024, LO_ENOTSUP, "moe_gemm(w4 tile): K = %lld is more than 128 K groups",
+             static_cast<long long>(a.K));
+  // one token block per expert, by and large: the slots spread over the routed experts fill half a block
+  const bool stream = a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * 32;
+#define LO_W4_TILE_LAUNCH(FA, FS, ST)                                                                          \
+  do {                                                                                                         \
+    if (lds > 32 * 1024) {                                                                                     \
+      static unsigned long long lds_done = 0; /* per instantiation: one bit per device */                      \
+      const int rc_lds = reserve_lds_once(reinterpret_cast<const void *>(&moe_gemm_w4_tile_kernel<FA, FS, ST>), \
+                                          128 * 1024, &lds_done);                                              \
+      if (rc_lds) return rc_lds;                                                                               \
+    }                                                                                                          \
+    hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<FA, FS, ST>), g, b, static_cast<size_t>(lds), s, a, mbi, gi);  \
+  } while (0)
+#define LO_W4_TILE_PICK(FA, FS)              \
+  do {                                       \
+    if (stream) LO_W4_TILE_LAUNCH(FA, FS, true); \
+    else LO_W4_TILE_LAUNCH(FA, FS, false);   \
+  } while (0)
   if (fused_act) {
-    if (fast) hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<true, true>), g, b, 0, s, a, mbi, gi);
-    else hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<true, false>), g, b, 0, s, a, mbi, gi);
+    if (fast) LO_W4_TILE_PICK(true, true);
+    else LO_W4_TILE_PICK(true, false);
   } else {
-    if (fast) hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<false, true>), g, b, 0, s, a, mbi, gi);
-    else hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<false, false>), g, b, 0, s, a, mbi, gi);
+    if (fast) LO_W4_TILE_PICK(false, true);
+    else LO_W4_TILE_PICK(false, false);
   }
+#undef LO_W4_TILE_PICK
+#undef LO_W4_TILE_LAUNCH
   return check_launch(fused_act ? "moe_gemm1_silu_quant(w4 tile)" : "moe_gemm(w4 tile)");
 }
 
