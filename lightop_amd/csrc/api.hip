@@ -135,11 +135,20 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
     if (H < 4096 && per_expert >= 96.0 && per_expert < 192.0) return 64;
     return 128;
   }
+  // Per-channel form: no scale arithmetic in the K loop, so the accumulators of 128 tokens fit
+  // and the larger tile halves the weight bytes requested from L2 per multiply-add; with about one
+  // token block per expert the LDS-tiled kernels stream the weights with the non-temporal hint and
+  // take over from the weight-streaming kernel at half a dozen slots per expert.  Measured (us, whole
+  // path, 16 / 32 / 64 / 128): Qwen3-30B-A3B-shaped layer at 64 tokens 122 / 122 / 121 / 126, at 128:
+  // 130 / 132 / 127 / 130, at 256: 188 / 147 / 135 / 138, at 512: 296 / 223 / 152 / 153, at 1024:
+  // 489 / 361 / 223 / 173; DeepSeek-V3 share of 32 experts at 128 tokens 252 / 251 / 253 / 253, at
+  // 256: 268 / 268 / 270 / 262, at 512: 365 / 296 / 297 / 285, at 1024: 627 / 476 / 336 / 319.
+  if (form == LO_FORM_CHANNEL) {
+    if (per_expert <= 6.0) return 16;
+    return (H >= 4096 || per_expert >= 48.0) ? 128 : 64;
+  }
   if (per_expert <= 12.0) return 16;
   if (per_expert <= 24.0) return 32;
-  // Per-channel form: no scale arithmetic in the K loop, so the accumulators of 128 tokens fit
-  // and the larger tile halves the weight bytes requested from L2 per multiply-add.
-  if (form == LO_FORM_CHANNEL && per_expert >= 64.0) return 128;
   // Row-major block-form weights: 64-token LDS tiles, two workgroups per CU; their 128-token
   // kernel is one phase-locked workgroup per CU and measured slower on every layer shape tried.
   return 64;

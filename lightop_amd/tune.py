@@ -69,11 +69,16 @@ def main(argv=None):
     w1, w2, w1s, w2s = wl.make_weights(layer, seed=0, device=dev, gen_device="cuda")
     if layer.weight_bits == 4:
         w1, w2 = preshuffle_moe_weight_int4(w1), preshuffle_moe_weight_int4(w2)
-        w1s, w2s = preshuffle_moe_scale_int4(w1s), preshuffle_moe_scale_int4(w2s)
+        if layer.quant != "channel":  # K-group scales go K-group-major; per-channel scales stay [E, N, 1]
+            w1s, w2s = preshuffle_moe_scale_int4(w1s), preshuffle_moe_scale_int4(w2s)
     else:
         w1, w2 = preshuffle_moe_weight(w1), preshuffle_moe_weight(w2)
-    # which form of the path the layer asks for: block-INT8, per-channel INT8 or W4A8 with K-group scales
-    block_shape = [1, 128] if layer.weight_bits == 4 else (None if layer.quant == "channel" else [128, 128])
+    # which form of the path the layer asks for: block-INT8, per-channel INT8, W4A8 with K-group scales, or
+    # W4A8 with per-token and per-channel scales
+    if layer.quant == "channel":
+        block_shape = None
+    else:
+        block_shape = [1, 128] if layer.weight_bits == 4 else [128, 128]
 
     def run(x, tw, ids, cache13, bs):
         if layer.weight_bits == 4:
@@ -107,7 +112,7 @@ def main(argv=None):
             ms[bs] = time_ms(lambda: run(x, tw, ids, cache13, bs), args.steps, flush)
         best = min(ms, key=ms.get)
         c1, c2 = get_w8a8moe_json(M, layer.E, 2 * layer.I, layer.H, layer.I, True, block_shape, layer.top_k,
-                                  layer.E_global)
+                                  layer.E_global, int4=layer.weight_bits == 4)
         pick = c1["BLOCK_SIZE_M"]
         loss = ms[pick] / ms[best] - 1.0
         rows.append((M, best, pick, loss))
@@ -122,7 +127,10 @@ def main(argv=None):
         props = torch.cuda.get_device_properties(dev)
         devname = f"{props.gcnArchName.split(':')[0]}_{props.multi_processor_count}cu"
         # file names as the reference's reader builds them (w8a8_get_cache_json.py:133-149)
-        kind = "W4A8INT8[1,128]" if layer.weight_bits == 4 else ("W8A8INT8" if block_shape is None else "BLOCKINT8[128,128]")
+        if layer.weight_bits == 4:
+            kind = "W4A8INT8" if block_shape is None else "W4A8INT8[1,128]"
+        else:
+            kind = "W8A8INT8" if block_shape is None else "BLOCKINT8[128,128]"
         name = (f"MOE_{kind}_E={layer.E}_N1={2 * layer.I}_N2={layer.H}_K={layer.I}_"
                 f"TOPK{layer.top_k}_{devname}.json")
         with open(os.path.join(args.out, name), "w") as f:

@@ -83,9 +83,13 @@ def test_version_and_tile_table(lib):
     assert lib.lo_moe_tile_query_form(_lib.LO_FORM_BLOCK, 0, 2048, 128, 128, 8, 2048, 768, t1, t2) == 0
     assert t1.block_size_m == 64
     assert lib.lo_moe_tile_query(2048, 128, 128, 8, 2048, 1536, t1, t2) == 0 and t1.block_size_m == 64
-    # per-channel form: same small tiles, 128 tokens once an expert sees that many
-    for M, want in ((1, 16), (64, 16), (1024, 64), (2048, 128), (8192, 128)):
+    # per-channel form: streaming tiles up to half a dozen slots per expert, then the LDS-tiled kernels
+    # (128 tokens on a long K; on a short K 64 tokens until an expert sees 48)
+    for M, want in ((1, 16), (64, 16), (192, 16), (256, 128), (1024, 128), (8192, 128)):
         assert lib.lo_moe_tile_query_form(_lib.LO_FORM_CHANNEL, 0, M, 32, 256, 8, 7168, 2048, t1, t2) == 0
+        assert t1.block_size_m == want and t2.block_size_m == want
+    for M, want in ((64, 16), (128, 64), (512, 64), (1024, 128)):
+        assert lib.lo_moe_tile_query_form(_lib.LO_FORM_CHANNEL, 0, M, 128, 128, 8, 2048, 768, t1, t2) == 0
         assert t1.block_size_m == want and t2.block_size_m == want
     # W4A8: streaming for a handful of slots per expert, the 64-token LDS tile from 8 on, 128 tokens from 48 on
     for M, want in ((1, 16), (128, 16), (256, 16), (512, 64), (1024, 64), (2048, 128), (8192, 128)):
