@@ -7,7 +7,7 @@ For every token count the whole path is timed with each token-block size the ker
 offer (16, 32: weight-streaming; 64, 128: LDS-tiled), caches flushed between calls.  The
 report shows the best size per token count next to what the compiled-in table
 (``pick_block_m`` in csrc/api.hip, ``lo_moe_tile_query``) picks and how much slower that pick
-is, so the table's thresholds (slots per expert <= 12 -> 16, <= 24 -> 32, else 64) can be
+is, so the table's thresholds (slots per expert at which the next larger block takes over) can be
 re-derived after a kernel change.  With ``--out`` the winners are also written in the JSON
 layout the reference keeps per device (reference: test/moe_w8a8/tune_int8.py writes, and
 python/lightop/_lmslim_native/vllm_compat/w8a8_get_cache_json.py:12-174 reads,
