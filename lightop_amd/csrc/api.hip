@@ -130,10 +130,20 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   if (form == LO_FORM_BLOCK && preshuffled && allow160) {
     if (H >= 4096 ? (per_expert >= 104.0 && per_expert < 134.0) : (per_expert >= 80.0 && per_expert < 152.0)) return 160;
   }
+  // With about one token block per expert the 64-token kernel with register-fed weights
+  // (gemm_tile.hip) streams them with the non-temporal hint as well, and its shorter start-up and
+  // epilogue put it ahead on a short K.  Measured (us, whole path, 16 / 64 / 128): Qwen3-30B-A3B layer
+  // at 64 tokens 117 / 117 / 130, at 128: 126 / 119 / 133, at 256: 184 / 126 / 140, at 512: 289 / 135 /
+  // 157, at 768: - / 162 / 176, at 1024: - / 218 / 194; DeepSeek-V3 share at 512 tokens 356 / 251 / 251,
+  // at 768: 508 / 264 / 264, at 1024: 638 / 276 / 283, at 1536: 847 / 292 / 303, at 2048: - / 428 / 333.
   if (form == LO_FORM_BLOCK && preshuffled) {
-    if (per_expert < (H >= 4096 ? 4.0 : 12.0)) return 16;
-    if (H < 4096 && per_expert >= 96.0 && per_expert < 192.0) return 64;
-    return 128;
+    if (H < 4096) {
+      if (per_expert < 6.0) return 16;
+      if (per_expert <= 48.0 || (per_expert >= 96.0 && per_expert < 192.0)) return 64;
+      return 128;
+    }
+    if (per_expert < 4.0) return 16;
+    return (per_expert >= 28.0 && per_expert <= 48.0) ? 64 : 128; // equal within 0.2 % from 16 to 24
   }
   // Per-channel form: no scale arithmetic in the K loop, so the accumulators of 128 tokens fit
   // and the larger tile halves the weight bytes requested from L2 per multiply-add; with about one

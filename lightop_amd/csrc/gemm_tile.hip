@@ -31,9 +31,17 @@ constexpr int kTileRow = 144;    // LDS row pitch in bytes: 128 + 16 keeps ds_re
 // WT = number of 64-token halves per workgroup: 2 -> 128-token tile, 8 waves, one
 // workgroup per CU; 1 -> 64-token tile, 4 waves, two workgroups per CU that are not
 // synchronised with each other, so one computes while the other waits at its barrier.
-template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int WT>
+//
+// STREAM (64-token tiles of pre-shuffled weights): an expert's weights are read by one token block,
+// by and large, and are loaded with the streaming cache policy (first GEMM of the Qwen3-30B-A3B
+// layer at 512 tokens 132 -> 74 us).  With several token blocks per expert the blocks share the
+// weights through L2 and the default policy is the faster one; with row-major weights, where a
+// 128-byte line serves several k-steps of a lane, the hint costs 50 %.
+template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int WT, bool STREAM = false>
 __global__ __launch_bounds__(256 * WT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
+  static_assert(!STREAM || (SHUF && WT == 1), "streaming policy: 64-token tiles of pre-shuffled weights");
+  constexpr int kWAux = STREAM ? kCacheStream : kCacheDefault;
   constexpr int kTileM = 64 * WT; // tokens per workgroup
   __shared__ __attribute__((aligned(16))) int8_t sA[2][kTileM * kTileRow];
   __shared__ float sS[2][kTileM];
@@ -168,7 +176,7 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks)
-        wreg[b][rb][ks] = SHUF ? bld16(rW, woff[rb], kc * wkstride + ks * 512)
+        wreg[b][rb][ks] = SHUF ? bld16<kWAux>(rW, woff[rb], kc * wkstride + ks * 512)
                                : bld16(rW, woff[rb], kc * kGroup + ks * 16);
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) bsc[b][rb] = wsrow[rb][kc];
@@ -353,9 +361,16 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int block_size_m, int f
     if (wt == 2) hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, SH, 2>), g, b, 0, s, a, mbi, static_cast<int>(G)); \
     else hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, SH, 1>), g, b, 0, s, a, mbi, static_cast<int>(G));         \
   } while (0)
+  // one token block per expert, by and large (measured up to 48 slots per expert on average: first GEMM
+  // of the Qwen3-30B-A3B layer at 768 tokens 135 -> 88 us; at 64 the second GEMM loses more than
+  // the first one gains)
+  const bool stream = a.w_shuffled && wt == 1 &&
+                      a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * 48;
 #define LO_TILE_LAUNCH(FA, FS)                         \
   do {                                                 \
-    if (a.w_shuffled) LO_TILE_LAUNCH2(FA, FS, true);   \
+    if (stream)                                        \
+      hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, true, 1, true>), g, b, 0, s, a, mbi, static_cast<int>(G)); \
+    else if (a.w_shuffled) LO_TILE_LAUNCH2(FA, FS, true);   \
     else LO_TILE_LAUNCH2(FA, FS, false);               \
   } while (0)
   if (fused_act) {

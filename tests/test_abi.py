@@ -68,14 +68,18 @@ def test_version_and_tile_table(lib):
     assert sizes[1] == 16 and sizes[64] == 16 and sizes[4096] == 160 and sizes[8192] == 128
     assert lib.lo_moe_tile_query(-1, 32, 256, 8, 7168, 2048, t1, t2) < 0
     assert b"moe_tile_query" in lib.lo_last_error()
-    # the block-form table as the tuning harness last derived it (pre-shuffled weights): 128-token
-    # blocks from a handful of slots per expert on, 160-token blocks around 128 slots per expert (where a
-    # 128-token block would spill a few tokens into a second pass over the expert's weights)
-    for M, want in ((64, 16), (128, 128), (1024, 128), (3072, 128), (3584, 160), (4096, 160), (4352, 128)):
+    # the block-form table as the tuning harness last derived it (pre-shuffled weights): LDS-tiled
+    # kernels from a handful of slots per expert on (64-token tiles while there is about one token block
+    # per expert, on a short K up to 48 slots per expert), 160-token blocks around 128 slots per expert
+    # (where a 128-token block would spill a few tokens into a second pass over the expert's weights)
+    for M, want in ((64, 16), (128, 128), (256, 128), (512, 128), (1024, 64), (1280, 64), (1536, 64), (2048, 128), (3072, 128),
+                    (3584, 160), (4096, 160), (4352, 128)):
         assert lib.lo_moe_tile_query(M, 32, 256, 8, 7168, 2048, t1, t2) == 0 and t1.block_size_m == want
-    for M, want in ((128, 16), (192, 128), (1024, 128), (1280, 160), (1536, 160), (2048, 160), (2304, 160),
-                    (2560, 64), (3072, 128), (8192, 128)):
+    for M, want in ((64, 16), (128, 64), (512, 64), (768, 64), (1024, 128), (1280, 160), (1536, 160), (2048, 160),
+                    (2304, 160), (2560, 64), (3072, 128), (8192, 128)):
         assert lib.lo_moe_tile_query(M, 128, 128, 8, 2048, 768, t1, t2) == 0 and t1.block_size_m == want
+    assert lib.lo_moe_tile_query(512, 128, 128, 8, 2048, 768, t1, t2) == 0
+    assert t1.kernel == _lib.LO_KERNEL_TILE == t2.kernel
     # 160-token blocks: the same direct-to-LDS kernel for both GEMMs, the first one without its fused epilogue
     assert lib.lo_moe_tile_query(4096, 32, 256, 8, 7168, 2048, t1, t2) == 0
     assert t1.kernel == _lib.LO_KERNEL_T128 == t2.kernel and (t1.waves, t1.block_n) == (4, 256)
@@ -132,7 +136,8 @@ def test_tile_query_names_the_kernel_that_is_launched(lib):
     assert q(_lib.LO_FORM_BLOCK, 0, 8192, *qwen) == 0
     assert (t1.block_size_m, t1.kernel, t1.waves) == (64, _lib.LO_KERNEL_TILE, 4)
     assert q(_lib.LO_FORM_BLOCK, 0, 256, *qwen) == 0 and t1.block_size_m == 32 and t1.kernel == _lib.LO_KERNEL_WS
-    assert q(_lib.LO_FORM_BLOCK, pre, 256, *qwen) == 0 and t1.block_size_m == 128
+    assert q(_lib.LO_FORM_BLOCK, pre, 256, *qwen) == 0 and (t1.block_size_m, t1.kernel) == (64, _lib.LO_KERNEL_TILE)
+    assert q(_lib.LO_FORM_BLOCK, pre, 256, *dsv3) == 0 and (t1.block_size_m, t1.kernel) == (128, _lib.LO_KERNEL_T128)
     # forced streaming is honoured
     assert q(_lib.LO_FORM_BLOCK, pre | _lib.LO_GEMM_FORCE_STREAMING, 8192, *qwen) == 0 and t1.kernel == _lib.LO_KERNEL_WS
     # per-channel and int4 forms
