@@ -165,6 +165,8 @@ class Point:
         out = torch.empty(self.M, L.H, dtype=torch.bfloat16, device=self.dev)
         if L.quant == "channel":
             return self.stage_times_channel(steps, warmup, flush, bs), bs
+        a2q_buf = torch.empty(S, L.I, dtype=torch.int8, device=self.dev)
+        a2s_buf = torch.empty(S, L.I // 128, dtype=torch.float32, device=self.dev)
         names = ["quant", "align", "gemm1_silu_quant", "gemm2", "moe_sum"]
         acc = {n: [] for n in names}
         # With an expert_map the whole path leaves the rows of other ranks' slots untouched and
@@ -189,8 +191,8 @@ class Point:
             if bs == 160:  # 160-token blocks: plain first GEMM, activation and quantisation in a launch of their own
                 c1 = self.cache13[: S * 2 * L.I].view(S, 2 * L.I)
                 moe.invoke_fused_moe_kernel_int8(a1q, self.w1, c1, a1s, self.w1s, tw, s, e, p, False, L.top_k, cfg,
-                                                 fused_scale=fused_scale, flags=wflag, global_num_experts=L.E_global)
-                a2q, a2s = moe.act_and_mul_group_quant(c1)
+                                                 fused_scale=fused_scale, flags=g2flag, global_num_experts=L.E_global)
+                a2q, a2s = moe.act_and_mul_group_quant(c1, row_mask=mask, out=(a2q_buf, a2s_buf))
             else:
                 a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
                                                                  L.top_k, S, cfg, fused_scale=fused_scale,

@@ -244,9 +244,11 @@ int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t I, void *ac
  * q [rows, I] int8, s [rows, I/128] f32.  Replaces the pair of calls between the two GEMMs where the
  * first GEMM's epilogue does not do it: silu_and_mul + per_token_group_quant_int8 (int8.py:811-823) or
  * gelu_and_mul + per_token_group_quant_int8 (int8.py:826-838).  activation: LO_ACT_SILU / LO_ACT_GELU.
+ * row_mask (may be NULL): one byte per row as lo_moe_align_block_size_mask writes it; rows whose byte
+ * is 0 (slots of experts on other ranks) are neither read nor written.
  */
 int lo_act_mul_group_quant(const void *c1, int dtype, int activation, int64_t rows, int64_t I, int8_t *q,
-                           float *s, lo_stream_t stream);
+                           float *s, const uint8_t *row_mask, lo_stream_t stream);
 /* The 65536 values T(act(g)), indexed by the bit pattern of g, that the kernels look up for activation
  * LO_ACT_SILU / LO_ACT_GELU and element type LO_BF16 / LO_F16, copied to table_out (device memory,
  * 128 KB).  For tests; no counterpart in the reference. */

@@ -61,7 +61,7 @@ SIGNATURES = {
     "lo_silu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "lo_gelu_and_mul": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "lo_activation_table": (c_int, [c_int, c_int, c_void_p, c_void_p]),
-    "lo_act_mul_group_quant": (c_int, [c_void_p, c_int, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),
+    "lo_act_mul_group_quant": (c_int, [c_void_p, c_int, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lo_moe_sum": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int32, c_int64, c_float,
                            c_void_p, c_void_p]),
     "lo_topk_softmax": (c_int, [c_void_p, c_int, c_int64, c_int32, c_int32, c_int, c_void_p, c_void_p, c_int,

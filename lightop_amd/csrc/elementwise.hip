@@ -590,7 +590,7 @@ extern "C" int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
 }
 
 extern "C" int lo_act_mul_group_quant(const void *c1, int dtype, int activation, int64_t rows, int64_t I, int8_t *q,
-                                      float *s, lo_stream_t stream) {
+                                      float *s, const uint8_t *row_mask, lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(c1 && q && s, LO_EINVAL, "act_mul_group_quant: null pointer");
   LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "act_mul_group_quant: bf16 or fp16");
@@ -600,7 +600,7 @@ extern "C" int lo_act_mul_group_quant(const void *c1, int dtype, int activation,
              "act_mul_group_quant: the output width (%lld) must be a multiple of 128", (long long)I);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0, LO_EINVAL,
              "act_mul_group_quant: input must be 16-byte and q 8-byte aligned");
-  return launch_act_mul_group_quant(c1, dtype, activation, rows, I, q, s, nullptr, static_cast<hipStream_t>(stream));
+  return launch_act_mul_group_quant(c1, dtype, activation, rows, I, q, s, row_mask, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int lo_activation_table(int activation, int dtype, void *table_out, lo_stream_t stream) {

@@ -284,20 +284,31 @@ def gelu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
                                               _lib.stream_of(x)))
 
 
-def act_and_mul_group_quant(x: torch.Tensor, activation: str = "silu") -> Tuple[torch.Tensor, torch.Tensor]:
+def act_and_mul_group_quant(x: torch.Tensor, activation: str = "silu", row_mask: Optional[torch.Tensor] = None,
+                            out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+                            ) -> Tuple[torch.Tensor, torch.Tensor]:
     """The gated activation of ``x`` [rows, 2I] and the 1x128 group quantisation of the result in one
     launch: (q [rows, I] int8, s [rows, I/128] f32).  The pair silu_and_mul / gelu_and_mul +
-    per_token_group_quant_int8 of int8.py:811-838."""
+    per_token_group_quant_int8 of int8.py:811-838.  ``row_mask`` (bool or uint8 [rows], as the alignment
+    writes its slot mask): rows whose entry is 0 are neither read nor written.  ``out``: (q, s) to write
+    into."""
     _require_cuda(x)
     assert x.is_contiguous() and x.dim() == 2 and x.shape[1] % 256 == 0
     assert activation in ("silu", "gelu")
     rows, I = x.shape[0], x.shape[1] // 2
-    q = torch.empty(rows, I, dtype=torch.int8, device=x.device)
-    s = torch.empty(rows, I // 128, dtype=torch.float32, device=x.device)
+    if out is None:
+        q = torch.empty(rows, I, dtype=torch.int8, device=x.device)
+        s = torch.empty(rows, I // 128, dtype=torch.float32, device=x.device)
+    else:
+        q, s = out
+        assert q.is_contiguous() and s.is_contiguous() and q.dtype == torch.int8 and s.dtype == torch.float32
+        assert q.shape == (rows, I) and s.shape == (rows, I // 128)
+    if row_mask is not None:
+        assert row_mask.is_contiguous() and row_mask.numel() == rows and row_mask.element_size() == 1
     with _on_device(x):
         _lib.check(_lib.lib().lo_act_mul_group_quant(
             _lib.ptr(x), _act_dtype(x), _lib.LO_ACT_GELU if activation == "gelu" else _lib.LO_ACT_SILU, rows, I,
-            _lib.ptr(q), _lib.ptr(s), _lib.stream_of(x)))
+            _lib.ptr(q), _lib.ptr(s), None if row_mask is None else _lib.ptr(row_mask), _lib.stream_of(x)))
     return q, s
 
 

@@ -140,6 +140,27 @@ def test_act_and_mul_group_quant_bit_exact(dev, oracle, rows, I, activation):
     assert torch.equal(s.cpu(), rs) and torch.equal(q.cpu(), rq)
 
 
+def test_act_and_mul_group_quant_row_mask_and_out(dev, oracle):
+    """Rows whose mask byte is 0 are neither read (NaN there must not matter) nor written."""
+    from lightop_amd.moe import act_and_mul_group_quant
+
+    say("act_and_mul_group_quant with a row mask")
+    g = torch.Generator().manual_seed(5)
+    rows, I = 77, 384
+    c1 = (torch.randn(rows, 2 * I, generator=g) * 3).to(torch.bfloat16)
+    mask = torch.rand(rows, generator=g) > 0.4
+    mask[0], mask[1] = True, False
+    c1[~mask] = float("nan")
+    rq, rs = oracle.per_token_group_quant_int8(oracle.silu_and_mul(torch.where(mask[:, None], c1, torch.zeros_like(c1))))
+    q = torch.full((rows, I), 77, dtype=torch.int8, device=dev)
+    s = torch.full((rows, I // 128), -5.0, dtype=torch.float32, device=dev)
+    q2, s2 = act_and_mul_group_quant(c1.to(dev), "silu", row_mask=mask.to(dev), out=(q, s))
+    torch.cuda.synchronize()
+    assert q2.data_ptr() == q.data_ptr() and s2.data_ptr() == s.data_ptr()
+    assert torch.equal(q.cpu()[mask], rq[mask]) and torch.equal(s.cpu()[mask], rs[mask])
+    assert (q.cpu()[~mask] == 77).all() and (s.cpu()[~mask] == -5.0).all()
+
+
 def _run(layer, wd, x, tw, ids, emap, dev, bs, **kw):
     from lightop_amd.moe import fused_experts_impl_int8
 
