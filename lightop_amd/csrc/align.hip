@@ -310,36 +310,17 @@ __global__ __launch_bounds__(256) void moe_align_count_kernel(
                             slots_per_token, sorted, sorted_cap, static_cast<int>(gridDim.x));
 }
 
-// The first nchunks workgroups count, the others quantise the activations: the quantisation does
-// not depend on the alignment, and on its own launch it would only wait for the counting to end.
 template <typename IdT>
-__global__ __launch_bounds__(256) void quant_align_count_kernel(
-    const uint16_t *__restrict__ x, int64_t groups, float eps, int8_t *__restrict__ q, float *__restrict__ qs,
-    const IdT *__restrict__ ids, int64_t numel, int E, const int32_t *__restrict__ expert_map,
-    int64_t chunk_slots, int32_t *__restrict__ cnt, uint8_t *__restrict__ slot_mask, int32_t *__restrict__ sorted,
-    int64_t sorted_cap, int nchunks) {
-  if (static_cast<int>(blockIdx.x) < nchunks) {
-    moe_align_count_body<IdT>(ids, numel, E, expert_map, 0, chunk_slots, cnt, slot_mask, nullptr, 1, sorted,
-                              sorted_cap, nchunks);
-  } else {
-    group_quant_body<LO_BF16>(x, groups, eps, q, qs,
-                              static_cast<int64_t>(blockIdx.x - nchunks) * 16 + (threadIdx.x >> 4),
-                              static_cast<int64_t>(gridDim.x - nchunks) * 16, threadIdx.x & 15);
-  }
-}
-
-template <typename IdT>
-__global__ __launch_bounds__(256) void moe_align_scatter_kernel(
+__device__ __forceinline__ void moe_align_scatter_body(
     const IdT *__restrict__ ids, int64_t numel, int E, int bs, const int32_t *__restrict__ expert_map,
     int ignore_invalid, int64_t chunk_slots, const int32_t *__restrict__ cnt,
     int32_t *__restrict__ sorted, int64_t sorted_cap, int32_t *__restrict__ expert_ids,
     int64_t expert_ids_cap, int32_t *__restrict__ ntpp, int key_bits,
-    const int32_t *__restrict__ num_local_tokens, int slots_per_token) {
+    const int32_t *__restrict__ num_local_tokens, int slots_per_token, int chunk, int nchunks) {
   extern __shared__ int32_t lds[];
   numel = local_slots(numel, num_local_tokens, slots_per_token);
   constexpr int nw = 4;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int chunk = blockIdx.x, nchunks = gridDim.x;
   int32_t *offs = lds;              // [E + 1] padded exclusive prefix
   int32_t *total = lds + (E + 1);   // [E]
   int32_t *cbase = total + E;       // [E] slots of expert e in earlier chunks
@@ -478,6 +459,39 @@ __global__ __launch_bounds__(256) void moe_align_scatter_kernel(
   }
 }
 
+template <typename IdT>
+__global__ __launch_bounds__(256) void moe_align_scatter_kernel(
+    const IdT *__restrict__ ids, int64_t numel, int E, int bs, const int32_t *__restrict__ expert_map,
+    int ignore_invalid, int64_t chunk_slots, const int32_t *__restrict__ cnt,
+    int32_t *__restrict__ sorted, int64_t sorted_cap, int32_t *__restrict__ expert_ids,
+    int64_t expert_ids_cap, int32_t *__restrict__ ntpp, int key_bits,
+    const int32_t *__restrict__ num_local_tokens, int slots_per_token) {
+  moe_align_scatter_body<IdT>(ids, numel, E, bs, expert_map, ignore_invalid, chunk_slots, cnt, sorted, sorted_cap,
+                              expert_ids, expert_ids_cap, ntpp, key_bits, num_local_tokens, slots_per_token,
+                              static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x));
+}
+
+// The first nchunks workgroups scatter, the others quantise the activations: the quantisation does
+// not depend on the alignment, and the scatter (a chain of dependent round trips on a few compute
+// units) costs nothing beside it.  The counting, which the scatter waits for, is a launch of its own
+// before this one.
+template <typename IdT>
+__global__ __launch_bounds__(256) void quant_align_scatter_kernel(
+    const uint16_t *__restrict__ x, int64_t groups, float eps, int8_t *__restrict__ q, float *__restrict__ qs,
+    const IdT *__restrict__ ids, int64_t numel, int E, int bs, const int32_t *__restrict__ expert_map,
+    int64_t chunk_slots, const int32_t *__restrict__ cnt, int32_t *__restrict__ sorted, int64_t sorted_cap,
+    int32_t *__restrict__ expert_ids, int64_t expert_ids_cap, int32_t *__restrict__ ntpp, int key_bits,
+    int nchunks) {
+  if (static_cast<int>(blockIdx.x) < nchunks) {
+    moe_align_scatter_body<IdT>(ids, numel, E, bs, expert_map, 0, chunk_slots, cnt, sorted, sorted_cap, expert_ids,
+                                expert_ids_cap, ntpp, key_bits, nullptr, 1, static_cast<int>(blockIdx.x), nchunks);
+  } else {
+    group_quant_body<LO_BF16>(x, groups, eps, q, qs,
+                              static_cast<int64_t>(blockIdx.x - nchunks) * 16 + (threadIdx.x >> 4),
+                              static_cast<int64_t>(gridDim.x - nchunks) * 16, threadIdx.x & 15);
+  }
+}
+
 // chunks for the multi-workgroup path: about 1024 slots each, at most 256 chunks
 static void single_wg_shape(int64_t numel, int64_t sorted_cap, int32_t num_experts, int *nw, size_t *lds_bytes) {
   // waves per workgroup: as many as the per-wave LDS counters allow (<= 60 KB)
@@ -519,7 +533,7 @@ int launch_quant_align(const void *x, int64_t M, int64_t H, float eps, int8_t *q
   int key_bits = 1;
   while ((1 << key_bits) < num_experts) ++key_bits;
   const int64_t groups = M * (H / kGroup);
-  if (want > 0) { // many slots: counting + quantisation, then the scatter
+  if (want > 0) { // many slots: counting, then the scatter beside the quantisation
     int nchunks;
     int64_t cs;
     align_chunks(numel, &nchunks, &cs);
@@ -528,23 +542,23 @@ int launch_quant_align(const void *x, int64_t M, int64_t H, float eps, int8_t *q
     const size_t lds2 = (static_cast<size_t>(4 + 3) * num_experts + 1) * 4;
     int64_t qb = (groups + 15) / 16;
     if (qb > 8192) qb = 8192;
-    const dim3 grid1(static_cast<unsigned>(nchunks + qb));
+    const dim3 grid2(static_cast<unsigned>(nchunks + qb));
     if (ids_dtype == LO_I32) {
-      hipLaunchKernelGGL(quant_align_count_kernel<int32_t>, grid1, dim3(256), lds1, stream,
+      hipLaunchKernelGGL(moe_align_count_kernel<int32_t>, dim3(nchunks), dim3(256), lds1, stream,
+                         static_cast<const int32_t *>(topk_ids), numel, num_experts, expert_map, 0, cs, cnt, slot_mask,
+                         nullptr, 1, sorted_ids, sorted_cap);
+      hipLaunchKernelGGL(quant_align_scatter_kernel<int32_t>, grid2, dim3(256), lds2, stream,
                          static_cast<const uint16_t *>(x), groups, eps, q, qs, static_cast<const int32_t *>(topk_ids),
-                         numel, num_experts, expert_map, cs, cnt, slot_mask, sorted_ids, sorted_cap, nchunks);
-      hipLaunchKernelGGL(moe_align_scatter_kernel<int32_t>, dim3(nchunks), dim3(256), lds2, stream,
-                         static_cast<const int32_t *>(topk_ids), numel, num_experts, block_size, expert_map, 0, cs,
-                         cnt, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, num_tokens_post_pad, key_bits,
-                         nullptr, 1);
+                         numel, num_experts, block_size, expert_map, cs, cnt, sorted_ids, sorted_cap, expert_ids,
+                         expert_ids_cap, num_tokens_post_pad, key_bits, nchunks);
     } else {
-      hipLaunchKernelGGL(quant_align_count_kernel<int64_t>, grid1, dim3(256), lds1, stream,
+      hipLaunchKernelGGL(moe_align_count_kernel<int64_t>, dim3(nchunks), dim3(256), lds1, stream,
+                         static_cast<const int64_t *>(topk_ids), numel, num_experts, expert_map, 0, cs, cnt, slot_mask,
+                         nullptr, 1, sorted_ids, sorted_cap);
+      hipLaunchKernelGGL(quant_align_scatter_kernel<int64_t>, grid2, dim3(256), lds2, stream,
                          static_cast<const uint16_t *>(x), groups, eps, q, qs, static_cast<const int64_t *>(topk_ids),
-                         numel, num_experts, expert_map, cs, cnt, slot_mask, sorted_ids, sorted_cap, nchunks);
-      hipLaunchKernelGGL(moe_align_scatter_kernel<int64_t>, dim3(nchunks), dim3(256), lds2, stream,
-                         static_cast<const int64_t *>(topk_ids), numel, num_experts, block_size, expert_map, 0, cs,
-                         cnt, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, num_tokens_post_pad, key_bits,
-                         nullptr, 1);
+                         numel, num_experts, block_size, expert_map, cs, cnt, sorted_ids, sorted_cap, expert_ids,
+                         expert_ids_cap, num_tokens_post_pad, key_bits, nchunks);
     }
     return check_launch("quant_align(multi)");
   }
