@@ -100,7 +100,14 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   // than a dozen tokens (measured on the Qwen3-235B-A22B-shaped layer, whole path in us, 16 / 32 /
   // 64 / 128: at 128 tokens 247 / 254 / 401 / 267, at 256: 365 / 294 / 433 / 285, at 1024: 953 / 727 /
   // 842 / 382, at 2048: 1610 / 1224 / 1455 / 596).
-  if (form == LO_FORM_CHANNEL && int4_channel) return per_expert <= 12.0 ? 16 : 128;
+  // Around 128 slots per expert the 160-token form of that kernel holds an expert's tokens in one block
+  // (a remainder block is a second pass over the expert's weights): same layer, 128 / 160: at 1024
+  // tokens 345 / 358, at 1280: 394 / 386, at 1792: 488 / 422, at 2048: 541 / 444, at 2304: 629 / 517, at
+  // 2560: 658 / 620, at 3072: 686 / 754.
+  if (form == LO_FORM_CHANNEL && int4_channel) {
+    if (per_expert <= 12.0) return 16;
+    return (allow160 && per_expert >= 76.0 && per_expert < 170.0) ? 160 : 128;
+  }
   // W4A8: the streaming kernel re-reads the token rows per wave, which outweighs the half-size
   // weights early; the LDS-tiled kernel (64 tokens) wins above about 8 slots per expert.
   // From 48 slots per expert on the 128-token kernel takes over (measured, 64 / 128: 475 / 394 us at
@@ -179,10 +186,11 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
              "moe_tile_query_form: bad problem size");
   if (form == LO_FORM_W4) flags |= LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED;
   const bool pre = (flags & LO_GEMM_W_PRESHUFFLED) != 0;
-  const int32_t bm = pick_block_m(M, num_experts, top_k, H, form, pre,
-                                  form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4),
-                                  form == LO_FORM_BLOCK && pre && blocks_of_160_fit(H, I) &&
-                                      !(flags & LO_FUSED_ACT_GELU));
+  const bool int4_channel = form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4);
+  const int32_t bm = pick_block_m(M, num_experts, top_k, H, form, pre, int4_channel,
+                                  int4_channel ? (H / kGroup <= 128 && I / kGroup <= 128)
+                                               : (form == LO_FORM_BLOCK && pre && blocks_of_160_fit(H, I) &&
+                                                  !(flags & LO_FUSED_ACT_GELU)));
   // the argument blocks the stage entry points would build for this problem
   GemmArgs a{};
   a.num_valid = M * top_k;
@@ -372,9 +380,13 @@ extern "C" int lo_fused_experts_channel_int8(
              "fused_experts(channel): workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
   if (block_size_m == 0)
-    block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_CHANNEL, true, (flags & LO_GEMM_W4) != 0);
-  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128,
-             LO_EINVAL, "fused_experts(channel): block_size_m %d is not one of 16, 32, 64, 128", block_size_m);
+    block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_CHANNEL, true, (flags & LO_GEMM_W4) != 0,
+                                H / kGroup <= 128 && I / kGroup <= 128);
+  // 160: the 160-token form of the direct-to-LDS kernel, for int4 weights
+  const bool bs160 = block_size_m == 160 && (flags & LO_GEMM_W4) && H / kGroup <= 128 && I / kGroup <= 128;
+  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 || bs160,
+             LO_EINVAL, "fused_experts(channel): block_size_m %d is not one of 16, 32, 64, 128 (160: int4 weights)",
+             block_size_m);
   // the block layout is roomy enough: its scale segments hold one float per 128 values
   const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
   LO_REQUIRE(workspace_bytes >= L.total, LO_ENOSPC,

@@ -186,8 +186,8 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   int rc = validate_common("moe_gemm_w8a8", A, As, W, Ws, sorted_ids, expert_ids, num_tokens_post_pad, K,
                            top_k, E, a_rows);
   if (rc) return rc;
-  LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL, "moe_gemm_w8a8: block_size_m %d is not one of 16, 32, 64, 128",
-             block_size_m);
+  LO_REQUIRE(valid_block_m(block_size_m) || (block_size_m == 160 && (flags & LO_GEMM_W4)), LO_EINVAL,
+             "moe_gemm_w8a8: block_size_m %d is not one of 16, 32, 64, 128 (160: int4 weights only)", block_size_m);
   LO_REQUIRE(C, LO_EINVAL, "moe_gemm_w8a8: null output");
   LO_REQUIRE(c_dtype == LO_BF16 || c_dtype == LO_F16, LO_ENOTSUP, "moe_gemm_w8a8: the output is bf16 or fp16");
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm_w8a8: N (%lld) must be a multiple of 16", (long long)N);
@@ -213,6 +213,8 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   a.out_f16 = c_dtype == LO_F16 ? 1 : 0;
   a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);
+  LO_REQUIRE(block_size_m != 160 || gemm_t128_supports(a, false, 160), LO_ENOTSUP,
+             "moe_gemm_w8a8: 160-token blocks need N a multiple of 64 and K <= %d", kGroup * 128);
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 30), LO_EINVAL, "moe_gemm_w8a8: grid too large");
   if (mblocks == 0) return LO_OK;

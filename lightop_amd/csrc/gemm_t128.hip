@@ -43,7 +43,8 @@ constexpr int kTMaxKB = 128;                  // K blocks whose weight-block sca
 constexpr int kTBs = 2 * kTMaxKB * 4;         // [fragment][K block] weight-block scales of the tile
 constexpr int kTIds = kT * 4;                  // the tile's sorted ids, for the epilogues
 constexpr int kTLds = kTW + kTA + kTS + kTRed + kTBs + kTIds + 2 * kSiluBandN * 2;
-// NTB = 10: 160 tokens per workgroup (plain epilogue only: no amax exchange, no SiLU band), for layers
+// NTB = 10: 160 tokens per workgroup (plain epilogue only: no amax exchange, no SiLU band; int8 block
+// form, or int4 weights with per-channel scales, whose int32 accumulators need no fold registers), for layers
 // whose experts see a few tokens more than 128: a remainder block is a second pass over the expert's
 // weights, and at that size the weights are what the stage streams.
 constexpr int kT160 = 160;
@@ -71,7 +72,8 @@ template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM, bool W4, bool PC = false
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   static_assert(!PC || (W4 && !FUSED_ACT && !FAST_SCALE), "per-channel scales: plain int4 GEMM only");
-  static_assert(NTB == 8 || (NTB == 10 && !FUSED_ACT && !W4 && !PC), "160-token tiles: plain int8 block form only");
+  static_assert(NTB == 8 || (NTB == 10 && !FUSED_ACT && W4 == PC),
+                "160-token tiles: plain GEMM, int8 block form or int4 with per-channel scales");
   constexpr int T = 16 * NTB;        // tokens per workgroup
   constexpr int AST = T * kGroup;    // token rows of one K block
   constexpr int APW = NTB / 2;       // 1 KB pieces (eight token rows) of a token stage that a wave copies
@@ -673,8 +675,9 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 }
 
 bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
-  if (block_size_m == kT160) // 160-token tiles: the plain int8 block form only
-    return a.w_shuffled && !fused_act && !a.w4 && !a.per_channel && a.N % 64 == 0 && a.K / kGroup <= kTMaxKB;
+  if (block_size_m == kT160) // 160-token tiles: plain GEMM, int8 block form or int4 with per-channel scales
+    return a.w_shuffled && !fused_act && (a.w4 != 0) == (a.per_channel != 0) && a.N % 64 == 0 &&
+           a.K / kGroup <= kTMaxKB;
   if (block_size_m != 128 || !a.w_shuffled) return false;
   if (a.per_channel && (!a.w4 || fused_act)) return false; // int8 per-channel weights have gemm_pc.hip
   if (!fused_act && a.N % 64 != 0) return false;
@@ -730,7 +733,13 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int f
     if (rc_lds) return rc_lds;                                                                                  \
     hipLaunchKernelGGL((moe_gemm_t128_kernel<false, FS, true, false, false, 10>), g, b, kTLds160, s, a, mbi, gi); \
   } while (0)
-    if (fast) LO_T160_LAUNCH(true);
+    if (a.per_channel) {
+      static unsigned long long lds_done = 0;
+      const int rc_lds = reserve_lds_once(
+          reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, false, true, true, true, 10>), kTLds160, &lds_done);
+      if (rc_lds) return rc_lds;
+      hipLaunchKernelGGL((moe_gemm_t128_kernel<false, false, true, true, true, 10>), g, b, kTLds160, s, a, mbi, gi);
+    } else if (fast) LO_T160_LAUNCH(true);
     else LO_T160_LAUNCH(false);
 #undef LO_T160_LAUNCH
     return check_launch("moe_gemm(t160)");

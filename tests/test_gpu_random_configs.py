@@ -33,10 +33,11 @@ def _draw(rnd):
 
 
 def _block_size_offered(c):
-    """160-token blocks: int8 block-scaled weights in the load-time layout and 2I <= H."""
+    """160-token blocks: int8 block-scaled weights in the load-time layout and 2I <= H, or int4 weights
+    with per-channel scales."""
     if c["bs"] != 160:
         return True
-    return c["form"] == "block" and c["pre"] and 2 * c["I"] <= c["H"]
+    return c["form"] == "w4pc" or (c["form"] == "block" and c["pre"] and 2 * c["I"] <= c["H"])
 
 
 @pytest.mark.parametrize("seed", [11, 12])

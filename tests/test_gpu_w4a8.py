@@ -218,11 +218,13 @@ def channel_gemm_case(seed, M, k, E, Eg, N, K):
 
 @pytest.mark.parametrize("M,k,E,Eg,N,K", [(1, 2, 4, 4, 64, 128), (5, 2, 4, 4, 256, 512), (40, 4, 8, 8, 320, 1152),
                                           (100, 8, 4, 16, 512, 768), (300, 2, 3, 3, 128, 2048), (70, 2, 2, 2, 48, 384)])
-@pytest.mark.parametrize("bs", [16, 32, 64, 128])
+@pytest.mark.parametrize("bs", [16, 32, 64, 128, 160])
 def test_channel_form_gemm_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
     from lightop_amd.moe import invoke_fused_moe_kernel_w4a8, moe_align_block_size, preshuffle_moe_weight_int4
 
     say(f"w4a8 channel gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs}")
+    if bs == 160 and N % 64:
+        pytest.skip("160-token blocks need N a multiple of 64")
     Aq, As, W4, Ws, ids, tw, emap = channel_gemm_case(M + N + bs, M, k, E, Eg, N, K)
     rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
     s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
@@ -270,7 +272,7 @@ def run_channel_path(layer, weights_dev, x, tw, ids, emap, dev, bs, **kw):
     return out
 
 
-@pytest.mark.parametrize("bs", [0, 16, 32, 64, 128])
+@pytest.mark.parametrize("bs", [0, 16, 32, 64, 128, 160])
 @pytest.mark.parametrize("with_map", [False, True])
 def test_channel_form_whole_path_tiny_bit_exact(dev, oracle, bs, with_map):
     from lightop_amd import workloads as wl
@@ -293,6 +295,23 @@ def test_channel_form_whole_path_tiny_bit_exact(dev, oracle, bs, with_map):
         ref = oracle.fused_experts_w4a8_channel(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=layer.E,
                                                 expert_map=emap, shared_output=so, routed_scaling_factor=rsf)
         assert ref.float().abs().max() > 0.05
+        assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+def test_channel_form_blocks_of_160_filled(dev, oracle):
+    """Two experts, every token on both: blocks of 160 tokens with 1 ... 160 valid rows, every K-loop variant."""
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import preshuffle_moe_weight_int4
+
+    layer = wl.MoeLayer("w4pc-160", E=2, E_global=2, top_k=2, H=512, I=256, routing="softmax", weight_bits=4,
+                        quant="channel")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=2)
+    wd = (preshuffle_moe_weight_int4(w1.to(dev)), preshuffle_moe_weight_int4(w2.to(dev)), w1s.to(dev), w2s.to(dev))
+    for M in (1, 60, 65, 129, 150, 160, 161, 330):
+        say(f"w4a8 channel whole path, 160-token blocks, M={M}")
+        x, tw, ids = wl.make_inputs(layer, M, seed=M)
+        out = run_channel_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None, dev, 160)
+        ref = oracle.fused_experts_w4a8_channel(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=layer.E)
         assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
