@@ -229,9 +229,10 @@ int launch_gemm_pc(const GemmArgs &a0, int block_size_m, int64_t m_blocks, hipSt
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm_w8a8: grid too large");
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
-  // one token block per expert, by and large: the slots spread over the routed experts fill half a block
-  const bool stream =
-      a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * (block_size_m / 2);
+  // one token block per expert, by and large: up to 48 slots per expert on average with 64-token blocks
+  // (as measured for the block form's 64-token kernel), half a block with 128-token blocks
+  const bool stream = a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) *
+                                         (block_size_m == 64 ? 48 : 64);
 #define LO_PC_LAUNCH(KERN)                                                                    \
   do {                                                                                        \
     if (a.w_shuffled) {                                                                       \
