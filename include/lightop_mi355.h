@@ -447,8 +447,9 @@ int lo_fuse_silu_mul_quant_ids(const void *c1, int dtype, int64_t rows, int64_t 
  * W is the load-time layout of lo_preshuffle_weight_int4, K counts unpacked elements, every
  * nibble enters the sum as int8(nibble << 4), i.e. 16 times the signed int4, and
  *   C[f, n] = T(((f32(sum_k A*w16) [* topk_w[f]]) * As[f / top_k]) * Ws[e, n]).
- * With LO_GEMM_W4, block_size_m may also be 160 (N % 64 == 0, K <= 16384): 160-token blocks of the
- * direct-to-LDS kernel, for layers whose experts see a few tokens more than 128.
+ * With weights in the load-time layout (LO_GEMM_W_PRESHUFFLED; int8 or int4) block_size_m may also
+ * be 160 (N % 64 == 0, K <= 16384): 160-token blocks of the direct-to-LDS kernel with the int32 sums
+ * of the whole K in its accumulators, for layers whose experts see a few tokens more than 128.
  */
 int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *W, const float *Ws, void *C,
                      int c_dtype, const float *topk_w, const int32_t *sorted_ids,
@@ -467,8 +468,9 @@ int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *W, const fl
  * The workspace is the one of lo_fused_experts_workspace_bytes.
  * flags LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED: both stages are the int4 kernel described at
  * lo_moe_gemm_w8a8, which makes the call the reference's fused_experts_impl_w4a8 (w4a8.py:480-658)
- * with w1 [E, 2I, H/2] and w2 [E, H, I/2] in the layout of lo_preshuffle_weight_int4; block_size_m
- * may then also be 160 (H, I <= 16384), which the tile table picks around 128 slots per expert.
+ * with w1 [E, 2I, H/2] and w2 [E, H, I/2] in the layout of lo_preshuffle_weight_int4.
+ * With weights in the load-time layout (either kind) block_size_m may also be 160 (H, I <= 16384),
+ * which the tile table picks around 128 slots per expert.
  */
 int lo_fused_experts_channel_int8(const void *x, int dtype, int64_t M, int64_t H, int64_t I,
                                   int32_t E, int32_t num_experts, int32_t top_k, const int8_t *w1,

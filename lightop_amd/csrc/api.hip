@@ -160,8 +160,14 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   // 130 / 132 / 127 / 130, at 256: 188 / 147 / 135 / 138, at 512: 296 / 223 / 152 / 153, at 1024:
   // 489 / 361 / 223 / 173; DeepSeek-V3 share of 32 experts at 128 tokens 252 / 251 / 253 / 253, at
   // 256: 268 / 268 / 270 / 262, at 512: 365 / 296 / 297 / 285, at 1024: 627 / 476 / 336 / 319.
+  // Around 128 slots per expert the 160-token form of the direct-to-LDS kernel (int32 sums over the whole K
+  // in its accumulators) holds an expert's tokens in one block, where a 128-token block spills into a
+  // second pass over the expert's weights.  Measured, 128 / 160: DeepSeek-V3 share at 2048 tokens 378 / 384,
+  // at 2560: 476 / 418, at 3584: 616 / 475, at 4096: 629 / 514, at 4608: 659 / 686; Qwen3-shaped layer at
+  // 1024 tokens 173 / 192, at 1280: 222 / 201, at 2048: 259 / 226, at 2304: 285 / 250, at 2560: 273 / 306.
   if (form == LO_FORM_CHANNEL) {
     if (per_expert <= 6.0) return 16;
+    if (allow160 && per_expert >= 72.0 && per_expert < (H >= 4096 ? 140.0 : 152.0)) return 160;
     return (H >= 4096 || per_expert >= 48.0) ? 128 : 64;
   }
   if (per_expert <= 12.0) return 16;
@@ -188,9 +194,9 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
   const bool pre = (flags & LO_GEMM_W_PRESHUFFLED) != 0;
   const bool int4_channel = form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4);
   const int32_t bm = pick_block_m(M, num_experts, top_k, H, form, pre, int4_channel,
-                                  int4_channel ? (H / kGroup <= 128 && I / kGroup <= 128)
-                                               : (form == LO_FORM_BLOCK && pre && blocks_of_160_fit(H, I) &&
-                                                  !(flags & LO_FUSED_ACT_GELU)));
+                                  form == LO_FORM_CHANNEL ? (pre && H / kGroup <= 128 && I / kGroup <= 128)
+                                                          : (form == LO_FORM_BLOCK && pre && blocks_of_160_fit(H, I) &&
+                                                             !(flags & LO_FUSED_ACT_GELU)));
   // the argument blocks the stage entry points would build for this problem
   GemmArgs a{};
   a.num_valid = M * top_k;
@@ -381,12 +387,15 @@ extern "C" int lo_fused_experts_channel_int8(
   if (M == 0) return LO_OK;
   if (block_size_m == 0)
     block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_CHANNEL, true, (flags & LO_GEMM_W4) != 0,
-                                H / kGroup <= 128 && I / kGroup <= 128);
-  // 160: the 160-token form of the direct-to-LDS kernel, for int4 weights
-  const bool bs160 = block_size_m == 160 && (flags & LO_GEMM_W4) && H / kGroup <= 128 && I / kGroup <= 128;
+                                (flags & (LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED)) && H / kGroup <= 128 &&
+                                    I / kGroup <= 128);
+  // 160: the 160-token form of the direct-to-LDS kernel (weights in the load-time layout)
+  const bool bs160 = block_size_m == 160 && (flags & (LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED)) && H / kGroup <= 128 &&
+                     I / kGroup <= 128;
   LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 || bs160,
-             LO_EINVAL, "fused_experts(channel): block_size_m %d is not one of 16, 32, 64, 128 (160: int4 weights)",
-             block_size_m);
+             LO_EINVAL,
+             "fused_experts(channel): block_size_m %d is not one of 16, 32, 64, 128 (160: weights in the load-time "
+             "layout)", block_size_m);
   // the block layout is roomy enough: its scale segments hold one float per 128 values
   const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
   LO_REQUIRE(workspace_bytes >= L.total, LO_ENOSPC,

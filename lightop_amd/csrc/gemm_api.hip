@@ -186,8 +186,9 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   int rc = validate_common("moe_gemm_w8a8", A, As, W, Ws, sorted_ids, expert_ids, num_tokens_post_pad, K,
                            top_k, E, a_rows);
   if (rc) return rc;
-  LO_REQUIRE(valid_block_m(block_size_m) || (block_size_m == 160 && (flags & LO_GEMM_W4)), LO_EINVAL,
-             "moe_gemm_w8a8: block_size_m %d is not one of 16, 32, 64, 128 (160: int4 weights only)", block_size_m);
+  LO_REQUIRE(valid_block_m(block_size_m) || (block_size_m == 160 && (flags & LO_GEMM_W_PRESHUFFLED)), LO_EINVAL,
+             "moe_gemm_w8a8: block_size_m %d is not one of 16, 32, 64, 128 (160: weights in the load-time layout)",
+             block_size_m);
   LO_REQUIRE(C, LO_EINVAL, "moe_gemm_w8a8: null output");
   LO_REQUIRE(c_dtype == LO_BF16 || c_dtype == LO_F16, LO_ENOTSUP, "moe_gemm_w8a8: the output is bf16 or fp16");
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm_w8a8: N (%lld) must be a multiple of 16", (long long)N);

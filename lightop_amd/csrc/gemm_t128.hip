@@ -71,9 +71,10 @@ __device__ __forceinline__ void wait_copies_barrier() {
 template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM, bool W4, bool PC = false, int NTB = 8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
-  static_assert(!PC || (W4 && !FUSED_ACT && !FAST_SCALE), "per-channel scales: plain int4 GEMM only");
-  static_assert(NTB == 8 || (NTB == 10 && !FUSED_ACT && W4 == PC),
-                "160-token tiles: plain GEMM, int8 block form or int4 with per-channel scales");
+  static_assert(!PC || (!FUSED_ACT && !FAST_SCALE && (W4 || NTB == 10)),
+                "per-channel scales: plain GEMM, int4 weights or 160-token tiles of int8 weights");
+  static_assert(NTB == 8 || (NTB == 10 && !FUSED_ACT && (PC || !W4)),
+                "160-token tiles: plain GEMM, int8 block form or per-channel scales");
   constexpr int T = 16 * NTB;        // tokens per workgroup
   constexpr int AST = T * kGroup;    // token rows of one K block
   constexpr int APW = NTB / 2;       // 1 KB pieces (eight token rows) of a token stage that a wave copies
@@ -216,7 +217,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     const int which = tid >> 7, kbi = tid & (kTMaxKB - 1);
     int64_t nblk = FUSED_ACT ? (which ? I / kGroup : 0) + nt : static_cast<int64_t>(nt) * 2 + which;
     if (nblk >= NB) nblk = 0;
-    if (!W4 && kbi < KB) bs_mine = a.Ws[(static_cast<int64_t>(e) * NB + nblk) * KB + kbi];
+    if (!W4 && !PC && kbi < KB) bs_mine = a.Ws[(static_cast<int64_t>(e) * NB + nblk) * KB + kbi];
   }
   const float *const sBs0 = sBs + (FUSED_ACT ? 0 : (wave >> 1) * kTMaxKB);
   const float *const sBs1 = sBs + (FUSED_ACT ? kTMaxKB : (wave >> 1) * kTMaxKB);
@@ -561,10 +562,14 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               float v;
-              if constexpr (PC) { // left to right: routed weight, token scale, channel scale (w4a8.py:386-395)
+              if constexpr (PC && W4) { // left to right: routed weight, token scale, channel scale (w4a8.py:386-395)
                 v = static_cast<float>(acci[h][tb][rf][i]);
                 if (a.mul_routed) v = v * wgt;
                 v = v * pas[tb];
+                v = v * pbs[h][rf][i];
+              } else if constexpr (PC) { // int8 weights: (f32(d) * ts) * b_s, ts = w * a_s (moe_w8a8.cu:452, :466)
+                const float ts = a.mul_routed ? wgt * pas[tb] : pas[tb];
+                v = static_cast<float>(acci[h][tb][rf][i]) * ts;
                 v = v * pbs[h][rf][i];
               } else {
                 v = acc[h][tb][rf][i];
@@ -675,9 +680,8 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 }
 
 bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
-  if (block_size_m == kT160) // 160-token tiles: plain GEMM, int8 block form or int4 with per-channel scales
-    return a.w_shuffled && !fused_act && (a.w4 != 0) == (a.per_channel != 0) && a.N % 64 == 0 &&
-           a.K / kGroup <= kTMaxKB;
+  if (block_size_m == kT160) // 160-token tiles: plain GEMM, int8 block form or per-channel scales
+    return a.w_shuffled && !fused_act && (a.per_channel || !a.w4) && a.N % 64 == 0 && a.K / kGroup <= kTMaxKB;
   if (block_size_m != 128 || !a.w_shuffled) return false;
   if (a.per_channel && (!a.w4 || fused_act)) return false; // int8 per-channel weights have gemm_pc.hip
   if (!fused_act && a.N % 64 != 0) return false;
@@ -733,12 +737,18 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int f
     if (rc_lds) return rc_lds;                                                                                  \
     hipLaunchKernelGGL((moe_gemm_t128_kernel<false, FS, true, false, false, 10>), g, b, kTLds160, s, a, mbi, gi); \
   } while (0)
-    if (a.per_channel) {
+    if (a.per_channel && a.w4) {
       static unsigned long long lds_done = 0;
       const int rc_lds = reserve_lds_once(
           reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, false, true, true, true, 10>), kTLds160, &lds_done);
       if (rc_lds) return rc_lds;
       hipLaunchKernelGGL((moe_gemm_t128_kernel<false, false, true, true, true, 10>), g, b, kTLds160, s, a, mbi, gi);
+    } else if (a.per_channel) {
+      static unsigned long long lds_done = 0;
+      const int rc_lds = reserve_lds_once(
+          reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, false, true, false, true, 10>), kTLds160, &lds_done);
+      if (rc_lds) return rc_lds;
+      hipLaunchKernelGGL((moe_gemm_t128_kernel<false, false, true, false, true, 10>), g, b, kTLds160, s, a, mbi, gi);
     } else if (fast) LO_T160_LAUNCH(true);
     else LO_T160_LAUNCH(false);
 #undef LO_T160_LAUNCH

@@ -109,7 +109,7 @@ def gemm_case(seed, M, k, E, Eg, N, K):
 
 @pytest.mark.parametrize("M,k,E,Eg,N,K", [(1, 2, 4, 4, 64, 128), (5, 2, 4, 4, 256, 512), (40, 4, 8, 8, 320, 1152),
                                           (100, 8, 4, 16, 512, 768), (300, 2, 3, 3, 128, 2048), (70, 2, 2, 2, 48, 384)])
-@pytest.mark.parametrize("bs", [16, 32, 64, 128])
+@pytest.mark.parametrize("bs", [16, 32, 64, 128, 160])
 @pytest.mark.parametrize("shuf", [False, True])
 def test_moe_gemm_w8a8_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs, shuf):
     from lightop_amd import _lib
@@ -117,6 +117,8 @@ def test_moe_gemm_w8a8_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs, shuf):
     from lightop_amd.moe import moe_align_block_size, preshuffle_moe_weight
 
     say(f"channel gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs} shuf={shuf}")
+    if bs == 160 and (not shuf or N % 64):
+        pytest.skip("160-token blocks: weights in the load-time layout, N a multiple of 64")
     Aq, As, W, Ws, ids, tw, emap = gemm_case(M + N + bs, M, k, E, Eg, N, K)
     rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
     s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
@@ -169,7 +171,27 @@ def run_path(layer, weights_dev, x, tw, ids, emap, dev, bs, **kw):
     return out
 
 
-@pytest.mark.parametrize("bs", [0, 16, 32, 64, 128])
+def test_whole_path_blocks_of_160_filled(dev, oracle):
+    """Two experts, every token on both: blocks of 160 tokens with 1 ... 160 valid rows, every K-loop variant;
+    the router weight in the second GEMM's epilogue (ts = w * a_s) and on the input."""
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import preshuffle_moe_weight
+
+    layer = wl.MoeLayer("pc-160", E=2, E_global=2, top_k=2, H=512, I=256, routing="softmax", quant="channel")
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=2)
+    wd = (preshuffle_moe_weight(w1.to(dev)), preshuffle_moe_weight(w2.to(dev)), w1s.to(dev), w2s.to(dev))
+    for M in (1, 60, 65, 129, 150, 160, 161, 330):
+        for on_input in (False, True):
+            say(f"channel whole path, 160-token blocks, M={M} on_input={on_input}")
+            x, tw, ids = wl.make_inputs(layer, M, seed=M)
+            out = run_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None, dev, 160,
+                           apply_router_weight_on_input=on_input)
+            ref = oracle.fused_experts_channel_int8(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=layer.E,
+                                                    apply_router_weight_on_input=on_input)
+            assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("bs", [0, 16, 32, 64, 128, 160])
 @pytest.mark.parametrize("with_map", [False, True])
 @pytest.mark.parametrize("shuf", [False, True])
 def test_whole_path_tiny_bit_exact(dev, oracle, bs, with_map, shuf):
@@ -178,6 +200,8 @@ def test_whole_path_tiny_bit_exact(dev, oracle, bs, with_map, shuf):
 
     layer = wl.TINY_PC
     say(f"channel whole path tiny bs={bs} map={with_map} shuf={shuf}")
+    if bs == 160 and not shuf:
+        pytest.skip("160-token blocks: weights in the load-time layout")
     w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
     x, tw, ids = wl.make_inputs(layer, 96, seed=4)
     emap = None

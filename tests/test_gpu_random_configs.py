@@ -33,11 +33,12 @@ def _draw(rnd):
 
 
 def _block_size_offered(c):
-    """160-token blocks: int8 block-scaled weights in the load-time layout and 2I <= H, or int4 weights
-    with per-channel scales."""
+    """160-token blocks: weights in the load-time layout with block scales (2I <= H) or per-channel scales."""
     if c["bs"] != 160:
         return True
-    return c["form"] == "w4pc" or (c["form"] == "block" and c["pre"] and 2 * c["I"] <= c["H"])
+    if c["form"] == "w4pc" or (c["form"] == "channel" and c["pre"]):
+        return True
+    return c["form"] == "block" and c["pre"] and 2 * c["I"] <= c["H"]
 
 
 @pytest.mark.parametrize("seed", [11, 12])
