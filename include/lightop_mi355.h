@@ -28,9 +28,13 @@ enum {
   LO_ENOTSUP = -4   /* valid request that this build has no kernel for */
 };
 
-/* activation element types (LO_F32: router inputs only).  fp16 rows go the same way as bf16 ones except
- * that no kernel fuses the gated activation for them: the first GEMM writes [S, 2I] in fp16 and one launch
- * applies the activation and quantises (as with LO_FUSED_ACT_GELU), and the two-launch path is not taken. */
+/* activation element types.  fp16 rows go the same way as bf16 ones except that no kernel fuses the gated
+ * activation for them: the first GEMM writes [S, 2I] in fp16 and one launch applies the activation and
+ * quantises (as with LO_FUSED_ACT_GELU), and the two-launch path is not taken.  LO_F32 (besides router
+ * inputs): the block form with int8 weights and its stages (lo_per_token_group_quant_int8,
+ * lo_moe_gemm_block_int8, lo_silu_and_mul, lo_gelu_and_mul, lo_act_mul_group_quant, lo_moe_sum); nothing
+ * between the stages is rounded to 16 bits then (compute_type tl.float32, int8.py:689-696), and the GEMMs
+ * are the weight-streaming kernel at every size. */
 enum { LO_BF16 = 0, LO_F16 = 1, LO_F32 = 2 };
 /* gated activations */
 enum { LO_ACT_SILU = 0, LO_ACT_GELU = 1 };

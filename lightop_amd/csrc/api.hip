@@ -266,7 +266,8 @@ extern "C" int lo_fused_experts_block_int8(
   using namespace lo;
   LO_REQUIRE(x && w1 && w1s && w2 && w2s && topk_w && topk_ids && cache3 && out && workspace,
              LO_EINVAL, "fused_experts: null pointer");
-  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "fused_experts: activations are bf16 or fp16");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16 || (dtype == LO_F32 && !(flags & LO_GEMM_W4)), LO_ENOTSUP,
+             "fused_experts: activations are bf16, fp16 or (int8 weights) fp32");
   LO_REQUIRE(M >= 0 && H >= kGroup && H % kGroup == 0 && I >= kGroup && I % kGroup == 0, LO_EINVAL,
              "fused_experts: hidden (%lld) and intermediate (%lld) sizes must be multiples of 128",
              (long long)H, (long long)I);
@@ -278,6 +279,8 @@ extern "C" int lo_fused_experts_block_int8(
              "fused_experts: workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
   const bool block_size_m_auto = block_size_m == 0;
+  if (block_size_m == 0 && dtype == LO_F32) // fp32 rows go through the weight-streaming kernel at every size
+    block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_BLOCK, false);
   if (block_size_m == 0)
     block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
                                 (flags & LO_GEMM_W_PRESHUFFLED) != 0, false,
@@ -286,11 +289,11 @@ extern "C" int lo_fused_experts_block_int8(
   // 160: the 160-token form of the direct-to-LDS kernel (int8 block form, load-time layout), both GEMMs
   // with plain epilogues and the activation in a launch of its own
   const bool bs160 = block_size_m == 160 && (flags & LO_GEMM_W_PRESHUFFLED) && !(flags & LO_GEMM_W4) &&
-                     blocks_of_160_fit(H, I);
+                     dtype != LO_F32 && blocks_of_160_fit(H, I);
   LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 || bs160,
              LO_EINVAL,
              "fused_experts: block_size_m %d is not one of 16, 32, 64, 128 (160: int8 weights in the load-time "
-             "layout and 2I <= H only)", block_size_m);
+             "layout, 16-bit rows and 2I <= H only)", block_size_m);
   const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
   LO_REQUIRE(workspace_bytes >= L.total, LO_ENOSPC, "fused_experts: workspace holds %lld bytes, needs %lld",
              (long long)workspace_bytes, (long long)L.total);

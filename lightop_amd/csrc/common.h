@@ -46,6 +46,13 @@ int act_table(hipStream_t stream, int act, int dtype, const uint16_t **table);
 // row_mask (optional, [rows] bytes): rows whose byte is 0 are skipped.
 int launch_act_mul_group_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
                                const uint8_t *row_mask, hipStream_t stream);
+// fp32 rows (elementwise_f32.hip)
+int launch_group_quant_f32(const float *x, int64_t groups, float eps, int8_t *q, float *s, hipStream_t stream);
+int launch_act_mul_f32(const float *c1, int64_t rows, int64_t I, int act, float *out, hipStream_t stream);
+int launch_act_mul_group_quant_f32(const float *c1, int act, int64_t rows, int64_t I, int8_t *q, float *s,
+                                   const uint8_t *row_mask, hipStream_t stream);
+int launch_moe_sum_f32(const float *in, float *out, const float *bias, const uint8_t *mask, int64_t M, int32_t topk,
+                       int64_t H, float factor, const int32_t *num_local_tokens, hipStream_t stream);
 int launch_act_mul_row_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
                              const int32_t *num_local_tokens, int32_t top_k, const int32_t *row_ids,
                              hipStream_t stream);

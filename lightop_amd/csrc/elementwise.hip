@@ -452,6 +452,8 @@ int act_table(hipStream_t stream, int act, int dtype, const uint16_t **out) {
 // activation from its table and the quantisation of the form in one pass over c1 [rows, 2I].
 int launch_act_mul_group_quant(const void *c1, int dtype, int act, int64_t rows, int64_t I, int8_t *q, float *s,
                                const uint8_t *row_mask, hipStream_t stream) {
+  if (dtype == LO_F32)
+    return launch_act_mul_group_quant_f32(static_cast<const float *>(c1), act, rows, I, q, s, row_mask, stream);
   const uint16_t *table = nullptr;
   int rc = act_table(stream, act, dtype, &table);
   if (rc) return rc;
@@ -527,7 +529,8 @@ extern "C" int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t
                                              lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(x && q && s, LO_EINVAL, "per_token_group_quant_int8: null pointer");
-  LO_REQUIRE(x_dtype == LO_BF16 || x_dtype == LO_F16, LO_ENOTSUP, "per_token_group_quant_int8: the input is bf16 or fp16");
+  LO_REQUIRE(x_dtype == LO_BF16 || x_dtype == LO_F16 || x_dtype == LO_F32, LO_ENOTSUP,
+             "per_token_group_quant_int8: the input is bf16, fp16 or fp32");
   LO_REQUIRE(rows >= 0 && cols > 0 && cols % kGroup == 0, LO_EINVAL,
              "per_token_group_quant_int8: the last dimension (%lld) must be a multiple of 128",
              (long long)cols);
@@ -535,6 +538,8 @@ extern "C" int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t
              LO_EINVAL, "per_token_group_quant_int8: x must be 16-byte and q 8-byte aligned");
   const int64_t groups = rows * (cols / kGroup);
   if (groups == 0) return LO_OK;
+  if (x_dtype == LO_F32)
+    return launch_group_quant_f32(static_cast<const float *>(x), groups, eps, q, s, static_cast<hipStream_t>(stream));
   if (x_dtype == LO_F16)
     hipLaunchKernelGGL(group_quant_kernel<LO_F16>, dim3(grid_for(groups, 16)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(x), groups, eps, q, s);
@@ -548,12 +553,15 @@ extern "C" int lo_silu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
                                lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(c1 && act, LO_EINVAL, "silu_and_mul: null pointer");
-  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "silu_and_mul: bf16 or fp16");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16 || dtype == LO_F32, LO_ENOTSUP, "silu_and_mul: bf16, fp16 or fp32");
   LO_REQUIRE(rows >= 0 && I > 0 && I % 8 == 0, LO_EINVAL, "silu_and_mul: I (%lld) must be a multiple of 8",
              (long long)I);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(act) & 15) == 0,
              LO_EINVAL, "silu_and_mul: pointers must be 16-byte aligned");
   if (rows == 0) return LO_OK;
+  if (dtype == LO_F32)
+    return launch_act_mul_f32(static_cast<const float *>(c1), rows, I, LO_ACT_SILU, static_cast<float *>(act),
+                              static_cast<hipStream_t>(stream));
   if (dtype == LO_F16)
     hipLaunchKernelGGL(silu_mul_kernel<LO_F16>, dim3(grid_for(rows * (I / 8), 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const uint16_t *>(c1), rows, I,
@@ -569,11 +577,14 @@ extern "C" int lo_gelu_and_mul(const void *c1, int dtype, int64_t rows, int64_t 
                                lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(c1 && act, LO_EINVAL, "gelu_and_mul: null pointer");
-  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "gelu_and_mul: bf16 or fp16");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16 || dtype == LO_F32, LO_ENOTSUP, "gelu_and_mul: bf16, fp16 or fp32");
   LO_REQUIRE(rows >= 0 && I > 0 && I % 8 == 0, LO_EINVAL, "gelu_and_mul: I (%lld) must be a multiple of 8",
              (long long)I);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(c1) & 15) == 0 && (reinterpret_cast<uintptr_t>(act) & 15) == 0,
              LO_EINVAL, "gelu_and_mul: pointers must be 16-byte aligned");
+  if (dtype == LO_F32)
+    return launch_act_mul_f32(static_cast<const float *>(c1), rows, I, LO_ACT_GELU, static_cast<float *>(act),
+                              static_cast<hipStream_t>(stream));
   const uint16_t *table = nullptr;
   int rc = act_table(static_cast<hipStream_t>(stream), LO_ACT_GELU, dtype, &table);
   if (rc) return rc;
@@ -593,7 +604,8 @@ extern "C" int lo_act_mul_group_quant(const void *c1, int dtype, int activation,
                                       float *s, const uint8_t *row_mask, lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(c1 && q && s, LO_EINVAL, "act_mul_group_quant: null pointer");
-  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "act_mul_group_quant: bf16 or fp16");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16 || dtype == LO_F32, LO_ENOTSUP,
+             "act_mul_group_quant: bf16, fp16 or fp32");
   LO_REQUIRE(activation == LO_ACT_SILU || activation == LO_ACT_GELU, LO_EINVAL,
              "act_mul_group_quant: unknown activation %d", activation);
   LO_REQUIRE(rows >= 0 && I > 0 && I % kGroup == 0, LO_EINVAL,
@@ -621,13 +633,17 @@ extern "C" int lo_moe_sum(const void *in, void *out, const void *bias, const uin
                           const int32_t *num_local_tokens, lo_stream_t stream) {
   using namespace lo;
   LO_REQUIRE(in && out, LO_EINVAL, "moe_sum: null pointer");
-  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "moe_sum: bf16 or fp16");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16 || dtype == LO_F32, LO_ENOTSUP, "moe_sum: bf16, fp16 or fp32");
   LO_REQUIRE(M >= 0 && topk >= 1 && H > 0 && H % 8 == 0, LO_EINVAL,
              "moe_sum: hidden size (%lld) must be a multiple of 8, topk >= 1", (long long)H);
   LO_REQUIRE((reinterpret_cast<uintptr_t>(in) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
                  (reinterpret_cast<uintptr_t>(bias) & 15) == 0,
              LO_EINVAL, "moe_sum: pointers must be 16-byte aligned");
   if (M == 0) return LO_OK;
+  if (dtype == LO_F32)
+    return launch_moe_sum_f32(static_cast<const float *>(in), static_cast<float *>(out),
+                              static_cast<const float *>(bias), expert_mask, M, topk, H, factor, num_local_tokens,
+                              static_cast<hipStream_t>(stream));
   const int grid = grid_for(M * (H / 8), 256);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define LO_SUM_LAUNCH(DTV, HB, TK)                                                                   \

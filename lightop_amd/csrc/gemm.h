@@ -40,6 +40,7 @@ struct GemmArgs {
   int32_t w4;            // W is packed int4 (load-time layout), Ws is [E, K/128, N]
   int32_t per_channel;   // As is [a_rows], Ws is [E, N]: scales applied once, after the whole-K int32 sum
   int32_t out_f16;       // C holds IEEE half instead of bf16 (plain epilogues only)
+  int32_t out_f32;       // C holds the fp32 sums themselves (block form, weight-streaming kernel only)
 };
 
 // The 16-bit form a plain epilogue stores: bf16, or IEEE half when the caller's activations are fp16.

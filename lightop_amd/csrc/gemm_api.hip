@@ -33,6 +33,7 @@ static int validate_common(const char *who, const void *A, const void *As, const
 // per expert large enough for operand reuse to matter); smaller ones stream weights.  The tile
 // query (lo_moe_tile_query_form) reports this very choice.
 int pick_gemm_kernel(const GemmArgs &a, bool fused_act, int bs, int flags) {
+  if (a.out_f32) return LO_KERNEL_WS; // fp32 rows: the weight-streaming kernel's plain epilogue only
   if (bs == 160) return LO_KERNEL_T128; // 160-token blocks exist for that kernel only (the entry point checks)
   const bool tiled = !(flags & LO_GEMM_FORCE_STREAMING);
   if (a.w4 && a.per_channel) // the reference's own int4 form: 128-token LDS tiles, else streaming
@@ -103,7 +104,9 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   LO_REQUIRE(valid_block_m(block_size_m) || block_size_m == 160, LO_EINVAL,
              "moe_gemm: block_size_m %d is not one of 16, 32, 64, 128 (or 160)", block_size_m);
   LO_REQUIRE(C, LO_EINVAL, "moe_gemm: null output");
-  LO_REQUIRE(c_dtype == LO_BF16 || c_dtype == LO_F16, LO_ENOTSUP, "moe_gemm: the output is bf16 or fp16");
+  LO_REQUIRE(c_dtype == LO_BF16 || c_dtype == LO_F16 || c_dtype == LO_F32, LO_ENOTSUP,
+             "moe_gemm: the output is bf16, fp16 or fp32");
+  LO_REQUIRE(c_dtype != LO_F32 || block_size_m != 160, LO_ENOTSUP, "moe_gemm: fp32 rows have no 160-token blocks");
   LO_REQUIRE(N > 0 && N % 16 == 0, LO_EINVAL, "moe_gemm: N (%lld) must be a multiple of 16", (long long)N);
   LO_REQUIRE(N * K < (1ll << 31), LO_ENOTSUP, "moe_gemm: one expert's weights exceed 2 GiB");
   LO_REQUIRE(!mul_routed || topk_w, LO_EINVAL, "moe_gemm: mul_routed needs topk_weights");
@@ -120,6 +123,7 @@ extern "C" int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const in
   a.skip_nonlocal = (flags & LO_GEMM_SKIP_NONLOCAL) ? 1 : 0;
   a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
   a.out_f16 = c_dtype == LO_F16 ? 1 : 0;
+  a.out_f32 = c_dtype == LO_F32 ? 1 : 0;
   LO_REQUIRE(!a.w4 || a.w_shuffled, LO_ENOTSUP,
              "moe_gemm: int4 weights must be in the layout of lo_preshuffle_weight_int4 (LO_GEMM_W_PRESHUFFLED)");
   a.n_tiles = static_cast<int32_t>((N + 63) / 64);

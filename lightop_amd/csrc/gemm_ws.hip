@@ -108,7 +108,12 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
         if (valid[j])
 #pragma unroll
           for (int g = 0; g < NW; ++g)
-            if (n0 + g * 16 < N) *reinterpret_cast<v2i *>(a.C + f[j] * N + n0 + g * 16 + 4 * c) = v2i{0, 0};
+            if (n0 + g * 16 < N) {
+              if (a.out_f32)
+                *reinterpret_cast<v4i *>(reinterpret_cast<float *>(a.C) + f[j] * N + n0 + g * 16 + 4 * c) = v4i{0, 0, 0, 0};
+              else
+                *reinterpret_cast<v2i *>(a.C + f[j] * N + n0 + g * 16 + 4 * c) = v2i{0, 0};
+            }
       return;
     }
   } else {
@@ -380,6 +385,13 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
 #pragma unroll
       for (int g = 0; g < NW; ++g) {
         if (nrow[g] >= N) continue;
+        if (__builtin_expect(a.out_f32 != 0, 0)) { // fp32 rows: the sum itself, unrounded (compute_type tl.float32)
+          v4f o32;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o32[i] = a.mul_routed ? acc[g][j][i] * w : acc[g][j][i];
+          *reinterpret_cast<v4f *>(reinterpret_cast<float *>(a.C) + f[j] * N + nrow[g] + 4 * c) = o32;
+          continue;
+        }
         v4u16 o;
         with_out16(a.out_f16, [&](auto cvt) __attribute__((always_inline)) {
 #pragma unroll

@@ -384,9 +384,11 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     per_channel_quant=True, block_shape=None`` (one scale per token and per weight row,
     ``w1_scale`` [E, 2I, 1], ``w2_scale`` [E, H, 1]) with ``activation="silu"`` or ``"gelu"`` (the
     latter without the fused epilogue: one more launch and a bf16 round trip of [S, 2I]); every other
-    combination raises.  ``hidden_states`` is bfloat16 or float16 (float16 rows take the path without the
-    fused epilogue as well; every value between the stages is rounded to float16 then, as the reference's
-    compute_type does, int8.py:689-696); float32 raises.  ``cache13`` is the caller's workspace (dtype of ``hidden_states``,
+    combination raises.  ``hidden_states`` is bfloat16, float16 or, in the block form, float32 (float16 and
+    float32 rows take the path without the fused epilogue as well; every value between the stages is rounded
+    to float16, or not at all, as the reference's compute_type does, int8.py:689-696; float32 rows go
+    through the weight-streaming kernel at every size); float32 with per-channel scales raises.
+    ``cache13`` is the caller's workspace (dtype of ``hidden_states``,
     at least ``min(M, CHUNK) * topk * max(2I, H)`` elements); its first ``M*topk*H``
     elements receive the second GEMM's per-slot output.  The top-k reduction is always
     performed: ``out = routed_scaling_factor * sum_k(...) (+ shared_output)``.
@@ -408,8 +410,8 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
         raise NotImplementedError("lightop_amd: block_shape must be [128, 128], or None with per_channel_quant=True")
     if activation not in ("silu", "gelu"):
         raise ValueError(f"Unsupported FusedMoe activation: {activation}")
-    if hidden_states.dtype == torch.float32:
-        raise NotImplementedError("lightop_amd: hidden_states must be bfloat16 or float16")
+    if hidden_states.dtype == torch.float32 and channel:
+        raise NotImplementedError("lightop_amd: per-channel scales take bfloat16 or float16 hidden_states")
     assert w1_scale is not None and w2_scale is not None
     del w1_zp, w2_zp, a1_scale, a2_scale, use_nn_moe, i_q, i_s
     _require_cuda(hidden_states, w1, w2, topk_weights, topk_ids, cache13, w1_scale, w2_scale,

@@ -40,6 +40,8 @@ def _act_dtype(t: torch.Tensor) -> int:
         return _lib.LO_BF16
     if t.dtype == torch.float16:
         return _lib.LO_F16
+    if t.dtype == torch.float32:  # the block form's stages; entry points without an fp32 form say so
+        return _lib.LO_F32
     raise RuntimeError(f"lightop_amd: unsupported activation dtype {t.dtype}")
 
 

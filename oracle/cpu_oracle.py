@@ -125,6 +125,9 @@ def per_token_group_quant_int8(x, group_size=128, eps=1e-10):
     R = x.numel() // C
     q = torch.empty(x.shape, dtype=torch.int8)
     s = torch.empty(x.shape[:-1] + (C // 128,), dtype=torch.float32)
+    if x.dtype == torch.float32:
+        lib().orc_group_quant_int8_f32(_p(x), _i64(R), _i64(C), ctypes.c_float(eps), _p(q), _p(s))
+        return q, s
     with _elements_of(x):
         lib().orc_group_quant_int8(_p(x), _i64(R), _i64(C), ctypes.c_float(eps), _p(q), _p(s))
     return q, s
@@ -209,9 +212,12 @@ def moe_gemm_w4a8_channel(A, As, W4, Ws, sorted_ids, expert_ids, ntpp, topk_w, m
 def moe_gemm_block_int8(A, As, W, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_routed,
                         top_k, num_valid, block_size, dump_acc=False, out=None, _fn="orc_moe_gemm_block_int8"):
     """One grouped-GEMM stage.  Returns C[num_valid, N] bf16 (and the int32
-    per-128-block dot products when dump_acc)."""
+    per-128-block dot products when dump_acc).  With a float32 ``out`` the sums are stored unrounded."""
     E, N, K = W.shape
     C = torch.zeros(num_valid, N, dtype=torch.bfloat16) if out is None else out
+    if C.dtype == torch.float32:
+        assert _fn == "orc_moe_gemm_block_int8"
+        _fn = "orc_moe_gemm_block_int8_f32"
     acc = torch.zeros(num_valid, N, K // 128, dtype=torch.int32) if dump_acc else None
     tw = None if topk_w is None else topk_w.reshape(-1).to(torch.float32).contiguous()
     getattr(lib(), _fn)(
@@ -221,8 +227,17 @@ def moe_gemm_block_int8(A, As, W, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_
     return (C, acc) if dump_acc else C
 
 
+def _act_and_mul_f32(c1, activation):
+    S, N = c1.shape
+    act = torch.empty(S, N // 2, dtype=torch.float32)
+    lib().orc_act_and_mul_f32(_p(c1.contiguous()), _i64(S), _i64(N // 2), ctypes.c_int(activation), _p(act))
+    return act
+
+
 def silu_and_mul(c1):
     S, N = c1.shape
+    if c1.dtype == torch.float32:
+        return _act_and_mul_f32(c1, 0)
     act = torch.empty(S, N // 2, dtype=c1.dtype)
     with _elements_of(c1):
         lib().orc_silu_and_mul(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(act))
@@ -232,6 +247,8 @@ def silu_and_mul(c1):
 def gelu_and_mul(c1):
     """act = bf16(bf16(gelu(g)) * u), gelu with erf (activation_kernels_opt.cu:234-242)."""
     S, N = c1.shape
+    if c1.dtype == torch.float32:
+        return _act_and_mul_f32(c1, 1)
     act = torch.empty(S, N // 2, dtype=c1.dtype)
     with _elements_of(c1):
         lib().orc_gelu_and_mul(_p(c1.contiguous()), _i64(S), _i64(N // 2), _p(act))
@@ -256,9 +273,13 @@ def moe_sum(inp, bias=None, factor=1.0, num_local_tokens=None, out=None):
     """With num_local_tokens, rows from that index on keep what ``out`` held."""
     M, k, H = inp.shape
     res = torch.empty(M, H, dtype=inp.dtype)
-    with _elements_of(inp):
-        lib().orc_moe_sum(_p(inp.contiguous()), _i64(M), _i32(k), _i64(H),
-                          _p(None if bias is None else bias.contiguous()), ctypes.c_float(factor), _p(res))
+    if inp.dtype == torch.float32:
+        lib().orc_moe_sum_f32(_p(inp.contiguous()), _i64(M), _i32(k), _i64(H),
+                              _p(None if bias is None else bias.contiguous()), ctypes.c_float(factor), _p(res))
+    else:
+        with _elements_of(inp):
+            lib().orc_moe_sum(_p(inp.contiguous()), _i64(M), _i32(k), _i64(H),
+                              _p(None if bias is None else bias.contiguous()), ctypes.c_float(factor), _p(res))
     if num_local_tokens is not None:
         n = max(0, min(M, int(num_local_tokens)))
         res[n:] = out[n:]
@@ -353,6 +374,9 @@ def fused_experts_block_int8(x, w1, w2, w1_scale, w2_scale, topk_weights, topk_i
     tw = topk_weights.to(torch.float32).contiguous()
     emap = None if expert_map is None else expert_map.to(torch.int32).contiguous()
     assert shared_output is None or shared_output.dtype == dt
+    if dt == torch.float32:
+        assert _fn == "orc_fused_experts_block_int8", "fp32 rows: block form only"
+        _fn = "orc_fused_experts_block_int8_f32"
     lib().orc_set_activation(ctypes.c_int(1 if activation == "gelu" else 0))
     lib().orc_set_dtype(ctypes.c_int(1 if dt == torch.float16 else 0))
     try:

@@ -236,7 +236,8 @@ static void gemm_core(const int8_t *A, const float *As, const int8_t *W,
                       const int32_t *num_tokens_post_pad,
                       const float *topk_w, int mul_routed, int32_t top_k,
                       int64_t num_valid, int64_t N, int64_t K, int32_t bs,
-                      uint16_t *C, int32_t *acc_dump, int64_t group_n) {
+                      uint16_t *C, int32_t *acc_dump, int64_t group_n, float *Cf) {
+  /* Cf != NULL: fp32 rows (compute_type tl.float32, int8.py:689-696: the sum is stored unrounded) */
   int64_t KB = K / ORC_GROUP;
   int64_t NB = (N + group_n - 1) / group_n;
   int64_t P = num_tokens_post_pad[0];
@@ -247,9 +248,13 @@ static void gemm_core(const int8_t *A, const float *As, const int8_t *W,
       int64_t f = sorted[b * bs + i];
       if (f >= num_valid) continue;
       int32_t e = expert_ids[b];
-      uint16_t *c = C + f * N;
+      uint16_t *c = Cf ? NULL : C + f * N;
+      float *cf = Cf ? Cf + f * N : NULL;
       if (e < 0) {
-        for (int64_t n = 0; n < N; ++n) c[n] = 0;
+        for (int64_t n = 0; n < N; ++n) {
+          if (cf) cf[n] = 0.0f;
+          else c[n] = 0;
+        }
         continue;
       }
       int64_t row = f / top_k;
@@ -270,7 +275,8 @@ static void gemm_core(const int8_t *A, const float *As, const int8_t *W,
           acc = acc + t;
         }
         if (mul_routed) acc = acc * topk_w[f];
-        c[n] = f32_to_bf16(acc);
+        if (cf) cf[n] = acc;
+        else c[n] = f32_to_bf16(acc);
       }
     }
   }
@@ -284,7 +290,7 @@ void orc_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W,
                              int64_t num_valid, int64_t N, int64_t K, int32_t bs,
                              uint16_t *C, int32_t *acc_dump) {
   gemm_core(A, As, W, Ws, sorted, expert_ids, num_tokens_post_pad, topk_w, mul_routed, top_k,
-            num_valid, N, K, bs, C, acc_dump, ORC_GROUP);
+            num_valid, N, K, bs, C, acc_dump, ORC_GROUP, NULL);
 }
 
 /*
@@ -315,7 +321,7 @@ void orc_moe_gemm_rowscale_int8(const int8_t *A, const float *As, const int8_t *
                                 int64_t num_valid, int64_t N, int64_t K, int32_t bs,
                                 uint16_t *C, int32_t *acc_dump) {
   gemm_core(A, As, W, Ws, sorted, expert_ids, num_tokens_post_pad, topk_w, mul_routed, top_k,
-            num_valid, N, K, bs, C, acc_dump, 1);
+            num_valid, N, K, bs, C, acc_dump, 1, NULL);
 }
 
 /* ------------------------------------------------------------ SiLU*mul -- */
@@ -481,12 +487,12 @@ static int fused_path(
                                     sorted, sorted_cap, expert_ids, expert_ids_cap, ntpp);
   if (rc == 0) {
     gemm_core(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w,
-              apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL, group_n);
+              apply_router_weight_on_input, top_k, S, 2 * I, H, bs, c1, NULL, group_n, NULL);
     if (g_activation == 1) orc_gelu_and_mul(c1, S, I, act);
     else orc_silu_and_mul(c1, S, I, act);
     orc_group_quant_int8(act, S, I, 1e-10f, a2q, a2s);
     gemm_core(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w,
-              !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL, group_n);
+              !apply_router_weight_on_input, 1, S, H, I, bs, c3, NULL, group_n, NULL);
     orc_moe_sum(c3, M, top_k, H, shared_output, routed_scaling_factor, out);
   }
   if (own_a1q) free(a1q);
@@ -529,6 +535,119 @@ int orc_fused_experts_w4a8(
                     expert_map, bs, apply_router_weight_on_input, routed_scaling_factor, shared_output,
                     out, sorted, sorted_cap, expert_ids, expert_ids_cap, ntpp, a1q, a1s, c1, act, a2q, a2s,
                     c3, 1);
+}
+
+/* ------------------------------------------------------------------------- *
+ * The block form with fp32 activations (hidden_states.dtype == torch.float32: compute_type
+ * tl.float32, int8.py:689-696).  Nothing between the stages is rounded to 16 bits:
+ *   quant     the same rule on fp32 inputs (int8_utils.py:74-122 widens to fp32 anyway)
+ *   GEMM      C[f, n] = acc (the fp32 sum itself; with mul_routed acc * topk_w[f])
+ *   SiLU*mul  act = (g / (1 + exp(-g))) * u in fp32 (vLLM's silu_and_mul, called at int8.py:811:
+ *             T(float(x) / (1.0f + expf(float(-x)))) * y with T = float); exp is orc_expf, the
+ *             fixed sequence of IEEE operations used for the 16-bit tables, so the last place of
+ *             the reference's device expf is unpinned
+ *   GELU*mul  act = ((g * 0.5f) * (1 + erf(g * ALPHA))) * u, erf correctly rounded (as above)
+ *   moe_sum   sequential fp32 sum over the k slots, * factor, + bias
+ *             (moe_align_sum_kernels.cu:619-633, :886-909 with T = float)
+ * ------------------------------------------------------------------------- */
+void orc_group_quant_int8_f32(const float *x, int64_t R, int64_t C, float eps, int8_t *q, float *s) {
+  int64_t G = C / ORC_GROUP;
+#pragma omp parallel for schedule(static)
+  for (int64_t g = 0; g < R * G; ++g) {
+    const float *xg = x + g * ORC_GROUP;
+    float amax = 0.0f;
+    for (int i = 0; i < ORC_GROUP; ++i) {
+      float a = fabsf(xg[i]);
+      if (a > amax) amax = a;
+    }
+    if (!(amax > eps)) amax = eps;
+    float sc = amax / 127.0f;
+    s[g] = sc;
+    for (int i = 0; i < ORC_GROUP; ++i) {
+      float v = xg[i] / sc;
+      if (v < -128.0f) v = -128.0f;
+      if (v > 127.0f) v = 127.0f;
+      q[g * ORC_GROUP + i] = (int8_t)(int32_t)v;
+    }
+  }
+}
+
+void orc_moe_gemm_block_int8_f32(const int8_t *A, const float *As, const int8_t *W, const float *Ws,
+                                 const int32_t *sorted, const int32_t *expert_ids,
+                                 const int32_t *num_tokens_post_pad, const float *topk_w, int mul_routed,
+                                 int32_t top_k, int64_t num_valid, int64_t N, int64_t K, int32_t bs, float *C,
+                                 int32_t *acc_dump) {
+  gemm_core(A, As, W, Ws, sorted, expert_ids, num_tokens_post_pad, topk_w, mul_routed, top_k, num_valid, N, K, bs,
+            NULL, acc_dump, ORC_GROUP, C);
+}
+
+float orc_silu_f32(float g) { return g / (1.0f + orc_expf(-g)); }
+
+float orc_gelu_f32(float g) {
+  const float alpha = 0.70710678118654752440f;
+  const float e = (float)erf((double)(g * alpha));
+  return (g * 0.5f) * (1.0f + e);
+}
+
+void orc_act_and_mul_f32(const float *c1, int64_t S, int64_t I, int activation, float *act) {
+#pragma omp parallel for schedule(static)
+  for (int64_t f = 0; f < S; ++f)
+    for (int64_t i = 0; i < I; ++i) {
+      const float g = c1[f * 2 * I + i], u = c1[f * 2 * I + I + i];
+      act[f * I + i] = (activation == 1 ? orc_gelu_f32(g) : orc_silu_f32(g)) * u;
+    }
+}
+
+void orc_moe_sum_f32(const float *in, int64_t M, int32_t k, int64_t H, const float *bias, float factor,
+                     float *out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t t = 0; t < M; ++t)
+    for (int64_t h = 0; h < H; ++h) {
+      float acc = 0.0f;
+      for (int32_t j = 0; j < k; ++j) acc = acc + in[(t * k + j) * H + h];
+      acc = acc * factor;
+      if (bias) acc = acc + bias[t * H + h];
+      out[t * H + h] = acc;
+    }
+}
+
+int orc_fused_experts_block_int8_f32(
+    const float *x, int64_t M, int64_t H, int64_t I, int32_t E_local, int32_t num_experts_global, int32_t top_k,
+    const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s, const float *topk_w,
+    const int32_t *topk_ids, const int32_t *expert_map, int32_t bs, int apply_router_weight_on_input,
+    float routed_scaling_factor, const float *shared_output, float *out, int32_t *sorted, int64_t sorted_cap,
+    int32_t *expert_ids, int64_t expert_ids_cap, int32_t *ntpp, int8_t *a1q, float *a1s, float *c1, float *act,
+    int8_t *a2q, float *a2s, float *c3) {
+  (void)E_local;
+  int64_t S = M * top_k;
+  int own_a1q = !a1q, own_a1s = !a1s, own_c1 = !c1, own_act = !act, own_a2q = !a2q, own_a2s = !a2s, own_c3 = !c3;
+  if (own_a1q) a1q = (int8_t *)malloc((size_t)(M * H));
+  if (own_a1s) a1s = (float *)malloc(sizeof(float) * (size_t)(M * (H / ORC_GROUP)));
+  if (own_c1) c1 = (float *)calloc((size_t)(S * 2 * I), 4);
+  if (own_act) act = (float *)malloc(4 * (size_t)(S * I));
+  if (own_a2q) a2q = (int8_t *)malloc((size_t)(S * I));
+  if (own_a2s) a2s = (float *)malloc(sizeof(float) * (size_t)(S * (I / ORC_GROUP)));
+  if (own_c3) c3 = (float *)calloc((size_t)(S * H), 4);
+  orc_group_quant_int8_f32(x, M, H, 1e-10f, a1q, a1s);
+  int rc = orc_moe_align_block_size(topk_ids, S, num_experts_global, bs, expert_map, 0, sorted, sorted_cap,
+                                    expert_ids, expert_ids_cap, ntpp);
+  if (rc == 0) {
+    gemm_core(a1q, a1s, w1, w1s, sorted, expert_ids, ntpp, topk_w, apply_router_weight_on_input, top_k, S, 2 * I, H,
+              bs, NULL, NULL, ORC_GROUP, c1);
+    orc_act_and_mul_f32(c1, S, I, g_activation, act);
+    orc_group_quant_int8_f32(act, S, I, 1e-10f, a2q, a2s);
+    gemm_core(a2q, a2s, w2, w2s, sorted, expert_ids, ntpp, topk_w, !apply_router_weight_on_input, 1, S, H, I, bs,
+              NULL, NULL, ORC_GROUP, c3);
+    orc_moe_sum_f32(c3, M, top_k, H, shared_output, routed_scaling_factor, out);
+  }
+  if (own_a1q) free(a1q);
+  if (own_a1s) free(a1s);
+  if (own_c1) free(c1);
+  if (own_act) free(act);
+  if (own_a2q) free(a2q);
+  if (own_a2s) free(a2s);
+  if (own_c3) free(c3);
+  return rc;
 }
 
 /* ------------------------------------------------------------------------- *

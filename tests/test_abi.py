@@ -192,7 +192,8 @@ def test_validation_happens_before_any_launch(lib):
     assert lib.lo_moe_align_block_size(p, 0, 8, 8, 16, null, 0, p, 10, p, 8, p, null) == -2      # buffer too small
     assert b"sorted_ids holds 10" in lib.lo_last_error()
     assert lib.lo_per_token_group_quant_int8(p, 0, 1, 100, 1e-10, p, p, null) == -1              # cols % 128
-    assert lib.lo_per_token_group_quant_int8(p, 2, 1, 128, 1e-10, p, p, null) == -4              # fp32 rows are not built
+    assert lib.lo_per_token_group_quant_int8(p, 3, 1, 128, 1e-10, p, p, null) == -4              # no such element type
+    assert lib.lo_per_token_quant_int8(p, 2, 1, 128, p, p, null) == -4                           # per-channel form: no fp32 rows
     assert lib.lo_moe_sum(p, p, null, null, 0, 1, 8, 100, 1.0, null, null) == -1                       # H % 8
     assert lib.lo_preshuffle_weight_int8(p, p, 1, 16, 128, null) == -1                           # src == dst
 

@@ -196,14 +196,14 @@ def test_float16_qwen3_layer_sampled_tokens(dev, oracle):
     assert torch.equal(out[tokens].cpu().view(torch.int16), ref.view(torch.int16))
 
 
-def test_float32_rows_still_raise(dev):
+def test_float32_rows_with_per_channel_scales_raise(dev):
     from lightop_amd import workloads as wl
     from lightop_amd.moe import fused_experts_impl_int8
 
-    layer = wl.TINY
+    layer = wl.TINY_PC
     w1, w2, w1s, w2s = (t.to(dev) for t in wl.make_weights(layer, seed=0))
     x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, 4, seed=0))
     cache13 = torch.empty(4 * 2 * 1024, dtype=torch.float32, device=dev)
     with pytest.raises(NotImplementedError):
-        fused_experts_impl_int8(x.float(), w1, w2, tw, ids, cache13, use_int8_w8a8=True, w1_scale=w1s, w2_scale=w2s,
-                                block_shape=[128, 128])
+        fused_experts_impl_int8(x.float(), w1, w2, tw, ids, cache13, use_int8_w8a8=True, per_channel_quant=True,
+                                w1_scale=w1s, w2_scale=w2s, block_shape=None)

@@ -16,6 +16,8 @@ Pinning status per oracle function
                               pinned by closed-form cases and the torch restatement.
   orc_expf / orc_silu_and_mul pinned against libm expf over all 65536 bf16 inputs.
   orc_moe_sum                 pinned: k=1 identity, torch.sum, hand-worked roundings.
+  orc_*_f32 (fp32 rows)       pinned: hand-worked quantisation and reduce cases, the bf16
+                              functions' results after one rounding, float64 torch.
   orc_fused_experts_block_int8 pinned against the torch restatement within the path's
                               tolerance (the reference holds no end-to-end assertion
                               for the block-INT8 path).
@@ -488,3 +490,140 @@ def test_fused_path_expert_parallel_share(oracle):
     assert (r["expert_ids"][: r["num_tokens_post_pad"].item() // 16] >= -1).all()
     nonlocal_slots = emap.long()[ids.reshape(-1).long()] < 0
     assert (r["c3"][nonlocal_slots] == 0).all()
+
+
+# ------------------------------------------------------- fp32 activations ----
+# (hidden_states.dtype == torch.float32: compute_type tl.float32, int8.py:689-696)
+
+def test_float_rows_quant_and_gemm_pins(oracle):
+    """fp32 quantisation: hand-worked truncations, and on bf16-representable rows the result of the bf16
+    rule.  fp32 GEMM output: the sum itself - rounded to bf16 it is the (pinned) bf16 output, with and without
+    the router weight, zero rows for experts of other ranks included."""
+    row = [127.0, 1.5, -1.5, 2.5, -2.5, 0.75, -0.75, 126.5] + [0.0] * 120
+    q, s = oracle.per_token_group_quant_int8(torch.tensor([row]))
+    assert s.item() == 1.0 and q[0, :8].tolist() == [127, 1, -1, 2, -2, 0, 0, 126]
+    q, s = oracle.per_token_group_quant_int8(torch.zeros(1, 128))
+    assert s.item() == np.float32(1e-10) / np.float32(127) and not q.any()
+    g = torch.Generator().manual_seed(3)
+    x16 = (torch.randn(9, 512, generator=g) * 4).to(torch.bfloat16)
+    q16, s16 = oracle.per_token_group_quant_int8(x16)
+    q32, s32 = oracle.per_token_group_quant_int8(x16.float())
+    assert torch.equal(q16, q32) and torch.equal(s16, s32)
+    # a value that is not bf16-representable decides the scale
+    x = x16.float()
+    x[0, 5] = 1000.0625
+    q, s = oracle.per_token_group_quant_int8(x)
+    assert s[0, 0].item() == np.float32(1000.0625) / np.float32(127) and q[0, 5] == 127
+    M, k, E, Eg, N, K = 23, 2, 3, 5, 192, 256
+    Aq = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    W = torch.randint(-127, 128, (E, N, K), generator=g, dtype=torch.int8)
+    As = torch.rand(M, K // 128, generator=g) * 0.05 + 0.005
+    Ws = torch.exp(torch.randn(E, 2, K // 128, generator=g) * 0.3 + math.log(1e-3))
+    ids = torch.stack([torch.randperm(Eg, generator=g)[:k] for _ in range(M)]).to(torch.int32)
+    tw = torch.rand(M, k, generator=g) + 0.1
+    emap = torch.full((Eg,), -1, dtype=torch.int32)
+    emap[:E] = torch.arange(E, dtype=torch.int32)
+    s_, e_, p_ = oracle.moe_align_block_size(ids, 16, Eg, expert_map=emap)
+    for mul in (False, True):
+        c32 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s_, e_, p_, tw, mul, k, M * k, 16,
+                                         out=torch.full((M * k, N), 9.0))
+        c16 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s_, e_, p_, tw, mul, k, M * k, 16)
+        assert torch.equal(c32.to(torch.bfloat16).view(torch.int16), c16.view(torch.int16))
+        assert not torch.equal(c32, c16.float())  # ... and it is not the rounded value
+        local = emap.long()[ids.reshape(-1).long()] >= 0
+        assert (c32[~local] == 0).all() and (c32[local].abs().sum(1) > 0).all()
+
+
+def test_float_rows_activations_pins(oracle):
+    """fp32 SiLU / GELU: rounded to bf16 they are the (pinned) bf16 tables on every finite bf16 gate; against
+    float64 torch within two fp32 ulps (GELU of negative gates, where 1 + erf cancels: plus the rounding of
+    erf); the product with the up value is one fp32 multiplication."""
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = pats.float().isfinite()
+    gates = pats[finite].float()
+    ones = torch.ones_like(gates)
+    for name, fn, table in (("silu", oracle.silu_and_mul, oracle.activation_table("silu")),
+                            ("gelu", oracle.gelu_and_mul, oracle.activation_table("gelu"))):
+        act = fn(torch.stack([gates, ones], dim=1).reshape(-1, 2).contiguous()).reshape(-1)
+        assert act.dtype == torch.float32
+        assert torch.equal(act.to(torch.bfloat16).view(torch.int16), table[finite]), name
+        g64 = gates.double()
+        ref = g64 / (1 + torch.exp(-g64)) if name == "silu" else torch.nn.functional.gelu(g64)
+        ulp = torch.maximum(ref.abs().float(), torch.tensor(1.2e-38)) * 2.0 ** -23
+        err = (act.double() - ref).abs()
+        if name == "gelu":  # negative gates: 1 + erf cancels, the rounding of erf (2^-24) stays, times |g| / 2
+            slack = torch.where(gates < 0, gates.abs().double() / 2 * 2.0 ** -23, torch.zeros(()).double())
+            assert (err <= 2 * ulp.double() + slack).all(), name
+        else:  # below -87 the fixed-sequence exp saturates: silu is then -0 or a denormal
+            keep = gates > -87.0
+            assert (err[keep] <= 2 * ulp[keep].double()).all(), name
+    g = torch.Generator().manual_seed(5)
+    c1 = torch.randn(7, 2 * 64, generator=g) * 3
+    for name, fn in (("silu", oracle.silu_and_mul), ("gelu", oracle.gelu_and_mul)):
+        one = fn(torch.cat([c1[:, :64], torch.ones(7, 64)], dim=1).contiguous())
+        assert torch.equal(fn(c1), torch.from_numpy(one.numpy() * c1[:, 64:].numpy()))
+    assert oracle.silu_and_mul(torch.tensor([[0.0, 5.0]])).item() == 0.0
+    assert oracle.silu_and_mul(torch.tensor([[100.0, 1.0]])).item() == 100.0
+    assert oracle.gelu_and_mul(torch.tensor([[100.0, 0.5]])).item() == 50.0
+    assert oracle.gelu_and_mul(torch.tensor([[-100.0, 1.0]])).item() == 0.0
+
+
+def test_float_rows_moe_sum_pins(oracle):
+    """Sequential fp32 sum in slot order, then the factor, then the bias: a hand-worked case that every other
+    order gets wrong."""
+    x = torch.tensor([[[1e8], [1.0], [-1e8], [1.0]]])          # ((1e8 + 1) - 1e8) + 1 = 1 in fp32; pairwise: 2
+    assert oracle.moe_sum(x).item() == 1.0
+    assert oracle.moe_sum(x, factor=2.5).item() == 2.5
+    assert oracle.moe_sum(x, bias=torch.tensor([[0.25]]), factor=2.5).item() == 2.75    # (sum * factor) + bias
+    big = torch.tensor([[[3.0], [1e-8]]])
+    assert oracle.moe_sum(big, bias=torch.tensor([[1e8]]), factor=1.0).item() == np.float32(1e8) + np.float32(3.0)
+    g = torch.Generator().manual_seed(2)
+    y = torch.randn(5, 6, 40, generator=g)
+    b = torch.randn(5, 40, generator=g)
+    acc = np.zeros((5, 40), dtype=np.float32)
+    for j in range(6):
+        acc = acc + y[:, j].numpy()
+    assert torch.equal(oracle.moe_sum(y, b, 1.5), torch.from_numpy(acc * np.float32(1.5) + b.numpy()))
+
+
+@pytest.mark.parametrize("activation", ["silu", "gelu"])
+def test_float_rows_whole_path(oracle, activation):
+    """The fp32 chain is the composition of its (pinned) stages, differs from the bf16 chain by roundings
+    only, and agrees with a float64 restatement on dequantised weights within the path's tolerance."""
+    from lightop_amd import workloads as wl
+
+    layer = wl.TINY
+    w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
+    M = 12
+    x, tw, ids = wl.make_inputs(layer, M, seed=2)
+    x32 = x.float() * 1.37
+    r = oracle.fused_experts_block_int8(x32, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True,
+                                        activation=activation)
+    out = r["out"]
+    assert out.dtype == torch.float32 and r["c1"].dtype == torch.float32
+    a1q, a1s = oracle.per_token_group_quant_int8(x32)
+    assert torch.equal(r["a1q"], a1q) and torch.equal(r["a1s"], a1s)
+    act = (oracle.silu_and_mul if activation == "silu" else oracle.gelu_and_mul)(r["c1"])
+    assert torch.equal(r["act"], act)
+    a2q, a2s = oracle.per_token_group_quant_int8(act)
+    assert torch.equal(r["a2q"], a2q) and torch.equal(r["a2s"], a2s)
+    assert torch.equal(out, oracle.moe_sum(r["c3"].view(M, layer.top_k, layer.H)))
+    W1 = w1.double() * w1s.double().repeat_interleave(128, 1).repeat_interleave(128, 2)
+    W2 = w2.double() * w2s.double().repeat_interleave(128, 1).repeat_interleave(128, 2)
+    a1 = a1q.double() * a1s.double().repeat_interleave(128, dim=1)
+    ref = torch.zeros(M, layer.H, dtype=torch.float64)
+    for t in range(M):
+        for j in range(layer.top_k):
+            e = int(ids[t, j])
+            c1 = W1[e] @ a1[t]
+            gate, up = c1[: layer.I], c1[layer.I:]
+            a = (gate / (1 + torch.exp(-gate)) if activation == "silu" else torch.nn.functional.gelu(gate)) * up
+            q, s = oracle.per_token_group_quant_int8(a.float().reshape(1, -1))
+            ref[t] += float(tw[t, j]) * (W2[e] @ (q.double() * s.double().repeat_interleave(128, dim=1))[0])
+    err = (out.double() - ref).abs()
+    assert ref.abs().max() > 0.05
+    assert err.max() <= 1e-2 * ref.abs().max() and err.sum() <= 2e-3 * ref.abs().sum()
+    out16 = oracle.fused_experts_block_int8(x32.to(torch.bfloat16), w1, w2, w1s, w2s, tw, ids, 16,
+                                            activation=activation)
+    d = (out - out16.float()).abs()
+    assert 0 < d.max() <= 3e-2 * out.abs().max()
