@@ -123,6 +123,25 @@ def test_whole_path_tiny_bit_exact(dev, oracle, bs, with_map):
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
+@pytest.mark.parametrize("bs", [16, 32, 64, 128])
+def test_whole_path_long_k_bit_exact(dev, oracle, bs):
+    """K = 4608 and 5120: more than 32 K groups, so the copy of the row scales into LDS takes a second pass
+    (streaming kernel and 64-token kernel), and both K-block parities end the loop."""
+    from lightop_amd import _lib, workloads as wl
+    from lightop_amd.moe import preshuffle_moe_weight_int4
+
+    for H, I in ((4608, 256), (256, 5120), (7168, 128)):  # 7168: more than 48 KB of scales in LDS
+        layer = wl.MoeLayer("w4-long-k", E=2, E_global=2, top_k=2, H=H, I=I, routing="softmax", weight_bits=4)
+        say(f"w4a8 whole path H={H} I={I} bs={bs}")
+        w1, w2, w1s, w2s = wl.make_weights(layer, seed=H)
+        x, tw, ids = wl.make_inputs(layer, 40, seed=H)
+        wd = (preshuffle_moe_weight_int4(w1.to(dev)), preshuffle_moe_weight_int4(w2.to(dev)), w1s.to(dev), w2s.to(dev))
+        out = run_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None, dev, bs,
+                       _lib.LO_GEMM_CANONICAL_ORDER | _lib.LO_FUSED_NO_DECODE_PATH)
+        ref = oracle.fused_experts_w4a8(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=layer.E)
+        assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
 @pytest.mark.parametrize("M", [1, 5, 40, 200])
 @pytest.mark.parametrize("with_map", [False, True])
 def test_two_launch_path_w4a8_bit_exact(dev, oracle, M, with_map):
