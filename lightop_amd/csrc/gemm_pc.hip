@@ -27,6 +27,7 @@ constexpr int kPcRow = 144; // LDS row pitch in bytes: 128 + 16 keeps ds_read_b1
 
 template <bool SHUF, int TB, bool STREAM>
 __device__ __forceinline__ void moe_gemm_pc_body(const GemmArgs &a, int m_blocks, int group_m) {
+  static_assert(!STREAM || SHUF, "streaming policy: pre-shuffled weights only");
   constexpr int kWAux = STREAM ? kCacheStream : kCacheDefault;
   constexpr int kTileM = 32 * TB;       // tokens per workgroup
   constexpr int kThrPerTok = 256 / kTileM; // threads that gather one token row
@@ -231,17 +232,16 @@ int launch_gemm_pc(const GemmArgs &a0, int block_size_m, int64_t m_blocks, hipSt
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
   // one token block per expert, by and large: up to 48 slots per expert on average with 64-token blocks
   // (as measured for the block form's 64-token kernel), half a block with 128-token blocks
-  const bool stream = a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) *
+  // (pre-shuffled weights only: a 128-byte line of row-major weights serves several k-steps of a lane,
+  // and the hint would have it fetched again for each)
+  const bool stream = a.w_shuffled &&
+                      a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) *
                                          (block_size_m == 64 ? 48 : 64);
 #define LO_PC_LAUNCH(KERN)                                                                    \
   do {                                                                                        \
-    if (a.w_shuffled) {                                                                       \
-      if (stream) hipLaunchKernelGGL((KERN<true, true>), g, b, 0, s, a, mbi, gi);             \
-      else hipLaunchKernelGGL((KERN<true, false>), g, b, 0, s, a, mbi, gi);                   \
-    } else {                                                                                  \
-      if (stream) hipLaunchKernelGGL((KERN<false, true>), g, b, 0, s, a, mbi, gi);            \
-      else hipLaunchKernelGGL((KERN<false, false>), g, b, 0, s, a, mbi, gi);                  \
-    }                                                                                         \
+    if (stream) hipLaunchKernelGGL((KERN<true, true>), g, b, 0, s, a, mbi, gi);               \
+    else if (a.w_shuffled) hipLaunchKernelGGL((KERN<true, false>), g, b, 0, s, a, mbi, gi);   \
+    else hipLaunchKernelGGL((KERN<false, false>), g, b, 0, s, a, mbi, gi);                    \
   } while (0)
   if (block_size_m == 128) LO_PC_LAUNCH(moe_gemm_pc_kernel_128);
   else LO_PC_LAUNCH(moe_gemm_pc_kernel_64);
