@@ -158,6 +158,7 @@ class Point:
         if bs == 0:
             shape = None if L.quant == "channel" else ([1, 128] if L.weight_bits == 4 else [128, 128])
             bs = moe.get_w8a8moe_json(self.M, L.E, 2 * L.I, L.H, L.I, True, shape, L.top_k, L.E_global,
+                                      preshuffled=bool(getattr(self.w1, "lo_preshuffled", False)),
                                       int4=L.weight_bits == 4)[0]["BLOCK_SIZE_M"]
         cfg = {"BLOCK_SIZE_M": bs}
         S = self.M * L.top_k
