@@ -283,7 +283,7 @@ def test_channel_path_rejects_mixed_arguments(dev):
                                 block_shape=None)
 
 
-@pytest.mark.parametrize("M", [1, 32, 512, 8192])
+@pytest.mark.parametrize("M", [1, 32, 512, 2048, 8192])
 def test_qwen3_channel_layer_sampled_tokens(dev, oracle, M):
     """A token's output depends on that token only: a sample of tokens goes through the oracle with
     just the experts it uses."""
