@@ -5,8 +5,10 @@
                     [--sweep {default,none,full}] [--no-cpu-baseline]
 
 A step is one call of ``fused_experts_impl_int8`` on one batch of synthetic tokens with
-every input already resident in HBM.  Between steps a 512 MiB buffer is overwritten so
-that weights are streamed from HBM and not served from the 256 MB Infinity Cache; the
+every input already resident in HBM.  Between steps a 512 MiB buffer is read through so
+that weights are streamed from HBM and not served from the 256 MB Infinity Cache (read, not
+overwritten: an overwrite leaves the cache full of dirty lines whose write-back takes place
+inside the timed step - 5 to 25 us of it, `--flush write` shows the difference); the
 step time is taken with HIP events on the launching stream and excludes that flush.
 ms_per_step is the median of the timed steps (mean and min are reported next to it).  The
 headline is timed in the library's default arithmetic (canonical scale order, the mode the GPU
@@ -66,6 +68,8 @@ def parse_args():
     p.add_argument("--tokens", type=int, default=8192)
     p.add_argument("--sweep", default="default", choices=["default", "none", "full"])
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--flush", default="read", choices=["read", "write"],
+                   help="how the Infinity Cache is evicted between steps: by reading 512 MiB or by overwriting them")
     p.add_argument("--block-size-m", type=int, default=0)
     p.add_argument("--row-major-weights", action="store_true",
                    help="keep w1/w2 row-major instead of the load-time pre-shuffled layout")
@@ -76,15 +80,19 @@ def parse_args():
 
 
 class Flusher:
-    """Evicts the Infinity Cache between steps by overwriting 512 MiB."""
+    """Evicts the Infinity Cache between steps: a max-reduction reads 512 MiB ("write": a fill overwrites them)."""
 
-    def __init__(self, dev):
-        self.buf = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.int32, device=dev)
+    def __init__(self, dev, mode="read"):
+        self.buf = torch.zeros(512 * 1024 * 1024 // 4, dtype=torch.int32, device=dev)
         self.i = 0
+        self.mode = mode
 
     def __call__(self):
         self.i += 1
-        self.buf.fill_(self.i)
+        if self.mode == "read":
+            self.buf.max()
+        else:
+            self.buf.fill_(self.i)
 
 
 def time_steps(fn, steps, warmup, flush):
@@ -447,7 +455,7 @@ def main():
     _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    flush = Flusher(dev)
+    flush = Flusher(dev, args.flush)
     flags_default = _lib.LO_GEMM_FUSED_SCALE if args.fused_scale == 1 else 0
     flags_other = 0 if args.fused_scale == 1 else _lib.LO_GEMM_FUSED_SCALE
 
@@ -562,7 +570,8 @@ def main():
                                   "per-channel INT8" if L.quant == "channel" else "block-INT8[128,128]")
                                + f", M={args.tokens}",
                    "tokens": args.tokens, "block_size_m": bs_used, "routing": L.routing,
-                   "gemm1_kernel": tile1["kernel_name"], "gemm2_kernel": tile2["kernel_name"]},
+                   "gemm1_kernel": tile1["kernel_name"], "gemm2_kernel": tile2["kernel_name"],
+                   "cache_flush": f"512 MiB {args.flush} between steps, outside the timed region"},
         "int8_tops": head["int8_tops"], "hbm_gbs": head["hbm_gbs"], "frac_hbm": head["frac_hbm"],
         "frac_mfma": head["frac_mfma"], "stage_ms": {k: round(v, 4) for k, v in stages.items()},
         "roofline": roofline, "cpu_baseline": cpu, "routers": router_times(layer, args.tokens, dev, 50, 5),
