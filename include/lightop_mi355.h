@@ -485,6 +485,25 @@ int lo_fused_experts_channel_int8(const void *x, int dtype, int64_t M, int64_t H
                                   void *cache13, void *out, void *workspace, int64_t workspace_bytes,
                                   int32_t block_size_m, int flags, lo_stream_t stream);
 
+/*
+ * The same with the activations already quantised per token by the caller: the i_q / i_s arguments of
+ * fused_experts_impl_int8 (int8.py:652-653), which moe_kernel_prepare_input takes in place of
+ * per_token_quant_int8(hidden_states) when LMSLIM_USE_FUSED_RMS_QUANT is set (int8.py:291-293; the
+ * producer is the fused RMS-norm + quant upstream of the layer).
+ *   x_q [M, H] int8, x_s [M] f32: neither is written; the quantisation launch is left out.
+ *   dtype: the type of cache13, shared_output and out (LO_BF16 / LO_F16).
+ * Everything else as lo_fused_experts_channel_int8.
+ */
+int lo_fused_experts_channel_int8_prequant(const int8_t *x_q, const float *x_s, int dtype, int64_t M, int64_t H,
+                                           int64_t I, int32_t E, int32_t num_experts, int32_t top_k,
+                                           const int8_t *w1, const float *w1s, const int8_t *w2,
+                                           const float *w2s, const float *topk_w, const void *topk_ids,
+                                           int ids_dtype, const int32_t *expert_map,
+                                           int apply_router_weight_on_input, float routed_scaling_factor,
+                                           const void *shared_output, void *cache13, void *out, void *workspace,
+                                           int64_t workspace_bytes, int32_t block_size_m, int flags,
+                                           lo_stream_t stream);
+
 /* ---- routers upstream of the path (they produce topk_ids / topk_weights) ---------- */
 
 /*

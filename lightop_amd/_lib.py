@@ -86,6 +86,11 @@ SIGNATURES = {
                                               c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                               c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,
                                               c_void_p, c_void_p, c_int64, c_int32, c_int, c_void_p]),
+    "lo_fused_experts_channel_int8_prequant": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int32,
+                                                       c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                       c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p,
+                                                       c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int,
+                                                       c_void_p]),
     "lo_fused_experts_block_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int32, c_int32,
                                             c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p,

@@ -367,15 +367,17 @@ extern "C" int lo_fused_experts_block_int8(
 // block_shape=None): per-token quant -> align -> moe_gemm_w8a8 -> fuse_silu_mul_quant ->
 // moe_gemm_w8a8 (routed weight in its epilogue) -> moe_sum.  cache13 holds the first GEMM's
 // output [S, 2I] and then the second's [S, H], as in the reference (int8.py:681-682).
-extern "C" int lo_fused_experts_channel_int8(
-    const void *x, int dtype, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts,
-    int32_t top_k, const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s,
+// x_q / x_s: the activations already quantised per token by the caller (the i_q / i_s of int8.py:291-293,
+// LMSLIM_USE_FUSED_RMS_QUANT); then x is not read and the quantisation launch is left out.
+static int fused_experts_channel(
+    const void *x, const int8_t *x_q, const float *x_s, int dtype, int64_t M, int64_t H, int64_t I, int32_t E,
+    int32_t num_experts, int32_t top_k, const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s,
     const float *topk_w, const void *topk_ids, int ids_dtype, const int32_t *expert_map,
     int apply_router_weight_on_input, float routed_scaling_factor, const void *shared_output,
     void *cache13, void *out, void *workspace, int64_t workspace_bytes, int32_t block_size_m,
     int flags, lo_stream_t stream) {
   using namespace lo;
-  LO_REQUIRE(x && w1 && w1s && w2 && w2s && topk_w && topk_ids && cache13 && out && workspace,
+  LO_REQUIRE((x || (x_q && x_s)) && w1 && w1s && w2 && w2s && topk_w && topk_ids && cache13 && out && workspace,
              LO_EINVAL, "fused_experts(channel): null pointer");
   LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16, LO_ENOTSUP, "fused_experts(channel): activations are bf16 or fp16");
   LO_REQUIRE(M >= 0 && H >= kGroup && H % kGroup == 0 && I >= kGroup && I % kGroup == 0, LO_EINVAL,
@@ -405,8 +407,8 @@ extern "C" int lo_fused_experts_channel_int8(
              "fused_experts(channel): workspace holds %lld bytes, needs %lld", (long long)workspace_bytes,
              (long long)L.total);
   char *ws = static_cast<char *>(workspace);
-  int8_t *a1q = reinterpret_cast<int8_t *>(ws + L.off[0]);
-  float *a1s = reinterpret_cast<float *>(ws + L.off[1]);
+  const int8_t *a1q = x_q ? x_q : reinterpret_cast<int8_t *>(ws + L.off[0]);
+  const float *a1s = x_q ? x_s : reinterpret_cast<float *>(ws + L.off[1]);
   int32_t *sorted = reinterpret_cast<int32_t *>(ws + L.off[2]);
   int32_t *eids = reinterpret_cast<int32_t *>(ws + L.off[3]);
   int32_t *ntpp = reinterpret_cast<int32_t *>(ws + L.off[4]);
@@ -415,7 +417,10 @@ extern "C" int lo_fused_experts_channel_int8(
   uint8_t *mask = expert_map ? reinterpret_cast<uint8_t *>(ws + L.off[7]) : nullptr;
   const int64_t S = M * top_k;
 
-  int rc = lo_per_token_quant_int8(x, dtype, M, H, a1q, a1s, stream);
+  int rc = LO_OK;
+  if (!x_q)
+    rc = lo_per_token_quant_int8(x, dtype, M, H, reinterpret_cast<int8_t *>(ws + L.off[0]),
+                                 reinterpret_cast<float *>(ws + L.off[1]), stream);
   if (rc) return rc;
   rc = lo_moe_align_block_size_ws(topk_ids, ids_dtype, S, num_experts, block_size_m, expert_map, 0,
                                   sorted, L.sorted_cap, eids, L.blocks_cap, ntpp, mask, ws + L.off[8],
@@ -438,6 +443,32 @@ extern "C" int lo_fused_experts_channel_int8(
   if (rc) return rc;
   return lo_moe_sum(cache13, out, shared_output, mask, dtype, M, top_k, H, routed_scaling_factor, nullptr,
                     stream);
+}
+
+extern "C" int lo_fused_experts_channel_int8(
+    const void *x, int dtype, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts,
+    int32_t top_k, const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s,
+    const float *topk_w, const void *topk_ids, int ids_dtype, const int32_t *expert_map,
+    int apply_router_weight_on_input, float routed_scaling_factor, const void *shared_output,
+    void *cache13, void *out, void *workspace, int64_t workspace_bytes, int32_t block_size_m,
+    int flags, lo_stream_t stream) {
+  LO_REQUIRE(x, LO_EINVAL, "fused_experts(channel): null pointer");
+  return fused_experts_channel(x, nullptr, nullptr, dtype, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w,
+                               topk_ids, ids_dtype, expert_map, apply_router_weight_on_input, routed_scaling_factor,
+                               shared_output, cache13, out, workspace, workspace_bytes, block_size_m, flags, stream);
+}
+
+extern "C" int lo_fused_experts_channel_int8_prequant(
+    const int8_t *x_q, const float *x_s, int dtype, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts,
+    int32_t top_k, const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s,
+    const float *topk_w, const void *topk_ids, int ids_dtype, const int32_t *expert_map,
+    int apply_router_weight_on_input, float routed_scaling_factor, const void *shared_output,
+    void *cache13, void *out, void *workspace, int64_t workspace_bytes, int32_t block_size_m,
+    int flags, lo_stream_t stream) {
+  LO_REQUIRE(x_q && x_s, LO_EINVAL, "fused_experts(channel, quantised input): null pointer");
+  return fused_experts_channel(nullptr, x_q, x_s, dtype, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w,
+                               topk_ids, ids_dtype, expert_map, apply_router_weight_on_input, routed_scaling_factor,
+                               shared_output, cache13, out, workspace, workspace_bytes, block_size_m, flags, stream);
 }
 
 // ---- whole path for callers that cannot allocate -------------------------------------------

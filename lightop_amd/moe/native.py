@@ -413,7 +413,16 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     if hidden_states.dtype == torch.float32 and channel:
         raise NotImplementedError("lightop_amd: per-channel scales take bfloat16 or float16 hidden_states")
     assert w1_scale is not None and w2_scale is not None
-    del w1_zp, w2_zp, a1_scale, a2_scale, use_nn_moe, i_q, i_s
+    del w1_zp, w2_zp, a1_scale, a2_scale, use_nn_moe
+    # int8.py:291-293: the per-channel form takes the caller's own per-token quantisation of the input
+    # (the fused RMS-norm + quant upstream) when the flag is set; the block form never does (:297-301).
+    prequant = None
+    if channel and envs.LMSLIM_USE_FUSED_RMS_QUANT and i_q is not None and i_s is not None:
+        assert i_q.dtype == torch.int8 and i_q.is_contiguous() and i_q.shape == hidden_states.shape
+        assert i_s.numel() == hidden_states.shape[0]
+        prequant = (i_q, i_s if i_s.dtype == torch.float32 and i_s.is_contiguous()
+                    else i_s.to(torch.float32).contiguous())
+        _require_cuda(*prequant)
     _require_cuda(hidden_states, w1, w2, topk_weights, topk_ids, cache13, w1_scale, w2_scale,
                   expert_map, shared_output)
 
@@ -443,7 +452,7 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
                               apply_router_weight_on_input, global_num_experts, expert_map, w1_scale, w2_scale,
                               routed_scaling_factor, shared_output, I, flags,
                               int(extra.get("lightop_amd_block_size_m", 0)), channel=channel,
-                              workspace=extra.get("lightop_amd_workspace"))
+                              workspace=extra.get("lightop_amd_workspace"), prequant=prequant)
 
 
 def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
@@ -551,7 +560,7 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
 
 def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace, apply_router_weight_on_input,
                        global_num_experts, expert_map, w1_scale, w2_scale, routed_scaling_factor, shared_output,
-                       I, flags, block_size_m, channel=False, workspace=None):
+                       I, flags, block_size_m, channel=False, workspace=None, prequant=None):
     """Chunk loop shared by the block-INT8, per-channel and W4A8 entry points (int8.py:703-888)."""
     num_tokens, H = hidden_states.shape
     E = w1.shape[0]
@@ -598,9 +607,14 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
             if m <= 0:
                 break
             x = hidden_states[begin:end]
-            entry = lib.lo_fused_experts_channel_int8 if channel else lib.lo_fused_experts_block_int8
+            if prequant is not None:  # the chunk's rows of the caller's quantised input
+                entry = lib.lo_fused_experts_channel_int8_prequant
+                head = (_lib.ptr(prequant[0][begin:end]), _lib.ptr(prequant[1].reshape(-1)[begin:end]))
+            else:
+                entry = lib.lo_fused_experts_channel_int8 if channel else lib.lo_fused_experts_block_int8
+                head = (_lib.ptr(x),)
             _lib.check(entry(
-                _lib.ptr(x), _act_dtype(x), m, H, I, E, global_num_experts, top_k_num,
+                *head, _act_dtype(x), m, H, I, E, global_num_experts, top_k_num,
                 _lib.ptr(w1), _lib.ptr(w1_scale), _lib.ptr(w2), _lib.ptr(w2_scale),
                 _lib.ptr(topk_weights[begin:end]), _lib.ptr(topk_ids[begin:end]), _ids_dtype(topk_ids),
                 _lib.ptr(expert_map), 1 if apply_router_weight_on_input else 0,

@@ -267,6 +267,86 @@ def test_whole_path_in_chunks(dev, oracle, monkeypatch):
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
+def _staged_reference(oracle, layer, i_q, i_s, w, tw, ids, bs, emap=None, shared=None, factor=1.0):
+    """The per-channel path from its stages on the CPU, starting from a given quantised input."""
+    w1, w2, w1s, w2s = w
+    M, k = ids.shape
+    S = M * k
+    srt, eids, ntpp = oracle.moe_align_block_size(ids, bs, layer.E_global, expert_map=emap)
+    c1 = oracle.moe_gemm_w8a8(i_q, i_s, w1, w1s, srt, eids, ntpp, None, False, k, S, bs)
+    a2q, a2s = oracle.fuse_silu_mul_quant(c1)
+    c3 = oracle.moe_gemm_w8a8(a2q, a2s, w2, w2s, srt, eids, ntpp, tw, True, 1, S, bs)
+    return oracle.moe_sum(c3.view(M, k, layer.H), shared, factor)
+
+
+@pytest.mark.parametrize("bs", [0, 16, 64, 128])
+@pytest.mark.parametrize("chunk", [None, 48])
+def test_caller_quantised_input(dev, oracle, monkeypatch, bs, chunk):
+    """i_q / i_s with LMSLIM_USE_FUSED_RMS_QUANT (int8.py:291-293): the path starts from the caller's int8 rows
+    and per-token scales - here unrelated to hidden_states, which must not be read - and without the flag,
+    or in the block form, they are ignored."""
+    from lightop_amd import workloads as wl
+    from lightop_amd.moe import fused_experts_impl_int8
+
+    say(f"channel whole path from i_q / i_s, bs={bs} chunk={chunk}")
+    layer = wl.TINY_PC
+    w = wl.make_weights(layer, seed=0)
+    wd = tuple(t.to(dev) for t in w)
+    M = 100
+    x, tw, ids = wl.make_inputs(layer, M, seed=8)
+    g = torch.Generator().manual_seed(5)
+    i_q = torch.randint(-127, 128, (M, layer.H), generator=g, dtype=torch.int8)
+    i_s = (torch.rand(M, 1, generator=g) * 0.04 + 0.005).to(torch.float32)
+    shared = (torch.randn(M, layer.H, generator=g) * 0.1).to(torch.bfloat16)
+    ref = _staged_reference(oracle, layer, i_q, i_s, w, tw, ids, bs or 16, shared=shared, factor=2.0)
+    assert ref.float().abs().max() > 0.05
+    plain = oracle.fused_experts_channel_int8(x, *w, tw, ids, 16, shared_output=shared, routed_scaling_factor=2.0)
+    assert not torch.equal(plain, ref)
+    kw = dict(shared_output=shared.to(dev), routed_scaling_factor=2.0, i_q=i_q.to(dev), i_s=i_s.to(dev))
+    if chunk:
+        monkeypatch.setenv("LMSLIM_FUSED_MOE_CHUNK_SIZE", str(chunk))
+    # without the flag the arguments are ignored
+    monkeypatch.delenv("LMSLIM_USE_FUSED_RMS_QUANT", raising=False)
+    monkeypatch.delenv("USE_FUSED_RMS_QUANT", raising=False)
+    out = run_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None, dev, bs, **kw)
+    assert torch.equal(out.cpu().view(torch.int16), plain.view(torch.int16))
+    monkeypatch.setenv("LMSLIM_USE_FUSED_RMS_QUANT", "1")
+    poison = torch.full_like(x, float("nan")).to(dev)  # any read of hidden_states would show
+    out = run_path(layer, wd, poison, tw.to(dev), ids.to(dev), None, dev, bs, **kw)
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+    # the block form quantises hidden_states itself whatever the flag says (int8.py:297-301)
+    lb = wl.TINY
+    wb = wl.make_weights(lb, seed=0)
+    xb, twb, idsb = wl.make_inputs(lb, M, seed=8)
+    cache13 = torch.empty(M * lb.top_k * max(2 * lb.I, lb.H), dtype=torch.bfloat16, device=dev)
+    outb = fused_experts_impl_int8(xb.to(dev), wb[0].to(dev), wb[1].to(dev), twb.to(dev), idsb.to(dev), cache13,
+                                   use_int8_w8a8=True, w1_scale=wb[2].to(dev), w2_scale=wb[3].to(dev),
+                                   block_shape=[128, 128], i_q=i_q.to(dev), i_s=i_s.to(dev))
+    torch.cuda.synchronize()
+    refb = oracle.fused_experts_block_int8(xb, *wb, twb, idsb, 16)
+    assert torch.equal(outb.cpu().view(torch.int16), refb.view(torch.int16))
+
+
+def test_caller_quantised_input_on_an_expert_parallel_share(dev, oracle, monkeypatch):
+    from lightop_amd import workloads as wl
+
+    say("channel whole path from i_q / i_s, expert-parallel share")
+    monkeypatch.setenv("LMSLIM_USE_FUSED_RMS_QUANT", "1")
+    layer = wl.MoeLayer("ep-pc-q", E=4, E_global=32, top_k=8, H=512, I=256, routing="grouped_sigmoid", n_group=8,
+                        topk_group=4, routed_scaling=2.5, quant="channel")
+    w = wl.make_weights(layer, seed=2)
+    M = 77
+    x, tw, ids = wl.make_inputs(layer, M, seed=2)
+    emap = wl.expert_map_for(layer)
+    g = torch.Generator().manual_seed(9)
+    i_q = torch.randint(-127, 128, (M, layer.H), generator=g, dtype=torch.int8)
+    i_s = (torch.rand(M, generator=g) * 0.04 + 0.005).to(torch.float32)
+    ref = _staged_reference(oracle, layer, i_q, i_s, w, tw, ids, 16, emap=emap)
+    out = run_path(layer, tuple(t.to(dev) for t in w), x.to(dev), tw.to(dev), ids.to(dev), emap.to(dev), dev, 0,
+                   i_q=i_q.to(dev), i_s=i_s.to(dev))
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
 def test_channel_path_rejects_mixed_arguments(dev):
     from lightop_amd import workloads as wl
     from lightop_amd.moe import fused_experts_impl_int8
