@@ -12,6 +12,7 @@ _NATIVE_APIS = {
     "preshuffle_moe_weight_int4",
     "preshuffle_moe_scale_int4",
     "get_w8a8moe_json",
+    "get_moe_cuda_config",
     "invoke_fused_moe_kernel_int8",
     "invoke_fused_moe_kernel_w4a8",
     "invoke_fused_moe_gemm1_silu_quant",
@@ -40,6 +41,7 @@ __all__ = [
     "fused_experts_workspace_bytes",
     "fused_experts_workspace_views",
     "get_moe_cache",
+    "get_moe_cuda_config",
     "gelu_and_mul",
     "get_w8a8moe_json",
     "invoke_fused_moe_gemm1_silu_quant",

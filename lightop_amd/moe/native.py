@@ -43,6 +43,27 @@ def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bo
     return as_dict(t1), as_dict(t2)
 
 
+def get_moe_cuda_config(E: int, M: int, N1: int, K1: int, N2: int, K2: int, topk: int,
+                        device_name: Optional[str] = None, num_cus: Optional[int] = None,
+                        dtype: Optional[str] = None, block_n: Optional[int] = None,
+                        block_k: Optional[int] = None, is_ep: Optional[bool] = False,
+                        ep_size: Optional[int] = 16) -> Tuple[Dict[str, Any], Dict[str, Any], bool]:
+    """Configurations of the two per-channel GEMMs for ``M`` tokens and whether they were found
+    (reference: lightop.moe.get_moe_cuda_config, python/lightop/config.py:33-131, which reads per-device
+    JSON files keyed by GEMM shape and token count; the per-channel branch of fused_experts_impl_int8
+    asks it first, int8.py:735-741).  ``N1, K1`` = 2*I, H and ``N2, K2`` = H, I.  The table is the one
+    compiled into the library, so the answer is always found; ``MODE`` and ``DELTA``, which select among
+    the reference's per-gfx kernels, are carried as 0 and read by nothing here.  ``is_ep``: ``E`` experts
+    are resident out of ``E * ep_size`` that the router chooses from."""
+    del device_name, num_cus, dtype, block_n, block_k
+    assert N1 % 2 == 0 and K1 == N2 and K2 == N1 // 2, "shapes of one gated layer: N1 = 2*I, K1 = N2 = H, K2 = I"
+    c1, c2 = get_w8a8moe_json(M, E, N1, N2, K2, True, None, topk,
+                              global_num_experts=E * int(ep_size) if is_ep else E)
+    for c in (c1, c2):
+        c.update(MODE=0, DELTA=0)
+    return c1, c2, True
+
+
 def _scale_flags(fused_scale: Optional[bool]) -> int:
     """None or False: the canonical (d * a_s) * b_s + acc, which is the library's default;
     True: acc = fma(d, a_s * b_s, acc) everywhere (last-ulp differences)."""
@@ -630,7 +651,8 @@ def ctypes_void(addr: int):
     return ctypes.c_void_p(addr)
 
 
-__all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "preshuffle_moe_weight",
+__all__ = ["fused_experts_impl_int8", "fused_experts_impl_w4a8", "get_w8a8moe_json", "get_moe_cuda_config",
+           "preshuffle_moe_weight",
            "preshuffle_moe_weight_int4", "preshuffle_moe_scale_int4", "invoke_fused_moe_kernel_int8",
            "invoke_fused_moe_kernel_w4a8",
            "invoke_fused_moe_gemm1_silu_quant", "silu_and_mul", "gelu_and_mul", "act_and_mul_group_quant", "fused_experts_workspace_bytes",

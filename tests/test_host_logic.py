@@ -148,6 +148,23 @@ def test_tile_config_dictionary():
     assert c1["BLOCK_SIZE_M"] == c2["BLOCK_SIZE_M"] == 16  # the alignment block serves both GEMMs (int8.py:767)
 
 
+def test_per_channel_config_lookup_mirrors_the_reference_call():
+    """get_moe_cuda_config as the per-channel branch calls it (int8.py:739): two dictionaries and a status."""
+    from lightop_amd.moe import get_moe_cuda_config
+
+    E, M, H, I, k = 128, 512, 2048, 768, 8
+    c1, c2, status = get_moe_cuda_config(E, M, 2 * I, H, H, I, k, "gfx950", 256, "bf16")
+    assert status is True
+    for c in (c1, c2):
+        assert {"BLOCK_SIZE_M", "MODE", "DELTA"} <= set(c)
+    assert c1["BLOCK_SIZE_M"] == c2["BLOCK_SIZE_M"] in (16, 32, 64, 128, 160)
+    # an expert-parallel share: an eighth of the slots per resident expert's block choice
+    e1, _, _ = get_moe_cuda_config(32, 64, 4096, 7168, 7168, 2048, 8, "gfx950", 256, "bf16", is_ep=True, ep_size=8)
+    assert e1["BLOCK_SIZE_M"] == 16
+    with pytest.raises(AssertionError):
+        get_moe_cuda_config(E, M, 2 * I, H, H + 128, I, k, "gfx950", 256, "bf16")
+
+
 # ------------------------------------------------------------------ workloads --
 
 def test_routing_generators():
