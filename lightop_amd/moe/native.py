@@ -432,6 +432,8 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
     if activation not in ("silu", "gelu"):
         raise ValueError(f"Unsupported FusedMoe activation: {activation}")
     if hidden_states.dtype == torch.float32 and channel:
+        # the reference's per-channel GEMM refuses them too (moe_w8a8_gemm: bf16 or fp16 outputs only,
+        # csrc/moe_gemm/w8a8/moe_w8a8.cu:2585-2784)
         raise NotImplementedError("lightop_amd: per-channel scales take bfloat16 or float16 hidden_states")
     assert w1_scale is not None and w2_scale is not None
     del w1_zp, w2_zp, a1_scale, a2_scale, use_nn_moe
