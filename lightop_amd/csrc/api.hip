@@ -103,10 +103,15 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   // Around 128 slots per expert the 160-token form of that kernel holds an expert's tokens in one block
   // (a remainder block is a second pass over the expert's weights): same layer, 128 / 160: at 1024
   // tokens 345 / 358, at 1280: 394 / 386, at 1792: 488 / 422, at 2048: 541 / 444, at 2304: 629 / 517, at
-  // 2560: 658 / 620, at 3072: 686 / 754.
+  // 2560: 658 / 620, at 3072: 686 / 754.  The same happens around 256 slots per expert, where two 160-token
+  // blocks hold what would spill into a third 128-token block (at 3840 tokens 779 / 796, at 4096: 869 / 797,
+  // at 4352: 938 / 830, at 4608: 964 / 868, at 4864: 997 / 924, at 5120: 1012 / 1030); the int8 forms,
+  // whose tiles are bound by arithmetic at that size, gain nothing there.
   if (form == LO_FORM_CHANNEL && int4_channel) {
     if (per_expert <= 12.0) return 16;
-    return (allow160 && per_expert >= 76.0 && per_expert < 170.0) ? 160 : 128;
+    const bool one_block = per_expert >= 76.0 && per_expert < 170.0;
+    const bool two_blocks = per_expert >= 248.0 && per_expert < 312.0;
+    return (allow160 && (one_block || two_blocks)) ? 160 : 128;
   }
   // W4A8: the streaming kernel re-reads the token rows per wave, which outweighs the half-size
   // weights early; the LDS-tiled kernel (64 tokens) wins above about 8 slots per expert.

@@ -150,6 +150,10 @@ def test_tile_query_names_the_kernel_that_is_launched(lib):
     assert q(_lib.LO_FORM_CHANNEL, pre | _lib.LO_GEMM_W4, 2048, *qwen) == 0
     assert t1.kernel == _lib.LO_KERNEL_T128 == t2.kernel and t1.block_size_m == 160 == t2.block_size_m
     assert q(_lib.LO_FORM_CHANNEL, pre | _lib.LO_GEMM_W4, 1024, *qwen) == 0 and t1.block_size_m == 128
+    # ... and again around 256, where two such blocks hold what would need a third of 128 tokens
+    for M, want in ((3072, 128), (3840, 128), (4096, 160), (4608, 160), (5120, 128)):
+        assert q(_lib.LO_FORM_CHANNEL, pre | _lib.LO_GEMM_W4, M, *qwen) == 0 and t1.block_size_m == want, M
+    assert q(_lib.LO_FORM_CHANNEL, pre, 4096, *qwen) == 0 and t1.block_size_m == 128  # int8 weights: no second window
     assert q(_lib.LO_FORM_CHANNEL, pre, 2048, *qwen) == 0 and (t1.block_size_m, t1.kernel) == (160, _lib.LO_KERNEL_T128)
     assert q(_lib.LO_FORM_CHANNEL, 0, 2048, *qwen) == 0 and t1.block_size_m == 128  # row-major weights: no such form
     assert q(_lib.LO_FORM_W4, 0, 2, *dsv3) == 0 and t1.kernel == _lib.LO_KERNEL_DEC  # int4: up to 16 slots

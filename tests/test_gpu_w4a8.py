@@ -360,7 +360,7 @@ def test_channel_form_ep_share_variants_bit_exact(dev, oracle, M, variant):
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
-@pytest.mark.parametrize("M", [1, 32, 512, 2048])
+@pytest.mark.parametrize("M", [1, 32, 512, 2048, 4096])
 def test_channel_form_int4_layer_sampled_tokens(dev, oracle, M):
     """Qwen3-235B-A22B-shaped layer in the reference's own int4 form, sampled tokens against the oracle."""
     from lightop_amd import workloads as wl
