@@ -151,7 +151,10 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   if (form == LO_FORM_BLOCK && preshuffled) {
     if (H < 4096) {
       if (per_expert < 6.0) return 16;
-      if (per_expert <= 48.0 || (per_expert >= 96.0 && per_expert < 192.0)) return 64;
+      // 96 to 152 (where 160-token blocks cannot be used): the remainder blocks' second pass costs the
+      // 64-token tiles less; from 160 slots per expert on the 128-token kernel is ahead again (at 2560
+      // tokens 313 / 303, at 2816: 325 / 306)
+      if (per_expert <= 48.0 || (per_expert >= 96.0 && per_expert < 152.0)) return 64;
       return 128;
     }
     if (per_expert < 4.0) return 16;
