@@ -267,14 +267,17 @@ def test_whole_path_in_chunks(dev, oracle, monkeypatch):
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
-def _staged_reference(oracle, layer, i_q, i_s, w, tw, ids, bs, emap=None, shared=None, factor=1.0):
+def _staged_reference(oracle, layer, i_q, i_s, w, tw, ids, bs, emap=None, shared=None, factor=1.0, activation="silu"):
     """The per-channel path from its stages on the CPU, starting from a given quantised input."""
     w1, w2, w1s, w2s = w
     M, k = ids.shape
     S = M * k
     srt, eids, ntpp = oracle.moe_align_block_size(ids, bs, layer.E_global, expert_map=emap)
     c1 = oracle.moe_gemm_w8a8(i_q, i_s, w1, w1s, srt, eids, ntpp, None, False, k, S, bs)
-    a2q, a2s = oracle.fuse_silu_mul_quant(c1)
+    if activation == "gelu":  # gelu_and_mul, then per_token_quant_int8 with its floor (int8.py:826-838)
+        a2q, a2s = oracle.per_token_quant_int8(oracle.gelu_and_mul(c1))
+    else:
+        a2q, a2s = oracle.fuse_silu_mul_quant(c1)
     c3 = oracle.moe_gemm_w8a8(a2q, a2s, w2, w2s, srt, eids, ntpp, tw, True, 1, S, bs)
     return oracle.moe_sum(c3.view(M, k, layer.H), shared, factor)
 
@@ -325,6 +328,24 @@ def test_caller_quantised_input(dev, oracle, monkeypatch, bs, chunk):
     torch.cuda.synchronize()
     refb = oracle.fused_experts_block_int8(xb, *wb, twb, idsb, 16)
     assert torch.equal(outb.cpu().view(torch.int16), refb.view(torch.int16))
+
+
+def test_caller_quantised_input_with_gelu(dev, oracle, monkeypatch):
+    from lightop_amd import workloads as wl
+
+    say("channel whole path from i_q / i_s, GELU")
+    monkeypatch.setenv("LMSLIM_USE_FUSED_RMS_QUANT", "1")
+    layer = wl.TINY_PC
+    w = wl.make_weights(layer, seed=1)
+    M = 50
+    x, tw, ids = wl.make_inputs(layer, M, seed=3)
+    g = torch.Generator().manual_seed(13)
+    i_q = torch.randint(-127, 128, (M, layer.H), generator=g, dtype=torch.int8)
+    i_s = (torch.rand(M, 1, generator=g) * 0.04 + 0.005).to(torch.float32)
+    ref = _staged_reference(oracle, layer, i_q, i_s, w, tw, ids, 16, activation="gelu")
+    out = run_path(layer, tuple(t.to(dev) for t in w), x.to(dev), tw.to(dev), ids.to(dev), None, dev, 16,
+                   i_q=i_q.to(dev), i_s=i_s.to(dev), activation="gelu")
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
 def test_caller_quantised_input_on_an_expert_parallel_share(dev, oracle, monkeypatch):
