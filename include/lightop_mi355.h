@@ -43,19 +43,23 @@ enum { LO_I32 = 0, LO_I64 = 1 };
 
 /* flags of lo_moe_gemm_block_int8 / lo_fused_experts_block_int8 */
 enum {
+  /* Per 128-wide K block every kernel accumulates acc = fma(f32(d) * a_s, b_s, acc) (d: the block's
+   * exact int32 sum): the order the reference's Triton line
+   *   accumulator += tl.dot(a, b) * a_scale[:, None] * b_scale[None, :]
+   * (python/lightop/_lmslim_native/layers/fused_moe/int8.py:499-508) compiles to under the AMD
+   * backend's default enable_fp_fusion. */
   LO_GEMM_DEFAULT = 0,
-  /* accumulate acc = fma(f32(d), a_s * b_s, acc) per 128-K block instead of the canonical
-   * acc = acc + (f32(d) * a_s) * b_s, which every kernel computes by default.  The int32
-   * partial sums are identical; the fp32 rounding differs in the last ulp, so outputs (and the
-   * re-quantised int8 activations between the GEMMs) are no longer bit-identical to the
-   * canonical ones, only within the path's tolerance.  Halves the scale arithmetic of the
-   * compute-bound kernels. */
+  /* accumulate acc = fma(f32(d), a_s * b_s, acc) instead.  The int32 partial sums are identical; the
+   * fp32 rounding differs in the last ulp, so outputs (and the re-quantised int8 activations
+   * between the GEMMs) are no longer bit-identical to the default ones, only within the path's
+   * tolerance.  Two vector instructions per accumulator element and K block instead of three. */
   LO_GEMM_FUSED_SCALE = 1,
   /* always use the weight-streaming kernels, also where the LDS-tiled kernel applies */
   LO_GEMM_FORCE_STREAMING = 2,
-  /* canonical order in every kernel: the default, kept as an explicit flag; it wins over
+  /* accumulate acc = acc + (f32(d) * a_s) * b_s, every operation rounded on its own: the same
+   * reference line compiled without fp fusion (four vector instructions).  Wins over
    * LO_GEMM_FUSED_SCALE. */
-  LO_GEMM_CANONICAL_ORDER = 4,
+  LO_GEMM_SEPARATE_ORDER = 4,
   /* W (for the whole path: w1 and w2) is in the layout of lo_preshuffle_weight_int8 */
   LO_GEMM_W_PRESHUFFLED = 8,
   /* leave the output rows of blocks whose expert id is -1 untouched instead of zeroing

@@ -10,7 +10,7 @@ LIB_PATH = os.environ.get("LIGHTOP_AMD_LIB") or os.path.join(_CSRC, "liblightop_
 
 LO_BF16, LO_F16, LO_F32 = 0, 1, 2
 LO_I32, LO_I64 = 0, 1
-LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE, LO_GEMM_FORCE_STREAMING, LO_GEMM_CANONICAL_ORDER = 0, 1, 2, 4
+LO_GEMM_DEFAULT, LO_GEMM_FUSED_SCALE, LO_GEMM_FORCE_STREAMING, LO_GEMM_SEPARATE_ORDER = 0, 1, 2, 4
 LO_GEMM_W_PRESHUFFLED = 8
 LO_GEMM_SKIP_NONLOCAL = 16
 LO_GEMM_W4 = 32

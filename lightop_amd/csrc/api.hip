@@ -329,7 +329,7 @@ extern "C" int lo_fused_experts_block_int8(
     const int rc2 = launch_decode_path(x, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w, topk_ids, ids_dtype,
                                        expert_map, apply_router_weight_on_input, routed_scaling_factor, shared_output,
                                        cache3, out, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0, (flags & LO_GEMM_W4) != 0,
-                                       static_cast<hipStream_t>(stream));
+                                       flags, static_cast<hipStream_t>(stream));
     if (rc2 != LO_ENOTSUP) return rc2;
   }
 

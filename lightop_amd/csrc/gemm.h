@@ -53,13 +53,41 @@ __device__ __forceinline__ void with_out16(int f16, Body body) {
   else body([](float v) { return f32_to_bf16(v); });
 }
 
-// Order of the scale arithmetic per 128-wide K block.  Every kernel computes the canonical
-// acc = acc + (f32(d) * a_s) * b_s (three roundings, the order the CPU checker restates) unless the
-// caller asks for LO_GEMM_FUSED_SCALE: acc = fma(f32(d), a_s * b_s, acc), two vector instructions per
-// accumulator element instead of four, last-ulp differences in fp32.
-inline bool fused_scale_order(int flags) {
-  return (flags & LO_GEMM_FUSED_SCALE) != 0 && (flags & LO_GEMM_CANONICAL_ORDER) == 0;
+// Order of the scale arithmetic per 128-wide K block (d = the block's exact int32 sum):
+//   kOrdContract   acc = fma(f32(d) * a_s, b_s, acc)    the default: what the reference's Triton line
+//                  `accumulator += tl.dot(a, b) * a_scale * b_scale` (int8.py:499-508) compiles to with
+//                  the AMD backend's default enable_fp_fusion; three vector instructions per element
+//   kOrdSeparate   acc = acc + (f32(d) * a_s) * b_s     the same line without fp fusion; four instructions
+//                  (LO_GEMM_SEPARATE_ORDER)
+//   kOrdFusedScale acc = fma(f32(d), a_s * b_s, acc)    two instructions, last-ulp differences in fp32
+//                  (LO_GEMM_FUSED_SCALE)
+// The CPU checker restates the first two bit for bit.
+constexpr int kOrdSeparate = 0, kOrdFusedScale = 1, kOrdContract = 2;
+inline int scale_order(int flags) {
+  if (flags & LO_GEMM_SEPARATE_ORDER) return kOrdSeparate;
+  return (flags & LO_GEMM_FUSED_SCALE) ? kOrdFusedScale : kOrdContract;
 }
+// One accumulator element.  sc = a_s * b_s is read by kOrdFusedScale only, as and bs by the other two.
+template <int ORD>
+__device__ __forceinline__ float fold_elem(int d, float sc, float as, float bs, float acc) {
+  if constexpr (ORD == kOrdFusedScale) {
+    return __builtin_fmaf(static_cast<float>(d), sc, acc);
+  } else if constexpr (ORD == kOrdContract) {
+    return __builtin_fmaf(static_cast<float>(d) * as, bs, acc);
+  } else {
+    float t = static_cast<float>(d) * as;
+    t = t * bs;
+    return acc + t;
+  }
+}
+// Three-way dispatch of a launcher macro on the order: LO_ORD_DISPATCH(ord, MACRO, args...) expands to
+// MACRO(order constant, args...).
+#define LO_ORD_DISPATCH(ord, MACRO, ...)                                   \
+  do {                                                                     \
+    if ((ord) == ::lo::kOrdContract) MACRO(::lo::kOrdContract, __VA_ARGS__);      \
+    else if ((ord) == ::lo::kOrdSeparate) MACRO(::lo::kOrdSeparate, __VA_ARGS__); \
+    else MACRO(::lo::kOrdFusedScale, __VA_ARGS__);                         \
+  } while (0)
 
 __device__ __forceinline__ v4i ld16(const int8_t *p) { return *reinterpret_cast<const v4i *>(p); }
 
@@ -145,7 +173,8 @@ void decode_path_waves(int32_t top_k, int64_t H, int *gemm1_waves, int *gemm2_wa
 int launch_decode_path(const void *x, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts, int32_t top_k,
                        const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s, const float *topk_w,
                        const void *topk_ids, int ids_dtype, const int32_t *expert_map, int apply_router_weight_on_input,
-                       float factor, const void *shared_output, void *act, void *out, bool force, bool w4, hipStream_t stream);
+                       float factor, const void *shared_output, void *act, void *out, bool force, bool w4, int flags,
+                       hipStream_t stream);
 
 // Weight-streaming kernels (gemm_ws.hip): block_size_m in {16, 32, 64, 128}.
 int launch_gemm_ws(const GemmArgs &a, bool fused_act, int block_size_m, int flags, int64_t m_blocks,

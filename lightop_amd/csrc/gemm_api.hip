@@ -223,6 +223,6 @@ extern "C" int lo_moe_gemm_w8a8(const int8_t *A, const float *As, const int8_t *
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);
   LO_REQUIRE(mblocks * a.n_tiles < (1ll << 30), LO_EINVAL, "moe_gemm_w8a8: grid too large");
   if (mblocks == 0) return LO_OK;
-  return launch_gemm(a, false, block_size_m, flags & ~(LO_GEMM_FUSED_SCALE | LO_GEMM_CANONICAL_ORDER), mblocks,
+  return launch_gemm(a, false, block_size_m, flags & ~(LO_GEMM_FUSED_SCALE | LO_GEMM_SEPARATE_ORDER), mblocks,
                      static_cast<hipStream_t>(stream));
 }

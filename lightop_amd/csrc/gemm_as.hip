@@ -22,7 +22,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 // knows how many memory operations follow each weight load and waits for exactly those; in the
 // general form the stores sit in a branch, the wait counts assume they did not happen, and after
 // every tile the wave waits for loads it has only just issued.
-template <bool FAST_SCALE, bool SHUF, int KBT = 0>
+template <int ORD, bool SHUF, int KBT = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
                                                           int n_groups, int n_cnt, int sub_shift) {
@@ -149,18 +149,9 @@ void moe_gemm_as_kernel(const GemmArgs a, int m_blocks, int group_m,
     for (int rb = 0; rb < 2; ++rb) bsc[b][rb] = bld_f32(rWs, wsoff[rb], ss);
   };
   auto fold = [&](const v16i &d, float as, float bs, float *dst) __attribute__((always_inline)) {
-    if constexpr (FAST_SCALE) {
-      const float sc = as * bs;
+    const float sc = ORD == kOrdFusedScale ? as * bs : 0.0f;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) dst[i] = __builtin_fmaf(static_cast<float>(d[i]), sc, dst[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float t = static_cast<float>(d[i]) * as;
-        t = t * bs;
-        dst[i] = dst[i] + t;
-      }
-    }
+    for (int i = 0; i < 16; ++i) dst[i] = fold_elem<ORD>(d[i], sc, as, bs, dst[i]);
     // The accumulators must be final here: an empty asm that "modifies" them stops the
     // optimiser from postponing the fold (and keeping the int32 fragment alive instead).
 #pragma unroll
@@ -319,7 +310,7 @@ int launch_gemm_as(const GemmArgs &a0, int flags, int block_size_m, int64_t m_bl
   const int64_t chunks = (m_blocks + G - 1) / G;
   const int64_t grid = (chunks + 7) / 8 * (G * n_groups) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
-  const bool fast = fused_scale_order(flags);
+  const int ord = scale_order(flags);
   const size_t lds = static_cast<size_t>(as_lds_bytes(a.K));
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), Gi = static_cast<int>(G);
@@ -336,13 +327,8 @@ int launch_gemm_as(const GemmArgs &a0, int flags, int block_size_m, int64_t m_bl
     if (rc_lds) return rc_lds;                                                                        \
     hipLaunchKernelGGL(kern, g, b, lds, s, a, mbi, Gi, n_groups, n_cnt, sub_shift);                   \
   } while (0)
-  if (fast) {
-    if (a.w_shuffled) LO_AS_LAUNCH(true, true);
-    else LO_AS_LAUNCH(true, false);
-  } else {
-    if (a.w_shuffled) LO_AS_LAUNCH(false, true);
-    else LO_AS_LAUNCH(false, false);
-  }
+  if (a.w_shuffled) LO_ORD_DISPATCH(ord, LO_AS_LAUNCH, true);
+  else LO_ORD_DISPATCH(ord, LO_AS_LAUNCH, false);
 #undef LO_AS_LAUNCH
 #undef LO_AS_LAUNCH_K
   return check_launch("moe_gemm(activation-stationary)");

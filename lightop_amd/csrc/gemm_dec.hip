@@ -14,10 +14,11 @@
 //                      K blocks of the 16 gate rows and the matching 16 up rows from HBM, all
 //                      loads in flight at once, quantises its K range of the token rows
 //                      (1x128 groups, layers/gemm/int8_utils.py:74-122) into LDS while they
-//                      fly, and keeps one term (f32(d) * a_s) * b_s per K block.  The canonical
-//                      sum adds the terms in K order, so the running sum is handed from wave to
-//                      wave through LDS; the last wave ends with SiLU * mul (int8.py:811-813)
-//                      and writes the bf16 activations [S, I].
+//                      fly, and leaves one product f32(d) * a_s per K block in LDS.  The sum over
+//                      K runs in K order (acc = fma(product, b_s, acc), or acc + product * b_s
+//                      with LO_GEMM_SEPARATE_ORDER), so after one barrier the last wave walks
+//                      the products; it ends with SiLU * mul (int8.py:811-813) and writes the
+//                      bf16 activations [S, I].
 //   dec_gemm2_kernel   one workgroup per (token, 16 output columns), one wave per routed slot
 //                      of the token: the wave re-quantises its slot's activation row
 //                      (int8.py:813-823) into LDS while its expert's 16 weight rows are on
@@ -29,6 +30,7 @@
 // The second kernel reads an expert's weights once per slot routed to it, which is why the path
 // is taken only while slots rarely share an expert.
 #include <cstdlib>
+#include <type_traits>
 
 #include "gemm.h"
 
@@ -51,6 +53,7 @@ struct DecArgs {
   uint16_t *out;             // [M, H]
   float factor;
   int32_t ids64, M, S, top_k, E, Eg, H, I, kbw, mul_on_input;
+  int32_t contract;          // acc = fma(f32(d) * a_s, b_s, acc) (the default order); 0: acc + (f32(d) * a_s) * b_s
 };
 
 // Global expert id of flat slot s (returned through g) and the local expert that serves it, or -1.
@@ -117,12 +120,14 @@ __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
   const int I = a.I, N = 2 * I;
   const int pitch = KBw * kGroup + 16;
 
-  // LDS: slot list, counter, the terms of every K block, per-wave token tiles
+  // LDS: slot list, counter, the products of every K block and their weight scales, per-wave token tiles
   int32_t *const sSlots = reinterpret_cast<int32_t *>(smem);                    // [S rounded up to 4]
   int32_t *const sMeta = sSlots + ((a.S + 3) & ~3);                             // [4]
   float *const sT = reinterpret_cast<float *>(sMeta + 4);                       // [KB][8 values][4 c][TP tokens]
-  float *const sAs = sT + KB * 128 + wave * (kDecTP * KBW);              // [TP][KBw] of this wave
-  int8_t *const sA = reinterpret_cast<int8_t *>(sT + KB * 128 + W * (kDecTP * KBW)) + wave * (kDecTP * pitch);
+  constexpr int SB = W4 ? 32 : 2; // weight scales per K block: one per row (W4: [8 values][4 c]), else gate block, up block
+  float *const sB = sT + KB * 128;                                              // [KB][SB]
+  float *const sAs = sB + KB * SB + wave * (kDecTP * KBW);                      // [TP][KBw] of this wave
+  int8_t *const sA = reinterpret_cast<int8_t *>(sB + KB * SB + W * (kDecTP * KBW)) + wave * (kDecTP * pitch);
 
   // ---- requests that do not wait for the routing: the slot's own token row ----------------------
   const int sub = lane & 15, gq = lane >> 4;
@@ -238,8 +243,8 @@ __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
     }
     __builtin_amdgcn_wave_barrier();
 
-    // ---- one term per K block: weights from registers, tokens from LDS; the terms of the pass's
-    //      tokens go to LDS, K block by K block -----------------------------------------------------
+    // ---- one product f32(d) * a_s per K block: weights from registers, tokens from LDS; the products
+    //      of the pass's tokens and the weight scales they meet go to LDS, K block by K block --------
 #pragma unroll
     for (int p = 0; p < KBW; ++p) {
       if (p < KBw) {
@@ -264,9 +269,12 @@ __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
           d = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, b1, d, 0, 0, 0);
           if (n < nc) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const float t = static_cast<float>(d[i]) * as;
-              sT[((kb0 + p) * 8 + g * 4 + i) * 16 + c * kDecTP + n] = t * (W4 ? wsc[W4 ? p : 0][g][i] * 0.0625f : bs[g]);
+            for (int i = 0; i < 4; ++i)
+              sT[((kb0 + p) * 8 + g * 4 + i) * 16 + c * kDecTP + n] = static_cast<float>(d[i]) * as;
+            if constexpr (W4) { // the scales of the lane's four rows, as loaded ([c][i]; the factor 1/16 is applied by the reader)
+              if (n == 0) *reinterpret_cast<v4f *>(sB + ((kb0 + p) * 2 + g) * 16 + c * 4) = wsc[W4 ? p : 0][g];
+            } else {
+              if (lane == 0) sB[(kb0 + p) * 2 + g] = bs[g];
             }
           }
         }
@@ -279,24 +287,39 @@ __device__ __forceinline__ void dec_gemm1_body(const DecArgs &a) {
     //      and the up terms of activation column 4c + i. ---------------------------------------------
     if (wave == W - 1) {
       float accg = 0.0f, accu = 0.0f;
-      int kb = 0;
-      for (; kb + 4 <= KB; kb += 4) {
-        float tg[4], tu[4];
+      auto sum_k = [&](auto CONTRACT) __attribute__((always_inline)) {
+        auto add = [](float acc, float t, float b) __attribute__((always_inline)) {
+          if constexpr (W4) b = b * 0.0625f; // int4 nibbles are unpacked 16 times too large
+          if constexpr (decltype(CONTRACT)::value) return __builtin_fmaf(t, b, acc);
+          const float tb = t * b;
+          return acc + tb;
+        };
+        // lane (i, c, token): row 4c + i of the fragment
+        const int brow = ((lane >> 2) & 3) * 4 + (lane >> 4);
+        const float *const bg = sB + (W4 ? brow : 0), *const bu = sB + (W4 ? 16 + brow : 1);
+        int kb = 0;
+        for (; kb + 4 <= KB; kb += 4) {
+          float tg[4], tu[4], sg[4], su[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          tg[j] = sT[(kb + j) * 128 + lane];
-          tu[j] = sT[(kb + j) * 128 + 64 + lane];
-        }
+          for (int j = 0; j < 4; ++j) {
+            tg[j] = sT[(kb + j) * 128 + lane];
+            tu[j] = sT[(kb + j) * 128 + 64 + lane];
+            sg[j] = bg[(kb + j) * SB];
+            su[j] = bu[(kb + j) * SB];
+          }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          accg = accg + tg[j];
-          accu = accu + tu[j];
+          for (int j = 0; j < 4; ++j) {
+            accg = add(accg, tg[j], sg[j]);
+            accu = add(accu, tu[j], su[j]);
+          }
         }
-      }
-      for (; kb < KB; ++kb) {
-        accg = accg + sT[kb * 128 + lane];
-        accu = accu + sT[kb * 128 + 64 + lane];
-      }
+        for (; kb < KB; ++kb) {
+          accg = add(accg, sT[kb * 128 + lane], bg[kb * SB]);
+          accu = add(accu, sT[kb * 128 + 64 + lane], bu[kb * SB]);
+        }
+      };
+      if (a.contract) sum_k(std::true_type{});
+      else sum_k(std::false_type{});
       const int i = lane >> 4, cc = (lane >> 2) & 3, tok = lane & 3;
       if (tok < nc) {
         const int64_t fslot = sSlots[chunk0 + tok];
@@ -417,8 +440,12 @@ __global__ __launch_bounds__(512) void dec_gemm2_kernel(const DecArgs a) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             float tt = static_cast<float>(d[i]) * as;
-            tt = tt * (W4 ? bs4[i] : bs);
-            acc[i] = acc[i] + tt;
+            if (a.contract) {
+              acc[i] = __builtin_fmaf(tt, W4 ? bs4[i] : bs, acc[i]);
+            } else {
+              tt = tt * (W4 ? bs4[i] : bs);
+              acc[i] = acc[i] + tt;
+            }
           }
         }
       }
@@ -509,7 +536,8 @@ void decode_path_waves(int32_t top_k, int64_t H, int *gemm1_waves, int *gemm2_wa
 int launch_decode_path(const void *x, int64_t M, int64_t H, int64_t I, int32_t E, int32_t num_experts, int32_t top_k,
                        const int8_t *w1, const float *w1s, const int8_t *w2, const float *w2s, const float *topk_w,
                        const void *topk_ids, int ids_dtype, const int32_t *expert_map, int apply_router_weight_on_input,
-                       float factor, const void *shared_output, void *act, void *out, bool force, bool w4, hipStream_t stream) {
+                       float factor, const void *shared_output, void *act, void *out, bool force, bool w4, int flags,
+                       hipStream_t stream) {
   if (!decode_path_applies(M, top_k, H, I, num_experts, force, w4)) return LO_ENOTSUP;
   const int64_t S = M * top_k;
   const int KB1 = static_cast<int>(H / kGroup), KB2 = static_cast<int>(I / kGroup);
@@ -526,8 +554,10 @@ int launch_decode_path(const void *x, int64_t M, int64_t H, int64_t I, int32_t E
   a.M = static_cast<int>(M); a.S = static_cast<int>(S); a.top_k = top_k; a.E = E; a.Eg = num_experts;
   a.H = static_cast<int>(H); a.I = static_cast<int>(I); a.kbw = KB1 / W1;
   a.mul_on_input = apply_router_weight_on_input ? 1 : 0;
+  // two orders only: LO_GEMM_FUSED_SCALE buys nothing at this size and gets the default order
+  a.contract = scale_order(flags) == kOrdSeparate ? 0 : 1;
 
-  const size_t l1 = static_cast<size_t>((S + 3) & ~int64_t(3)) * 4 + 16 + static_cast<size_t>(KB1) * 128 * 4 +
+  const size_t l1 = static_cast<size_t>((S + 3) & ~int64_t(3)) * 4 + 16 + static_cast<size_t>(KB1) * (128 + (w4 ? 32 : 2)) * 4 +
                     static_cast<size_t>(W1) * kDecTP * kDecMaxKBw * 4 +
                     static_cast<size_t>(W1) * kDecTP * (a.kbw * kGroup + 16);
   const size_t l2 = ((static_cast<size_t>(top_k) * 33 + 15) & ~size_t(15)) + ((static_cast<size_t>(W2) * KB2 * 4 + 15) & ~size_t(15)) +

@@ -68,10 +68,10 @@ __device__ __forceinline__ void wait_copies_barrier() {
 // python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341-395): one scale per token row and one
 // per weight row, both applied in the epilogue, so the int32 sums run over the whole K inside the
 // MFMA accumulators and the K loop has no scale arithmetic at all.
-template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM, bool W4, bool PC = false, int NTB = 8>
+template <bool FUSED_ACT, int ORD, bool STREAM, bool W4, bool PC = false, int NTB = 8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
-  static_assert(!PC || (!FUSED_ACT && !FAST_SCALE && (W4 || NTB == 10)),
+  static_assert(!PC || (!FUSED_ACT && ORD == kOrdSeparate && (W4 || NTB == 10)),
                 "per-channel scales: plain GEMM, int4 weights or 160-token tiles of int8 weights");
   static_assert(NTB == 8 || (NTB == 10 && !FUSED_ACT && (PC || !W4)),
                 "160-token tiles: plain GEMM, int8 block form or per-channel scales");
@@ -282,30 +282,14 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   // One scale per weight row: bs4[i] for row 4q + i.
   auto fold4 = [&](const v4i &d, float as, const v4f &bs4, float *dst) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if constexpr (FAST_SCALE) {
-        dst[i] = __builtin_fmaf(static_cast<float>(d[i]), as * bs4[i], dst[i]); // bs4 already holds scale / 16
-      } else {
-        float t = static_cast<float>(d[i]) * as;
-        t = t * bs4[i];
-        dst[i] = dst[i] + t;
-      }
-    }
+    for (int i = 0; i < 4; ++i) // bs4 already holds scale / 16
+      dst[i] = fold_elem<ORD>(d[i], ORD == kOrdFusedScale ? as * bs4[i] : 0.0f, as, bs4[i], dst[i]);
 #pragma unroll
     for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(dst[i])); // keep the fold here
   };
   auto fold = [&](const v4i &d, float sc, float as, float bs, float *dst) __attribute__((always_inline)) {
-    if constexpr (FAST_SCALE) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dst[i] = __builtin_fmaf(static_cast<float>(d[i]), sc, dst[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float t = static_cast<float>(d[i]) * as;
-        t = t * bs;
-        dst[i] = dst[i] + t;
-      }
-    }
+    for (int i = 0; i < 4; ++i) dst[i] = fold_elem<ORD>(d[i], sc, as, bs, dst[i]);
 #pragma unroll
     for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(dst[i])); // keep the fold here
   };
@@ -389,7 +373,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
         fold4(dprev[1], as_p, wsc[h][1], acc[h][tb][1]);
         return;
       }
-      if (FAST_SCALE && h == 0) {
+      if (ORD == kOrdFusedScale && h == 0) {
         sc0 = as_p * bs0;
         sc1 = FUSED_ACT ? as_p * bs1 : sc0;
       }
@@ -697,7 +681,7 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int f
   const int64_t chunks = (m_blocks + G - 1) / G;
   const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
-  const bool fast = fused_scale_order(flags);
+  const int ord = scale_order(flags);
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
 #define LO_T128_LAUNCH(FA, FS, ST, W)                                                                           \
@@ -712,11 +696,11 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int f
   do {                                                                                                          \
     static unsigned long long lds_done = 0;                                                                     \
     const int rc_lds = reserve_lds_once(                                                                        \
-        reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, false, ST, true, true>), kTLds, &lds_done); \
+        reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, kOrdSeparate, ST, true, true>), kTLds, &lds_done); \
     if (rc_lds) return rc_lds;                                                                                  \
-    hipLaunchKernelGGL((moe_gemm_t128_kernel<false, false, ST, true, true>), g, b, kTLds, s, a, mbi, gi);       \
+    hipLaunchKernelGGL((moe_gemm_t128_kernel<false, kOrdSeparate, ST, true, true>), g, b, kTLds, s, a, mbi, gi);       \
   } while (0)
-#define LO_T128_PICK(FA, FS)                                                                                    \
+#define LO_T128_PICK(FS, FA)                                                                                    \
   do {                                                                                                          \
     if (a.w4) {                                                                                                 \
       if (stream) LO_T128_LAUNCH(FA, FS, true, true);                                                           \
@@ -740,17 +724,18 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int f
     if (a.per_channel && a.w4) {
       static unsigned long long lds_done = 0;
       const int rc_lds = reserve_lds_once(
-          reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, false, true, true, true, 10>), kTLds160, &lds_done);
+          reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, kOrdSeparate, true, true, true, 10>), kTLds160, &lds_done);
       if (rc_lds) return rc_lds;
-      hipLaunchKernelGGL((moe_gemm_t128_kernel<false, false, true, true, true, 10>), g, b, kTLds160, s, a, mbi, gi);
+      hipLaunchKernelGGL((moe_gemm_t128_kernel<false, kOrdSeparate, true, true, true, 10>), g, b, kTLds160, s, a, mbi, gi);
     } else if (a.per_channel) {
       static unsigned long long lds_done = 0;
       const int rc_lds = reserve_lds_once(
-          reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, false, true, false, true, 10>), kTLds160, &lds_done);
+          reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, kOrdSeparate, true, false, true, 10>), kTLds160, &lds_done);
       if (rc_lds) return rc_lds;
-      hipLaunchKernelGGL((moe_gemm_t128_kernel<false, false, true, false, true, 10>), g, b, kTLds160, s, a, mbi, gi);
-    } else if (fast) LO_T160_LAUNCH(true);
-    else LO_T160_LAUNCH(false);
+      hipLaunchKernelGGL((moe_gemm_t128_kernel<false, kOrdSeparate, true, false, true, 10>), g, b, kTLds160, s, a, mbi, gi);
+    } else if (ord == kOrdContract) LO_T160_LAUNCH(kOrdContract);
+    else if (ord == kOrdSeparate) LO_T160_LAUNCH(kOrdSeparate);
+    else LO_T160_LAUNCH(kOrdFusedScale);
 #undef LO_T160_LAUNCH
     return check_launch("moe_gemm(t160)");
   }
@@ -760,11 +745,9 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int f
     if (stream) LO_T128_LAUNCH_PC(true);
     else LO_T128_LAUNCH_PC(false);
   } else if (fused_act) {
-    if (fast) LO_T128_PICK(true, true);
-    else LO_T128_PICK(true, false);
+    LO_ORD_DISPATCH(ord, LO_T128_PICK, true);
   } else {
-    if (fast) LO_T128_PICK(false, true);
-    else LO_T128_PICK(false, false);
+    LO_ORD_DISPATCH(ord, LO_T128_PICK, false);
   }
 #undef LO_T128_PICK
 #undef LO_T128_LAUNCH_PC

@@ -37,7 +37,7 @@ constexpr int kTileRow = 144;    // LDS row pitch in bytes: 128 + 16 keeps ds_re
 // layer at 512 tokens 132 -> 74 us).  With several token blocks per expert the blocks share the
 // weights through L2 and the default policy is the faster one; with row-major weights, where a
 // 128-byte line serves several k-steps of a lane, the hint costs 50 %.
-template <bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int WT, bool STREAM = false>
+template <bool FUSED_ACT, int ORD, bool SHUF, int WT, bool STREAM = false>
 __global__ __launch_bounds__(256 * WT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   static_assert(!STREAM || (SHUF && WT == 1), "streaming policy: 64-token tiles of pre-shuffled weights");
@@ -182,18 +182,9 @@ void moe_gemm_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
     for (int rb = 0; rb < 2; ++rb) bsc[b][rb] = wsrow[rb][kc];
   };
   auto fold = [&](const v16i &d, float as, float bs, float *dst) {
-    if constexpr (FAST_SCALE) {
-      const float sc = as * bs;
+    const float sc = ORD == kOrdFusedScale ? as * bs : 0.0f;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) dst[i] = __builtin_fmaf(static_cast<float>(d[i]), sc, dst[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float t = static_cast<float>(d[i]) * as;
-        t = t * bs;
-        dst[i] = dst[i] + t;
-      }
-    }
+    for (int i = 0; i < 16; ++i) dst[i] = fold_elem<ORD>(d[i], sc, as, bs, dst[i]);
     // The accumulators must be final here: an empty asm that "modifies" them stops the
     // optimiser from postponing the fold (and keeping the int32 fragment alive instead).
 #pragma unroll
@@ -352,7 +343,7 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int block_size_m, int f
   const int64_t chunks = (m_blocks + G - 1) / G;
   const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm: grid too large");
-  const bool fast = fused_scale_order(flags);
+  const int ord = scale_order(flags);
   const int wt = block_size_m / 64;
   const dim3 g(static_cast<unsigned>(grid)), b(256 * wt);
   const int mbi = static_cast<int>(m_blocks);
@@ -366,20 +357,15 @@ int launch_gemm_tile(const GemmArgs &a0, bool fused_act, int block_size_m, int f
   // the first one gains)
   const bool stream = a.w_shuffled && wt == 1 &&
                       a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * 48;
-#define LO_TILE_LAUNCH(FA, FS)                         \
+#define LO_TILE_LAUNCH(FS, FA)                         \
   do {                                                 \
     if (stream)                                        \
       hipLaunchKernelGGL((moe_gemm_tile_kernel<FA, FS, true, 1, true>), g, b, 0, s, a, mbi, static_cast<int>(G)); \
     else if (a.w_shuffled) LO_TILE_LAUNCH2(FA, FS, true);   \
     else LO_TILE_LAUNCH2(FA, FS, false);               \
   } while (0)
-  if (fused_act) {
-    if (fast) LO_TILE_LAUNCH(true, true);
-    else LO_TILE_LAUNCH(true, false);
-  } else {
-    if (fast) LO_TILE_LAUNCH(false, true);
-    else LO_TILE_LAUNCH(false, false);
-  }
+  if (fused_act) LO_ORD_DISPATCH(ord, LO_TILE_LAUNCH, true);
+  else LO_ORD_DISPATCH(ord, LO_TILE_LAUNCH, false);
 #undef LO_TILE_LAUNCH
 #undef LO_TILE_LAUNCH2
   return check_launch(fused_act ? "moe_gemm1_silu_quant(tile)" : "moe_gemm(tile)");

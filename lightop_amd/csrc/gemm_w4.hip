@@ -33,7 +33,7 @@ constexpr int kW4Row = 144; // LDS row pitch in bytes: 128 + 16 keeps ds_read_b1
 // loaded with the streaming cache policy (first GEMM of a 4096 x 1536 layer with 16 or 32 slots per
 // expert: 227 -> 180 us).  With several token blocks per expert the blocks share the weights through
 // L2 and the default policy is the faster one.
-template <bool FUSED_ACT, bool FAST_SCALE, bool STREAM>
+template <bool FUSED_ACT, int ORD, bool STREAM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
   constexpr int kTileM = 64;
@@ -190,15 +190,8 @@ void moe_gemm_w4_tile_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
     for (int tf = 0; tf < 4; ++tf)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if constexpr (FAST_SCALE) {
-          dst[tf][i] = __builtin_fmaf(static_cast<float>(d[tf][i]), as[tf] * bs16[i], dst[tf][i]);
-        } else {
-          float t = static_cast<float>(d[tf][i]) * as[tf];
-          t = t * bs16[i];
-          dst[tf][i] = dst[tf][i] + t;
-        }
-      }
+      for (int i = 0; i < 4; ++i)
+        dst[tf][i] = fold_elem<ORD>(d[tf][i], ORD == kOrdFusedScale ? as[tf] * bs16[i] : 0.0f, as[tf], bs16[i], dst[tf][i]);
 #pragma unroll
     for (int tf = 0; tf < 4; ++tf)
 #pragma unroll
@@ -378,7 +371,7 @@ int launch_gemm_w4_tile(const GemmArgs &a0, bool fused_act, int flags, int64_t m
   const int64_t chunks = (m_blocks + G - 1) / G;
   const int64_t grid = (chunks + 7) / 8 * (G * a.n_tiles) * 8;
   LO_REQUIRE(grid < (1ll << 31), LO_EINVAL, "moe_gemm(w4): grid too large");
-  const bool fast = fused_scale_order(flags);
+  const int ord = scale_order(flags);
   const dim3 g(static_cast<unsigned>(grid)), b(256);
   const int mbi = static_cast<int>(m_blocks), gi = static_cast<int>(G);
   // the row scales of the workgroup's 256 rows, every K block, sit in LDS next to 28 KB of static arrays
@@ -398,18 +391,13 @@ int launch_gemm_w4_tile(const GemmArgs &a0, bool fused_act, int flags, int64_t m
     }                                                                                                          \
     hipLaunchKernelGGL((moe_gemm_w4_tile_kernel<FA, FS, ST>), g, b, static_cast<size_t>(lds), s, a, mbi, gi);  \
   } while (0)
-#define LO_W4_TILE_PICK(FA, FS)              \
+#define LO_W4_TILE_PICK(FS, FA)              \
   do {                                       \
     if (stream) LO_W4_TILE_LAUNCH(FA, FS, true); \
     else LO_W4_TILE_LAUNCH(FA, FS, false);   \
   } while (0)
-  if (fused_act) {
-    if (fast) LO_W4_TILE_PICK(true, true);
-    else LO_W4_TILE_PICK(true, false);
-  } else {
-    if (fast) LO_W4_TILE_PICK(false, true);
-    else LO_W4_TILE_PICK(false, false);
-  }
+  if (fused_act) LO_ORD_DISPATCH(ord, LO_W4_TILE_PICK, true);
+  else LO_ORD_DISPATCH(ord, LO_W4_TILE_PICK, false);
 #undef LO_W4_TILE_PICK
 #undef LO_W4_TILE_LAUNCH
   return check_launch(fused_act ? "moe_gemm1_silu_quant(w4 tile)" : "moe_gemm(w4 tile)");

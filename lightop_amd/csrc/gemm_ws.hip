@@ -53,7 +53,7 @@ namespace lo {
 // python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341-395): the nibbles enter the sum as
 // int8(nibble << 4), the factor 16 stays in it, and C = bf16(((f32(d) [* topk_w[f]]) * As[row])
 // * Ws[e, n]).
-template <int TM, bool FUSED_ACT, bool FAST_SCALE, bool SHUF, int NWAVES, int PD, int RPW, bool W4 = false,
+template <int TM, bool FUSED_ACT, int ORD, bool SHUF, int NWAVES, int PD, int RPW, bool W4 = false,
           bool PC = false>
 __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs a) {
   static_assert(!W4 || SHUF, "int4 weights exist in the load-time layout only");
@@ -325,17 +325,10 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
       for (int j = 0; j < TM; ++j) {
 #pragma unroll
         for (int g = 0; g < NW; ++g) {
-          if constexpr (FAST_SCALE) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              acc[g][j][i] = __builtin_fmaf(static_cast<float>(d[g][j][i]), as[j] * bs[g][W4 ? i : 0], acc[g][j][i]);
-          } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              float t = static_cast<float>(d[g][j][i]) * as[j];
-              t = t * bs[g][W4 ? i : 0];
-              acc[g][j][i] = acc[g][j][i] + t;
-            }
+          for (int i = 0; i < 4; ++i) {
+            const float b = bs[g][W4 ? i : 0];
+            acc[g][j][i] = fold_elem<ORD>(d[g][j][i], ORD == kOrdFusedScale ? as[j] * b : 0.0f, as[j], b, acc[g][j][i]);
           }
         }
       }
@@ -444,7 +437,7 @@ __global__ __launch_bounds__(NWAVES * 64) void moe_gemm_ws_kernel(const GemmArgs
   }
 }
 
-template <int TM, bool FUSED_ACT, bool FAST_SCALE>
+template <int TM, bool FUSED_ACT, int ORD>
 static int launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
   constexpr int NWAVES = FUSED_ACT ? 8 : LO_WS_PLAIN_WAVES;
   // A plain-GEMM wave takes RPW consecutive 16-row fragments so that it streams a few
@@ -455,14 +448,14 @@ static int launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
   GemmArgs a = a0;
   if (!FUSED_ACT) a.n_tiles = static_cast<int32_t>((a.N + 16 * NWAVES * RPW - 1) / (16 * NWAVES * RPW));
   const dim3 grid(static_cast<unsigned>(m_blocks * a.n_tiles)), block(NWAVES * 64);
-  if constexpr (!FUSED_ACT && !FAST_SCALE) {
+  if constexpr (!FUSED_ACT && ORD == kOrdSeparate) {
     if (a.per_channel) {
       if (a.w4)
-        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, true, NWAVES, PD, RPW, true, true>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, kOrdSeparate, true, NWAVES, PD, RPW, true, true>), grid, block, 0, s, a);
       else if (a.w_shuffled)
-        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, true, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, kOrdSeparate, true, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
       else
-        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, false, false, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, false, kOrdSeparate, false, NWAVES, PD, RPW, false, true>), grid, block, 0, s, a);
       return LO_OK;
     }
   }
@@ -472,7 +465,7 @@ static int launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
     const int64_t lds = a.K / kGroup * ROWS * 4;
     LO_REQUIRE(lds <= 128 * 1024, LO_ENOTSUP, "moe_gemm(int4): K = %lld is more than this kernel's %d K groups",
                static_cast<long long>(a.K), 128 * 1024 / (ROWS * 4));
-    const auto kern = &moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, true, NWAVES, PD, RPW, true>;
+    const auto kern = &moe_gemm_ws_kernel<TM, FUSED_ACT, ORD, true, NWAVES, PD, RPW, true>;
     if (lds > 48 * 1024) {
       static unsigned long long lds_done = 0; // per instantiation: one bit per device
       const int rc_lds = reserve_lds_once(reinterpret_cast<const void *>(kern), 128 * 1024, &lds_done);
@@ -480,20 +473,22 @@ static int launch_ws(const GemmArgs &a0, int64_t m_blocks, hipStream_t s) {
     }
     hipLaunchKernelGGL(kern, grid, block, static_cast<size_t>(lds), s, a);
   } else if (a.w_shuffled)
-    hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, true, NWAVES, PD, RPW>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, ORD, true, NWAVES, PD, RPW>), grid, block, 0, s, a);
   else
-    hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, FAST_SCALE, false, NWAVES, PD, RPW>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((moe_gemm_ws_kernel<TM, FUSED_ACT, ORD, false, NWAVES, PD, RPW>), grid, block, 0, s, a);
   return LO_OK;
 }
 
 template <bool FUSED_ACT>
 static int dispatch_ws(const GemmArgs &a, int bs, int flags, int64_t m_blocks, hipStream_t s) {
-  const bool fast = fused_scale_order(flags) && !a.per_channel;
+  // per-channel scales are applied once, in the epilogue: one instantiation (tagged kOrdSeparate)
+  const int ord = a.per_channel ? kOrdSeparate : scale_order(flags);
   int rc = LO_OK;
 #define LO_WS_CASE(TMV)                                               \
   case 16 * TMV:                                                      \
-    rc = fast ? launch_ws<TMV, FUSED_ACT, true>(a, m_blocks, s)       \
-              : launch_ws<TMV, FUSED_ACT, false>(a, m_blocks, s);     \
+    rc = ord == kOrdContract   ? launch_ws<TMV, FUSED_ACT, kOrdContract>(a, m_blocks, s)     \
+         : ord == kOrdSeparate ? launch_ws<TMV, FUSED_ACT, kOrdSeparate>(a, m_blocks, s)     \
+                               : launch_ws<TMV, FUSED_ACT, kOrdFusedScale>(a, m_blocks, s);  \
     break;
   switch (bs) {
     LO_WS_CASE(1)

@@ -65,11 +65,10 @@ def get_moe_cuda_config(E: int, M: int, N1: int, K1: int, N2: int, K2: int, topk
 
 
 def _scale_flags(fused_scale: Optional[bool]) -> int:
-    """None or False: the canonical (d * a_s) * b_s + acc, which is the library's default;
-    True: acc = fma(d, a_s * b_s, acc) everywhere (last-ulp differences)."""
-    if fused_scale is None:
-        return 0
-    return _lib.LO_GEMM_FUSED_SCALE if fused_scale else _lib.LO_GEMM_CANONICAL_ORDER
+    """None or False: the library's default order, acc = fma(f32(d) * a_s, b_s, acc) per K block;
+    True: acc = fma(f32(d), a_s * b_s, acc) everywhere (last-ulp differences).  The order without
+    fp fusion, acc + (f32(d) * a_s) * b_s, is ``flags=LO_GEMM_SEPARATE_ORDER``."""
+    return _lib.LO_GEMM_FUSED_SCALE if fused_scale else 0
 
 
 def preshuffle_moe_weight(w: torch.Tensor) -> torch.Tensor:

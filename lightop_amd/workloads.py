@@ -6,7 +6,11 @@ top-k (renormalised), DeepSeek-V3 grouped sigmoid top-k (8 groups, top-4 groups,
 score = sum of the group's two best experts, renormalised, x2.5; reference form:
 test/ci_tests/test_fused_moe_gate.py:9-61), optionally Zipf-skewed.  Everything is
 drawn from a seeded torch.Generator on the CPU (or, for layers too large to copy, on
-the device) so that a CPU checker and the GPU see the same bits.
+the device) so that a CPU checker and the GPU see the same bits.  Exponentials (the
+lognormal scales, softmax, sigmoid) and the renormalising sums are taken in float64 and
+rounded to float32 once: torch's float32 exp differs in the last place between CPUs
+(vector width), and the committed fixtures must not depend on the host that regenerates
+their inputs.
 """
 from __future__ import annotations
 
@@ -78,8 +82,8 @@ def make_weights(layer: MoeLayer, seed: int = 0, device="cpu", gen_device: Optio
             return torch.randint(0, 256, shape, generator=g, dtype=torch.int16, device=gen_device).to(torch.uint8)
 
         def s4(shape):
-            return torch.exp(torch.randn(shape, generator=g, dtype=torch.float32, device=gen_device) * 0.3
-                             + math.log(1e-2))
+            z = torch.randn(shape, generator=g, dtype=torch.float32, device=gen_device) * 0.3 + math.log(1e-2)
+            return torch.exp(z.double()).float()
 
         if layer.quant == "channel":
             return tuple(t.to(device) for t in (w4((E, 2 * I, H // 2)), w4((E, H, I // 2)),
@@ -91,8 +95,8 @@ def make_weights(layer: MoeLayer, seed: int = 0, device="cpu", gen_device: Optio
         return torch.randint(-127, 128, shape, generator=g, dtype=torch.int8, device=gen_device)
 
     def s(shape):
-        return torch.exp(torch.randn(shape, generator=g, dtype=torch.float32, device=gen_device) * 0.3
-                         + math.log(1e-3))
+        z = torch.randn(shape, generator=g, dtype=torch.float32, device=gen_device) * 0.3 + math.log(1e-3)
+        return torch.exp(z.double()).float()
 
     w1 = w((E, 2 * I, H))
     w2 = w((E, H, I))
@@ -116,11 +120,11 @@ def route(layer: MoeLayer, logits: torch.Tensor) -> Tuple[torch.Tensor, torch.Te
     """(topk_weights [M,k] f32, topk_ids [M,k] int32) from router logits [M, E_global]."""
     k = layer.top_k
     if layer.routing == "softmax":
-        p = torch.softmax(logits.float(), dim=-1)
+        p = torch.softmax(logits.double(), dim=-1)
         w, ids = torch.topk(p, k, dim=-1)
         w = w / w.sum(dim=-1, keepdim=True)
-        return w.contiguous(), ids.to(torch.int32).contiguous()
-    scores = torch.sigmoid(logits.float())
+        return w.float().contiguous(), ids.to(torch.int32).contiguous()
+    scores = torch.sigmoid(logits.double())
     M, Eg = scores.shape
     per = Eg // layer.n_group
     group_scores = scores.view(M, layer.n_group, per).topk(2, dim=-1)[0].sum(dim=-1)
@@ -132,7 +136,7 @@ def route(layer: MoeLayer, logits: torch.Tensor) -> Tuple[torch.Tensor, torch.Te
     ids = torch.topk(masked, k, dim=-1, sorted=False)[1]
     w = scores.gather(1, ids)
     w = w / w.sum(dim=-1, keepdim=True) * layer.routed_scaling
-    return w.contiguous(), ids.to(torch.int32).contiguous()
+    return w.float().contiguous(), ids.to(torch.int32).contiguous()
 
 
 def make_inputs(layer: MoeLayer, M: int, seed: int = 0, device="cpu"):
@@ -142,9 +146,9 @@ def make_inputs(layer: MoeLayer, M: int, seed: int = 0, device="cpu"):
     logits = torch.randn((M, layer.E_global), generator=g, dtype=torch.float32)
     if layer.routing.endswith("zipf"):
         perm = torch.randperm(layer.E_global, generator=g)
-        zipf = 1.0 / torch.arange(1, layer.E_global + 1, dtype=torch.float32) ** 1.2
+        zipf = 1.0 / torch.arange(1, layer.E_global + 1, dtype=torch.float64) ** 1.2
         bias = torch.empty(layer.E_global)
-        bias[perm] = torch.log(zipf / zipf.sum())
+        bias[perm] = torch.log(zipf / zipf.sum()).float()
         logits = logits + bias
     w, ids = route(layer, logits)
     return x.to(device), w.to(device), ids.to(device)

@@ -47,6 +47,22 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+SCALE_ORDERS = ("contract", "separate")
+
+
+@contextlib.contextmanager
+def scale_order(order: str):
+    """Scale arithmetic of the block-form GEMMs per 128-wide K block inside the ``with`` block:
+    "contract" (the default: acc = fma(f32(d) * a_s, b_s, acc)) or "separate"
+    (acc = acc + (f32(d) * a_s) * b_s)."""
+    assert order in SCALE_ORDERS, order
+    lib().orc_set_scale_order(ctypes.c_int(1 if order == "contract" else 0))
+    try:
+        yield order
+    finally:
+        lib().orc_set_scale_order(ctypes.c_int(1))
+
+
 def _p(t: Optional[torch.Tensor]):
     if t is None:
         return ctypes.c_void_p(0)

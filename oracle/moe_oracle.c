@@ -221,7 +221,9 @@ void orc_group_quant_int8(const uint16_t *x, int64_t R, int64_t C, float eps,
  * For every block b < P/bs with e = expert_ids[b] and every row
  * f = sorted[b*bs + i] < num_valid:
  *   acc = 0;  for kb: d = sum_k A*W (int32, exact);
- *             acc = acc + (f32(d) * As[row, kb]) * Ws[e, n/128, kb]   (int8.py:499-508)
+ *             t = f32(d) * As[row, kb];                               (int8.py:499-508)
+ *             acc = fma(t, Ws[e, n/128, kb], acc)    contracted order (the default), or
+ *             acc = acc + t * Ws[e, n/128, kb]       separate order (orc_set_scale_order(0))
  *   if mul_routed: acc = acc * topk_w[f]                              (int8.py:521-525)
  *   C[f, n] = bf16(acc);  e == -1 -> C[f, :] = 0                      (int8.py:441-449)
  *
@@ -229,6 +231,20 @@ void orc_group_quant_int8(const uint16_t *x, int64_t R, int64_t C, float eps,
  * per-128-block integer dot products, so that the integer part can be checked
  * on its own.
  */
+/*
+ * Order of the scale arithmetic per 128-wide K block.  The reference line is
+ *   accumulator += tl.dot(a, b) * a_scale[:, None] * b_scale[None, :]      (int8.py:499-508)
+ * and the kernel is compiled without an enable_fp_fusion override (launch at int8.py:596-626),
+ * so Triton's AMD backend, whose default is enable_fp_fusion = True, lets LLVM contract the last
+ * multiplication and the addition: acc = fma(f32(d) * a_s, b_s, acc), two roundings per K
+ * block.  That contracted order is the default here (g_contract = 1).  The separate order,
+ * acc = acc + (f32(d) * a_s) * b_s with three roundings, is what the same line gives with fp
+ * fusion off; orc_set_scale_order(0) selects it.  The first multiplication feeds a multiplication,
+ * not an addition, so it is never contracted.  A switch for the test harness, like the dtype's.
+ */
+static int g_contract = 1;
+void orc_set_scale_order(int contract) { g_contract = contract; }
+
 /* group_n = rows of W that share a scale: 128 (block-INT8) or 1 (one scale per row and K group) */
 static void gemm_core(const int8_t *A, const float *As, const int8_t *W,
                       const float *Ws, const int32_t *sorted,
@@ -271,8 +287,12 @@ static void gemm_core(const int8_t *A, const float *As, const int8_t *W,
             d += (int32_t)a[kb * ORC_GROUP + k] * (int32_t)wn[kb * ORC_GROUP + k];
           if (acc_dump) acc_dump[(f * N + n) * KB + kb] = d;
           float t = (float)d * as[kb];
-          t = t * ws[(n / group_n) * KB + kb];
-          acc = acc + t;
+          if (g_contract) {
+            acc = fmaf(t, ws[(n / group_n) * KB + kb], acc);
+          } else {
+            t = t * ws[(n / group_n) * KB + kb];
+            acc = acc + t;
+          }
         }
         if (mul_routed) acc = acc * topk_w[f];
         if (cf) cf[n] = acc;
@@ -301,8 +321,8 @@ void orc_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W,
  * (python/lightop/_lmslim_native/layers/fused_moe/w4a8.py:341, :375-377).  The reference
  * itself scales per token and per channel in the epilogue only (w4a8.py:395); the K-group
  * form restated here has no reference implementation, so its parity is unpinned beyond the
- * arithmetic it shares with the block-INT8 path:
- *   acc = acc + (f32(sum_k A*w) * As[row, kb]) * Ws[e, n, kb]
+ * arithmetic it shares with the block-INT8 path (both scale orders, see gemm_core):
+ *   acc = fma(f32(sum_k A*w) * As[row, kb], Ws[e, n, kb], acc)
  */
 void orc_unpack_int4(const uint8_t *packed, int64_t n_bytes, int8_t *out) {
   for (int64_t i = 0; i < n_bytes; ++i) {

@@ -10,9 +10,12 @@ tree, checks the HIP path against fixed bytes as well as against the live oracle
 
   small_layer.npz    every input and every intermediate of one small fused-MoE call
                      (E=4 of 8 global, top-2, H=256, I=128, M=9, block 16, expert_map,
-                     shared_output, routed_scaling_factor 2.5)
+                     shared_output, routed_scaling_factor 2.5); ref_* in the default (contracted)
+                     scale order, ref_sep_* the stages that differ in the separate order
   tiny_config1.json  the tiny benchmark configuration (E=8, top-2, H=1024, I=512, M=64, seed 0):
-                     routing outputs in full, sha256 of every other stage's bytes
+                     routing outputs in full, sha256 of every other stage's bytes in both scale
+                     orders ("sha256": the default, acc = fma(f32(d) * a_s, b_s, acc);
+                     "sha256_separate_order": acc = acc + (f32(d) * a_s) * b_s)
   tiny_forms.json    the same tiny layer in the per-channel W8A8 form and in the W4A8 form with
                      K-group scales (M=64, seed 0, block 16): sha256 of the inputs and of every stage
   align_docstring.json  the one literal known answer the reference holds
@@ -43,6 +46,9 @@ def sha(t: torch.Tensor) -> str:
     return hashlib.sha256(raw(t).tobytes()).hexdigest()
 
 
+STAGES_AFTER_GEMM1 = ("c1", "act", "a2q", "a2s", "c3", "out")  # what the scale order can change
+
+
 def small_layer():
     layer = wl.MoeLayer("golden-small", E=4, E_global=8, top_k=2, H=256, I=128, routing="softmax")
     w1, w2, w1s, w2s = wl.make_weights(layer, seed=11)
@@ -56,6 +62,11 @@ def small_layer():
     arrays = dict(x=raw(x), w1=raw(w1), w2=raw(w2), w1_scale=raw(w1s), w2_scale=raw(w2s),
                   topk_weights=raw(tw), topk_ids=raw(ids), expert_map=raw(emap), shared_output=raw(shared))
     arrays.update({"ref_" + k: raw(v) for k, v in r.items()})
+    with cpu_oracle.scale_order("separate"):
+        rs = cpu_oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=8,
+                                                 expert_map=emap, routed_scaling_factor=2.5,
+                                                 shared_output=shared, return_intermediates=True)
+    arrays.update({"ref_sep_" + k: raw(rs[k]) for k in STAGES_AFTER_GEMM1})
     np.savez_compressed(os.path.join(HERE, "small_layer.npz"), **arrays)
 
 
@@ -64,6 +75,8 @@ def tiny_config1():
     w1, w2, w1s, w2s = wl.make_weights(layer, seed=0)
     x, tw, ids = wl.make_inputs(layer, 64, seed=0)
     r = cpu_oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
+    with cpu_oracle.scale_order("separate"):
+        rs = cpu_oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
     P = int(r["num_tokens_post_pad"].item())
     doc = {
         "config": "E=8 top-2 H=1024 I=512 M=64 seed 0 block_size_m=16",
@@ -76,6 +89,8 @@ def tiny_config1():
         "sha256": {k: sha(r[k]) for k in ("a1q", "a1s", "c1", "act", "a2q", "a2s", "c3", "out")},
         "out_first_row_bf16_bits": raw(r["out"])[0, :16].tolist(),
         "out_abs_max": float(r["out"].float().abs().max()),
+        "sha256_separate_order": {k: sha(rs[k]) for k in STAGES_AFTER_GEMM1},
+        "out_first_row_bf16_bits_separate_order": raw(rs["out"])[0, :16].tolist(),
     }
     with open(os.path.join(HERE, "tiny_config1.json"), "w") as f:
         json.dump(doc, f, indent=1)
@@ -91,10 +106,14 @@ def tiny_forms():
         doc[name] = {
             "config": f"{layer.name}: E=8 top-2 H=1024 I=512 M=64 seed 0 block_size_m=16",
             "inputs_sha256": {"x": sha(x), "w1": sha(w1), "w2": sha(w2), "w1_scale": sha(w1s), "w2_scale": sha(w2s),
-                              "topk_ids": sha(ids)},
+                              "topk_weights": sha(tw), "topk_ids": sha(ids)},
             "sha256": {k: sha(r[k]) for k in ("a1q", "a1s", "c1", "a2q", "a2s", "c3", "out")},
             "out_first_row_bf16_bits": raw(r["out"])[0, :16].tolist(),
         }
+        if name == "w4a8":  # K-group scales: the scale order matters (the per-channel form scales once, at the end)
+            with cpu_oracle.scale_order("separate"):
+                rs = fn(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
+            doc[name]["sha256_separate_order"] = {k: sha(rs[k]) for k in ("c1", "a2q", "a2s", "c3", "out")}
     with open(os.path.join(HERE, "tiny_forms.json"), "w") as f:
         json.dump(doc, f, indent=1)
 

@@ -53,12 +53,13 @@ def run(dev, layer, M, seed, flags=None, shared=False, on_input=False, ids64=Fal
     return (x, w1, w2, w1s, w2s, tw, ids, emap, sh), outs
 
 
-def oracle_out(oracle, layer, data, on_input=False, shared=False):
+def oracle_out(oracle, layer, data, on_input=False, shared=False, order="contract"):
     x, w1, w2, w1s, w2s, tw, ids, emap, sh = data
-    return oracle.fused_experts_block_int8(
-        x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=layer.E_global, expert_map=emap,
-        apply_router_weight_on_input=on_input, routed_scaling_factor=2.5 if shared else layer.routed_scaling,
-        shared_output=sh)
+    with oracle.scale_order(order):
+        return oracle.fused_experts_block_int8(
+            x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=layer.E_global, expert_map=emap,
+            apply_router_weight_on_input=on_input, routed_scaling_factor=2.5 if shared else layer.routed_scaling,
+            shared_output=sh)
 
 
 def layers():
@@ -77,16 +78,20 @@ def layers():
 
 @pytest.mark.parametrize("name", ["tiny", "ep", "longk", "longk2", "few"])
 @pytest.mark.parametrize("M", [1, 3, 16, 64])
-def test_decode_path_bit_exact(dev, oracle, name, M):
+@pytest.mark.parametrize("order", ["contract", "separate"])
+def test_decode_path_bit_exact(dev, oracle, name, M, order):
+    """Both scale orders the checker restates: the default (acc = fma(f32(d) * a_s, b_s, acc)) and the one without
+    fp fusion (LO_GEMM_SEPARATE_ORDER)."""
     from lightop_amd import _lib
 
     layer = layers()[name]
-    say(f"decode path {name} M={M}")
-    data, outs = run(dev, layer, M, 7, repeat=3)
-    ref = oracle_out(oracle, layer, data)
+    say(f"decode path {name} M={M} order={order}")
+    oflag = _lib.LO_GEMM_SEPARATE_ORDER if order == "separate" else 0
+    data, outs = run(dev, layer, M, 7, repeat=3, flags=_lib.LO_FUSED_FORCE_DECODE_PATH | oflag)
+    ref = oracle_out(oracle, layer, data, order=order)
     for i, out in enumerate(outs):  # repeated calls: the counters of the kernels are back at zero each time
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"call {i}"
-    _, (plain,) = run(dev, layer, M, 7, flags=_lib.LO_FUSED_NO_DECODE_PATH)
+    _, (plain,) = run(dev, layer, M, 7, flags=_lib.LO_FUSED_NO_DECODE_PATH | oflag)
     assert torch.equal(plain.view(torch.int16), ref.view(torch.int16))
 
 

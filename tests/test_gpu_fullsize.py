@@ -118,7 +118,7 @@ CASES = [  # (layer name, M, block sizes)
 
 @pytest.mark.parametrize("name,M,block_sizes", CASES)
 def test_full_size_sampled_tokens_vs_oracle(dev, oracle, name, M, block_sizes):
-    """The library's default arithmetic (the canonical order, the one the benchmark times) at the
+    """The library's default arithmetic (acc = fma(f32(d) * a_s, b_s, acc) per K block, the one the benchmark times) at the
     benchmark's sizes: output rows, int8 activations between the GEMMs and their scales of sampled
     tokens equal the oracle's bit for bit, with both weight layouts and both kernel families; the
     optional fused-scale order stays within the path's tolerance of the oracle."""
@@ -151,6 +151,16 @@ def test_full_size_sampled_tokens_vs_oracle(dev, oracle, name, M, block_sizes):
         assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16))
         assert torch.equal(a2q[loc], ref["a2q"][loc]), f"a2q differs from the oracle in the default order (bs={bs})"
         assert torch.equal(a2s[loc].view(torch.int32), ref["a2s"][loc].view(torch.int32)), f"a2s differs (bs={bs})"
+        # the order without fp fusion: bit-exact against the oracle in that order
+        if bs == block_sizes[-1]:
+            with oracle.scale_order("separate"):
+                ref_s = oracle_rows(oracle, layer, weights, x, tw, ids, emap, tokens, 16, intermediates=True)
+            out_s, a2q_s, a2s_s = run_with_intermediates(layer, weights, x, tw, ids, emap, dev, bs,
+                                                         _lib.LO_GEMM_SEPARATE_ORDER, tokens)
+            assert torch.equal(out_s[tokens].cpu().view(torch.int16), ref_s["out"].view(torch.int16)), \
+                f"separate order: sampled rows differ from the oracle (bs={bs})"
+            assert torch.equal(a2q_s[loc], ref_s["a2q"][loc]) and \
+                torch.equal(a2s_s[loc].view(torch.int32), ref_s["a2s"][loc].view(torch.int32)), f"separate order (bs={bs})"
         # the optional fused-scale order: last-ulp differences in fp32, within the tolerance of the ORACLE
         out_f, a2q_f, a2s_f = run_with_intermediates(layer, weights, x, tw, ids, emap, dev, bs,
                                                      _lib.LO_GEMM_FUSED_SCALE, tokens)

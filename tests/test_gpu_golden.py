@@ -92,7 +92,9 @@ def test_tiny_config1_digests(dev):
     doc = json.load(open(os.path.join(GOLDEN, "tiny_config1.json")))
     w1, w2, w1s, w2s = (t.to(dev) for t in wl.make_weights(wl.TINY, seed=0))
     x, tw, ids = (t.to(dev) for t in wl.make_inputs(wl.TINY, 64, seed=0))
-    assert sha(x) == doc["inputs_sha256"]["x"] and sha(w1) == doc["inputs_sha256"]["w1"]
+    for name, t in (("x", x), ("w1", w1), ("w2", w2), ("w1_scale", w1s), ("w2_scale", w2s), ("topk_weights", tw),
+                    ("topk_ids", ids)):
+        assert sha(t) == doc["inputs_sha256"][name], f"this host's workload generator does not reproduce {name}"
     a1q, a1s = per_token_group_quant_int8(x, 128)
     assert sha(a1q) == doc["sha256"]["a1q"] and sha(a1s) == doc["sha256"]["a1s"]
     s, e, p = moe.moe_align_block_size(ids, 16, 8)
@@ -108,6 +110,21 @@ def test_tiny_config1_digests(dev):
     assert sha(cache13[: 128 * 1024].view(128, 1024)) == doc["sha256"]["c3"]
     assert sha(out) == doc["sha256"]["out"]
     assert bits(out.cpu())[0, :16].tolist() == doc["out_first_row_bf16_bits"]
+    # the order without fp fusion (its c1, act and c3 differ from the default's on this input)
+    from lightop_amd import _lib
+
+    sep = doc["sha256_separate_order"]
+    c1 = torch.zeros(64, 2, 1024, dtype=torch.bfloat16, device=dev)
+    moe.invoke_fused_moe_kernel_int8(a1q, w1, c1, a1s, w1s, tw, s, e, p, False, 2, {"BLOCK_SIZE_M": 16},
+                                     flags=_lib.LO_GEMM_SEPARATE_ORDER)
+    assert sha(c1) == sep["c1"] and sep["c1"] != doc["sha256"]["c1"]
+    out = moe.fused_experts_impl_int8(x, w1, w2, tw, ids, cache13, use_int8_w8a8=True, w1_scale=w1s, w2_scale=w2s,
+                                      block_shape=[128, 128], lightop_amd_block_size_m=16,
+                                      lightop_amd_flags=_lib.LO_GEMM_SEPARATE_ORDER)
+    torch.cuda.synchronize()
+    assert sha(cache13[: 128 * 1024].view(128, 1024)) == sep["c3"] and sep["c3"] != doc["sha256"]["c3"]
+    assert sha(out) == sep["out"]
+    assert bits(out.cpu())[0, :16].tolist() == doc["out_first_row_bf16_bits_separate_order"]
 
 
 @pytest.mark.parametrize("form", ["channel", "w4a8"])
@@ -120,7 +137,9 @@ def test_tiny_forms_digests(dev, form):
     layer = {"channel": wl.TINY_PC, "w4a8": wl.TINY_W4}[form]
     w1, w2, w1s, w2s = (t.to(dev) for t in wl.make_weights(layer, seed=0))
     x, tw, ids = (t.to(dev) for t in wl.make_inputs(layer, 64, seed=0))
-    assert sha(x) == doc["inputs_sha256"]["x"] and sha(w1) == doc["inputs_sha256"]["w1"]
+    for name, t in (("x", x), ("w1", w1), ("w2", w2), ("w1_scale", w1s), ("w2_scale", w2s), ("topk_weights", tw),
+                    ("topk_ids", ids)):
+        assert sha(t) == doc["inputs_sha256"][name], f"this host's workload generator does not reproduce {name}"
     cache13 = torch.empty(64 * 2 * 1024, dtype=torch.bfloat16, device=dev)
     if form == "channel":
         out = moe.fused_experts_impl_int8(x, w1, w2, tw, ids, cache13, use_int8_w8a8=True, per_channel_quant=True,
@@ -128,8 +147,15 @@ def test_tiny_forms_digests(dev, form):
     else:
         out = moe.fused_experts_impl_w4a8(x, moe.preshuffle_moe_weight_int4(w1), moe.preshuffle_moe_weight_int4(w2), tw,
                                           ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=[1, 128],
-                                          lightop_amd_block_size_m=16, lightop_amd_flags=_lib.LO_GEMM_CANONICAL_ORDER)
+                                          lightop_amd_block_size_m=16, lightop_amd_flags=0)
     torch.cuda.synchronize()
     assert sha(cache13[: 128 * 1024].view(128, 1024)) == doc["sha256"]["c3"]
     assert sha(out) == doc["sha256"]["out"]
     assert bits(out.cpu())[0, :16].tolist() == doc["out_first_row_bf16_bits"]
+    if form == "w4a8":  # K-group scales: the order without fp fusion has digests of its own
+        out = moe.fused_experts_impl_w4a8(x, moe.preshuffle_moe_weight_int4(w1), moe.preshuffle_moe_weight_int4(w2), tw,
+                                          ids, cache13, w1_scale=w1s, w2_scale=w2s, block_shape=[1, 128],
+                                          lightop_amd_block_size_m=16, lightop_amd_flags=_lib.LO_GEMM_SEPARATE_ORDER)
+        torch.cuda.synchronize()
+        assert sha(cache13[: 128 * 1024].view(128, 1024)) == doc["sha256_separate_order"]["c3"]
+        assert sha(out) == doc["sha256_separate_order"]["out"]

@@ -235,6 +235,17 @@ def test_moe_sum_expert_mask(dev, oracle):
 
 # --------------------------------------------------------------------- GEMM ----
 
+# The two scale orders the CPU checker restates bit for bit: the library's default, acc = fma(f32(d) * a_s, b_s, acc),
+# and the order without fp fusion, acc = acc + (f32(d) * a_s) * b_s (flag LO_GEMM_SEPARATE_ORDER).
+ORDERS = ["contract", "separate"]
+
+
+def order_flag(order):
+    from lightop_amd import _lib
+
+    return _lib.LO_GEMM_SEPARATE_ORDER if order == "separate" else 0
+
+
 def gemm_case(seed, M, k, E, Eg, N, K, small_values=False):
     g = torch.Generator().manual_seed(seed)
     lo, hi = (-7, 8) if small_values else (-127, 128)
@@ -259,10 +270,11 @@ def gemm_case(seed, M, k, E, Eg, N, K, small_values=False):
                                           (64, 2, 8, 8, 1024, 1024), (100, 8, 4, 16, 512, 768),
                                           (300, 2, 3, 3, 128, 2048)])
 @pytest.mark.parametrize("bs", BS_ALL)
-def test_gemm_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
+@pytest.mark.parametrize("order", ORDERS)
+def test_gemm_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs, order):
     from lightop_amd.moe import invoke_fused_moe_kernel_int8, moe_align_block_size, preshuffle_moe_weight
 
-    say(f"gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs}")
+    say(f"gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs} order={order}")
     Aq, As, W, Ws, ids, tw, emap = gemm_case(M + N + bs, M, k, E, Eg, N, K)
     rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
     S = M * k
@@ -271,13 +283,14 @@ def test_gemm_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
     Wd = W.to(dev)
     Wsh = preshuffle_moe_weight(Wd)
     for mul in (False, True):
-        ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, k, S, bs)
+        with oracle.scale_order(order):
+            ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, k, S, bs)
         for force_streaming in impls:
             for Wx in (Wd, Wsh):  # row-major and load-time pre-shuffled weights
                 C = torch.full((M, k, N), 7.0, dtype=torch.bfloat16, device=dev)
                 s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
                 invoke_fused_moe_kernel_int8(Aq.to(dev), Wx, C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p,
-                                             mul, k, {"BLOCK_SIZE_M": bs}, fused_scale=False, flags=force_streaming)
+                                             mul, k, {"BLOCK_SIZE_M": bs}, flags=force_streaming | order_flag(order))
                 torch.cuda.synchronize()
                 assert torch.equal(C.view(S, N).cpu().view(torch.int16), ref.view(torch.int16)), \
                     f"mul_routed={mul} flags={force_streaming} preshuffled={Wx is Wsh}"
@@ -314,10 +327,11 @@ def test_gemm_int32_accumulators_exact(dev, oracle, bs):
 @pytest.mark.parametrize("M,k,E,Eg,I,K", [(1, 2, 4, 4, 128, 256), (9, 2, 4, 4, 256, 512), (64, 2, 8, 8, 512, 1024),
                                           (50, 8, 4, 16, 256, 768), (200, 4, 6, 6, 384, 1024)])
 @pytest.mark.parametrize("bs", BS_ALL)
-def test_gemm1_silu_quant_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
+@pytest.mark.parametrize("order", ORDERS)
+def test_gemm1_silu_quant_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs, order):
     from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_weight
 
-    say(f"gemm1+silu+quant M={M} k={k} E={E}/{Eg} I={I} K={K} bs={bs}")
+    say(f"gemm1+silu+quant M={M} k={k} E={E}/{Eg} I={I} K={K} bs={bs} order={order}")
     Aq, As, W, Ws, ids, tw, emap = gemm_case(M + I + bs + 1, M, k, E, Eg, 2 * I, K)
     Ws = Ws * 30  # bring the gate into the range where SiLU is neither 0 nor identity
     rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
@@ -325,13 +339,14 @@ def test_gemm1_silu_quant_bit_exact(dev, oracle, M, k, E, Eg, I, K, bs):
     s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
     impls = (0, 2) if bs >= 64 else (0,)
     for mul in (False, True):
-        c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, k, S, bs)
+        with oracle.scale_order(order):
+            c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, k, S, bs)
         rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
         for force_streaming in impls:
             for Wx in (W.to(dev), preshuffle_moe_weight(W.to(dev))):
                 q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wx, As.to(dev), Ws.to(dev), tw.to(dev),
-                                                          s, e, p, mul, k, S, {"BLOCK_SIZE_M": bs}, fused_scale=False,
-                                                          flags=force_streaming)
+                                                          s, e, p, mul, k, S, {"BLOCK_SIZE_M": bs},
+                                                          flags=force_streaming | order_flag(order))
                 torch.cuda.synchronize()
                 local = torch.ones(S, dtype=torch.bool) if emap is None else emap.long()[ids.reshape(-1).long()] >= 0
                 what = f"mul_routed={mul}, flags={force_streaming}, preshuffled={hasattr(Wx, 'lo_preshuffled')}"
@@ -445,7 +460,8 @@ def test_gemm_sorted_ids_with_gaps(dev, oracle, bs):
 
 @pytest.mark.parametrize("count,K", [(c, 384) for c in (1, 31, 32, 33, 64, 65, 96, 97, 127, 128, 129, 200)] +
                          [(c, k) for k in (128, 256, 1024) for c in (40, 128, 250)])
-def test_gemm_128_token_blocks_fill_levels(dev, oracle, count, K):
+@pytest.mark.parametrize("order", ORDERS)
+def test_gemm_128_token_blocks_fill_levels(dev, oracle, count, K, order):
     """128-token blocks holding 1 ... 128 valid tokens: the K loop of the 128-token kernel comes in
     variants by the number of 32-token pieces in use, and padded pieces are skipped.  One, two and
     eight K blocks as well: the full-tile variant reads a K block's first operands during the
@@ -453,7 +469,7 @@ def test_gemm_128_token_blocks_fill_levels(dev, oracle, count, K):
     from lightop_amd.moe import (invoke_fused_moe_gemm1_silu_quant, invoke_fused_moe_kernel_int8,
                                  moe_align_block_size, preshuffle_moe_weight)
 
-    say(f"128-token blocks, {count} tokens on expert 0, K = {K}")
+    say(f"128-token blocks, {count} tokens on expert 0, K = {K}, order={order}")
     bs, E, I = 128, 2, 128
     M = count + 3
     Aq, As, W, Ws, _, tw, _ = gemm_case(count, M, 1, E, E, 2 * I, K)
@@ -463,16 +479,17 @@ def test_gemm_128_token_blocks_fill_levels(dev, oracle, count, K):
     rs, re, rp = oracle.moe_align_block_size(ids, bs, E)
     s, e, p = moe_align_block_size(ids.to(dev), bs, E)
     Wsh = preshuffle_moe_weight(W.to(dev))
-    ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, True, 1, M, bs)
+    with oracle.scale_order(order):
+        ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, True, 1, M, bs)
+        c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, False, 1, M, bs)
     C = torch.full((M, 1, 2 * I), 7.0, dtype=torch.bfloat16, device=dev)
     invoke_fused_moe_kernel_int8(Aq.to(dev), Wsh, C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, True, 1,
-                                 {"BLOCK_SIZE_M": bs}, fused_scale=False)
+                                 {"BLOCK_SIZE_M": bs}, flags=order_flag(order))
     torch.cuda.synchronize()
     assert torch.equal(C.view(M, -1).cpu().view(torch.int16), ref.view(torch.int16))
-    c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, False, 1, M, bs)
     rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
     q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wsh, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, False, 1,
-                                              M, {"BLOCK_SIZE_M": bs}, fused_scale=False)
+                                              M, {"BLOCK_SIZE_M": bs}, flags=order_flag(order))
     torch.cuda.synchronize()
     assert torch.equal(sc.cpu(), rsc) and torch.equal(q.cpu(), rq)
 
@@ -519,13 +536,16 @@ def run_fused(dev, layer, M, seed, bs=0, flags=0, shared=False, on_input=False, 
 
 @pytest.mark.parametrize("bs", BS_ALL)
 @pytest.mark.parametrize("preshuffle", [False, True])
-def test_fused_experts_tiny_config_bit_exact(dev, oracle, bs, preshuffle):
+@pytest.mark.parametrize("order", ORDERS)
+def test_fused_experts_tiny_config_bit_exact(dev, oracle, bs, preshuffle, order):
     """The tiny benchmark configuration: E=8, top-2, H=1024, I=512, M=64, seed 0."""
     from lightop_amd import workloads as wl
 
-    say(f"fused tiny bs={bs} preshuffle={preshuffle}")
-    (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, wl.TINY, 64, 0, bs=bs, preshuffle=preshuffle)
-    ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, bs)
+    say(f"fused tiny bs={bs} preshuffle={preshuffle} order={order}")
+    (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, wl.TINY, 64, 0, bs=bs, preshuffle=preshuffle,
+                                                              flags=order_flag(order))
+    with oracle.scale_order(order):
+        ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, bs)
     assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
 
@@ -557,6 +577,10 @@ def test_fused_experts_default_tile_and_fused_scale(dev, oracle):
         (x, w1, w2, w1s, w2s, tw, ids, emap, sh), out = run_fused(dev, layer, 200, 1, preshuffle=pre)
         ref = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 64)
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"default order, preshuffle={pre}"
+        _, out_s = run_fused(dev, layer, 200, 1, flags=_lib.LO_GEMM_SEPARATE_ORDER, preshuffle=pre)
+        with oracle.scale_order("separate"):
+            ref_s = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 64)
+        assert torch.equal(out_s.view(torch.int16), ref_s.view(torch.int16)), f"separate order, preshuffle={pre}"
         _, out_f = run_fused(dev, layer, 200, 1, flags=_lib.LO_GEMM_FUSED_SCALE, preshuffle=pre)
         assert within_tolerance(out_f, ref)
 

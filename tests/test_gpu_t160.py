@@ -57,19 +57,23 @@ def test_gemm_160_token_blocks_fill_levels(dev, oracle, count, K):
     s, e, p = moe_align_block_size(ids.to(dev), bs, E)
     assert torch.equal(s.cpu()[: int(rp[0])], rs[: int(rp[0])]) and torch.equal(e.cpu()[: int(rp[0]) // bs], re[: int(rp[0]) // bs])
     Wsh = preshuffle_moe_weight(W.to(dev))
+    from lightop_amd import _lib
+
     for mul in (False, True):
-        for fused_scale in (False, True):
-            ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, 1, M, bs)
+        # the default order, the order without fp fusion (both bit-exact) and the fused-scale order
+        for order, flags in (("contract", 0), ("separate", _lib.LO_GEMM_SEPARATE_ORDER), ("fused", _lib.LO_GEMM_FUSED_SCALE)):
+            with oracle.scale_order("contract" if order == "fused" else order):
+                ref = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, 1, M, bs)
             C = torch.full((M, 1, N), 7.0, dtype=torch.bfloat16, device=dev)
             invoke_fused_moe_kernel_int8(Aq.to(dev), Wsh, C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, mul, 1,
-                                         {"BLOCK_SIZE_M": bs}, fused_scale=fused_scale)
+                                         {"BLOCK_SIZE_M": bs}, flags=flags)
             torch.cuda.synchronize()
             got = C.view(M, -1).cpu()
-            if fused_scale:  # the optional order: last-ulp differences in fp32
+            if order == "fused":  # the optional order: last-ulp differences in fp32
                 err = (got.float() - ref.float()).abs()
                 assert err.max() <= 1e-2 * ref.float().abs().max()
             else:
-                assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"mul_routed={mul}"
+                assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"mul_routed={mul} order={order}"
 
 
 @pytest.mark.parametrize("M,k,E,Eg,N,K", [(5, 2, 4, 4, 256, 512), (400, 4, 8, 8, 320, 1152), (900, 8, 4, 16, 512, 768),

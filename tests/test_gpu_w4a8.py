@@ -39,21 +39,24 @@ def gemm_case(seed, M, k, E, Eg, N, K):
 @pytest.mark.parametrize("M,k,E,Eg,N,K", [(1, 2, 4, 4, 64, 128), (5, 2, 4, 4, 256, 512), (40, 4, 8, 8, 320, 1024),
                                           (100, 8, 4, 16, 512, 768), (300, 2, 3, 3, 128, 2048)])
 @pytest.mark.parametrize("bs", [16, 32, 64, 128])
-def test_gemm_w4a8_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs):
+@pytest.mark.parametrize("order", ["contract", "separate"])
+def test_gemm_w4a8_bit_exact(dev, oracle, M, k, E, Eg, N, K, bs, order):
     from lightop_amd import _lib
     from lightop_amd.moe import (invoke_fused_moe_kernel_int8, moe_align_block_size, preshuffle_moe_scale_int4,
                                  preshuffle_moe_weight_int4)
 
-    say(f"w4a8 gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs}")
+    say(f"w4a8 gemm M={M} k={k} E={E}/{Eg} N={N} K={K} bs={bs} order={order}")
+    oflag = _lib.LO_GEMM_SEPARATE_ORDER if order == "separate" else 0
     Aq, As, W4, Ws, ids, tw, emap = gemm_case(M + N + bs, M, k, E, Eg, N, K)
     rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
     s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
     Wd = preshuffle_moe_weight_int4(W4.to(dev))
     for mul in (False, True):
-        ref = oracle.moe_gemm_w4a8(Aq, As, W4, Ws, rs, re, rp, tw, mul, k, M * k, bs)
+        with oracle.scale_order(order):
+            ref = oracle.moe_gemm_w4a8(Aq, As, W4, Ws, rs, re, rp, tw, mul, k, M * k, bs)
         C = torch.empty((M, k, N), dtype=torch.bfloat16, device=dev)
         invoke_fused_moe_kernel_int8(Aq.to(dev), Wd, C, As.to(dev), preshuffle_moe_scale_int4(Ws.to(dev)), tw.to(dev), s, e, p, mul, k,
-                                     {"BLOCK_SIZE_M": bs}, fused_scale=False, flags=_lib.LO_GEMM_W4)
+                                     {"BLOCK_SIZE_M": bs}, flags=_lib.LO_GEMM_W4 | oflag)
         torch.cuda.synchronize()
         assert torch.equal(C.cpu().view(M * k, N).view(torch.int16), ref.view(torch.int16)), f"mul_routed={mul}"
 
@@ -116,7 +119,7 @@ def test_whole_path_tiny_bit_exact(dev, oracle, bs, with_map):
               preshuffle_moe_weight_int4(w2[:5].contiguous().to(dev)), w1s[:5].contiguous().to(dev),
               w2s[:5].contiguous().to(dev))
     out = run_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None if emap is None else emap.to(dev), dev, bs,
-                   _lib.LO_GEMM_CANONICAL_ORDER)
+                   0)
     ref = oracle.fused_experts_w4a8(x, w1[:5] if with_map else w1, w2[:5] if with_map else w2,
                                     w1s[:5] if with_map else w1s, w2s[:5] if with_map else w2s, tw, ids, 16,
                                     global_num_experts=layer.E, expert_map=emap)
@@ -137,14 +140,15 @@ def test_whole_path_long_k_bit_exact(dev, oracle, bs):
         x, tw, ids = wl.make_inputs(layer, 40, seed=H)
         wd = (preshuffle_moe_weight_int4(w1.to(dev)), preshuffle_moe_weight_int4(w2.to(dev)), w1s.to(dev), w2s.to(dev))
         out = run_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None, dev, bs,
-                       _lib.LO_GEMM_CANONICAL_ORDER | _lib.LO_FUSED_NO_DECODE_PATH)
+                       _lib.LO_FUSED_NO_DECODE_PATH)
         ref = oracle.fused_experts_w4a8(x, w1, w2, w1s, w2s, tw, ids, 16, global_num_experts=layer.E)
         assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
 @pytest.mark.parametrize("M", [1, 5, 40, 200])
 @pytest.mark.parametrize("with_map", [False, True])
-def test_two_launch_path_w4a8_bit_exact(dev, oracle, M, with_map):
+@pytest.mark.parametrize("order", ["contract", "separate"])
+def test_two_launch_path_w4a8_bit_exact(dev, oracle, M, with_map, order):
     """The two-launch path for a few tokens on packed int4 weights (forced beyond its default size)."""
     from lightop_amd import _lib, workloads as wl
     from lightop_amd.moe import preshuffle_moe_weight_int4
@@ -160,11 +164,13 @@ def test_two_launch_path_w4a8_bit_exact(dev, oracle, M, with_map):
         emap[:n] = torch.arange(n, dtype=torch.int32)
     wd = (preshuffle_moe_weight_int4(w1[:n].contiguous().to(dev)), preshuffle_moe_weight_int4(w2[:n].contiguous().to(dev)),
           w1s[:n].contiguous().to(dev), w2s[:n].contiguous().to(dev))
-    ref = oracle.fused_experts_w4a8(x, w1[:n], w2[:n], w1s[:n], w2s[:n], tw, ids, 16, global_num_experts=layer.E,
-                                    expert_map=emap)
+    with oracle.scale_order(order):
+        ref = oracle.fused_experts_w4a8(x, w1[:n], w2[:n], w1s[:n], w2s[:n], tw, ids, 16, global_num_experts=layer.E,
+                                        expert_map=emap)
+    oflag = _lib.LO_GEMM_SEPARATE_ORDER if order == "separate" else 0
     for _ in range(2):
         out = run_path(layer, wd, x.to(dev), tw.to(dev), ids.to(dev), None if emap is None else emap.to(dev), dev, 0,
-                       _lib.LO_FUSED_FORCE_DECODE_PATH)
+                       _lib.LO_FUSED_FORCE_DECODE_PATH | oflag)
         assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
@@ -211,9 +217,14 @@ def test_baseline_int4_layer_sampled_tokens(dev, oracle, M):
     sel = used.to(dev)
     ref = oracle.fused_experts_w4a8(x[tokens].cpu(), w1[sel].cpu(), w2[sel].cpu(), w1s[sel].cpu(), w2s[sel].cpu(),
                                     tw[tokens].cpu(), remap[sub_ids].to(torch.int32), 16)
-    out = run_path(layer, (w1p, w2p, w1sp, w2sp), x, tw, ids, None, dev, 0, _lib.LO_GEMM_CANONICAL_ORDER)
+    out = run_path(layer, (w1p, w2p, w1sp, w2sp), x, tw, ids, None, dev, 0, 0)
     assert torch.equal(out[tokens].cpu().view(torch.int16), ref.view(torch.int16))
-    out2 = run_path(layer, (w1p, w2p, w1sp, w2sp), x, tw, ids, None, dev, 0, 0)  # library default order
+    with oracle.scale_order("separate"):
+        ref_s = oracle.fused_experts_w4a8(x[tokens].cpu(), w1[sel].cpu(), w2[sel].cpu(), w1s[sel].cpu(), w2s[sel].cpu(),
+                                          tw[tokens].cpu(), remap[sub_ids].to(torch.int32), 16)
+    out_s = run_path(layer, (w1p, w2p, w1sp, w2sp), x, tw, ids, None, dev, 0, _lib.LO_GEMM_SEPARATE_ORDER)
+    assert torch.equal(out_s[tokens].cpu().view(torch.int16), ref_s.view(torch.int16))
+    out2 = run_path(layer, (w1p, w2p, w1sp, w2sp), x, tw, ids, None, dev, 0, _lib.LO_GEMM_FUSED_SCALE)  # within the tolerance
     err = (out2.float() - out.float()).abs()
     assert err.max() <= 1e-2 * out.float().abs().max() and err.sum() <= 2e-3 * out.float().abs().sum()
 

@@ -244,6 +244,12 @@ def test_golden_tiny_config1_oracle(oracle):
     assert r["expert_ids"][: P // 16].tolist() == doc["expert_ids"]
     for k, h in doc["sha256"].items():
         assert sha(r[k]) == h, k
+    # the order without fp fusion: its digests differ from the default's in c1, act and c3 on this input
+    with oracle.scale_order("separate"):
+        rs = oracle.fused_experts_block_int8(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
+    for k, h in doc["sha256_separate_order"].items():
+        assert sha(rs[k]) == h, k
+    assert any(doc["sha256_separate_order"][k] != doc["sha256"][k] for k in doc["sha256_separate_order"])
 
 
 @pytest.mark.parametrize("form", ["channel", "w4a8"])
@@ -266,6 +272,10 @@ def test_golden_tiny_forms_oracle(oracle, form):
     r = fn(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
     for k, h in doc["sha256"].items():
         assert sha(r[k]) == h, k
+    with oracle.scale_order("separate"):  # the per-channel form scales once, at the end: no order to choose
+        rs = fn(x, w1, w2, w1s, w2s, tw, ids, 16, return_intermediates=True)
+    for k, h in doc.get("sha256_separate_order", {k: doc["sha256"][k] for k in ("c1", "c3", "out")}).items():
+        assert sha(rs[k]) == h, k
 
 
 def test_golden_align_docstring(oracle):

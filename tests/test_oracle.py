@@ -181,19 +181,85 @@ def test_gemm_int32_exact_vs_python_integers(oracle):
 
 
 def test_gemm_scale_order_and_router_weight(oracle):
-    # one token, one expert, K=256: acc = (d0*as0)*ws0 + (d1*as1)*ws1, then * w, then bf16
+    # the order without fp fusion: one token, one expert, K=256: acc = (d0*as0)*ws0 + (d1*as1)*ws1, then * w, then bf16
     Aq = torch.zeros(1, 256, dtype=torch.int8); Aq[0, 0] = 100; Aq[0, 128] = -7
     W = torch.zeros(1, 16, 256, dtype=torch.int8); W[0, :, 0] = 3; W[0, :, 128] = 11
     As = torch.tensor([[0.37, 1.9]]); Ws = torch.tensor([[[0.0123, 0.5]]])
     ids = torch.zeros(1, 1, dtype=torch.int32); tw = torch.tensor([[0.731]])
     s, e, p = oracle.moe_align_block_size(ids, 16, 1)
-    C = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, tw, True, 1, 1, 16)
+    with oracle.scale_order("separate"):
+        C = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, tw, True, 1, 1, 16)
     f = np.float32
     acc = f(0) + (f(300) * f(0.37)) * f(0.0123)
     acc = acc + (f(-77) * f(1.9)) * f(0.5)
     acc = acc * f(0.731)
     assert C[0, 0].item() == torch.tensor(float(acc)).to(torch.bfloat16).item()
     assert (C[0] == C[0, 0]).all()
+
+
+def _round_to_f32(q):
+    """The float32 nearest to the rational q, ties to even: exact integer arithmetic, no float operation decides."""
+    from fractions import Fraction
+
+    if q == 0:
+        return np.float32(0.0)
+    c = np.float32(float(q))  # a float32 within an ulp or two of q; the neighbours are compared exactly
+    cands = [c, np.nextafter(c, np.float32(np.inf)), np.nextafter(c, np.float32(-np.inf))]
+    cands += [np.nextafter(cands[1], np.float32(np.inf)), np.nextafter(cands[2], np.float32(-np.inf))]
+    best = min(cands, key=lambda v: (abs(Fraction(float(v)) - q), int(np.float32(v).view(np.uint32)) & 1))
+    return np.float32(best)
+
+
+def test_gemm_contracted_order_hand_worked(oracle):
+    """The default order, acc = fma(f32(d) * a_s, b_s, acc): the product f32(d) * a_s is rounded, the second
+    product and the sum are rounded once, together.  Expected values from exact rational arithmetic; the
+    sixteen rows carry different sums, the fp32 output shows every rounding, and the two orders must differ
+    on some row, so that taking one for the other fails here."""
+    from fractions import Fraction
+
+    Aq = torch.zeros(1, 384, dtype=torch.int8); Aq[0, 0] = 100; Aq[0, 128] = -7; Aq[0, 256] = 53
+    W = torch.zeros(1, 16, 384, dtype=torch.int8)
+    for n in range(16):
+        W[0, n, 0] = 3 + 7 * n; W[0, n, 128] = 11 - 5 * n; W[0, n, 256] = 9 * n - 60
+    As = torch.tensor([[0.37, 1.9, 0.0421]]); Ws = torch.tensor([[[0.0123, 0.5003, 0.00917]]])
+    ids = torch.zeros(1, 1, dtype=torch.int32); tw = torch.tensor([[0.731]])
+    s, e, p = oracle.moe_align_block_size(ids, 16, 1)
+    f = np.float32
+    want_c, want_s = [], []
+    for n in range(16):
+        d = [100 * (3 + 7 * n), -7 * (11 - 5 * n), 53 * (9 * n - 60)]
+        acc_c, acc_s = f(0), f(0)
+        for kb in range(3):
+            t = f(d[kb]) * f(As[0, kb].item())                      # rounded on its own in both orders
+            b = f(Ws[0, 0, kb].item())
+            acc_c = _round_to_f32(Fraction(float(t)) * Fraction(float(b)) + Fraction(float(acc_c)))
+            acc_s = acc_s + t * b                                   # numpy float32: every operation rounded
+        want_c.append(acc_c); want_s.append(acc_s)
+    assert any(a != b for a, b in zip(want_c, want_s)), "the case no longer tells the orders apart"
+    for order, want in (("contract", want_c), ("separate", want_s)):
+        with oracle.scale_order(order):
+            Cf = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, None, False, 1, 1, 16,
+                                            out=torch.zeros(1, 16, dtype=torch.float32))
+            Cw = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, tw, True, 1, 1, 16)
+        assert Cf[0].tolist() == [float(v) for v in want], order
+        assert Cw[0].tolist() == [torch.tensor(float(v * f(0.731))).to(torch.bfloat16).item() for v in want], order
+    # the default is the contracted order
+    Cd = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, None, False, 1, 1, 16, out=torch.zeros(1, 16, dtype=torch.float32))
+    assert Cd[0].tolist() == [float(v) for v in want_c]
+
+
+def test_gemm_scale_orders_differ_in_bf16_somewhere(oracle):
+    """On a few thousand random sums the two orders give different bf16 outputs now and then (and never by more
+    than one bf16 ulp): a kernel test that compares bf16 rows can therefore tell them apart."""
+    Aq, As, W, Ws, ids, tw, Eg = _small_gemm_case(21, 64, 2, 2, 256, 1024, 16)
+    s, e, p = oracle.moe_align_block_size(ids, 16, Eg)
+    with oracle.scale_order("contract"):
+        Cc = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, None, False, 2, 128, 16)
+    with oracle.scale_order("separate"):
+        Cs = oracle.moe_gemm_block_int8(Aq, As, W, Ws, s, e, p, None, False, 2, 128, 16)
+    diff = (Cc.view(torch.int16) != Cs.view(torch.int16))
+    assert 0 < diff.sum().item() < 0.05 * diff.numel()
+    assert ((Cc.view(torch.int16).int() - Cs.view(torch.int16).int()).abs() <= 1).all()
 
 
 def test_gemm_vs_torch_restatement_and_skipped_experts(oracle):
