@@ -11,9 +11,12 @@ overwritten: an overwrite leaves the cache full of dirty lines whose write-back 
 inside the timed step - 5 to 25 us of it, `--flush write` shows the difference); the
 step time is taken with HIP events on the launching stream and excludes that flush.
 ms_per_step is the median of the timed steps (mean and min are reported next to it).  The
-headline is timed in the library's default arithmetic (canonical scale order, the mode the GPU
-parity tests compare bit for bit with the CPU checker); ms_per_step_fused_scale is the same call
-with LO_GEMM_FUSED_SCALE.  The last line printed is one JSON object (fields: metric, value, unit,
+headline is timed in the library's default arithmetic (acc = fma(f32(d) * a_s, b_s, acc) per K block, the
+mode the GPU parity tests compare bit for bit with the CPU checker); ms_per_step_separate_order and
+ms_per_step_fused_scale are the same call with LO_GEMM_SEPARATE_ORDER and LO_GEMM_FUSED_SCALE.  `roofline`
+also carries, as flat scalars, the sweep's figures for the targets of the path (the DeepSeek-V3-shaped
+layer at M >= 4096 against the int8 MFMA peak, M <= 64 against the HBM peak) and the ceiling the scale
+arithmetic puts on the matrix pipe (fold_insts_per_elem, mfma_cap_frac, achieved_over_cap).  The last line printed is one JSON object (fields: metric, value, unit,
 ms_per_step, roofline, cpu_baseline, stage_ms, routers, sweep).
 """
 from __future__ import annotations
@@ -73,9 +76,11 @@ def parse_args():
     p.add_argument("--block-size-m", type=int, default=0)
     p.add_argument("--row-major-weights", action="store_true",
                    help="keep w1/w2 row-major instead of the load-time pre-shuffled layout")
-    p.add_argument("--fused-scale", type=int, default=0,
-                   help="0: canonical scale order (the library default, bit-exact against the CPU checker); "
-                        "1: fused-scale order (LO_GEMM_FUSED_SCALE, tolerance-matched)")
+    p.add_argument("--scale-order", default="contract", choices=["contract", "separate", "fused"],
+                   help="scale arithmetic per 128-wide K block.  contract: acc = fma(f32(d) * a_s, b_s, acc), the "
+                        "library default, bit-exact against the CPU checker; separate: acc + (f32(d) * a_s) * b_s "
+                        "(LO_GEMM_SEPARATE_ORDER, bit-exact against the checker in that order); fused: "
+                        "fma(f32(d), a_s * b_s, acc) (LO_GEMM_FUSED_SCALE, tolerance-matched)")
     return p.parse_args()
 
 
@@ -156,7 +161,7 @@ class Point:
             expert_map=self.emap, w1_scale=self.w1s, w2_scale=self.w2s, block_shape=[128, 128],
             lightop_amd_block_size_m=bs, lightop_amd_flags=flags)
 
-    def stage_times(self, steps, warmup, flush, bs=0, fused_scale=None):
+    def stage_times(self, steps, warmup, flush, bs=0, order_flags=0):
         """Event-timed duration of each stage kernel launched on its own (ms, median)."""
         from lightop_amd import moe
         from lightop_amd.quant import per_token_group_quant_int8
@@ -200,15 +205,15 @@ class Point:
             if bs == 160:  # 160-token blocks: plain first GEMM, activation and quantisation in a launch of their own
                 c1 = self.cache13[: S * 2 * L.I].view(S, 2 * L.I)
                 moe.invoke_fused_moe_kernel_int8(a1q, self.w1, c1, a1s, self.w1s, tw, s, e, p, False, L.top_k, cfg,
-                                                 fused_scale=fused_scale, flags=g2flag, global_num_experts=L.E_global)
+                                                 flags=g2flag | order_flags, global_num_experts=L.E_global)
                 a2q, a2s = moe.act_and_mul_group_quant(c1, row_mask=mask, out=(a2q_buf, a2s_buf))
             else:
                 a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
-                                                                 L.top_k, S, cfg, fused_scale=fused_scale,
-                                                                 flags=wflag, global_num_experts=L.E_global)
+                                                                 L.top_k, S, cfg,
+                                                                 flags=wflag | order_flags, global_num_experts=L.E_global)
             ev[3].record()
             moe.invoke_fused_moe_kernel_int8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, True, 1, cfg,
-                                             fused_scale=fused_scale, flags=g2flag, global_num_experts=L.E_global)
+                                             flags=g2flag | order_flags, global_num_experts=L.E_global)
             ev[4].record()
             moe.moe_sum(c3, out, expert_mask=mask)
             ev[5].record()
@@ -456,8 +461,13 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     flush = Flusher(dev, args.flush)
-    flags_default = _lib.LO_GEMM_FUSED_SCALE if args.fused_scale == 1 else 0
-    flags_other = 0 if args.fused_scale == 1 else _lib.LO_GEMM_FUSED_SCALE
+    order_flag = {"contract": 0, "separate": _lib.LO_GEMM_SEPARATE_ORDER, "fused": _lib.LO_GEMM_FUSED_SCALE}
+    flags_default = order_flag[args.scale_order]
+    # vector instructions the fold spends per accumulator element and K block, and the share of the
+    # matrix pipe's time they leave it at best: an element's two MFMAs cost 8 cycles of matrix pipe, every
+    # vector instruction 4 cycles of the SIMD's vector ALU, and the two run side by side
+    fold_insts = {"contract": 3, "separate": 4, "fused": 2}[args.scale_order]
+    mfma_cap = min(1.0, 8.0 / (4.0 * fold_insts))
 
     from lightop_amd.moe import preshuffle_moe_scale_int4, preshuffle_moe_weight, preshuffle_moe_weight_int4
 
@@ -480,12 +490,26 @@ def main():
     weights = load_weights(layer, keep_cpu_copy=not args.no_cpu_baseline and layer.weight_bytes < 8e9)
     pt = Point(layer, weights, args.tokens, dev)
     head = measure_point(pt, args.steps, args.warmup, flush, args.block_size_m, flags_default)
-    # the other scale order, for comparison (block form only: the per-channel form has one order)
-    other = None
+    # the other scale orders, for comparison (block form only: the per-channel form has one order)
+    others = {}
     if layer.quant != "channel":
-        other = time_steps(lambda: pt.step(args.block_size_m, flags_other), args.steps, args.warmup, flush)
-    stages, bs_used = pt.stage_times(args.steps, args.warmup, flush, args.block_size_m,
-                                     fused_scale=args.fused_scale == 1)
+        for name, fl in order_flag.items():
+            if name != args.scale_order:
+                others[name] = time_steps(lambda: pt.step(args.block_size_m, fl), args.steps, args.warmup, flush)[1]
+    stages, bs_used = pt.stage_times(args.steps, args.warmup, flush, args.block_size_m, order_flags=flags_default)
+    # host time of one call at one token: launches and marshalling only, nothing waited for
+    host_us = None
+    if layer.quant != "channel":
+        p1 = Point(layer, weights, 1, dev, pool=1)
+        for _ in range(20):
+            p1.step(0, flags_default)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(200):
+            p1.step(0, flags_default)
+        host_us = (time.perf_counter() - t0) / 200 * 1e6
+        torch.cuda.synchronize()
+        del p1
     shape = None if layer.quant == "channel" else ([1, 128] if layer.weight_bits == 4 else [128, 128])
     from lightop_amd import moe as _moe
     tile1, tile2 = _moe.get_w8a8moe_json(args.tokens, layer.E, 2 * layer.I, layer.H, layer.I, True, shape, layer.top_k,
@@ -522,7 +546,9 @@ def main():
                                         "(SiLU*mul + 1x128 re-quant)" if bs_used == 160
                                    else "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)"),
                 "kernel_ms": round(stages[g1_name], 4),
-                "scale_order": "fused" if args.fused_scale == 1 else "canonical",
+                "scale_order": args.scale_order,
+                "fold_insts_per_elem": fold_insts if L.quant != "channel" else 0,
+                "mfma_cap_frac": round(mfma_cap, 3) if L.quant != "channel" else 1.0,
                 "profile": None if prof is None else prof["file"],
                 "profile_kernel_us": None if prof is None else {k: prof[k] for k in ("avg_us", "median_us", "min_us")},
                 "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately); kernel_ms is the "
@@ -555,14 +581,52 @@ def main():
     if cpu_weights:
         cpu = cpu_baseline(layer, cpu_weights, min(args.tokens, 8192))
 
+    # The targets of the path, as flat scalars next to the dominant kernel's figures: the DeepSeek-V3-shaped
+    # layer at M >= 4096 against the int8 MFMA peak, decode sizes against the HBM peak.
+    def sw(workload, M, key, scale=1.0):
+        for r in sweep:
+            if r["workload"] == workload and r["tokens"] == M:
+                return None if r.get(key) is None else round(r[key] * scale, 4)
+        return None
+
+    def hot_bucket():
+        for r in sweep:
+            if r["workload"] == "deepseek-v3-full":
+                for b in r.get("expert_buckets", []):
+                    if b["bucket"].startswith("compute-bound"):
+                        return b["frac_mfma"]
+        return None
+
+    roofline.update({
+        "achieved_over_cap": round(roofline["frac"] / roofline["mfma_cap_frac"], 4) if head["bound"] == "mfma" else None,
+        "gemm2_ms": round(stages.get("gemm2", 0.0), 4), "moe_sum_ms": round(stages.get("moe_sum", 0.0), 4),
+        "profile_avg_us": None if prof is None else prof["avg_us"],
+        "profile_median_us": None if prof is None else prof["median_us"],
+        "ms_per_step_fused_scale": None if "fused" not in others else round(others["fused"], 4),
+        "dsv3_full_M8192_ms": sw("deepseek-v3-full", 8192, "ms_per_step"),
+        "dsv3_full_M8192_frac_mfma": sw("deepseek-v3-full", 8192, "frac_mfma"),
+        "dsv3_full_hot_bucket_frac_mfma": hot_bucket(),
+        "dsv3_ep_M4096_ms": sw("deepseek-v3-ep8-share", 4096, "ms_per_step"),
+        "dsv3_ep_M4096_frac_hbm": sw("deepseek-v3-ep8-share", 4096, "frac_hbm"),
+        "dsv3_ep_M64_frac_hbm": sw("deepseek-v3-ep8-share", 64, "frac_hbm"),
+        "dsv3_ep_M16_frac_hbm": sw("deepseek-v3-ep8-share", 16, "frac_hbm"),
+        "dsv3_ep_M1_us": sw("deepseek-v3-ep8-share", 1, "ms_per_step", 1e3),
+        "qwen3_M2048_ms": sw("qwen3-30b-a3b", 2048, "ms_per_step"),
+        "qwen3_M32_frac_hbm": sw("qwen3-30b-a3b", 32, "frac_hbm"),
+        "qwen3_M8_frac_hbm": sw("qwen3-30b-a3b", 8, "frac_hbm"),
+        "qwen3_M1_us": sw("qwen3-30b-a3b", 1, "ms_per_step", 1e3),
+        "w4a8_M2048_ms": sw("qwen3-235b-a22b-w4a8", 2048, "ms_per_step"),
+        "w4a8_M256_frac_hbm": sw("qwen3-235b-a22b-w4a8", 256, "frac_hbm"),
+    })
+
     t = head["ms_per_step"] * 1e-3
     line = {
         "metric": "block-INT8 fused-MoE tokens/s", "value": round(args.tokens / t, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "ms_per_step_mean": head["ms_mean"], "ms_per_step_min": head["ms_min"],
-        "scale_order": "fused" if args.fused_scale == 1 else "canonical",
-        ("ms_per_step_canonical" if args.fused_scale == 1 else "ms_per_step_fused_scale"):
-            None if other is None else round(other[1], 4),
+        "scale_order": args.scale_order,
+        **{f"ms_per_step_{'fused_scale' if n == 'fused' else n + '_order'}": round(v, 4) for n, v in others.items()},
+        "host_us_per_call_M1": None if host_us is None else round(host_us, 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": f"{layer.name} E={L.E}/{L.E_global} top{L.top_k} H={L.H} I={L.I} "

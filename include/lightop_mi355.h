@@ -340,6 +340,16 @@ enum { LO_FORM_BLOCK = 0, LO_FORM_CHANNEL = 1, LO_FORM_W4 = 2 };
 int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_local, int32_t num_experts,
                            int32_t top_k, int64_t H, int64_t I, lo_moe_tile *gemm1,
                            lo_moe_tile *gemm2);
+/* The same for a given element type of the activations (LO_BF16 / LO_F16 / LO_F32: 16-bit rows other than
+ * bf16 and fp32 rows take other kernels) and a given block_size_m (0: the table's pick; otherwise the
+ * size a caller passes to lo_fused_experts_*, e.g. one read from a tuning file as get_w8a8moe_json does,
+ * vllm_compat/w8a8_get_cache_json.py:133-174).  flags may carry LO_FUSED_ACT_GELU and the decode-path
+ * flags as well.  The whole-path calls resolve block size, fused / plain first stage and the two-launch
+ * path through the very function this query reports from.  lo_moe_tile_query_form is this call with
+ * LO_BF16 and block_size_m = 0. */
+int lo_moe_tile_query_path(int form, int flags, int dtype, int32_t block_size_m, int64_t M, int32_t E_local,
+                           int32_t num_experts, int32_t top_k, int64_t H, int64_t I, lo_moe_tile *gemm1,
+                           lo_moe_tile *gemm2);
 
 /*
  * Whole path for one chunk of tokens: quant -> align -> GEMM1(+SiLU*mul+quant) -> GEMM2

@@ -15,6 +15,9 @@ Public surface (same names, argument order and defaults as the reference package
     lightop_amd.op                               (lightop.op: moe_align_block_size, moe_sum)
     lightop_amd.envs                             (lightop.envs: LMSLIM_* flags, read lazily)
 
+The repository also ships a package named ``lightop`` whose modules ARE these modules (``lightop.moe is
+lightop_amd.moe``), so that a caller of the reference keeps its imports.
+
 Importing the package touches neither the GPU nor the HIP library; the library
 (lightop_amd/csrc/liblightop_mi355.so, built by ``python -m lightop_amd.build``) is
 loaded on the first call and a missing library is a hard error - there is no CPU or

@@ -72,6 +72,8 @@ SIGNATURES = {
                                   ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
     "lo_moe_tile_query_form": (c_int, [c_int, c_int, c_int64, c_int32, c_int32, c_int32, c_int64, c_int64,
                                        ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
+    "lo_moe_tile_query_path": (c_int, [c_int, c_int, c_int, c_int32, c_int64, c_int32, c_int32, c_int32, c_int64,
+                                       c_int64, ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
     "lo_fused_experts_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
     "lo_fused_experts_workspace_offset": (c_int64, [c_int, c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
     "lo_per_token_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),

@@ -185,26 +185,78 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   return 64;
 }
 
+// What the block-form whole-path call (int8 weights, or int4 weights with K-group scales) does with a
+// problem: the token-block size and which launches follow.  One function for the call itself, for its
+// no-allocation variant's space check and for the tile query, so that the three cannot drift apart.
+struct BlockPlan {
+  int flags;            // the caller's flags, LO_GEMM_W4 implying LO_GEMM_W_PRESHUFFLED
+  int32_t block_size_m; // the caller's, or the table's pick when the caller passed 0
+  bool bs160;           // 160-token blocks: plain first GEMM, activation launch, plain second GEMM
+  bool unfused;         // the first GEMM writes [S, 2I] and one launch applies the activation and quantises
+  bool try_decode;      // the two-launch path is attempted first (it may still decline by size)
+};
+static int plan_block_path(int dtype, int flags, int64_t M, int32_t num_experts, int32_t top_k, int64_t H, int64_t I,
+                           int32_t block_size_m, BlockPlan *plan) {
+  if (flags & LO_GEMM_W4) flags |= LO_GEMM_W_PRESHUFFLED; // packed int4 exists in the load-time layout only
+  const bool w4 = (flags & LO_GEMM_W4) != 0, pre = (flags & LO_GEMM_W_PRESHUFFLED) != 0;
+  const bool gelu = (flags & LO_FUSED_ACT_GELU) != 0;
+  const bool block_size_m_auto = block_size_m == 0;
+  if (block_size_m == 0 && dtype == LO_F32) // fp32 rows go through the weight-streaming kernel at every size
+    block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_BLOCK, false);
+  if (block_size_m == 0)
+    block_size_m = pick_block_m(M, num_experts, top_k, H, w4 ? LO_FORM_W4 : LO_FORM_BLOCK, pre, false,
+                                !w4 && dtype == LO_BF16 && !gelu && blocks_of_160_fit(H, I));
+  // 160: the 160-token form of the direct-to-LDS kernel (int8 block form, load-time layout), both GEMMs
+  // with plain epilogues and the activation in a launch of its own
+  const bool bs160 = block_size_m == 160 && pre && !w4 && dtype != LO_F32 && blocks_of_160_fit(H, I);
+  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 || bs160,
+             LO_EINVAL,
+             "fused_experts: block_size_m %d is not one of 16, 32, 64, 128 (160: int8 weights in the load-time "
+             "layout, 16-bit rows and 2I <= H only)", block_size_m);
+  plan->flags = flags;
+  plan->block_size_m = block_size_m;
+  plan->bs160 = bs160;
+  // GELU and fp16 / fp32 activations have no fused epilogue
+  plan->unfused = gelu || dtype != LO_BF16 || bs160;
+  plan->try_decode = block_size_m_auto && pre && !plan->unfused && !(flags & LO_FUSED_NO_DECODE_PATH);
+  return LO_OK;
+}
+
 } // namespace lo
 
-extern "C" int lo_version(void) { return 100; }
+extern "C" int lo_version(void) { return 101; }
 
 extern "C" const char *lo_last_error(void) { return lo::g_err; }
 
-extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_local, int32_t num_experts,
-                                      int32_t top_k, int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
+extern "C" int lo_moe_tile_query_path(int form, int flags, int dtype, int32_t block_size_m, int64_t M, int32_t E_local,
+                                      int32_t num_experts, int32_t top_k, int64_t H, int64_t I, lo_moe_tile *gemm1,
+                                      lo_moe_tile *gemm2) {
   using namespace lo;
   LO_REQUIRE(form == LO_FORM_BLOCK || form == LO_FORM_CHANNEL || form == LO_FORM_W4, LO_EINVAL,
-             "moe_tile_query_form: unknown form %d", form);
+             "moe_tile_query: unknown form %d", form);
   LO_REQUIRE(M >= 0 && num_experts >= 1 && top_k >= 1 && H > 0 && I > 0, LO_EINVAL,
-             "moe_tile_query_form: bad problem size");
+             "moe_tile_query: bad problem size");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16 || dtype == LO_F32, LO_EINVAL, "moe_tile_query: unknown dtype %d", dtype);
   if (form == LO_FORM_W4) flags |= LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED;
+  int32_t bm = block_size_m;
+  bool fused = false, decode = false;
+  if (form == LO_FORM_CHANNEL) {
+    const bool pre = (flags & (LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED)) != 0;
+    if (bm == 0)
+      bm = pick_block_m(M, num_experts, top_k, H, form, true, (flags & LO_GEMM_W4) != 0,
+                        pre && H / kGroup <= 128 && I / kGroup <= 128);
+  } else {
+    BlockPlan plan;
+    const int rc = plan_block_path(dtype, flags, M, num_experts, top_k, H, I, block_size_m, &plan);
+    if (rc) return rc;
+    flags = plan.flags;
+    bm = plan.block_size_m;
+    fused = !plan.unfused;
+    decode = plan.try_decode && M > 0 &&
+             decode_path_applies(M, top_k, H, I, num_experts, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0,
+                                 (flags & LO_GEMM_W4) != 0);
+  }
   const bool pre = (flags & LO_GEMM_W_PRESHUFFLED) != 0;
-  const bool int4_channel = form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4);
-  const int32_t bm = pick_block_m(M, num_experts, top_k, H, form, pre, int4_channel,
-                                  form == LO_FORM_CHANNEL ? (pre && H / kGroup <= 128 && I / kGroup <= 128)
-                                                          : (form == LO_FORM_BLOCK && pre && blocks_of_160_fit(H, I) &&
-                                                             !(flags & LO_FUSED_ACT_GELU)));
   // the argument blocks the stage entry points would build for this problem
   GemmArgs a{};
   a.num_valid = M * top_k;
@@ -212,27 +264,32 @@ extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_
   a.experts_routed = num_experts;
   a.top_k = top_k;
   a.w_shuffled = pre ? 1 : 0;
-  a.w4 = (form == LO_FORM_W4 || (form == LO_FORM_CHANNEL && (flags & LO_GEMM_W4))) ? 1 : 0;
+  a.w4 = (flags & LO_GEMM_W4) ? 1 : 0;
   a.per_channel = form == LO_FORM_CHANNEL ? 1 : 0;
+  a.out_f16 = dtype == LO_F16 ? 1 : 0;
+  a.out_f32 = dtype == LO_F32 ? 1 : 0;
+  const int gflags = flags & ~(LO_FUSED_ACT_GELU | LO_FUSED_NO_DECODE_PATH | LO_FUSED_FORCE_DECODE_PATH);
   if (gemm1) {
     a.N = 2 * I; a.K = H; a.a_rows = M;
-    // the per-channel form and 160-token blocks apply the activation and quantise in a launch of their own
-    const bool fused = form != LO_FORM_CHANNEL && bm != 160;
-    describe_gemm_kernel(pick_gemm_kernel(a, fused, bm, flags), fused, bm, gemm1);
+    describe_gemm_kernel(pick_gemm_kernel(a, fused, bm, gflags), fused, bm, gemm1);
   }
   if (gemm2) {
     a.N = H; a.K = I; a.a_rows = M * top_k;
-    describe_gemm_kernel(pick_gemm_kernel(a, false, bm, flags), false, bm, gemm2);
+    describe_gemm_kernel(pick_gemm_kernel(a, false, bm, gflags), false, bm, gemm2);
   }
   // a few tokens: the whole-path call serves the block form with its two-launch path
-  if ((form == LO_FORM_BLOCK || form == LO_FORM_W4) && pre && !(flags & LO_FUSED_NO_DECODE_PATH) && M > 0 &&
-      decode_path_applies(M, top_k, H, I, num_experts, (flags & LO_FUSED_FORCE_DECODE_PATH) != 0, form == LO_FORM_W4)) {
+  if (decode) {
     int w1 = 0, w2 = 0;
     decode_path_waves(top_k, H, &w1, &w2);
     if (gemm1) { gemm1->kernel = LO_KERNEL_DEC; gemm1->waves = w1; gemm1->block_n = 16; }
     if (gemm2) { gemm2->kernel = LO_KERNEL_DEC; gemm2->waves = w2; gemm2->block_n = 16; }
   }
   return LO_OK;
+}
+
+extern "C" int lo_moe_tile_query_form(int form, int flags, int64_t M, int32_t E_local, int32_t num_experts,
+                                      int32_t top_k, int64_t H, int64_t I, lo_moe_tile *gemm1, lo_moe_tile *gemm2) {
+  return lo_moe_tile_query_path(form, flags, LO_BF16, 0, M, E_local, num_experts, top_k, H, I, gemm1, gemm2);
 }
 
 extern "C" int lo_moe_tile_query(int64_t M, int32_t E_local, int32_t num_experts, int32_t top_k,
@@ -286,22 +343,11 @@ extern "C" int lo_fused_experts_block_int8(
   LO_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, LO_EINVAL,
              "fused_experts: workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
-  const bool block_size_m_auto = block_size_m == 0;
-  if (block_size_m == 0 && dtype == LO_F32) // fp32 rows go through the weight-streaming kernel at every size
-    block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_BLOCK, false);
-  if (block_size_m == 0)
-    block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
-                                (flags & LO_GEMM_W_PRESHUFFLED) != 0, false,
-                                !(flags & LO_GEMM_W4) && dtype == LO_BF16 && !(flags & LO_FUSED_ACT_GELU) &&
-                                    blocks_of_160_fit(H, I));
-  // 160: the 160-token form of the direct-to-LDS kernel (int8 block form, load-time layout), both GEMMs
-  // with plain epilogues and the activation in a launch of its own
-  const bool bs160 = block_size_m == 160 && (flags & LO_GEMM_W_PRESHUFFLED) && !(flags & LO_GEMM_W4) &&
-                     dtype != LO_F32 && blocks_of_160_fit(H, I);
-  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 || bs160,
-             LO_EINVAL,
-             "fused_experts: block_size_m %d is not one of 16, 32, 64, 128 (160: int8 weights in the load-time "
-             "layout, 16-bit rows and 2I <= H only)", block_size_m);
+  BlockPlan plan;
+  const int rc_plan = plan_block_path(dtype, flags, M, num_experts, top_k, H, I, block_size_m, &plan);
+  if (rc_plan) return rc_plan;
+  flags = plan.flags;
+  block_size_m = plan.block_size_m;
   const WsLayout L = ws_layout(M, top_k, H, I, num_experts, block_size_m);
   LO_REQUIRE(workspace_bytes >= L.total, LO_ENOSPC, "fused_experts: workspace holds %lld bytes, needs %lld",
              (long long)workspace_bytes, (long long)L.total);
@@ -318,13 +364,11 @@ extern "C" int lo_fused_experts_block_int8(
   uint8_t *mask = expert_map ? reinterpret_cast<uint8_t *>(ws + L.off[7]) : nullptr;
   const int64_t S = M * top_k;
 
-  // Decode sizes: routing, quantisation, both GEMMs and the reduction in two launches.
+  // Decode sizes: routing, quantisation, both GEMMs and the reduction in two launches (in the default scale
+  // order, or the one of LO_GEMM_SEPARATE_ORDER; LO_GEMM_FUSED_SCALE buys nothing there and gets the default).
   const bool gelu = (flags & LO_FUSED_ACT_GELU) != 0;
-  // GELU and fp16 activations have no fused epilogue: the first GEMM writes [S, 2I] in the activation
-  // type, one launch applies the gated activation and quantises
-  const bool unfused = gelu || dtype != LO_BF16 || bs160;
-  if (block_size_m_auto && (flags & (LO_GEMM_W_PRESHUFFLED | LO_GEMM_W4)) && !unfused &&
-      !(flags & LO_FUSED_NO_DECODE_PATH)) {
+  const bool unfused = plan.unfused;
+  if (plan.try_decode) {
     // (cache3 is the front of the caller's cache13: the path keeps its bf16 activations [S, I] there)
     const int rc2 = launch_decode_path(x, M, H, I, E, num_experts, top_k, w1, w1s, w2, w2s, topk_w, topk_ids, ids_dtype,
                                        expert_map, apply_router_weight_on_input, routed_scaling_factor, shared_output,
@@ -532,15 +576,14 @@ extern "C" int lo_fused_experts_block_int8_noalloc(
   using namespace lo;
   LO_REQUIRE(M >= 0 && top_k >= 1 && H >= kGroup && I >= kGroup && num_experts >= 1, LO_EINVAL,
              "fused_experts(noalloc): bad problem size");
+  LO_REQUIRE(dtype == LO_BF16 || dtype == LO_F16 || (dtype == LO_F32 && !(flags & LO_GEMM_W4)), LO_ENOTSUP,
+             "fused_experts(noalloc): activations are bf16, fp16 or (int8 weights) fp32");
+  // the block size the workspace form will resolve to (same function, same arguments), for the space check
+  BlockPlan plan;
+  const int rc_plan = plan_block_path(dtype, flags, M, num_experts, top_k, H, I, block_size_m, &plan);
+  if (rc_plan) return rc_plan;
   const int32_t block_size_m_arg = block_size_m;
-  if (block_size_m == 0)
-    block_size_m = pick_block_m(M, num_experts, top_k, H, (flags & LO_GEMM_W4) ? LO_FORM_W4 : LO_FORM_BLOCK,
-                                (flags & LO_GEMM_W_PRESHUFFLED) != 0, false,
-                                !(flags & LO_GEMM_W4) && dtype == LO_BF16 && !(flags & LO_FUSED_ACT_GELU) &&
-                                    blocks_of_160_fit(H, I));
-  LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 ||
-                 block_size_m == 160,
-             LO_EINVAL, "fused_experts(noalloc): block_size_m %d is not one of 16, 32, 64, 128, 160", block_size_m);
+  block_size_m = plan.block_size_m;
   const int64_t need = ws_layout(M, top_k, H, I, num_experts, block_size_m).total;
   LO_REQUIRE(need <= kScratchBytes, LO_ENOSPC,
              "fused_experts(noalloc): this problem needs %lld bytes of scratch, the built-in scratch holds %lld; "

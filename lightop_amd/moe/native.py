@@ -8,24 +8,32 @@ from typing import Any, Dict, List, Optional, Tuple
 import torch
 
 from .. import _lib, envs
+from ..gemmopt import moe_gemm_w8a8
 from ..op import _act_dtype, _ids_dtype, _on_device, _require_cuda
 
 
 def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bool,
                      block_shape: Optional[List[int]], topk: int,
                      global_num_experts: int = -1, preshuffled: bool = True,
-                     int4: bool = False) -> Tuple[Dict[str, Any], Dict[str, Any]]:
+                     int4: bool = False, dtype: torch.dtype = torch.bfloat16,
+                     activation: str = "silu") -> Tuple[Dict[str, Any], Dict[str, Any]]:
     """Tile configuration of both GEMMs for ``m`` tokens (reference: get_w8a8moe_json,
-    int8.py:220-256, backed there by per-device JSON files).  Here the table is compiled
-    into the library; the dictionaries keep the reference's keys.  ``n1`` = 2*I, ``n2`` = H,
-    ``k`` = I.  ``block_shape=None`` asks for the per-channel form (the reference consults
-    get_moe_cuda_config first there, int8.py:735-741), ``[1, 128]`` for W4A8 with K-group scales.
-    ``int4`` with ``block_shape=None``: the reference's own W4A8 form (w4a8.py:587, which passes only
-    the first five arguments).
+    int8.py:220-256, backed there by per-device JSON files).  ``n1`` = 2*I, ``n2`` = H, ``k`` = I.
+    ``block_shape=None`` asks for the per-channel form (the reference consults get_moe_cuda_config first
+    there, int8.py:735-741), ``[1, 128]`` for W4A8 with K-group scales.  ``int4`` with ``block_shape=None``:
+    the reference's own W4A8 form (w4a8.py:587, which passes only the first five arguments).
+
+    The block size comes from a tuning file when ``TRITON_JSON_DIR`` names a directory that holds one for
+    this layer shape (``lightop_amd.moe.tile_files``: the reference's file names and keys, written by
+    ``python -m lightop_amd.tune --out``), else from the table compiled into the library.  The dictionaries
+    keep the reference's keys; ``kernel`` / ``num_warps`` / ``BLOCK_SIZE_N`` describe the kernel the
+    whole-path call launches for that block size, ``source`` says where the block size came from.
     ``preshuffled``: the weights are in the load-time layout of ``preshuffle_moe_weight`` (the table
-    differs for row-major weights).  ``kernel`` / ``num_warps`` / ``BLOCK_SIZE_N`` describe the kernel
-    the stage calls launch for that ``BLOCK_SIZE_M``."""
+    differs for row-major weights); ``dtype`` / ``activation``: rows other than bfloat16 and GELU take the
+    path without the fused epilogue."""
     del use_int8_w8a8
+    from . import tile_files
+
     t1, t2 = _lib.LoMoeTile(), _lib.LoMoeTile()
     Eg = E if global_num_experts in (-1, None) else global_num_experts
     form = _lib.LO_FORM_CHANNEL if block_shape is None else (
@@ -33,12 +41,17 @@ def get_w8a8moe_json(m: int, E: int, n1: int, n2: int, k: int, use_int8_w8a8: bo
     flags = _lib.LO_GEMM_W_PRESHUFFLED if preshuffled else 0
     if int4 and block_shape is None:
         flags |= _lib.LO_GEMM_W4 | _lib.LO_GEMM_W_PRESHUFFLED
-    _lib.check(_lib.lib().lo_moe_tile_query_form(form, flags, m, E, Eg, topk, n2, k, t1, t2))
+    if activation == "gelu":
+        flags |= _lib.LO_FUSED_ACT_GELU
+    dt = {torch.bfloat16: _lib.LO_BF16, torch.float16: _lib.LO_F16, torch.float32: _lib.LO_F32}[dtype]
+    bs_file = tile_files.block_size_m(m, E, n1, n2, k, topk, block_shape, int4=int4 or form == _lib.LO_FORM_W4)
+    _lib.check(_lib.lib().lo_moe_tile_query_path(form, flags, dt, bs_file, m, E, Eg, topk, n2, k, t1, t2))
 
     def as_dict(t):
         return {"BLOCK_SIZE_M": t.block_size_m, "BLOCK_SIZE_N": t.block_n, "BLOCK_SIZE_K": 128,
                 "GROUP_SIZE_M": 1, "num_warps": t.waves, "num_stages": 0, "kernel": t.kernel,
-                "kernel_name": _lib.KERNEL_NAMES.get(t.kernel, "?")}
+                "kernel_name": _lib.KERNEL_NAMES.get(t.kernel, "?"),
+                "source": "file" if bs_file else "compiled"}
 
     return as_dict(t1), as_dict(t2)
 
@@ -204,40 +217,6 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
             _scale_flags(fused_scale) | flags | (_lib.LO_GEMM_W_PRESHUFFLED if _is_preshuffled(B) else 0),
             _lib.stream_of(A)))
     return a2q, a2s
-
-
-def moe_gemm_w8a8(input: torch.Tensor, b_qweight: torch.Tensor, output: torch.Tensor, a_scale: torch.Tensor,
-                  b_scale: torch.Tensor, topk_weights: Optional[torch.Tensor], sorted_token_ids: torch.Tensor,
-                  experts_ids: torch.Tensor, num_tokens_post_pad: torch.Tensor, top_k: int,
-                  config: Dict[str, Any], flags: int = 0, global_num_experts: int = 0) -> torch.Tensor:
-    """One grouped GEMM stage in the per-channel form (reference: moe_gemm_w8a8, gemmopt.py:437-457):
-    output[f] = T((sum_k input[f // top_k] * b_qweight[e]) * ts * b_scale[e]) with
-    ts = a_scale[f // top_k], times topk_weights[f] when they are given (the second stage).
-    ``a_scale`` [rows(, 1)], ``b_scale`` [E, N(, 1)]; ``config`` needs ``BLOCK_SIZE_M`` (the reference's
-    ``MODE`` / ``DELTA`` pick among its tuned kernels and are ignored)."""
-    _require_cuda(input, b_qweight, output, a_scale, b_scale, topk_weights, sorted_token_ids, experts_ids,
-                  num_tokens_post_pad)
-    assert input.dtype == torch.int8 and b_qweight.dtype == torch.int8
-    assert input.is_contiguous() and b_qweight.is_contiguous() and output.is_contiguous()
-    E, N, K = b_qweight.shape
-    assert input.shape[1] == K and output.shape[-1] == N
-    assert a_scale.dtype == torch.float32 and a_scale.is_contiguous() and a_scale.numel() == input.shape[0]
-    assert b_scale.dtype == torch.float32 and b_scale.is_contiguous() and b_scale.numel() == E * N
-    assert sorted_token_ids.dtype == torch.int32 and experts_ids.dtype == torch.int32
-    num_valid = output.numel() // N
-    tw = None
-    if topk_weights is not None:
-        tw = topk_weights if topk_weights.dtype == torch.float32 and topk_weights.is_contiguous() \
-            else topk_weights.to(torch.float32).contiguous()
-    with _on_device(input):
-        _lib.check(_lib.lib().lo_moe_gemm_w8a8(
-            _lib.ptr(input), _lib.ptr(a_scale), _lib.ptr(b_qweight), _lib.ptr(b_scale), _lib.ptr(output),
-            _act_dtype(output), _lib.ptr(tw), _lib.ptr(sorted_token_ids), _lib.ptr(experts_ids),
-            _lib.ptr(num_tokens_post_pad), sorted_token_ids.numel(), num_valid, input.shape[0], E,
-            int(global_num_experts or 0), N, K, int(top_k),
-            int(config["BLOCK_SIZE_M"]), 1 if tw is not None else 0,
-            flags | (_lib.LO_GEMM_W_PRESHUFFLED if _is_preshuffled(b_qweight) else 0), _lib.stream_of(input)))
-    return output
 
 
 def invoke_fused_moe_kernel_w4a8(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, A_scale: torch.Tensor,
@@ -580,6 +559,27 @@ def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
                               int(extra.get("lightop_amd_block_size_m", 0)), workspace=extra.get("lightop_amd_workspace"))
 
 
+@functools.lru_cache(maxsize=256)
+def _workspace_bytes_cached(M: int, top_k: int, H: int, I: int, num_experts: int) -> int:
+    return fused_experts_workspace_bytes(M, top_k, H, I, num_experts, 0)
+
+
+_ws_cache: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _cached_workspace(nbytes: int, device: torch.device, stream_key: int) -> torch.Tensor:
+    """The library's scratch for a whole-path call, kept per (device, stream) and grown on demand, so that a
+    serving loop does not allocate on every call (the reference keeps its own workspace, cache13, in a
+    process-wide cache the same way: vllm_compat/fused_moe_cache.py:19-24).  Calls on one stream run in
+    order, so they can share it; calls on different streams get workspaces of their own."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_key)
+    ws = _ws_cache.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _ws_cache[key] = ws
+    return ws
+
+
 def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace, apply_router_weight_on_input,
                        global_num_experts, expert_map, w1_scale, w2_scale, routed_scaling_factor, shared_output,
                        I, flags, block_size_m, channel=False, workspace=None, prequant=None):
@@ -608,9 +608,11 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
         shared_output = shared_output.contiguous()
 
     lib = _lib.lib()
-    ws_bytes = fused_experts_workspace_bytes(M, top_k_num, H, I, global_num_experts, 0)
+    ws_bytes = _workspace_bytes_cached(M, top_k_num, H, I, global_num_experts)
     if workspace is None:
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=hidden_states.device)
+        workspace = _cached_workspace(ws_bytes, hidden_states.device,
+                                      torch.cuda.current_stream(hidden_states.device).cuda_stream)
+        ws_bytes = workspace.numel()
     else:  # the caller's own scratch (tests read the intermediates out of it afterwards)
         assert workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.numel() >= ws_bytes
         assert workspace.device == hidden_states.device
@@ -621,6 +623,11 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
     if _is_preshuffled(w1):
         flags |= _lib.LO_GEMM_W_PRESHUFFLED
 
+    from . import tile_files
+
+    use_files = block_size_m == 0 and tile_files.json_dir() is not None
+    w4 = bool(flags & _lib.LO_GEMM_W4)
+    file_shape = None if channel else ([1, 128] if w4 else [128, 128])
     with _on_device(hidden_states):
         stream = _lib.stream_of(hidden_states)
         for chunk in range((num_tokens // CHUNK_SIZE) + 1):
@@ -629,6 +636,8 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
             if m <= 0:
                 break
             x = hidden_states[begin:end]
+            if use_files:  # a tuning file under TRITON_JSON_DIR wins over the compiled-in table
+                block_size_m = tile_files.block_size_m(m, E, 2 * I, H, I, top_k_num, file_shape, int4=w4)
             if prequant is not None:  # the chunk's rows of the caller's quantised input
                 entry = lib.lo_fused_experts_channel_int8_prequant
                 head = (_lib.ptr(prequant[0][begin:end]), _lib.ptr(prequant[1].reshape(-1)[begin:end]))

@@ -8,10 +8,22 @@ from typing import Optional, Tuple
 import torch
 
 from .. import op
-from ..moe_fused_gate import moe_fused_gate
 
 # reference: moe/routing.py:20
 topk_softmax = op.topk_softmax
+
+
+def moe_fused_gate(x, bias, num_expert_group, topk_group, topk, n_share_experts_fusion, routed_scaling_factor,
+                   apply_routed_scaling_factor_on_output=True, output_indices_int64=False):
+    """Grouped top-k router of DeepSeek-style layers: sigmoid scores plus ``bias`` pick ``topk_group`` of
+    ``num_expert_group`` expert groups (a group's score is the sum of its two best experts) and then ``topk``
+    experts inside them; the weights are the unbiased sigmoid scores, renormalised and, when
+    ``apply_routed_scaling_factor_on_output``, multiplied by ``routed_scaling_factor``.  Returns
+    ``(topk_weights [T, topk] f32, topk_ids [T, topk] int32 or int64)``.  Same arguments as the reference's
+    lightop.moe_fused_gate (python/lightop/moe_fused_gate.py:10-31; kernel
+    csrc/kernels/moe_gate/moe_fused_gate.cu:76-312)."""
+    return op.moe_fused_gate(x, bias, num_expert_group, topk_group, topk, n_share_experts_fusion,
+                             routed_scaling_factor, apply_routed_scaling_factor_on_output, output_indices_int64)
 
 
 def round_up(x: int, y: int) -> int:

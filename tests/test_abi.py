@@ -216,3 +216,55 @@ def test_stage_entry_points_reject_a_bad_block_size(lib):
         assert rc == -1 and b"block_size_m" in lib.lo_last_error(), bad
         rc = lib.lo_moe_gemm_w8a8(p, p, p, p, p, 0, null, p, p, p, 128, 8, 8, 1, 1, 16, 128, 1, bad, 0, 0, null)
         assert rc == -1 and b"block_size_m" in lib.lo_last_error(), bad
+
+
+def test_tile_query_path_follows_element_type_activation_and_block_size(lib):
+    """The whole-path call resolves its block size, fused / plain first stage and the two-launch path in one
+    function; lo_moe_tile_query_path reports from that function for any element type, activation and
+    caller-chosen block size, so what it says is what the call launches."""
+    from lightop_amd import _lib
+
+    t1, t2 = _lib.LoMoeTile(), _lib.LoMoeTile()
+    pre = _lib.LO_GEMM_W_PRESHUFFLED
+    qwen, dsv3 = (128, 128, 8, 2048, 768), (32, 256, 8, 7168, 2048)
+
+    def q(form, flags, dtype, bs, M, shape):
+        assert lib.lo_moe_tile_query_path(form, flags, dtype, bs, M, *shape, t1, t2) == 0
+        return (t1.block_size_m, t1.kernel), (t2.block_size_m, t2.kernel)
+
+    # bf16 + SiLU: exactly lo_moe_tile_query_form
+    for M in (1, 8, 64, 512, 2048, 8192):
+        for shape in (qwen, dsv3):
+            want = q(_lib.LO_FORM_BLOCK, pre, _lib.LO_BF16, 0, M, shape)
+            assert lib.lo_moe_tile_query_form(_lib.LO_FORM_BLOCK, pre, M, *shape, t1, t2) == 0
+            assert ((t1.block_size_m, t1.kernel), (t2.block_size_m, t2.kernel)) == want
+    # one token: bf16 + SiLU takes the two-launch path; GELU and fp16 rows have no fused epilogue and never do
+    assert q(_lib.LO_FORM_BLOCK, pre, _lib.LO_BF16, 0, 1, qwen)[0][1] == _lib.LO_KERNEL_DEC
+    assert q(_lib.LO_FORM_BLOCK, pre | _lib.LO_FUSED_ACT_GELU, _lib.LO_BF16, 0, 1, qwen)[0][1] == _lib.LO_KERNEL_WS
+    assert q(_lib.LO_FORM_BLOCK, pre, _lib.LO_F16, 0, 1, qwen)[0][1] == _lib.LO_KERNEL_WS
+    # the plain first GEMM of those paths has the plain workgroup shape (four waves), not the fused one (eight)
+    q(_lib.LO_FORM_BLOCK, pre, _lib.LO_F16, 0, 16, dsv3)
+    assert (t1.kernel, t1.waves) == (_lib.LO_KERNEL_WS, 4)
+    q(_lib.LO_FORM_BLOCK, pre, _lib.LO_BF16, 0, 16, dsv3)
+    assert (t1.kernel, t1.waves) == (_lib.LO_KERNEL_WS, 8)
+    # 160-token blocks are the table's pick for bf16 + SiLU only; fp16 rows and GELU get 64 / 128 there
+    assert q(_lib.LO_FORM_BLOCK, pre, _lib.LO_BF16, 0, 2048, qwen)[0][0] == 160
+    assert q(_lib.LO_FORM_BLOCK, pre, _lib.LO_F16, 0, 2048, qwen)[0][0] == 64
+    assert q(_lib.LO_FORM_BLOCK, pre | _lib.LO_FUSED_ACT_GELU, _lib.LO_BF16, 0, 2048, qwen)[0][0] == 64
+    assert q(_lib.LO_FORM_BLOCK, pre, _lib.LO_F16, 160, 2048, qwen)[0] == (160, _lib.LO_KERNEL_T128)  # on request
+    # fp32 rows: the row-major table and the weight-streaming kernel at every size, whatever the layout
+    for M in (1, 512, 8192):
+        a, b = q(_lib.LO_FORM_BLOCK, pre, _lib.LO_F32, 0, M, qwen)
+        assert a[1] == _lib.LO_KERNEL_WS == b[1]
+        assert a[0] == q(_lib.LO_FORM_BLOCK, 0, _lib.LO_BF16, 0, M, qwen)[0][0]
+    assert lib.lo_moe_tile_query_path(_lib.LO_FORM_BLOCK, pre, _lib.LO_F32, 160, 2048, *qwen, t1, t2) < 0  # refused, as the call does
+    # a caller's block size (for instance from a tuning file) is described as it would be launched, and
+    # switches the two-launch path off, as it does in the call
+    assert q(_lib.LO_FORM_BLOCK, pre, _lib.LO_BF16, 64, 8192, qwen)[0] == (64, _lib.LO_KERNEL_TILE)
+    assert q(_lib.LO_FORM_BLOCK, pre, _lib.LO_BF16, 16, 1, qwen)[0] == (16, _lib.LO_KERNEL_WS)
+    assert lib.lo_moe_tile_query_path(_lib.LO_FORM_BLOCK, pre, _lib.LO_BF16, 48, 64, *qwen, t1, t2) < 0
+    assert lib.lo_moe_tile_query_path(_lib.LO_FORM_BLOCK, pre, 9, 0, 64, *qwen, t1, t2) < 0
+    # int4 weights imply the load-time layout in the whole-path call, at every size
+    assert q(_lib.LO_FORM_W4, 0, _lib.LO_BF16, 0, 2, dsv3)[0][1] == _lib.LO_KERNEL_DEC
+    assert q(_lib.LO_FORM_BLOCK, _lib.LO_GEMM_W4, _lib.LO_BF16, 0, 2048, dsv3) == \
+        q(_lib.LO_FORM_W4, 0, _lib.LO_BF16, 0, 2048, dsv3)

@@ -82,6 +82,35 @@ def test_moe_fused_gate_vs_oracle(dev, oracle, E, G, tg, topk, nshare, T):
         assert torch.equal(w.cpu().view(torch.int32), rw.view(torch.int32))
 
 
+# From 65 rows on and up to 128 experts the gate runs with 16 lanes per row; a group's two best experts are then
+# merged across the 16 / G lanes that share the group (two, four and eight lanes here; sixteen with one group,
+# one lane with sixteen groups above).
+GATE16_CONFIGS = [(128, 8, 4, 8, 0), (64, 4, 2, 6, 0), (96, 2, 1, 7, 1), (128, 2, 2, 8, 0), (32, 4, 3, 4, 0),
+                  (128, 4, 2, 16, 0), (48, 8, 5, 6, 0)]
+
+
+@pytest.mark.parametrize("E,G,tg,topk,nshare", GATE16_CONFIGS)
+@pytest.mark.parametrize("T", [65, 1000, 4096])
+@pytest.mark.parametrize("ties", [False, True])
+def test_moe_fused_gate_16_lane_rows_merge_groups_across_lanes(dev, oracle, E, G, tg, topk, nshare, T, ties):
+    from lightop_amd.moe import moe_fused_gate
+
+    say(f"moe_fused_gate (16 lanes per row) E={E} G={G} tg={tg} topk={topk} shared={nshare} T={T} ties={ties}")
+    g = torch.Generator().manual_seed(3 * E + T + G)
+    if ties:  # coarse scores: equal experts inside groups and equal group scores, decided by the lower id
+        x = torch.randint(-2, 3, (T, E), generator=g).float() * 0.5
+        bias = torch.randint(-1, 2, (E,), generator=g).float() * 0.25
+    else:
+        x = torch.randn(T, E, generator=g)
+        bias = torch.randn(E, generator=g)
+    for apply, i64 in ((True, False), (False, True)):
+        w, idx = moe_fused_gate(x.to(dev), bias.to(dev), G, tg, topk, nshare, 2.5, apply, i64)
+        torch.cuda.synchronize()
+        rw, ridx = oracle.moe_fused_gate(x, bias, G, tg, topk, nshare, 2.5, apply)
+        assert torch.equal(idx.cpu().long(), ridx.long())
+        assert torch.equal(w.cpu().view(torch.int32), rw.view(torch.int32))
+
+
 def test_moe_fused_gate_16_bit_inputs_and_ties(dev, oracle):
     from lightop_amd.moe import moe_fused_gate
 

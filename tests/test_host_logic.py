@@ -65,7 +65,8 @@ def test_signatures_match_the_reference():
                                    "w1_scale", "w2_scale", "w1_zp", "w2_zp", "a1_scale", "a2_scale", "block_shape",
                                    "use_nn_moe", "routed_scaling_factor", "shared_output", "_"]
     # gemmopt.py:437-447 (a trailing private `flags` is this build's)
-    from lightop_amd import fuse_silu_mul_quant, gemmopt, moe_fused_gate as gate_mod, op
+    from lightop_amd import fuse_silu_mul_quant, gemmopt, op
+    from lightop_amd.moe import routing as gate_mod
 
     assert list(inspect.signature(gemmopt.moe_gemm_w8a8).parameters)[:11] == [
         "input", "b_qweight", "output", "a_scale", "b_scale", "topk_weights", "sorted_token_ids", "experts_ids",
@@ -323,3 +324,81 @@ def test_moe_cache_is_keyed_and_grows(monkeypatch):
     assert cache.moe_cache_singleton is c
     cache.release_moe_cache()
     assert cache.moe_cache_singleton is None
+
+
+def test_lightop_is_an_importable_name():
+    """A caller of the reference keeps its imports: the ``lightop`` package's modules are the modules of
+    ``lightop_amd`` themselves (reference import paths: python/lightop/moe/__init__.py:57-78,
+    python/lightop/quant/int8.py, python/lightop/gemmopt.py:437, python/lightop/moe_fused_gate.py:10)."""
+    import lightop
+    import lightop_amd
+    from lightop.moe import fused_experts_impl_int8, fused_experts_impl_w4a8, moe_align_block_size, moe_sum, topk_softmax
+    from lightop.moe.native import fused_experts_impl_int8 as native_entry
+    from lightop.quant import per_token_group_quant_int8, per_token_quant_int8
+    from lightop.quant.int8 import per_token_group_quant_int8 as q2
+    from lightop.gemmopt import moe_gemm_w8a8
+    from lightop.moe_fused_gate import moe_fused_gate
+    from lightop.fuse_silu_mul_quant import fuse_silu_mul_quant as fsq
+    from lightop import envs, fuse_silu_mul_quant, op
+
+    assert lightop.moe is lightop_amd.moe and lightop.quant is lightop_amd.quant and op is lightop_amd.op
+    assert fused_experts_impl_int8 is lightop_amd.moe.fused_experts_impl_int8 is native_entry
+    assert fused_experts_impl_w4a8 is lightop_amd.moe.fused_experts_impl_w4a8
+    assert moe_align_block_size is lightop_amd.moe.moe_align_block_size and moe_sum is lightop_amd.moe.moe_sum
+    assert topk_softmax is lightop_amd.op.topk_softmax and moe_fused_gate is lightop_amd.moe.moe_fused_gate
+    assert per_token_group_quant_int8 is q2 is lightop_amd.quant.per_token_group_quant_int8
+    assert per_token_quant_int8 is lightop_amd.quant.per_token_quant_int8
+    assert moe_gemm_w8a8 is lightop_amd.gemmopt.moe_gemm_w8a8 is lightop_amd.moe.moe_gemm_w8a8
+    assert fuse_silu_mul_quant is fsq is lightop_amd.fuse_silu_mul_quant  # the function, as in the reference
+    assert envs.LMSLIM_FUSED_MOE_CHUNK_SIZE == lightop_amd.envs.LMSLIM_FUSED_MOE_CHUNK_SIZE
+    with pytest.raises(AttributeError):  # an operator family outside the path
+        lightop.RMSNorm
+    with pytest.raises(AttributeError):
+        lightop.moe.fused_experts_impl_fp8_marlin
+
+
+def test_tuning_files_override_the_compiled_table(monkeypatch, tmp_path):
+    """TRITON_JSON_DIR (vllm_compat/w8a8_get_cache_json.py:24) names a directory of tuning files in the
+    reference's layout; the block size such a file holds for the nearest tuned token count comes back from
+    get_w8a8moe_json (reference lookup: int8.py:220-256) together with the kernel that size launches."""
+    from lightop_amd import _lib, moe
+    from lightop_amd.moe import tile_files
+
+    E, k, H, I = 128, 8, 2048, 768
+    monkeypatch.delenv("TRITON_JSON_DIR", raising=False)
+    tile_files.forget()
+    c1, c2 = moe.get_w8a8moe_json(8192, E, 2 * I, H, I, True, [128, 128], k)
+    assert (c1["BLOCK_SIZE_M"], c1["source"], c1["kernel"]) == (128, "compiled", _lib.LO_KERNEL_T128)
+    assert tile_files.block_size_m(8192, E, 2 * I, H, I, k, [128, 128]) == 0
+
+    cfg = lambda bs, **kw: dict({"BLOCK_SIZE_M": bs, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128, "GROUP_SIZE_M": 1,
+                                 "num_warps": 4, "num_stages": 0}, **kw)
+    table = {"1": {"config1": cfg(16, lightop_amd_two_launch=True), "config2": cfg(16, lightop_amd_two_launch=True)},
+             "64": {"config1": cfg(32), "config2": cfg(32)},
+             "8192": {"config1": cfg(64), "config2": cfg(64)}}
+    name = tile_files.file_name(E, 2 * I, H, I, k, [128, 128], False)
+    assert name == "MOE_BLOCKINT8[128,128]_E=128_N1=1536_N2=2048_K=768_TOPK8_gfx950_256cu.json"
+    with open(tmp_path / name, "w") as f:
+        json.dump({f"{2 * I}_{H}_{I}": table}, f)
+    monkeypatch.setenv("TRITON_JSON_DIR", str(tmp_path))
+    tile_files.forget()
+    c1, c2 = moe.get_w8a8moe_json(8192, E, 2 * I, H, I, True, [128, 128], k)
+    assert (c1["BLOCK_SIZE_M"], c2["BLOCK_SIZE_M"], c1["source"]) == (64, 64, "file")
+    assert c1["kernel"] == _lib.LO_KERNEL_TILE           # the kernel that block size launches, not the table's
+    # nearest tuned count on a logarithmic scale: 3000 -> 8192, 500 -> 64 (a factor 7.8 away, 8192 is 16.4), 40 -> 64
+    assert tile_files.block_size_m(3000, E, 2 * I, H, I, k, [128, 128]) == 64
+    assert tile_files.block_size_m(500, E, 2 * I, H, I, k, [128, 128]) == 32
+    assert tile_files.block_size_m(40, E, 2 * I, H, I, k, [128, 128]) == 32
+    # the tuner's mark "the library's own pick was fastest" (the two-launch path): nothing is forced
+    assert tile_files.block_size_m(2, E, 2 * I, H, I, k, [128, 128]) == 0
+    c1, _ = moe.get_w8a8moe_json(1, E, 2 * I, H, I, True, [128, 128], k)
+    assert (c1["kernel"], c1["source"]) == (_lib.LO_KERNEL_DEC, "compiled")
+    # another layer shape has no file: the compiled-in table answers
+    c1, _ = moe.get_w8a8moe_json(8192, 32, 4096, 7168, 2048, True, [128, 128], k, global_num_experts=256)
+    assert (c1["BLOCK_SIZE_M"], c1["source"]) == (128, "compiled")
+    # per-channel and int4 forms have file names of their own (w8a8_get_cache_json.py:133-149)
+    assert tile_files.file_name(8, 1024, 1024, 512, 2, None, False).startswith("MOE_W8A8INT8_E=8_")
+    assert tile_files.file_name(8, 1024, 1024, 512, 2, [1, 128], True).startswith("MOE_W4A8INT8[1,128]_E=8_")
+    assert tile_files.file_name(8, 1024, 1024, 512, 2, None, True).startswith("MOE_W4A8INT8_E=8_")
+    monkeypatch.delenv("TRITON_JSON_DIR")
+    tile_files.forget()
