@@ -2,6 +2,7 @@
 python/lightop/_lmslim_native/layers/fused_moe/int8.py:543-908)."""
 from __future__ import annotations
 
+import ctypes
 import functools
 from typing import Any, Dict, List, Optional, Tuple
 
@@ -453,7 +454,7 @@ def fused_experts_impl_int8(hidden_states: torch.Tensor,
                               apply_router_weight_on_input, global_num_experts, expert_map, w1_scale, w2_scale,
                               routed_scaling_factor, shared_output, I, flags,
                               int(extra.get("lightop_amd_block_size_m", 0)), channel=channel,
-                              workspace=extra.get("lightop_amd_workspace"), prequant=prequant)
+                              workspace=extra.get("lightop_amd_workspace"), prequant=prequant, chunk_size=CHUNK_SIZE)
 
 
 def fused_experts_impl_w4a8(hidden_states: torch.Tensor,
@@ -582,12 +583,12 @@ def _cached_workspace(nbytes: int, device: torch.device, stream_key: int) -> tor
 
 def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, inplace, apply_router_weight_on_input,
                        global_num_experts, expert_map, w1_scale, w2_scale, routed_scaling_factor, shared_output,
-                       I, flags, block_size_m, channel=False, workspace=None, prequant=None):
+                       I, flags, block_size_m, channel=False, workspace=None, prequant=None, chunk_size=None):
     """Chunk loop shared by the block-INT8, per-channel and W4A8 entry points (int8.py:703-888)."""
     num_tokens, H = hidden_states.shape
     E = w1.shape[0]
     top_k_num = topk_ids.shape[1]
-    CHUNK_SIZE = envs.LMSLIM_FUSED_MOE_CHUNK_SIZE
+    CHUNK_SIZE = envs.LMSLIM_FUSED_MOE_CHUNK_SIZE if chunk_size is None else chunk_size
     M = min(num_tokens, CHUNK_SIZE)
     out_hidden_states = hidden_states if inplace else torch.empty_like(hidden_states)
     if num_tokens == 0:
@@ -609,9 +610,9 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
 
     lib = _lib.lib()
     ws_bytes = _workspace_bytes_cached(M, top_k_num, H, I, global_num_experts)
+    stream_handle = torch.cuda.current_stream(hidden_states.device).cuda_stream
     if workspace is None:
-        workspace = _cached_workspace(ws_bytes, hidden_states.device,
-                                      torch.cuda.current_stream(hidden_states.device).cuda_stream)
+        workspace = _cached_workspace(ws_bytes, hidden_states.device, stream_handle)
         ws_bytes = workspace.numel()
     else:  # the caller's own scratch (tests read the intermediates out of it afterwards)
         assert workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.numel() >= ws_bytes
@@ -629,7 +630,7 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
     w4 = bool(flags & _lib.LO_GEMM_W4)
     file_shape = None if channel else ([1, 128] if w4 else [128, 128])
     with _on_device(hidden_states):
-        stream = _lib.stream_of(hidden_states)
+        stream = ctypes_void(stream_handle)
         for chunk in range((num_tokens // CHUNK_SIZE) + 1):
             begin, end = chunk * CHUNK_SIZE, min((chunk + 1) * CHUNK_SIZE, num_tokens)
             m = end - begin
@@ -656,8 +657,6 @@ def _run_fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, cache13, i
 
 
 def ctypes_void(addr: int):
-    import ctypes
-
     return ctypes.c_void_p(addr)
 
 

@@ -236,10 +236,11 @@ def moe_gemm_block_int8(A, As, W, Ws, sorted_ids, expert_ids, ntpp, topk_w, mul_
         _fn = "orc_moe_gemm_block_int8_f32"
     acc = torch.zeros(num_valid, N, K // 128, dtype=torch.int32) if dump_acc else None
     tw = None if topk_w is None else topk_w.reshape(-1).to(torch.float32).contiguous()
-    getattr(lib(), _fn)(
-        _p(A.contiguous()), _p(As.contiguous()), _p(W.contiguous()), _p(Ws.contiguous()),
-        _p(sorted_ids), _p(expert_ids), _p(ntpp), _p(tw), ctypes.c_int(1 if mul_routed else 0),
-        _i32(top_k), _i64(num_valid), _i64(N), _i64(K), _i32(block_size), _p(C), _p(acc))
+    with (_elements_of(C) if C.dtype != torch.float32 else contextlib.nullcontext()):  # a float16 ``out``: rounded to half
+        getattr(lib(), _fn)(
+            _p(A.contiguous()), _p(As.contiguous()), _p(W.contiguous()), _p(Ws.contiguous()),
+            _p(sorted_ids), _p(expert_ids), _p(ntpp), _p(tw), ctypes.c_int(1 if mul_routed else 0),
+            _i32(top_k), _i64(num_valid), _i64(N), _i64(K), _i32(block_size), _p(C), _p(acc))
     return (C, acc) if dump_acc else C
 
 
