@@ -16,12 +16,15 @@ mode the GPU parity tests compare bit for bit with the CPU checker); ms_per_step
 ms_per_step_fused_scale are the same call with LO_GEMM_SEPARATE_ORDER and LO_GEMM_FUSED_SCALE.  `roofline`
 also carries, as flat scalars, the sweep's figures for the targets of the path (the DeepSeek-V3-shaped
 layer at M >= 4096 against the int8 MFMA peak, M <= 64 against the HBM peak) and the ceiling the scale
-arithmetic puts on the matrix pipe (fold_insts_per_elem, mfma_cap_frac, achieved_over_cap).  The last line printed is one JSON object (fields: metric, value, unit,
+arithmetic puts on the matrix pipe (fold_insts_per_elem; mfma_cap_frac = the rate lo_measure_mfma_issue_rate
+reports for MFMAs with that many vector instructions between them over the published peak, measured in
+this run; achieved_over_cap; issue_ceiling_tops holds the measured rates).  The last line printed is one JSON object (fields: metric, value, unit,
 ms_per_step, roofline, cpu_baseline, stage_ms, routers, sweep).
 """
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import statistics
@@ -463,11 +466,23 @@ def main():
     flush = Flusher(dev, args.flush)
     order_flag = {"contract": 0, "separate": _lib.LO_GEMM_SEPARATE_ORDER, "fused": _lib.LO_GEMM_FUSED_SCALE}
     flags_default = order_flag[args.scale_order]
-    # vector instructions the fold spends per accumulator element and K block, and the share of the
-    # matrix pipe's time they leave it at best: an element's two MFMAs cost 8 cycles of matrix pipe, every
-    # vector instruction 4 cycles of the SIMD's vector ALU, and the two run side by side
+    # Vector instructions the fold spends per accumulator element and K block, and the rate the matrix pipe
+    # reaches at best under that load: measured live with a loop of nothing but int8 MFMAs, each followed by
+    # its share of the fold (two elements per v_mfma_i32_16x16x64_i8) as independent v_fma_f32, two waves per
+    # SIMD, on random operand bytes (the clock this chip holds depends on how many operand bits toggle; the
+    # same loop on zeros and the MFMAs alone are reported next to it).
     fold_insts = {"contract": 3, "separate": 4, "fused": 2}[args.scale_order]
-    mfma_cap = min(1.0, 8.0 / (4.0 * fold_insts))
+
+    def issue_rate(valu_per_mfma, random_operands):
+        out = ctypes.c_double(0.0)
+        _lib.check(_lib.lib().lo_measure_mfma_issue_rate(valu_per_mfma, int(random_operands), 40000,
+                                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+                                                         ctypes.byref(out)))
+        return out.value / 1e12
+
+    issue = {"mfma_only_zero_operands_tops": issue_rate(0, False), "mfma_only_tops": issue_rate(0, True),
+             "mfma_with_fold_tops": issue_rate(2 * fold_insts, True)}
+    mfma_cap = min(1.0, issue["mfma_with_fold_tops"] / INT8_PEAK_TOPS)
 
     from lightop_amd.moe import preshuffle_moe_scale_int4, preshuffle_moe_weight, preshuffle_moe_weight_int4
 
@@ -549,6 +564,7 @@ def main():
                 "scale_order": args.scale_order,
                 "fold_insts_per_elem": fold_insts if L.quant != "channel" else 0,
                 "mfma_cap_frac": round(mfma_cap, 3) if L.quant != "channel" else 1.0,
+                "issue_ceiling_tops": {k: round(v, 1) for k, v in issue.items()},
                 "profile": None if prof is None else prof["file"],
                 "profile_kernel_us": None if prof is None else {k: prof[k] for k in ("avg_us", "median_us", "min_us")},
                 "note": "TFLOP/s stands for int8 TOP/s (multiply and add counted separately); kernel_ms is the "

@@ -352,6 +352,21 @@ int lo_moe_tile_query_path(int form, int flags, int dtype, int32_t block_size_m,
                            lo_moe_tile *gemm2);
 
 /*
+ * Measurement aid; no counterpart in the reference.  The block-INT8 GEMMs fold each 128-wide K block's int32
+ * sums into fp32 accumulators with 2, 3 or 4 vector instructions per element (LO_GEMM_FUSED_SCALE, the default
+ * contracted order, LO_GEMM_SEPARATE_ORDER): 4, 6 or 8 per v_mfma_i32_16x16x64_i8, issued by the wave that
+ * issues the MFMA.  This call times a loop of nothing but such MFMAs, each followed by valu_per_mfma (0, 4, 6
+ * or 8) independent v_fma_f32, two waves per SIMD on every compute unit, for `iters` groups of eight MFMAs per
+ * wave, on operand registers holding pseudo-random bytes (random_operands != 0) or zeros, and returns the
+ * int8 operations per second (multiply and add counted separately) the device sustained: the ceiling the
+ * chip's issue logic and clock management put on a K loop with that much scale arithmetic.  It allocates
+ * 256 bytes for the duration of the call and waits for its own kernel.  bench.py reports the result beside
+ * the dominant kernel's rate.
+ */
+int lo_measure_mfma_issue_rate(int valu_per_mfma, int random_operands, int iters, void *stream,
+                               double *int8_ops_per_second);
+
+/*
  * Whole path for one chunk of tokens: quant -> align -> GEMM1(+SiLU*mul+quant) -> GEMM2
  * -> weighted top-k reduce.  Replaces the body of fused_experts_impl_int8
  * (int8.py:703-888); the reduce is always performed.

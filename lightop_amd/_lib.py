@@ -74,6 +74,7 @@ SIGNATURES = {
                                        ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
     "lo_moe_tile_query_path": (c_int, [c_int, c_int, c_int, c_int32, c_int64, c_int32, c_int32, c_int32, c_int64,
                                        c_int64, ctypes.POINTER(LoMoeTile), ctypes.POINTER(LoMoeTile)]),
+    "lo_measure_mfma_issue_rate": (c_int, [c_int, c_int, c_int, c_void_p, ctypes.POINTER(ctypes.c_double)]),
     "lo_fused_experts_workspace_bytes": (c_int64, [c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
     "lo_fused_experts_workspace_offset": (c_int64, [c_int, c_int64, c_int32, c_int64, c_int64, c_int32, c_int32]),
     "lo_per_token_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),

@@ -635,3 +635,28 @@ def test_fused_experts_rejects_unsupported(dev):
     with pytest.raises(AssertionError):
         fused_experts_impl_int8(x[:, :128], w1, w2, tw, ids, c, use_int8_w8a8=True, block_shape=[128, 128],
                                 w1_scale=s1, w2_scale=s2)
+
+
+def test_issue_rate_measurement_is_sane(dev):
+    """lo_measure_mfma_issue_rate: positive rates below the published int8 peak, and the more vector instructions
+    between the MFMAs the lower the rate; bad arguments are refused."""
+    import ctypes
+
+    from lightop_amd import _lib
+
+    def rate(valu, random_operands, iters=4000):
+        out = ctypes.c_double(0.0)
+        rc = _lib.lib().lo_measure_mfma_issue_rate(valu, random_operands, iters,
+                                                   ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+                                                   ctypes.byref(out))
+        return rc, out.value
+
+    rates = {}
+    for valu in (0, 4, 6, 8):
+        rc, v = rate(valu, 1)
+        assert rc == 0 and 0.0 < v < 5.2e15
+        rates[valu] = v
+    assert rates[0] > rates[4] > rates[6] > rates[8]
+    rc, zero = rate(0, 0)
+    assert rc == 0 and zero >= 0.9 * rates[0]   # zeros toggle nothing: never slower than random bytes
+    assert rate(5, 1)[0] == -1 and rate(6, 1, iters=0)[0] == -1   # LO_EINVAL
