@@ -182,8 +182,6 @@ class Point:
         out = torch.empty(self.M, L.H, dtype=torch.bfloat16, device=self.dev)
         if L.quant == "channel":
             return self.stage_times_channel(steps, warmup, flush, bs), bs
-        a2q_buf = torch.empty(S, L.I, dtype=torch.int8, device=self.dev)
-        a2s_buf = torch.empty(S, L.I // 128, dtype=torch.float32, device=self.dev)
         names = ["quant", "align", "gemm1_silu_quant", "gemm2", "moe_sum"]
         acc = {n: [] for n in names}
         # With an expert_map the whole path leaves the rows of other ranks' slots untouched and
@@ -205,15 +203,9 @@ class Point:
                 mask = None
                 s, e, p = moe.moe_align_block_size(ids, bs, L.E_global, self.emap)
             ev[2].record()
-            if bs == 160:  # 160-token blocks: plain first GEMM, activation and quantisation in a launch of their own
-                c1 = self.cache13[: S * 2 * L.I].view(S, 2 * L.I)
-                moe.invoke_fused_moe_kernel_int8(a1q, self.w1, c1, a1s, self.w1s, tw, s, e, p, False, L.top_k, cfg,
-                                                 flags=g2flag | order_flags, global_num_experts=L.E_global)
-                a2q, a2s = moe.act_and_mul_group_quant(c1, row_mask=mask, out=(a2q_buf, a2s_buf))
-            else:
-                a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
-                                                                 L.top_k, S, cfg,
-                                                                 flags=wflag | order_flags, global_num_experts=L.E_global)
+            a2q, a2s = moe.invoke_fused_moe_gemm1_silu_quant(a1q, self.w1, a1s, self.w1s, tw, s, e, p, False,
+                                                             L.top_k, S, cfg,
+                                                             flags=wflag | order_flags, global_num_experts=L.E_global)
             ev[3].record()
             moe.invoke_fused_moe_kernel_int8(a2q, self.w2, c3, a2s, self.w2s, tw, s, e, p, True, 1, cfg,
                                              flags=g2flag | order_flags, global_num_experts=L.E_global)
@@ -557,8 +549,7 @@ def main():
                 "frac": round(ach / peak, 4), "traffic": None if prof is None else prof["traffic_bytes"],
                 "algorithmic_bytes": int(g1_bytes), "algorithmic_ops": int(g1_ops),
                 "kernel": kname + (" (GEMM1, per-channel scales in the epilogue)" if L.quant == "channel"
-                                   else " with 160-token blocks (plain GEMM1), then act_mul_group_quant_kernel "
-                                        "(SiLU*mul + 1x128 re-quant)" if bs_used == 160
+                                   else "<FUSED_ACT, 160-token blocks> (GEMM1 + SiLU*mul + 1x128 re-quant)" if bs_used == 160
                                    else "<FUSED_ACT> (GEMM1 + SiLU*mul + 1x128 re-quant)"),
                 "kernel_ms": round(stages[g1_name], 4),
                 "scale_order": args.scale_order,

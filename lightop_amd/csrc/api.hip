@@ -85,15 +85,24 @@ static WsLayout ws_layout(int64_t M, int32_t top_k, int64_t H, int64_t I, int32_
   return L;
 }
 
-// 160-token blocks: the first GEMM's bf16 output [S, 2I] has to fit the caller's [S, H] buffer, and both K
-// extents the kernel's scale table (128 K blocks).
-static bool blocks_of_160_fit(int64_t H, int64_t I) { return 2 * I <= H && H / kGroup <= 128 && I / kGroup <= 128; }
+// 160-token blocks: both K extents have to fit the kernel's scale table (128 K blocks); where the first GEMM
+// is not fused with the activation (fp16 rows, GELU) its 16-bit output [S, 2I] has to fit the caller's [S, H]
+// buffer as well.
+static bool blocks_of_160_fit(int64_t H, int64_t I, bool fused) {
+  return (fused || 2 * I <= H) && H / kGroup <= 128 && I / kGroup <= 128;
+}
 
 // gfx950 tile table.  The token tile (= alignment block) follows the expected number
 // of slots per expert: small tiles waste no MFMA columns on padding while the layer
 // is weight-streaming bound, larger ones amortise each pass over an expert's weights.
-static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64_t H, int form = LO_FORM_BLOCK,
-                            bool preshuffled = true, bool int4_channel = false, bool allow160 = false) {
+//
+// The key is (form, weight layout, shape class, expected slots per expert).  The shape class is the size of one
+// expert's weights, 3 * H * I bytes of int8: a handful of megabytes (Qwen3-30B-A3B: H 2048, I 768, 4.7 MB),
+// around twenty (Qwen3-235B-A22B: 4096 x 1536, 18.9 MB), forty and more (DeepSeek-V3: 7168 x 2048, 44 MB); the
+// thresholds below were measured on one layer of each class with `python -m lightop_amd.tune`.
+static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64_t H, int64_t I,
+                            int form = LO_FORM_BLOCK, bool preshuffled = true, bool int4_channel = false,
+                            bool allow160 = false) {
   const double per_expert = static_cast<double>(M) * top_k / (num_experts > 0 ? num_experts : 1);
   // Packed int4 weights with per-channel scales: the 128-token kernel has no scale arithmetic in
   // its K loop and skips the padded part of a block, so it takes over as soon as an expert sees more
@@ -140,7 +149,17 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
   // DeepSeek-V3 share at 3072 (96 per expert): 435 / 451, 3584: 544 / 468, 4096: 581 / 495, 4352:
   // 610 / 616, 4608: 620 / 660.
   if (form == LO_FORM_BLOCK && preshuffled && allow160) {
-    if (H >= 4096 ? (per_expert >= 104.0 && per_expert < 134.0) : (per_expert >= 80.0 && per_expert < 152.0)) return 160;
+    // With the first stage's fused epilogue in the 160-token form as well (no activation launch, no [S, 2I] round
+    // trip) the window widens; whole path in us, 128 / 160: Qwen3-30B-A3B layer at 1024 tokens (64 slots per
+    // expert) 184 / 193, at 1152: 230 / 197, at 2048: 279 / 221, at 2432: 306 / 276, at 2560: 298 / 307;
+    // DeepSeek-V3 share at 2560 (80 per expert): 380 / 367, at 3072: 381 / 373, at 4096: 541 / 428, at 4352:
+    // 561 / 570.
+    // Medium experts (Qwen3-235B-A22B-shaped layer, int8): at 1280 tokens (80 per expert) 573 / 580, at 1536: 606 /
+    // 596, at 2048: 775 / 659, at 2304: 889 / 742, at 2560: 911 / 934.
+    const bool medium = H >= 4096 && 3 * H * I < (32ll << 20);
+    if (medium ? (per_expert >= 88.0 && per_expert < 152.0)
+               : H >= 4096 ? (per_expert >= 76.0 && per_expert < 134.0) : (per_expert >= 68.0 && per_expert < 156.0))
+      return 160;
   }
   // With about one token block per expert the 64-token kernel with register-fed weights
   // (gemm_tile.hip) streams them with the non-temporal hint as well, and its shorter start-up and
@@ -156,6 +175,14 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
       // tokens 313 / 303, at 2816: 325 / 306)
       if (per_expert <= 48.0 || (per_expert >= 96.0 && per_expert < 152.0)) return 64;
       return 128;
+    }
+    if (3 * H * I < (32ll << 20)) {
+      // Medium experts, measured on the Qwen3-235B-A22B-shaped layer with int8 weights (us, whole path, 16 /
+      // 64 / 128): at 16 tokens 253 / 246 / 256, at 64: 416 / 376 / 391, at 128: 450 / 391 / 407, at 256: 631 /
+      // 414 / 427, at 512: 1022 / 444 / 461, at 768: - / 504 / 488, at 1024: - / 618 / 522, at 4096: - / 1392 /
+      // 1200.
+      if (per_expert < 1.0) return 16;
+      return per_expert <= 40.0 ? 64 : 128;
     }
     if (per_expert < 4.0) return 16;
     return (per_expert >= 28.0 && per_expert <= 48.0) ? 64 : 128; // equal within 0.2 % from 16 to 24
@@ -191,7 +218,7 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
 struct BlockPlan {
   int flags;            // the caller's flags, LO_GEMM_W4 implying LO_GEMM_W_PRESHUFFLED
   int32_t block_size_m; // the caller's, or the table's pick when the caller passed 0
-  bool bs160;           // 160-token blocks: plain first GEMM, activation launch, plain second GEMM
+  bool bs160;           // 160-token blocks of the direct-to-LDS kernel
   bool unfused;         // the first GEMM writes [S, 2I] and one launch applies the activation and quantises
   bool try_decode;      // the two-launch path is attempted first (it may still decline by size)
 };
@@ -202,22 +229,23 @@ static int plan_block_path(int dtype, int flags, int64_t M, int32_t num_experts,
   const bool gelu = (flags & LO_FUSED_ACT_GELU) != 0;
   const bool block_size_m_auto = block_size_m == 0;
   if (block_size_m == 0 && dtype == LO_F32) // fp32 rows go through the weight-streaming kernel at every size
-    block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_BLOCK, false);
+    block_size_m = pick_block_m(M, num_experts, top_k, H, I, LO_FORM_BLOCK, false);
   if (block_size_m == 0)
-    block_size_m = pick_block_m(M, num_experts, top_k, H, w4 ? LO_FORM_W4 : LO_FORM_BLOCK, pre, false,
-                                !w4 && dtype == LO_BF16 && !gelu && blocks_of_160_fit(H, I));
-  // 160: the 160-token form of the direct-to-LDS kernel (int8 block form, load-time layout), both GEMMs
-  // with plain epilogues and the activation in a launch of its own
-  const bool bs160 = block_size_m == 160 && pre && !w4 && dtype != LO_F32 && blocks_of_160_fit(H, I);
+    block_size_m = pick_block_m(M, num_experts, top_k, H, I, w4 ? LO_FORM_W4 : LO_FORM_BLOCK, pre, false,
+                                !w4 && dtype == LO_BF16 && !gelu && blocks_of_160_fit(H, I, true));
+  // 160: the 160-token form of the direct-to-LDS kernel (int8 block form, load-time layout) for both GEMMs; bf16
+  // rows with SiLU take its fused first stage, fp16 rows and GELU the plain one and the activation launch
+  const bool fused_ok = dtype == LO_BF16 && !gelu;
+  const bool bs160 = block_size_m == 160 && pre && !w4 && dtype != LO_F32 && blocks_of_160_fit(H, I, fused_ok);
   LO_REQUIRE(block_size_m == 16 || block_size_m == 32 || block_size_m == 64 || block_size_m == 128 || bs160,
              LO_EINVAL,
              "fused_experts: block_size_m %d is not one of 16, 32, 64, 128 (160: int8 weights in the load-time "
-             "layout, 16-bit rows and 2I <= H only)", block_size_m);
+             "layout and 16-bit rows; with fp16 rows or GELU 2I <= H as well)", block_size_m);
   plan->flags = flags;
   plan->block_size_m = block_size_m;
   plan->bs160 = bs160;
   // GELU and fp16 / fp32 activations have no fused epilogue
-  plan->unfused = gelu || dtype != LO_BF16 || bs160;
+  plan->unfused = !fused_ok;
   plan->try_decode = block_size_m_auto && pre && !plan->unfused && !(flags & LO_FUSED_NO_DECODE_PATH);
   return LO_OK;
 }
@@ -243,7 +271,7 @@ extern "C" int lo_moe_tile_query_path(int form, int flags, int dtype, int32_t bl
   if (form == LO_FORM_CHANNEL) {
     const bool pre = (flags & (LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED)) != 0;
     if (bm == 0)
-      bm = pick_block_m(M, num_experts, top_k, H, form, true, (flags & LO_GEMM_W4) != 0,
+      bm = pick_block_m(M, num_experts, top_k, H, I, form, true, (flags & LO_GEMM_W4) != 0,
                         pre && H / kGroup <= 128 && I / kGroup <= 128);
   } else {
     BlockPlan plan;
@@ -443,7 +471,7 @@ static int fused_experts_channel(
              "fused_experts(channel): workspace must be 256-byte aligned");
   if (M == 0) return LO_OK;
   if (block_size_m == 0)
-    block_size_m = pick_block_m(M, num_experts, top_k, H, LO_FORM_CHANNEL, true, (flags & LO_GEMM_W4) != 0,
+    block_size_m = pick_block_m(M, num_experts, top_k, H, I, LO_FORM_CHANNEL, true, (flags & LO_GEMM_W4) != 0,
                                 (flags & (LO_GEMM_W4 | LO_GEMM_W_PRESHUFFLED)) && H / kGroup <= 128 &&
                                     I / kGroup <= 128);
   // 160: the 160-token form of the direct-to-LDS kernel (weights in the load-time layout)

@@ -146,9 +146,8 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
   int rc = validate_common("moe_gemm1_silu_quant", A, As, W, Ws, sorted_ids, expert_ids,
                            num_tokens_post_pad, K, top_k, E, a_rows);
   if (rc) return rc;
-  LO_REQUIRE(valid_block_m(block_size_m), LO_EINVAL,
-             "moe_gemm1_silu_quant: block_size_m %d is not one of 16, 32, 64, 128 (160-token blocks have no fused "
-             "epilogue: lo_moe_gemm_block_int8, then lo_act_mul_group_quant)", block_size_m);
+  LO_REQUIRE(valid_block_m(block_size_m) || block_size_m == 160, LO_EINVAL,
+             "moe_gemm1_silu_quant: block_size_m %d is not one of 16, 32, 64, 128 (or 160)", block_size_m);
   LO_REQUIRE(A2q && A2s, LO_EINVAL, "moe_gemm1_silu_quant: null output");
   LO_REQUIRE(c_dtype == LO_BF16, LO_ENOTSUP, "moe_gemm1_silu_quant: only bf16 rounding is built");
   LO_REQUIRE(I > 0 && I % kGroup == 0, LO_EINVAL,
@@ -172,6 +171,9 @@ extern "C" int lo_moe_gemm1_silu_quant_block_int8(
              "moe_gemm1_silu_quant: int4 weights must be in the layout of lo_preshuffle_weight_int4 "
              "(LO_GEMM_W_PRESHUFFLED)");
   a.n_tiles = static_cast<int32_t>(I / kGroup);
+  LO_REQUIRE(block_size_m != 160 || gemm_t128_supports(a, true, 160), LO_ENOTSUP,
+             "moe_gemm1_silu_quant: 160-token blocks need int8 weights in the load-time layout "
+             "(LO_GEMM_W_PRESHUFFLED) and K <= %d", kGroup * 128);
   rc = silu_table(static_cast<hipStream_t>(stream), &a.silu);
   if (rc) return rc;
   const int64_t mblocks = grid_m_blocks(sorted_cap, num_valid, block_size_m);

@@ -73,8 +73,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   static_assert(!PC || (!FUSED_ACT && ORD == kOrdSeparate && (W4 || NTB == 10)),
                 "per-channel scales: plain GEMM, int4 weights or 160-token tiles of int8 weights");
-  static_assert(NTB == 8 || (NTB == 10 && !FUSED_ACT && (PC || !W4)),
-                "160-token tiles: plain GEMM, int8 block form or per-channel scales");
+  static_assert(NTB == 8 || (NTB == 10 && (PC || !W4)),
+                "160-token tiles: int8 block form (plain or fused epilogue) or per-channel scales");
   constexpr int T = 16 * NTB;        // tokens per workgroup
   constexpr int AST = T * kGroup;    // token rows of one K block
   constexpr int APW = NTB / 2;       // 1 KB pieces (eight token rows) of a token stage that a wave copies
@@ -82,10 +82,18 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   int8_t *const sA = smem + kTW;
   float *const sS = reinterpret_cast<float *>(smem + kTW + 2 * AST);
-  float *const sRed = reinterpret_cast<float *>(smem + kTW + 2 * AST + 2 * T * 4);
+  // 160-token tiles have no room for the fused epilogue's amax exchange and SiLU band beside the stages
+  // (two workgroups per compute unit): there every wave copies the band into its own weight stage once its K
+  // loop is done, and its row of the exchange lies behind the band.
+  constexpr bool kLateBand = FUSED_ACT && NTB == 10;
+  static_assert(!kLateBand || 2 * kSiluBandN * 2 + 160 * 4 <= kTWStage, "band and amax row fit a weight stage");
+  auto red_row = [&](int w) __attribute__((always_inline)) { // [token] amax of wave w's 32 columns
+    if constexpr (kLateBand) return reinterpret_cast<float *>(smem + w * kTWStage + 2 * kSiluBandN * 2);
+    else return reinterpret_cast<float *>(smem + kTW + 2 * AST + 2 * T * 4) + w * T;
+  };
   float *const sBs = reinterpret_cast<float *>(smem + kTW + 2 * AST + 2 * T * 4 + RED);
   int32_t *const sIds = reinterpret_cast<int32_t *>(smem + kTW + 2 * AST + 2 * T * 4 + RED + kTBs);
-  uint16_t *const sSilu = reinterpret_cast<uint16_t *>(smem + kTW + 2 * AST + 2 * T * 4 + RED + kTBs + T * 4);
+  uint16_t *const sSiluShared = reinterpret_cast<uint16_t *>(smem + kTW + 2 * AST + 2 * T * 4 + RED + kTBs + T * 4);
 
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
@@ -125,7 +133,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   }
 
   uint16_t band_regs[kSiluBandPer];
-  if constexpr (FUSED_ACT) silu_band_load(band_regs, a.silu, tid);
+  if constexpr (FUSED_ACT && !kLateBand) silu_band_load(band_regs, a.silu, tid);
 
   // ---- what this wave copies -----------------------------------------------------------------------
   const int NBLK = static_cast<int>(N / 16);
@@ -468,7 +476,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   __builtin_amdgcn_sched_barrier(0);
   if (tid < T) sS[tid] = s_now;
   sBs[tid] = bs_mine;
-  if constexpr (FUSED_ACT) silu_band_store(sSilu, band_regs, tid);
+  if constexpr (FUSED_ACT && !kLateBand) silu_band_store(sSiluShared, band_regs, tid);
   wait_copies<0>();
   read_w();
 
@@ -576,11 +584,29 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
       __builtin_amdgcn_wave_barrier();
     }
   } else {
+    const uint16_t *sSilu = sSiluShared;
+    if constexpr (kLateBand) {
+      // the band of the SiLU table (two runs of kSiluBandN entries, one per sign of the gate) straight into this
+      // wave's own weight stage, 256 bytes per copy
+      const brsrc rT = make_rsrc(a.silu, 65536 * 2);
+      constexpr int kRun = kSiluBandN * 2; // bytes per sign
+#pragma unroll
+      for (int sgn = 0; sgn < 2; ++sgn)
+#pragma unroll
+        for (int j = 0; j < (kRun + 255) / 256; ++j) {
+          int off = j * 256 + lane * 4;
+          off = off < kRun ? off : kRun - 4; // the last copy's surplus lanes repeat the run's last word
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rT, sWw + sgn * kRun + j * 256, 4,
+                                                   (sgn * 0x8000 + kSiluBandLo) * 2 + off, 0, 0, 0);
+        }
+      wait_copies<0>();
+      sSilu = reinterpret_cast<const uint16_t *>(sWw);
+    }
     // acc[h][tb][0] = gate, acc[h][tb][1] = up for activation columns nt*128 + wave*32 + 16h + 4q + i
-    float actf[8][2][4];
+    float actf[NTB][2][4];
     if (a.mul_routed) { // router weight on the first GEMM's output: rare, kept out of the main pass
 #pragma unroll
-      for (int tb = 0; tb < 8; ++tb) {
+      for (int tb = 0; tb < NTB; ++tb) {
         const int64_t ft = sIds[tb * 16 + r];
         const float wgt = ft < a.num_valid ? a.topk_w[ft] : 1.0f;
 #pragma unroll
@@ -594,7 +620,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     // Token fragments are in use in pairs (nst is a multiple of four stages).  A pair shares one
     // wave-uniform branch, so the LDS lookups of its two fragments are in flight together.
 #pragma unroll
-    for (int tb = 0; tb < 8; ++tb) {
+    for (int tb = 0; tb < NTB; ++tb) {
       if (2 * (tb & ~1) >= nst) continue; // the same condition for both fragments of a pair
       uint16_t g16[2][4], u16[2][4];
       bool special = false;
@@ -621,7 +647,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
         for (int i = 0; i < 4; ++i) amax = fmaxf(amax, fabsf(actf[tb][h][i]));
       amax = fmaxf(amax, __shfl_xor(amax, 16));
       amax = fmaxf(amax, __shfl_xor(amax, 32));
-      if (q == 0) sRed[wave * kT + tb * 16 + r] = amax;
+      if (q == 0) red_row(wave)[tb * 16 + r] = amax;
     }
     __syncthreads(); // also: every wave is done with the token stages
     const int64_t G = I / kGroup;
@@ -629,17 +655,17 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     int8_t *qst = sA;
     // scales of all eight fragments first, outside the branches on nst: the reads are in bounds
     // either way, and one batch of LDS reads and divisions replaces eight dependent chains
-    float sc_all[8], rsc_all[8];
+    float sc_all[NTB], rsc_all[NTB];
 #pragma unroll
-    for (int tb = 0; tb < 8; ++tb) {
+    for (int tb = 0; tb < NTB; ++tb) {
       const int t = tb * 16 + r;
-      float amax = fmaxf(fmaxf(sRed[t], sRed[kT + t]), fmaxf(sRed[2 * kT + t], sRed[3 * kT + t]));
+      float amax = fmaxf(fmaxf(red_row(0)[t], red_row(1)[t]), fmaxf(red_row(2)[t], red_row(3)[t]));
       amax = fmaxf(amax, 1e-10f);
       sc_all[tb] = amax / 127.0f;
       rsc_all[tb] = 1.0f / sc_all[tb];
     }
 #pragma unroll
-    for (int tb = 0; tb < 8; ++tb) {
+    for (int tb = 0; tb < NTB; ++tb) {
       if (2 * (tb & ~1) >= nst) continue;
       const int t = tb * 16 + r;
       const float sc = sc_all[tb], rsc = rsc_all[tb];
@@ -653,7 +679,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < kT * 8 / 256; ++j) {
+    for (int j = 0; j < T * 8 / 256; ++j) {
       const int id = tid + 256 * j, tok = id >> 3, piece = id & 7;
       const int64_t ft = sIds[tok];
       if (ft < a.num_valid)
@@ -664,8 +690,11 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 }
 
 bool gemm_t128_supports(const GemmArgs &a, bool fused_act, int block_size_m) {
-  if (block_size_m == kT160) // 160-token tiles: plain GEMM, int8 block form or per-channel scales
-    return a.w_shuffled && !fused_act && (a.per_channel || !a.w4) && a.N % 64 == 0 && a.K / kGroup <= kTMaxKB;
+  if (block_size_m == kT160) { // 160-token tiles: int8 block form (plain or fused epilogue) or per-channel scales
+    if (!a.w_shuffled || a.K / kGroup > kTMaxKB) return false;
+    if (fused_act) return !a.per_channel && !a.w4;
+    return (a.per_channel || !a.w4) && a.N % 64 == 0;
+  }
   if (block_size_m != 128 || !a.w_shuffled) return false;
   if (a.per_channel && (!a.w4 || fused_act)) return false; // int8 per-channel weights have gemm_pc.hip
   if (!fused_act && a.N % 64 != 0) return false;
@@ -712,14 +741,14 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int f
   } while (0)
   if (block_size_m == kT160) {
     // chosen where an expert's tokens fill one block, so a weight byte has one reader: streaming hint
-#define LO_T160_LAUNCH(FS)                                                                                      \
+#define LO_T160_LAUNCH(FS, FA)                                                                                  \
   do {                                                                                                          \
     static unsigned long long lds_done = 0;                                                                     \
     const int rc_lds = reserve_lds_once(                                                                        \
-        reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, FS, true, false, false, 10>), kTLds160,     \
+        reinterpret_cast<const void *>(&moe_gemm_t128_kernel<FA, FS, true, false, false, 10>), kTLds160,        \
         &lds_done);                                                                                             \
     if (rc_lds) return rc_lds;                                                                                  \
-    hipLaunchKernelGGL((moe_gemm_t128_kernel<false, FS, true, false, false, 10>), g, b, kTLds160, s, a, mbi, gi); \
+    hipLaunchKernelGGL((moe_gemm_t128_kernel<FA, FS, true, false, false, 10>), g, b, kTLds160, s, a, mbi, gi);  \
   } while (0)
     if (a.per_channel && a.w4) {
       static unsigned long long lds_done = 0;
@@ -733,11 +762,13 @@ int launch_gemm_t128(const GemmArgs &a0, bool fused_act, int block_size_m, int f
           reinterpret_cast<const void *>(&moe_gemm_t128_kernel<false, kOrdSeparate, true, false, true, 10>), kTLds160, &lds_done);
       if (rc_lds) return rc_lds;
       hipLaunchKernelGGL((moe_gemm_t128_kernel<false, kOrdSeparate, true, false, true, 10>), g, b, kTLds160, s, a, mbi, gi);
-    } else if (ord == kOrdContract) LO_T160_LAUNCH(kOrdContract);
-    else if (ord == kOrdSeparate) LO_T160_LAUNCH(kOrdSeparate);
-    else LO_T160_LAUNCH(kOrdFusedScale);
+    } else if (fused_act) {
+      LO_ORD_DISPATCH(ord, LO_T160_LAUNCH, true);
+    } else {
+      LO_ORD_DISPATCH(ord, LO_T160_LAUNCH, false);
+    }
 #undef LO_T160_LAUNCH
-    return check_launch("moe_gemm(t160)");
+    return check_launch(fused_act ? "moe_gemm1_silu_quant(t160)" : "moe_gemm(t160)");
   }
   // one token block per expert, by and large: the slots spread over the routed experts fill half a block
   const bool stream = a.num_valid <= static_cast<int64_t>(a.experts_routed > 0 ? a.experts_routed : 1) * (kT / 2);

@@ -48,6 +48,10 @@ DSV3_EP = MoeLayer("deepseek-v3-ep8-share", E=32, E_global=256, top_k=8, H=7168,
 DSV3_FULL = MoeLayer("deepseek-v3-full", E=256, E_global=256, top_k=8, H=7168, I=2048,
                      routing="grouped_sigmoid_zipf", n_group=8, topk_group=4, routed_scaling=2.5)
 
+# Qwen3-235B-A22B-shaped layer with int8 weights in the block form: a third shape class for the tile table
+# (H = 4096 between the other two layers' 2048 and 7168, I = 1536)
+QWEN3_235B = MoeLayer("qwen3-235b-a22b", E=128, E_global=128, top_k=8, H=4096, I=1536, routing="softmax")
+
 TINY_W4 = MoeLayer("tiny-e8-w4a8", E=8, E_global=8, top_k=2, H=1024, I=512, routing="softmax", weight_bits=4)
 QWEN3_235B_W4 = MoeLayer("qwen3-235b-a22b-w4a8", E=128, E_global=128, top_k=8, H=4096, I=1536, routing="softmax",
                          weight_bits=4)
@@ -64,7 +68,7 @@ QWEN3_30B_PC = MoeLayer("qwen3-30b-a3b-channel", E=128, E_global=128, top_k=8, H
 DSV3_EP_PC = MoeLayer("deepseek-v3-ep8-share-channel", E=32, E_global=256, top_k=8, H=7168, I=2048,
                       routing="grouped_sigmoid", n_group=8, topk_group=4, routed_scaling=2.5, quant="channel")
 
-LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL, TINY_W4, QWEN3_235B_W4, TINY_W4_PC,
+LAYERS = {l.name: l for l in (TINY, QWEN3_30B, DSV3_EP, DSV3_FULL, QWEN3_235B, TINY_W4, QWEN3_235B_W4, TINY_W4_PC,
                               QWEN3_235B_W4_PC, TINY_PC, QWEN3_30B_PC, DSV3_EP_PC)}
 
 

@@ -72,21 +72,25 @@ def test_version_and_tile_table(lib):
     # kernels from a handful of slots per expert on (64-token tiles while there is about one token block
     # per expert, on a short K up to 48 slots per expert), 160-token blocks around 128 slots per expert
     # (where a 128-token block would spill a few tokens into a second pass over the expert's weights)
-    for M, want in ((64, 16), (128, 128), (256, 128), (512, 128), (1024, 64), (1280, 64), (1536, 64), (2048, 128), (3072, 128),
-                    (3584, 160), (4096, 160), (4352, 128)):
+    for M, want in ((64, 16), (128, 128), (256, 128), (512, 128), (1024, 64), (1280, 64), (1536, 64), (2048, 128), (2304, 128),
+                    (2560, 160), (3072, 160), (3584, 160), (4096, 160), (4352, 128)):
         assert lib.lo_moe_tile_query(M, 32, 256, 8, 7168, 2048, t1, t2) == 0 and t1.block_size_m == want
-    for M, want in ((64, 16), (128, 64), (512, 64), (768, 64), (1024, 128), (1280, 160), (1536, 160), (2048, 160),
-                    (2304, 160), (2560, 128), (3072, 128), (8192, 128)):
+    for M, want in ((64, 16), (128, 64), (512, 64), (768, 64), (1024, 128), (1152, 160), (1280, 160), (1536, 160),
+                    (2048, 160), (2304, 160), (2432, 160), (2560, 128), (3072, 128), (8192, 128)):
         assert lib.lo_moe_tile_query(M, 128, 128, 8, 2048, 768, t1, t2) == 0 and t1.block_size_m == want
     assert lib.lo_moe_tile_query(512, 128, 128, 8, 2048, 768, t1, t2) == 0
     assert t1.kernel == _lib.LO_KERNEL_TILE == t2.kernel
-    # 160-token blocks: the same direct-to-LDS kernel for both GEMMs, the first one without its fused epilogue
+    # a third shape class by the size of an expert's weights (3 * H * I bytes: 4096 x 1536 lies between the two
+    # layers above): 64-token tiles up to 40 slots per expert, 160-token blocks from 88 to 152
+    for M, want in ((8, 16), (16, 64), (512, 64), (768, 128), (1280, 128), (1536, 160), (2304, 160), (2560, 128)):
+        assert lib.lo_moe_tile_query(M, 128, 128, 8, 4096, 1536, t1, t2) == 0 and t1.block_size_m == want
+    # 160-token blocks: the same direct-to-LDS kernel for both GEMMs
     assert lib.lo_moe_tile_query(4096, 32, 256, 8, 7168, 2048, t1, t2) == 0
     assert t1.kernel == _lib.LO_KERNEL_T128 == t2.kernel and (t1.waves, t1.block_n) == (4, 256)
-    # not with row-major weights, and not where the first GEMM's output would not fit the caller's [S, H] buffer
+    # not with row-major weights; the fused first stage needs no [S, 2I] buffer, so 2I > H is no obstacle
     assert lib.lo_moe_tile_query_form(_lib.LO_FORM_BLOCK, 0, 2048, 128, 128, 8, 2048, 768, t1, t2) == 0
     assert t1.block_size_m == 64
-    assert lib.lo_moe_tile_query(2048, 128, 128, 8, 2048, 1536, t1, t2) == 0 and t1.block_size_m == 64
+    assert lib.lo_moe_tile_query(2048, 128, 128, 8, 2048, 1536, t1, t2) == 0 and t1.block_size_m == 160
     # per-channel form: streaming tiles up to half a dozen slots per expert, then the LDS-tiled kernels
     # (128 tokens on a long K; on a short K 64 tokens until an expert sees 48)
     for M, want in ((1, 16), (64, 16), (192, 16), (256, 128), (1024, 128), (8192, 128)):

@@ -1,8 +1,8 @@
 """GPU parity of the 160-token form of the direct-to-LDS GEMM kernel (block size 160: chosen by the tile table
 around 128 slots per expert, where a 128-token block would spill a few tokens into a second pass over the
-expert's weights), through the C ABI, bit for bit against the oracle: the plain GEMM at every fill level
-of a block, the activation + group-quantisation launch that follows the first GEMM on this path, and the
-whole path, explicitly and where the table picks it."""
+expert's weights), through the C ABI, bit for bit against the oracle: the plain GEMM and the first stage with its
+fused SiLU*mul + re-quantisation at every fill level of a block, the activation + group-quantisation launch that
+follows the plain first GEMM with fp16 rows and GELU, and the whole path, explicitly and where the table picks it."""
 import math
 
 import pytest
@@ -116,9 +116,96 @@ def test_160_token_blocks_need_the_load_time_layout(dev):
     with pytest.raises(RuntimeError, match="160-token blocks"):  # row-major weights
         invoke_fused_moe_kernel_int8(Aq.to(dev), W.to(dev), C, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, False, 2,
                                      {"BLOCK_SIZE_M": 160})
-    with pytest.raises(RuntimeError, match="no fused"):  # the fused first stage has no 160-token form
+    with pytest.raises(RuntimeError, match="160-token blocks"):  # the fused first stage as well
         invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), W.to(dev), As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, False, 2,
                                           16, {"BLOCK_SIZE_M": 160})
+
+
+@pytest.mark.parametrize("count,K", [(c, 384) for c in (1, 32, 33, 64, 65, 127, 128, 129, 144, 145, 160, 161, 330)] +
+                         [(c, k) for k in (128, 256, 1024) for c in (40, 136, 160)])
+def test_gemm1_fused_160_token_blocks_fill_levels(dev, oracle, count, K):
+    """The first stage with its fused epilogue on blocks of 160 holding 1 ... 160 valid tokens, in both bit-exact
+    scale orders, with and without the router weight: int8 activations and group scales against the oracle.
+    (The SiLU band and the amax exchange of this form live in the waves' weight stages after the K loop.)"""
+    from lightop_amd import _lib
+    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_weight
+
+    say(f"fused first stage, 160-token blocks, {count} tokens on expert 0, K = {K}")
+    bs, E, I = 160, 2, 256
+    M = count + 3
+    Aq, As, W, Ws, _, tw, _ = gemm_case(1000 + count, M, 1, E, E, 2 * I, K)
+    Ws = Ws * 30  # gates where SiLU is neither 0 nor the identity
+    ids = torch.ones(M, 1, dtype=torch.int32)
+    ids[torch.randperm(M, generator=torch.Generator().manual_seed(count))[:count]] = 0
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, E)
+    s, e, p = moe_align_block_size(ids.to(dev), bs, E)
+    Wsh = preshuffle_moe_weight(W.to(dev))
+    for mul in (False, True):
+        for order, flags in (("contract", 0), ("separate", _lib.LO_GEMM_SEPARATE_ORDER)):
+            with oracle.scale_order(order):
+                c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, mul, 1, M, bs)
+            rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+            q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wsh, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, mul,
+                                                      1, M, {"BLOCK_SIZE_M": bs}, flags=flags)
+            torch.cuda.synchronize()
+            assert torch.equal(sc.cpu(), rsc), f"scales differ (mul_routed={mul}, order={order})"
+            assert torch.equal(q.cpu(), rq), f"int8 activations differ (mul_routed={mul}, order={order})"
+
+
+@pytest.mark.parametrize("M,k,E,Eg,I,K", [(9, 2, 4, 4, 256, 512), (400, 4, 8, 8, 384, 1152), (900, 8, 4, 16, 256, 768)])
+def test_gemm1_fused_160_bit_exact_with_expert_map(dev, oracle, M, k, E, Eg, I, K):
+    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_weight
+
+    say(f"fused first stage bs=160 M={M} k={k} E={E}/{Eg} I={I} K={K}")
+    bs = 160
+    Aq, As, W, Ws, ids, tw, emap = gemm_case(M + I, M, k, E, Eg, 2 * I, K)
+    Ws = Ws * 30
+    rs, re, rp = oracle.moe_align_block_size(ids, bs, Eg, expert_map=emap)
+    S = M * k
+    s, e, p = moe_align_block_size(ids.to(dev), bs, Eg, None if emap is None else emap.to(dev))
+    c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, False, k, S, bs)
+    rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+    q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), preshuffle_moe_weight(W.to(dev)), As.to(dev), Ws.to(dev),
+                                              tw.to(dev), s, e, p, False, k, S, {"BLOCK_SIZE_M": bs})
+    torch.cuda.synchronize()
+    local = torch.ones(S, dtype=torch.bool) if emap is None else emap.long()[ids.reshape(-1).long()] >= 0
+    assert torch.equal(sc.cpu()[local], rsc[local]) and torch.equal(q.cpu()[local], rq[local])
+
+
+def test_gemm1_fused_160_every_finite_bf16_gate_and_special_gates(dev, oracle):
+    """Every bf16 value below 1e18 in magnitude as the gate of the 160-token form's fused epilogue, then rows with
+    NaN and infinite gates next to ordinary rows (they leave the fast lookup by a wave-wide vote)."""
+    from lightop_amd.moe import invoke_fused_moe_gemm1_silu_quant, moe_align_block_size, preshuffle_moe_weight
+
+    say("fused first stage bs=160 over all bf16 gates")
+    bs, I, K = 160, 128, 128
+    pat = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    pat = pat[torch.isfinite(pat) & (pat.abs() < 1e18)]
+    g = torch.Generator().manual_seed(3)
+    special = torch.randn(200, generator=g) * 3
+    special[5], special[70], special[71], special[150] = float("inf"), float("-inf"), float("nan"), float("-inf")
+    W = torch.zeros(1, 2 * I, K, dtype=torch.int8)
+    W[0, :, 0] = 1
+    Wsh = preshuffle_moe_weight(W.to(dev))
+    for vals in (pat, special):
+        M = vals.numel()
+        Aq = torch.zeros(M, K, dtype=torch.int8)
+        Aq[:, 0] = 1
+        As = vals.reshape(M, 1).contiguous()
+        Ws = torch.ones(1, 2, 1)
+        ids = torch.zeros(M, 1, dtype=torch.int32)
+        tw = torch.ones(M, 1)
+        rs, re, rp = oracle.moe_align_block_size(ids, bs, 1)
+        c1 = oracle.moe_gemm_block_int8(Aq, As, W, Ws, rs, re, rp, tw, False, 1, M, bs)
+        rq, rsc = oracle.per_token_group_quant_int8(oracle.silu_and_mul(c1))
+        s, e, p = moe_align_block_size(ids.to(dev), bs, 1)
+        q, sc = invoke_fused_moe_gemm1_silu_quant(Aq.to(dev), Wsh, As.to(dev), Ws.to(dev), tw.to(dev), s, e, p, False,
+                                                  1, M, {"BLOCK_SIZE_M": bs})
+        torch.cuda.synchronize()
+        ordinary = torch.isfinite(vals)
+        assert torch.equal(sc.cpu()[ordinary], rsc[ordinary]) and torch.equal(q.cpu()[ordinary], rq[ordinary])
+        sp = ~ordinary
+        assert ((torch.isnan(sc.cpu()[sp]) == torch.isnan(rsc[sp])) & (torch.isinf(sc.cpu()[sp]) == torch.isinf(rsc[sp]))).all()
 
 
 @pytest.mark.parametrize("rows,I", [(1, 128), (7, 768), (33, 2048), (130, 256)])
