@@ -160,6 +160,11 @@ static int32_t pick_block_m(int64_t M, int32_t num_experts, int32_t top_k, int64
     if (medium ? (per_expert >= 88.0 && per_expert < 152.0)
                : H >= 4096 ? (per_expert >= 76.0 && per_expert < 134.0) : (per_expert >= 68.0 && per_expert < 156.0))
       return 160;
+    // Small experts again around 256 slots per expert, where two 160-token blocks hold what would spill into a
+    // third block of 128 (Qwen3-30B-A3B layer, 128 / 160: at 3840 tokens 365 / 381, at 4096: 391 / 376, at 4352:
+    // 415 / 382, at 4608: 429 / 427, at 5120: 445 / 491); the larger experts, whose tiles are bound by arithmetic
+    // at that size, gain nothing there (DeepSeek-V3 share at 8192 tokens 795 / 801).
+    if (H < 4096 && per_expert >= 248.0 && per_expert < 284.0) return 160;
   }
   // With about one token block per expert the 64-token kernel with register-fed weights
   // (gemm_tile.hip) streams them with the non-temporal hint as well, and its shorter start-up and

@@ -76,7 +76,8 @@ def test_version_and_tile_table(lib):
                     (2560, 160), (3072, 160), (3584, 160), (4096, 160), (4352, 128)):
         assert lib.lo_moe_tile_query(M, 32, 256, 8, 7168, 2048, t1, t2) == 0 and t1.block_size_m == want
     for M, want in ((64, 16), (128, 64), (512, 64), (768, 64), (1024, 128), (1152, 160), (1280, 160), (1536, 160),
-                    (2048, 160), (2304, 160), (2432, 160), (2560, 128), (3072, 128), (8192, 128)):
+                    (2048, 160), (2304, 160), (2432, 160), (2560, 128), (3072, 128), (4096, 160), (4352, 160), (4608, 128),
+                    (8192, 128)):
         assert lib.lo_moe_tile_query(M, 128, 128, 8, 2048, 768, t1, t2) == 0 and t1.block_size_m == want
     assert lib.lo_moe_tile_query(512, 128, 128, 8, 2048, 768, t1, t2) == 0
     assert t1.kernel == _lib.LO_KERNEL_TILE == t2.kernel
