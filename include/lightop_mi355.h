@@ -219,7 +219,8 @@ int lo_moe_gemm_block_int8(const int8_t *A, const float *As, const int8_t *W, co
  * int8.py:784-823 without materialising intermediate_cache1 / intermediate_cache2.
  *   W [E, 2I, K] (gate rows first, then up rows), Ws [E, 2I/128, K/128]
  *   A2q [num_valid, I] int8, A2s [num_valid, I/128] f32 (rows of -1 blocks untouched)
- * I % 128 == 0, K % 128 == 0; A, W and A2q 16-byte aligned.
+ * I % 128 == 0, K % 128 == 0; A, W and A2q 16-byte aligned.  block_size_m: 16, 32, 64, 128, or 160 with
+ * int8 weights in the load-time layout and K <= 16384.
  */
 int lo_moe_gemm1_silu_quant_block_int8(const int8_t *A, const float *As, const int8_t *W,
                                        const float *Ws, int8_t *A2q, float *A2s, int c_dtype,
@@ -304,9 +305,9 @@ int lo_preshuffle_weight_int8(const int8_t *src, int8_t *dst, int32_t E, int64_t
  * configs/w8a8/MOE_BLOCKINT8[128,128]_*.json.
  */
 typedef struct lo_moe_tile {
-  int32_t block_size_m; /* 16, 32, 64, 128 or 160; with 160 the first GEMM is the plain stage
-                         * (lo_moe_gemm_block_int8) followed by lo_act_mul_group_quant: the fused first
-                         * stage has no 160-token form */
+  int32_t block_size_m; /* 16, 32, 64, 128 or 160 (160: int8 weights in the load-time layout; bf16 rows with
+                         * SiLU keep the fused first stage, fp16 rows and GELU take the plain stage
+                         * followed by lo_act_mul_group_quant, as they do with every block size) */
   int32_t kernel;       /* LO_KERNEL_*: the kernel the stage entry points launch for this problem */
   int32_t waves;        /* wavefronts per workgroup of that kernel */
   int32_t block_n;      /* weight rows per workgroup of that kernel */
@@ -381,10 +382,10 @@ int lo_measure_mfma_issue_rate(int valu_per_mfma, int random_operands, int iters
  *   workspace: lo_fused_experts_workspace_bytes(...) bytes of device memory, 256-byte aligned
  *   block_size_m: 0 = take it from the tile table (lo_fused_experts_workspace_bytes(.., 0) is
  *   large enough for whatever the table picks and for every explicit block size); 16, 32, 64, 128,
- *   or 160 (int8 weights in the load-time layout, 2I <= H: 160-token blocks of the direct-to-LDS
- *   kernel with plain epilogues and lo_act_mul_group_quant between the GEMMs - what the table picks
- *   around 128 slots per expert, where a 128-token block would spill into a second pass over the
- *   expert's weights; cache3 then also receives the first GEMM's output [M*top_k, 2I])
+ *   or 160 (int8 weights in the load-time layout: 160-token blocks of the direct-to-LDS kernel - what
+ *   the table picks around 128 slots per expert, where a 128-token block would spill into a second
+ *   pass over the expert's weights; with fp16 rows or GELU the first GEMM is not fused with the
+ *   activation, cache3 also receives its output [M*top_k, 2I], and 2I <= H is required)
  */
 int64_t lo_fused_experts_workspace_bytes(int64_t M, int32_t top_k, int64_t H, int64_t I,
                                          int32_t num_experts, int32_t block_size_m);
