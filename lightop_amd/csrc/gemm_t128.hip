@@ -97,19 +97,37 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 
   int mb, nt;
   if (!tile_of(blockIdx.x, a.n_tiles, m_blocks, group_m, mb, nt)) return;
-  if (static_cast<int64_t>(mb) * T >= a.ntpp[0]) return;
-  // An expert_map entry outside the weight tensor is treated like an expert of another rank, but its
-  // rows are always zero-filled: the slot mask of the alignment counts such a slot as local.
-  const int e_raw = a.expert_ids[mb];
-  const bool e_oob = e_raw >= a.E;
-  const int e = e_oob ? -1 : e_raw;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // which 64 weight rows of the tile
   const int r = lane & 15, q = lane >> 4;
+  const int32_t *const sorted = a.sorted + static_cast<int64_t>(mb) * T;
+  // Everything the tile's start-up reads from memory by its block index alone is requested here, in one go:
+  // the number of blocks in use, the block's expert and the sorted ids this thread needs (token rows it
+  // copies, the last valid token, the token whose scales it carries).  Asked for one after the other, each
+  // behind the branch on the one before, they were three round trips in front of the first operand copy.
+  // (Not for the fused 160-token form: the values alive across the branches cost it registers it does not have.)
+  constexpr bool kEarlyIds = !(FUSED_ACT && NTB == 10);
+  const int32_t blocks_end = a.ntpp[0];
+  const int e_raw = a.expert_ids[mb];
+  int32_t lf_copy[APW];
+  int32_t lf_v0 = 0, lf_v1 = 0, lf_v2 = 0, lf_scale = 0;
+  auto load_ids = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < APW; ++j) lf_copy[j] = sorted[(wave * APW + j) * 8 + (lane >> 3)];
+    lf_v0 = sorted[lane];
+    lf_v1 = sorted[lane + 64];
+    if constexpr (NTB == 10) lf_v2 = sorted[128 + (lane & 31)];
+    lf_scale = sorted[NTB == 8 ? (tid & (T - 1)) : (tid < T ? tid : tid - T)];
+  };
+  if constexpr (kEarlyIds) load_ids();
+  if (static_cast<int64_t>(mb) * T >= blocks_end) return;
+  // An expert_map entry outside the weight tensor is treated like an expert of another rank, but its
+  // rows are always zero-filled: the slot mask of the alignment counts such a slot as local.
+  const bool e_oob = e_raw >= a.E;
+  const int e = e_oob ? -1 : e_raw;
   const int64_t K = a.K, N = a.N;
   const int KB = static_cast<int>(K / kGroup);
   const int64_t I = N / 2;
-  const int32_t *const sorted = a.sorted + static_cast<int64_t>(mb) * T;
 
   // first row of the wave's 64 (plain) or of its 32 gate rows (fused)
   const int64_t nrow0 = FUSED_ACT ? static_cast<int64_t>(nt) * kGroup + wave * 32
@@ -188,7 +206,7 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
 #pragma unroll
   for (int j = 0; j < APW; ++j) {
     const int t = (wave * APW + j) * 8 + (lane >> 3);
-    const int64_t lf = sorted[t];
+    const int64_t lf = kEarlyIds ? lf_copy[j] : sorted[t];
     const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
     const int piece = (lane & 7) ^ (t & 7); // slot lane & 7 of row t holds piece slot ^ (t & 7)
     avoff[j] = static_cast<int>(lrow * K) + piece * 16;
@@ -199,18 +217,23 @@ void moe_gemm_t128_kernel(const GemmArgs a, int m_blocks, int group_m) {
   // a caller's own sorted ids with gaps are still computed in full).
   int nst; // pipeline stages per K block: four per 32 tokens in use
   {
-    const uint64_t v0 = __builtin_amdgcn_ballot_w64(sorted[lane] < a.num_valid);
-    const uint64_t v1 = __builtin_amdgcn_ballot_w64(sorted[lane + 64] < a.num_valid);
+    if constexpr (!kEarlyIds) {
+      lf_v0 = sorted[lane];
+      lf_v1 = sorted[lane + 64];
+      if constexpr (NTB == 10) lf_v2 = sorted[128 + (lane & 31)];
+    }
+    const uint64_t v0 = __builtin_amdgcn_ballot_w64(lf_v0 < a.num_valid);
+    const uint64_t v1 = __builtin_amdgcn_ballot_w64(lf_v1 < a.num_valid);
     int last = v1 ? 127 - __builtin_clzll(v1) : (v0 ? 63 - __builtin_clzll(v0) : 0);
     if constexpr (NTB == 10) {
-      const uint64_t v2 = __builtin_amdgcn_ballot_w64(lane < 32 && sorted[128 + (lane & 31)] < a.num_valid);
+      const uint64_t v2 = __builtin_amdgcn_ballot_w64(lane < 32 && lf_v2 < a.num_valid);
       if (v2) last = 191 - __builtin_clzll(v2);
     }
     nst = __builtin_amdgcn_readfirstlane(4 * ((last >> 5) + 1)); // the K loop comes in variants of 2, 4, 6, 8 (, 10) fragments
   }
   int asoff; // thread t and thread t + T both carry the scale of token t
   {
-    const int64_t lf = sorted[NTB == 8 ? (tid & (T - 1)) : (tid < T ? tid : tid - T)];
+    const int64_t lf = kEarlyIds ? lf_scale : sorted[NTB == 8 ? (tid & (T - 1)) : (tid < T ? tid : tid - T)];
     const int64_t lrow = (lf < a.num_valid) ? lf / a.top_k : 0;
     asoff = static_cast<int>(lrow * (PC ? 1 : KB) * 4);
     // The epilogues take the ids from LDS: a global load in each of their exec-masked blocks is a
