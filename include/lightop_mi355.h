@@ -200,7 +200,9 @@ int lo_per_token_group_quant_int8(const void *x, int x_dtype, int64_t rows, int6
  *   sorted_ids / expert_ids / num_tokens_post_pad as produced by lo_moe_align_block_size
  *   with block_size == block_size_m (16, 32, 64 or 128; also 160 with int8 weights in the load-time
  *   layout, N % 64 == 0 and K <= 16384); sorted_cap is the extent of sorted_ids
- *   (any extent >= the alignment's own works, e.g. one rounded up by the caller).
+ *   (any extent >= the alignment's own works, e.g. one rounded up by the caller), and expert_ids
+ *   holds at least sorted_cap / block_size_m entries: a kernel may read the entry and the sorted ids of
+ *   any block below that bound before it knows num_tokens_post_pad (it uses them only for blocks in use).
  *   E: experts held by W.  num_experts: experts the routing spreads the slots over (the
  *   num_experts given to the alignment; 0 = E).  It only steers scheduling choices (tile order,
  *   cache hints), never the result.

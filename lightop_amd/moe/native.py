@@ -154,6 +154,16 @@ def _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num
     return E, N, K
 
 
+def _check_block_extents(sorted_token_ids, expert_ids, block_size_m, num_valid):
+    """``expert_ids`` must cover every token block the launch's grid can reach (the blocks ``sorted_token_ids``
+    has room for, at most one per routed slot): a kernel may read a block's entry before it knows how many
+    blocks are in use."""
+    blocks = min(sorted_token_ids.numel() // int(block_size_m), int(num_valid))
+    if expert_ids.numel() < blocks:
+        raise ValueError(f"expert_ids holds {expert_ids.numel()} entries, the {sorted_token_ids.numel()} sorted ids "
+                         f"span {blocks} blocks of {int(block_size_m)}")
+
+
 def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
                                  A_scale: torch.Tensor, B_scale: torch.Tensor,
                                  topk_weights: Optional[torch.Tensor],
@@ -171,6 +181,7 @@ def invoke_fused_moe_kernel_int8(A: torch.Tensor, B: torch.Tensor, C: torch.Tens
                                  w4=bool(flags & _lib.LO_GEMM_W4))
     assert C.is_contiguous() and C.shape[-1] == N
     num_valid = C.numel() // N
+    _check_block_extents(sorted_token_ids, expert_ids, config["BLOCK_SIZE_M"], num_valid)
     tw = None
     if topk_weights is not None:
         tw = topk_weights
@@ -201,6 +212,7 @@ def invoke_fused_moe_gemm1_silu_quant(A: torch.Tensor, B: torch.Tensor, A_scale:
     E, N, K = _check_gemm_inputs(A, A_scale, B, B_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
                                  w4=bool(flags & _lib.LO_GEMM_W4))
     I = N // 2
+    _check_block_extents(sorted_token_ids, expert_ids, config["BLOCK_SIZE_M"], num_valid)
     a2q = torch.empty(num_valid, I, dtype=torch.int8, device=A.device)
     a2s = torch.empty(num_valid, I // 128, dtype=torch.float32, device=A.device)
     tw = None
@@ -248,6 +260,7 @@ def invoke_fused_moe_kernel_w4a8(A: torch.Tensor, B: torch.Tensor, C: torch.Tens
     assert sorted_token_ids.dtype == torch.int32 and expert_ids.dtype == torch.int32
     assert topk_weights is not None or not mul_routed_weight
     num_valid = C.numel() // N
+    _check_block_extents(sorted_token_ids, expert_ids, config["BLOCK_SIZE_M"], num_valid)
     tw = None
     if mul_routed_weight:
         tw = topk_weights if topk_weights.dtype == torch.float32 and topk_weights.is_contiguous() \

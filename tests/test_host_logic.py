@@ -402,3 +402,18 @@ def test_tuning_files_override_the_compiled_table(monkeypatch, tmp_path):
     assert tile_files.file_name(8, 1024, 1024, 512, 2, None, True).startswith("MOE_W4A8INT8_E=8_")
     monkeypatch.delenv("TRITON_JSON_DIR")
     tile_files.forget()
+
+
+def test_expert_ids_must_cover_the_blocks_the_grid_reaches():
+    """The GEMM stubs refuse an expert_ids tensor shorter than the token blocks sorted_token_ids has room for
+    (the kernels may read any such block's entry before they know how many blocks are in use)."""
+    import pytest
+    import torch
+
+    from lightop_amd.moe.native import _check_block_extents
+
+    sorted_ids = torch.zeros(128 * 7 + 5, dtype=torch.int32)
+    _check_block_extents(sorted_ids, torch.zeros(7, dtype=torch.int32), 128, 10_000)   # 7 whole blocks
+    _check_block_extents(sorted_ids, torch.zeros(3, dtype=torch.int32), 128, 3)        # at most one block per slot
+    with pytest.raises(ValueError, match="span 7 blocks"):
+        _check_block_extents(sorted_ids, torch.zeros(6, dtype=torch.int32), 128, 10_000)
