@@ -105,9 +105,9 @@ def main(argv=None):
 
     rows, table = [], {}
     print(f"{layer.name}: E={layer.E}/{layer.E_global} top{layer.top_k} H={layer.H} I={layer.I}")
-    # 160-token blocks exist for the block form with int8 weights where the first GEMM's output fits [S, H],
+    # 160-token blocks exist for the block form with int8 weights (bf16 rows with SiLU keep the fused first stage)
     # and for per-channel scales
-    has160 = (layer.weight_bits == 8 and block_shape is not None and 2 * layer.I <= layer.H) or block_shape is None
+    has160 = (layer.weight_bits == 8 and block_shape is not None) or block_shape is None
     sizes = BLOCK_SIZES + ((160,) if has160 else ())
     print(f"{'tokens':>7} {'slots/expert':>12} | " + " ".join(f"bs={b:<4}" for b in sizes) + " | best  table  loss")
     for M in (int(v) for v in args.tokens.split(",")):
