@@ -61,3 +61,10 @@ def per_token_quant_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 
 __all__ = ["per_token_group_quant_int8", "per_token_quant_int8"]
+
+# ``quant.int8`` (python/lightop/quant/int8.py in the reference) is this module: the attribute makes
+# ``import lightop.quant.int8 as q`` and ``from lightop_amd.quant import int8`` resolve as well.
+import sys as _sys  # noqa: E402
+
+int8 = _sys.modules[__name__]
+_sys.modules.setdefault(__name__ + ".int8", int8)

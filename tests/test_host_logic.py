@@ -355,6 +355,11 @@ def test_lightop_is_an_importable_name():
         lightop.RMSNorm
     with pytest.raises(AttributeError):
         lightop.moe.fused_experts_impl_fp8_marlin
+    import lightop.quant.int8 as q8  # the attribute form of the dotted import
+    import lightop_amd.quant as q
+
+    assert q8 is q and q.int8 is q
+
 
 
 def test_tuning_files_override_the_compiled_table(monkeypatch, tmp_path):
