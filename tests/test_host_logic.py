@@ -361,7 +361,6 @@ def test_lightop_is_an_importable_name():
     assert q8 is q and q.int8 is q
 
 
-
 def test_tuning_files_override_the_compiled_table(monkeypatch, tmp_path):
     """TRITON_JSON_DIR (vllm_compat/w8a8_get_cache_json.py:24) names a directory of tuning files in the
     reference's layout; the block size such a file holds for the nearest tuned token count comes back from
