@@ -3,12 +3,12 @@
 Three kinds of checks:
   * size-independent properties of the routing alignment and the group quantisation;
   * two independent implementations (LDS-tiled and weight-streaming kernels, row-major
-    and pre-shuffled weights) must agree bit for bit in canonical order;
+    and pre-shuffled weights) must agree bit for bit in both bit-exact scale orders;
   * tokens of a MoE layer are independent, so a random sample of tokens is pushed through
     the CPU oracle with only the experts those tokens use, and the sampled output rows, int8
     activations and scales of the full-size GPU run must equal the oracle's bit for bit in the
-    library's default (canonical) order, or lie within the tolerance of the oracle in the optional
-    fused-scale order.
+    library's default (contracted) order and in the order without fp fusion, or lie within the tolerance of
+    the oracle in the optional fused-scale order.
 """
 import sys
 

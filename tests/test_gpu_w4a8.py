@@ -1,5 +1,5 @@
 """GPU parity of the W4A8 (packed int4 weights, K-group scales) path, through the C ABI, bit for
-bit against the oracle in canonical order; the benchmark's int4 configuration (Qwen3-235B-A22B-shaped
+bit against the oracle in both bit-exact scale orders; the benchmark's int4 configuration (Qwen3-235B-A22B-shaped
 layer, M in {1, 32, 256, 2048}) on sampled tokens."""
 import pytest
 import torch
